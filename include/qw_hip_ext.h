@@ -1,0 +1,48 @@
+/* Additions of the HIP backend that the reference's src/gpu.h has no counterpart for. None of them is needed by
+ * the reference's callers; they exist because HBM is not host memory, and for measurement.
+ *
+ * Host shadow rules (qw_buf.ptr is host memory, the kernels read HBM):
+ *   - host -> device, when a batch is submitted, for every buffer a dispatch of the batch binds:
+ *       a buffer of at most QW_HIP_SMALL_BYTES is copied every time;
+ *       a larger one is copied the first time it is bound and again only after qw_hip_buf_mark_dirty();
+ *       qw_buf_wrap() buffers are copied once; device-only buffers never.
+ *   - device -> host, when the batch completes, for every buffer bound in an output role:
+ *       always, unless the buffer is device-only or larger than QW_HIP_BIG_OUT_BYTES (then: qw_hip_buf_download()).
+ */
+#pragma once
+#include "gpu.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QW_HIP_SMALL_BYTES ((size_t)4 << 20)
+#define QW_HIP_BIG_OUT_BYTES ((size_t)256 << 20)
+
+/* Device memory without a host shadow (out->ptr = NULL). Zero-filled. For resident weights and scratch that the
+ * host never looks at. */
+bool qw_hip_buf_new_device(qw_gpu *g, size_t size, qw_buf *out);
+/* The host changed a large buffer after its first use: copy it again at the next submit. */
+void qw_hip_buf_mark_dirty(qw_buf *b);
+/* Explicit copies (synchronous). upload/download move [offset, offset + len) between the shadow and HBM;
+ * write/read move between caller memory and HBM (the only way to fill or inspect a device-only buffer). */
+bool qw_hip_buf_upload(qw_buf *b, size_t offset, size_t len);
+bool qw_hip_buf_download(qw_buf *b, size_t offset, size_t len);
+bool qw_hip_buf_write(qw_buf *b, size_t offset, const void *src, size_t len);
+bool qw_hip_buf_read(const qw_buf *b, size_t offset, void *dst, size_t len);
+/* Device address of a buffer (for tools that pass it to their own code). */
+void *qw_hip_buf_devptr(const qw_buf *b);
+
+/* Last error text of this device (empty string if none); cleared by qw_batch_begin. */
+const char *qw_hip_last_error(const qw_gpu *g);
+/* Number of compute units and the name of the code-object architecture the library was built for. */
+int qw_hip_cu_count(const qw_gpu *g);
+const char *qw_hip_arch(void);
+
+/* Average duration in seconds of the kernel whose entry-point name starts with `prefix`, over the dispatches of
+ * the last completed batch that ran with profiling enabled; count receives how many matched. */
+double qw_hip_profile_mean(const qw_gpu *g, const char *prefix, int *count);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,64 @@
+/* Host side of the quantized decode path, above the GPU interface of gpu.h.
+ *
+ * These functions restate, against gpu.h only, what the reference's engine does for this path: build the kernel
+ * name and the "#define" block, compile on a miss, bind by index, dispatch. They mirror
+ *     qmv_gg()      src/engine.c:689-724      qw_path_qmv_gg()
+ *     gg_router()   src/engine.c:544-552      qw_path_gg_router()
+ *     gg_kernel()   src/engine.c:460-517      (internal)
+ *     gg_moe()      src/engine.c:568-647      qw_path_gg_moe()
+ * with the same binding indices, macro names and dispatch order, so that a parity test written against them
+ * exercises exactly the call sequence engine.c would issue. The one extension is a token count above 8 (up to 16),
+ * which the reference splits into two passes (src/engine.c:8783-8814).
+ *
+ * Failure: where the reference prints and calls exit(1) (src/engine.c:508-514), these return false after printing
+ * the same kind of message to stderr; the batch must then be abandoned with qw_batch_end().
+ */
+#pragma once
+#include "gpu.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A quantized matrix in HBM: rows x cols values of one ggml type, rows contiguous (src/model.h:64-66). */
+typedef struct {
+    const qw_buf *buf;
+    size_t offset;
+    int type; /* ggml type: 8 = Q8_0, 21 = IQ3_S; router: 1 = F16, 30 = BF16 */
+} qw_tensor;
+
+/* One MoE layer's weights (the fields of the reference's qw_moe that this path reads, src/model.h). */
+typedef struct {
+    qw_tensor router;    /* [E][D], F16 or BF16 */
+    qw_tensor sh_gate_w; /* [D] shared-expert gate vector, same type as router */
+    qw_tensor gate, up;  /* routed, [E][I][D-row]; same type */
+    qw_tensor down;      /* routed, [E][D][I-row] */
+    qw_tensor sh_gate, sh_up, sh_down; /* shared expert */
+} qw_moe_layer;
+
+typedef struct qw_path qw_path;
+
+/* Scratch buffers (lookup tables, H, Psh, Pg, counter) for layers of this shape and up to nbmax <= 16 tokens.
+ * device_scratch: keep the intermediates in HBM only (no host shadow), as a serving loop would. */
+qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool device_scratch);
+void qw_path_close(qw_path *p);
+/* Bytes the caller must give the selection record and the logits for nb tokens. */
+size_t qw_path_sel_bytes(const qw_path *p, int nb);
+size_t qw_path_logits_bytes(const qw_path *p, int nb);
+/* Token count a kernel is built for when nb tokens are asked (1, 2, 4, 8, 16; src/engine.c:447 stops at 8). */
+int qw_path_nbv(int nb);
+
+/* y[b][0..N) = W x[b], b < nb; x stride K, y stride N; fout selects float (else binary16) output. */
+bool qw_path_qmv_gg(qw_path *p, qw_batch *b, const qw_tensor *W, int N, int K, const qw_buf *x, size_t xoff, const qw_buf *y,
+                    size_t yoff, int nb, bool fout);
+/* logits[nb][E + 1] alone. */
+bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg);
+/* The whole layer: x [nb][D] binary16 -> out [nb][D] binary16; lg and sel receive the logits and the selection. */
+bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
+                    const qw_buf *out);
+/* The scratch buffers, for tests: 0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg. */
+const qw_buf *qw_path_scratch(const qw_path *p, int which);
+
+#ifdef __cplusplus
+}
+#endif

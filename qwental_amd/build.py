@@ -1,0 +1,51 @@
+"""Build recipe of the HIP backend: kernels -> gfx950 code object -> embedded into libqwgpu_hip.so.
+
+    python -m qwental_amd.build
+
+Two steps, both cross-compile without a GPU:
+  1. hipcc --genco: csrc/kernels/qw_kernels.hip -> csrc/qw_kernels_gfx950.hsaco
+  2. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c -> qwental_amd/libqwgpu_hip.so
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.path.join(ROCM, "bin", "hipcc")
+CLANG = os.path.join(ROCM, "llvm", "bin", "clang")
+LIB = os.path.join(HERE, "libqwgpu_hip.so")
+HSACO = os.path.join(CSRC, "qw_kernels_gfx950.hsaco")
+# -packed-fp32-ops: packed FP32 instructions are kept out of every kernel of this library
+HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode:
+        sys.stderr.write(out + "\n")
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+    return out
+
+
+def build(verbose=False):
+    out = _run([HIPCC] + HIPFLAGS + ["--genco", "-I", os.path.join(CSRC, "kernels"), "-o", HSACO,
+                                    os.path.join(CSRC, "kernels", "qw_kernels.hip")])
+    if verbose and out.strip():
+        print(out)
+    out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+                "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), "-o", LIB,
+                "-L", os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    if verbose and out.strip():
+        print(out)
+    # command-line tool with the reference's dqtest contract
+    _run([CLANG, "-std=c23", "-O2", "-Wall", "-I", os.path.join(ROOT, "include"), os.path.join(CSRC, "tools", "dqhip.c"), "-o",
+          os.path.join(HERE, "dqhip"), "-L", HERE, "-lqwgpu_hip", "-Wl,-rpath," + HERE, "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,836 @@
+// HIP implementation of the GPU interface in include/gpu.h (the reference's src/gpu.h, implemented there by
+// src/gpu_metal.m). C23 over the HIP runtime's C API; the gfx950 code object built from kernels/qw_kernels.hip is
+// embedded below and loaded with hipModuleLoadData. No kernel is compiled at run time.
+//
+// What a dispatch means here: callers record dispatches in Metal terms (kernel by name, sticky bindings by index,
+// grid in threadgroups of 32-wide SIMD groups). Each kernel name was registered by qw_gpu_compile() from the
+// caller's "#define" block, which names a kernel family and its parameters. At qw_batch_dispatch() the family's
+// translator reads the bindings, checks every size, and records one or more HIP launches with this backend's own
+// wave64 geometry. A translation that fails a check marks the batch failed; nothing of a failed batch is launched.
+#define _GNU_SOURCE
+#define __HIP_PLATFORM_AMD__ 1
+#include "gpu.h"
+#include "qw_hip_ext.h"
+#include "kernels/qw_kargs.h"
+#include <hip/hip_runtime_api.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#include <unistd.h>
+
+static const unsigned char qw_code_object[] = {
+#embed "qw_kernels_gfx950.hsaco"
+};
+
+enum { QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 2048, QW_MAX_FUNCS = 96 };
+
+// ---------------------------------------------------------------- records
+typedef enum {
+    FAM_DQ_TEST, FAM_QMV_GG, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
+    FAM_BW_READ, FAM_COPY, FAM_FILL,
+} qw_family;
+
+typedef struct { // parameters taken from the define block
+    int F, K, RB, NB, yfloat;            // dq_test / qmv_gg
+    int E, topk, D, I, gnb;              // MoE
+    int fgu, fd, fsg, fsu, fsd, rbf, rwf; // formats; rbf: router inside moe_pre_gg; rwf: router weight type (1 / 30)
+} qw_kparams;
+
+struct qw_kernel {
+    char name[128];
+    qw_family fam;
+    qw_kparams p;
+};
+
+typedef struct qw_hbuf {
+    void *dptr;
+    void *host;      // shadow (NULL for device-only)
+    size_t size;
+    bool own_host;   // shadow allocated here (hipHostMalloc or calloc)
+    bool pinned;
+    bool wrapped, device_only;
+    bool dirty;      // host copy is newer than HBM (or HBM never received it)
+    unsigned mark;   // scratch for de-duplication while a batch is submitted
+} qw_hbuf;
+
+typedef struct {
+    hipFunction_t f;
+    const char *fname;
+    unsigned gx, gy, gz, bx;
+    unsigned char args[128];
+    size_t argsz;
+    const char *kname; // caller-visible kernel name (for profiling)
+    bool last_of_dispatch;
+} qw_launch;
+
+typedef struct { qw_hbuf *b; bool out; } qw_use;
+
+struct qw_batch {
+    qw_gpu *g;
+    int stream;
+    bool failed, submitted, prof;
+    struct qw_kernel *k;
+    struct { const qw_buf *buf; qw_hbuf *h; size_t off; } buf[QW_MAX_BIND];
+    unsigned char bytes[QW_MAX_BIND][QW_MAX_BYTES];
+    size_t blen[QW_MAX_BIND];
+    qw_launch *l;
+    int nl, capl, done_l; // done_l: launches already submitted by a flush
+    qw_use *use;
+    int nuse, capuse, done_use;
+    hipEvent_t ev[2 * 9]; // start/stop per submitted segment (end + at most 8 flushes)
+    int nseg;
+    hipEvent_t *pev;      // profiling: 2 events per dispatch
+    int npev;
+};
+
+struct qw_gpu {
+    int dev;
+    char name[256];
+    size_t total_mem;
+    int ncu;
+    hipModule_t mod;
+    hipStream_t stream[2];
+    int cur_stream;
+    struct qw_kernel *kernels;
+    int nkernels;
+    struct { char name[48]; hipFunction_t f; } funcs[QW_MAX_FUNCS];
+    int nfuncs;
+    char err[1024];
+    bool prof;
+    int nprof;
+    const char *prof_name[QW_PROF_MAX];
+    const char *prof_fname[QW_PROF_MAX];
+    double prof_us[QW_PROF_MAX];
+    unsigned mark;
+};
+
+static void set_err(qw_gpu *g, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g->err, sizeof g->err, fmt, ap);
+    va_end(ap);
+    if (getenv("QW_HIP_VERBOSE")) fprintf(stderr, "[qw_hip] %s\n", g->err);
+}
+#define HIPOK(g, call) (hip_ok((g), (call), #call))
+static bool hip_ok(qw_gpu *g, hipError_t e, const char *what) {
+    if (e == hipSuccess) return true;
+    set_err(g, "%s: %s", what, hipGetErrorString(e));
+    return false;
+}
+
+double qw_now(void) {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec + (double)ts.tv_nsec * 1e-9;
+}
+
+// ---------------------------------------------------------------- device
+qw_gpu *qw_gpu_open(void) {
+    int n = 0;
+    if (hipInit(0) != hipSuccess || hipGetDeviceCount(&n) != hipSuccess || n < 1) return NULL;
+    qw_gpu *g = calloc(1, sizeof *g);
+    if (!g) return NULL;
+    hipDeviceProp_t pr;
+    if (hipSetDevice(0) != hipSuccess || hipGetDeviceProperties(&pr, 0) != hipSuccess) { free(g); return NULL; }
+    snprintf(g->name, sizeof g->name, "%s (%s)", pr.name, pr.gcnArchName);
+    g->total_mem = pr.totalGlobalMem;
+    g->ncu = pr.multiProcessorCount;
+    if (strncmp(pr.gcnArchName, "gfx950", 6) != 0) {
+        fprintf(stderr, "qw_gpu_open: device is %s; this library holds gfx950 code only\n", pr.gcnArchName);
+        free(g);
+        return NULL;
+    }
+    if (hipModuleLoadData(&g->mod, qw_code_object) != hipSuccess) {
+        fprintf(stderr, "qw_gpu_open: the embedded gfx950 code object does not load\n");
+        free(g);
+        return NULL;
+    }
+    for (int i = 0; i < 2; i++)
+        if (hipStreamCreateWithFlags(&g->stream[i], hipStreamNonBlocking) != hipSuccess) { free(g); return NULL; }
+    g->kernels = calloc(QW_MAX_KERNELS, sizeof *g->kernels);
+    return g;
+}
+
+void qw_gpu_close(qw_gpu *g) {
+    if (!g) return;
+    (void)hipDeviceSynchronize();
+    for (int i = 0; i < 2; i++) (void)hipStreamDestroy(g->stream[i]);
+    (void)hipModuleUnload(g->mod);
+    free(g->kernels);
+    free(g);
+}
+
+const char *qw_gpu_name(const qw_gpu *g) { return g->name; }
+size_t qw_gpu_max_working_set(const qw_gpu *g) { return g->total_mem; }
+const char *qw_hip_last_error(const qw_gpu *g) { return g->err; }
+int qw_hip_cu_count(const qw_gpu *g) { return g->ncu; }
+const char *qw_hip_arch(void) { return "gfx950"; }
+
+static hipFunction_t get_func(qw_gpu *g, const char *fname) {
+    for (int i = 0; i < g->nfuncs; i++)
+        if (!strcmp(g->funcs[i].name, fname)) return g->funcs[i].f;
+    if (g->nfuncs >= QW_MAX_FUNCS) return NULL;
+    hipFunction_t f;
+    if (!HIPOK(g, hipModuleGetFunction(&f, g->mod, fname))) return NULL;
+    snprintf(g->funcs[g->nfuncs].name, sizeof g->funcs[0].name, "%s", fname);
+    g->funcs[g->nfuncs].f = f;
+    return g->funcs[g->nfuncs++].f;
+}
+
+// ---------------------------------------------------------------- define block -> kernels
+// The block is the run of "#define NAME VALUE" lines at the start of the source (src/engine.c:478-507, :709-710,
+// tools/dqtest.c:27). Later definitions of a name win, as in the preprocessor.
+typedef struct { char name[48], val[80]; } qw_def;
+
+static int parse_defs(const char *src, size_t len, qw_def *d, int max) {
+    int n = 0;
+    size_t i = 0;
+    while (i < len) {
+        while (i < len && (src[i] == ' ' || src[i] == '\t' || src[i] == '\r' || src[i] == '\n')) i++;
+        if (i + 7 >= len || strncmp(src + i, "#define", 7) != 0) break;
+        i += 7;
+        while (i < len && (src[i] == ' ' || src[i] == '\t')) i++;
+        size_t a = i;
+        while (i < len && src[i] != ' ' && src[i] != '\t' && src[i] != '\n' && src[i] != '\r') i++;
+        size_t nl = i - a;
+        while (i < len && (src[i] == ' ' || src[i] == '\t')) i++;
+        size_t b = i;
+        while (i < len && src[i] != '\n' && src[i] != '\r') i++;
+        size_t vl = i - b;
+        while (vl && (src[b + vl - 1] == ' ' || src[b + vl - 1] == '\t')) vl--;
+        if (n < max && nl && nl < sizeof d->name && vl < sizeof d->val) {
+            memcpy(d[n].name, src + a, nl); d[n].name[nl] = 0;
+            memcpy(d[n].val, src + b, vl); d[n].val[vl] = 0;
+            n++;
+        }
+    }
+    return n;
+}
+static const char *def_get(const qw_def *d, int n, const char *name) {
+    for (int i = n - 1; i >= 0; i--)
+        if (!strcmp(d[i].name, name)) return d[i].val;
+    return NULL;
+}
+static bool def_int(const qw_def *d, int n, const char *name, int *out) {
+    const char *v = def_get(d, n, name);
+    if (!v || !*v) return false;
+    char *end;
+    long x = strtol(v, &end, 0);
+    if (*end) return false;
+    *out = (int)x;
+    return true;
+}
+
+static bool fmt_ok(int f) { return f == 8 || f == 21; }
+static int fmt_qb(int f) { return f == 8 ? 32 : 256; }
+static int fmt_bb(int f) { return f == 8 ? 34 : 110; }
+static size_t fmt_rb(int f, int K) { return (size_t)(K / fmt_qb(f)) * (size_t)fmt_bb(f); }
+
+static bool reg_kernel(qw_gpu *g, const qw_def *d, int n, const char *base, qw_family fam, const qw_kparams *p, char *err, size_t errlen) {
+    const char *nm = def_get(d, n, base); // "#define base newname" renames the kernel (src/engine.c:149)
+    if (!nm || !*nm) nm = base;
+    for (int i = 0; i < g->nkernels; i++)
+        if (!strcmp(g->kernels[i].name, nm)) { g->kernels[i].fam = fam; g->kernels[i].p = *p; return true; }
+    if (g->nkernels >= QW_MAX_KERNELS) { snprintf(err, errlen, "too many kernels"); return false; }
+    struct qw_kernel *k = &g->kernels[g->nkernels++];
+    snprintf(k->name, sizeof k->name, "%s", nm);
+    k->fam = fam;
+    k->p = *p;
+    return true;
+}
+
+bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t errlen) {
+    char dummy[8];
+    if (!err || !errlen) { err = dummy; errlen = sizeof dummy; }
+    err[0] = 0;
+    qw_def *d = calloc(128, sizeof *d);
+    const int n = parse_defs(src, len, d, 128);
+    qw_kparams p = {0};
+    int v;
+    bool ok = true;
+#define FAIL(...) do { snprintf(err, errlen, __VA_ARGS__); ok = false; goto out; } while (0)
+    if (def_int(d, n, "DQ_TEST", &v)) { // tools/dqtest.c:27
+        if (!fmt_ok(v)) FAIL("dq_test: ggml type %d has no gfx950 build (have 8, 21)", v);
+        p.F = v;
+        if (!reg_kernel(g, d, n, "dq_test", FAM_DQ_TEST, &p, err, errlen)) { ok = false; goto out; }
+    }
+    if (def_get(d, n, "GF") && def_get(d, n, "KD")) { // src/engine.c:709-710
+        if (!def_int(d, n, "GF", &p.F) || !def_int(d, n, "KD", &p.K) || !def_int(d, n, "RB", &p.RB) || !def_int(d, n, "NB", &p.NB))
+            FAIL("qmv_gg: GF, KD, RB and NB must be integer macros");
+        if (!fmt_ok(p.F)) FAIL("qmv_gg: ggml type %d has no gfx950 build (have 8, 21)", p.F);
+        if (p.K <= 0 || p.K % fmt_qb(p.F) || (size_t)p.RB != fmt_rb(p.F, p.K)) FAIL("qmv_gg: K %d / row bytes %d do not fit type %d", p.K, p.RB, p.F);
+        if (p.NB < 1 || p.NB > 16) FAIL("qmv_gg: NB %d outside 1..16", p.NB);
+        const char *yt = def_get(d, n, "YT");
+        p.yfloat = yt && !strcmp(yt, "float");
+        if (yt && strcmp(yt, "float") && strcmp(yt, "half")) FAIL("qmv_gg: YT %s is neither half nor float", yt);
+        if (!reg_kernel(g, d, n, "qmv_gg", FAM_QMV_GG, &p, err, errlen)) { ok = false; goto out; }
+    }
+    const bool router = def_get(d, n, "GG_ROUTER") != NULL;
+    int part = -1;
+    if (router || def_int(d, n, "GG_PART", &part)) { // src/engine.c:478-507
+        p = (qw_kparams){0};
+        if (!def_int(d, n, "E", &p.E) || !def_int(d, n, "TOPK", &p.topk) || !def_int(d, n, "D", &p.D) || !def_int(d, n, "I", &p.I) || !def_int(d, n, "NB", &p.NB))
+            FAIL("moe_gg: E, TOPK, D, I and NB must be integer macros");
+        if (p.NB < 1 || p.NB > 16) FAIL("moe_gg: NB %d outside 1..16", p.NB);
+        if (p.E < 1 || p.E > 1024 || p.topk < 1 || p.topk > 16 || p.topk > p.E) FAIL("moe_gg: E %d / TOPK %d outside this build (E <= 1024, TOPK <= 16)", p.E, p.topk);
+        if (p.D % 256 || p.I % 256 || p.D > 2560 || p.D < 256 || p.I < 256) FAIL("moe_gg: D %d / I %d outside this build (multiples of 256, D <= 2560)", p.D, p.I);
+        p.gnb = p.NB <= 8 ? 8 : 16; // 8 = the reference's gg_sel layout; 16 = the wide layout
+        p.rwf = 30;
+        if (def_int(d, n, "RWF", &v)) { if (v != 1 && v != 30) FAIL("moe_gg: RWF %d (router weight type) must be 1 or 30", v); p.rwf = v; }
+        if (router) {
+            if (!reg_kernel(g, d, n, "moe_router_bf", FAM_ROUTER, &p, err, errlen)) { ok = false; goto out; }
+        } else if (part == 0) {
+            if (!reg_kernel(g, d, n, "gg_tab_init", FAM_TAB_INIT, &p, err, errlen) || !reg_kernel(g, d, n, "moe_sel_gg", FAM_SEL, &p, err, errlen)) { ok = false; goto out; }
+        } else if (part == 1) {
+            if (!def_int(d, n, "FSG", &p.fsg) || !def_int(d, n, "FSU", &p.fsu) || !def_int(d, n, "RBF", &p.rbf)) FAIL("moe_pre_gg: FSG, FSU, RBF missing");
+            if (!fmt_ok(p.fsg) || p.fsu != p.fsg) FAIL("moe_pre_gg: shared gate/up types %d/%d: this build needs equal types from {8, 21}", p.fsg, p.fsu);
+            if (!reg_kernel(g, d, n, "moe_pre_gg", FAM_PRE, &p, err, errlen)) { ok = false; goto out; }
+        } else if (part == 2) {
+            if (!def_int(d, n, "FGU", &p.fgu) || !def_int(d, n, "FSD", &p.fsd)) FAIL("moe_gu_gg: FGU, FSD missing");
+            if (!fmt_ok(p.fgu) || !fmt_ok(p.fsd)) FAIL("moe_gu_gg: types %d/%d have no gfx950 build (have 8, 21)", p.fgu, p.fsd);
+            if (!reg_kernel(g, d, n, "moe_gu_gg", FAM_GU, &p, err, errlen)) { ok = false; goto out; }
+        } else if (part == 3) {
+            if (!def_int(d, n, "FD", &p.fd)) FAIL("moe_dn_gg: FD missing");
+            if (!fmt_ok(p.fd)) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 21)", p.fd);
+            if (!reg_kernel(g, d, n, "moe_dn_gg", FAM_DN, &p, err, errlen) || !reg_kernel(g, d, n, "moe_cmb_gg", FAM_CMB, &p, err, errlen)) { ok = false; goto out; }
+        } else FAIL("moe_gg: GG_PART %d has no gfx950 build (have 0..3 and GG_ROUTER)", part);
+    }
+    if (def_get(d, n, "QW_HIP_MEM")) { // this backend's own measurement helpers
+        p = (qw_kparams){0};
+        if (!reg_kernel(g, d, n, "qw_bw_read", FAM_BW_READ, &p, err, errlen) || !reg_kernel(g, d, n, "qw_copy", FAM_COPY, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "qw_fill_random", FAM_FILL, &p, err, errlen)) { ok = false; goto out; }
+    }
+#undef FAIL
+out:
+    free(d);
+    return ok;
+}
+
+qw_kernel *qw_kernel_get(qw_gpu *g, const char *name) {
+    for (int i = 0; i < g->nkernels; i++)
+        if (!strcmp(g->kernels[i].name, name)) return &g->kernels[i];
+    return NULL;
+}
+unsigned qw_kernel_max_threads(const qw_kernel *k) { (void)k; return 1024; }
+unsigned qw_kernel_simd_width(const qw_kernel *k) { (void)k; return 64; }
+
+// ---------------------------------------------------------------- buffers
+static qw_hbuf *hbuf_new(qw_gpu *g, size_t size) {
+    qw_hbuf *h = calloc(1, sizeof *h);
+    if (!h) return NULL;
+    // the memset runs on the null stream; the batches run on non-blocking streams, so wait for it here
+    if (!HIPOK(g, hipMalloc(&h->dptr, size ? size : 1)) || !HIPOK(g, hipMemset(h->dptr, 0, size)) || !HIPOK(g, hipDeviceSynchronize())) { free(h); return NULL; }
+    h->size = size;
+    return h;
+}
+
+bool qw_buf_new(qw_gpu *g, size_t size, qw_buf *out) {
+    qw_hbuf *h = hbuf_new(g, size);
+    if (!h) return false;
+    if (size <= ((size_t)64 << 20) && hipHostMalloc(&h->host, size ? size : 1, hipHostMallocDefault) == hipSuccess) {
+        h->pinned = true;
+        memset(h->host, 0, size);
+    } else {
+        h->host = calloc(size ? size : 1, 1);
+        if (!h->host) { (void)hipFree(h->dptr); free(h); return false; }
+    }
+    h->own_host = true;
+    h->dirty = false; // both sides are zero
+    out->handle = h;
+    out->ptr = h->host;
+    out->size = size;
+    return true;
+}
+
+bool qw_hip_buf_new_device(qw_gpu *g, size_t size, qw_buf *out) {
+    qw_hbuf *h = hbuf_new(g, size);
+    if (!h) return false;
+    h->device_only = true;
+    out->handle = h;
+    out->ptr = NULL;
+    out->size = size;
+    return true;
+}
+
+bool qw_buf_wrap(qw_gpu *g, void *ptr, size_t len, qw_buf *out) {
+    const size_t page = (size_t)sysconf(_SC_PAGESIZE);
+    if ((uintptr_t)ptr % page) return false;
+    qw_hbuf *h = hbuf_new(g, len);
+    if (!h) return false;
+    h->host = ptr;
+    h->wrapped = true;
+    h->dirty = true; // copied to HBM at the first submit that binds it
+    out->handle = h;
+    out->ptr = ptr;
+    out->size = len;
+    return true;
+}
+
+void qw_buf_free(qw_buf *b) {
+    if (!b || !b->handle) return;
+    qw_hbuf *h = b->handle;
+    (void)hipFree(h->dptr);
+    if (h->own_host) {
+        if (h->pinned) (void)hipHostFree(h->host);
+        else free(h->host);
+    }
+    free(h);
+    b->handle = NULL;
+    b->ptr = NULL;
+    b->size = 0;
+}
+
+void *qw_pool_push(void) { return NULL; }
+void qw_pool_pop(void *pool) { (void)pool; }
+
+void qw_hip_buf_mark_dirty(qw_buf *b) { if (b && b->handle) ((qw_hbuf *)b->handle)->dirty = true; }
+void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle ? ((qw_hbuf *)b->handle)->dptr : NULL; }
+static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return off <= h->size && len <= h->size - off; }
+bool qw_hip_buf_upload(qw_buf *b, size_t off, size_t len) {
+    qw_hbuf *h = b ? b->handle : NULL;
+    return h && h->host && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, (char *)h->host + off, len, hipMemcpyHostToDevice) == hipSuccess;
+}
+bool qw_hip_buf_download(qw_buf *b, size_t off, size_t len) {
+    qw_hbuf *h = b ? b->handle : NULL;
+    return h && h->host && !h->wrapped && range_ok(h, off, len) && hipMemcpy((char *)h->host + off, (char *)h->dptr + off, len, hipMemcpyDeviceToHost) == hipSuccess;
+}
+bool qw_hip_buf_write(qw_buf *b, size_t off, const void *src, size_t len) {
+    qw_hbuf *h = b ? b->handle : NULL;
+    return h && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
+}
+bool qw_hip_buf_read(const qw_buf *b, size_t off, void *dst, size_t len) {
+    const qw_hbuf *h = b ? b->handle : NULL;
+    return h && range_ok(h, off, len) && hipMemcpy(dst, (const char *)h->dptr + off, len, hipMemcpyDeviceToHost) == hipSuccess;
+}
+
+// ---------------------------------------------------------------- batches: recording
+qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
+    (void)concurrent; // an in-order stream already gives the serial order; "concurrent" batches are serial too
+    qw_batch *b = calloc(1, sizeof *b);
+    if (!b) return NULL;
+    b->g = g;
+    b->stream = g->cur_stream;
+    b->prof = g->prof;
+    g->err[0] = 0;
+    return b;
+}
+
+void qw_batch_kernel(qw_batch *b, qw_kernel *k) {
+    b->k = k;
+    if (!k) { b->failed = true; set_err(b->g, "qw_batch_kernel: NULL kernel"); }
+}
+
+void qw_batch_buf(qw_batch *b, unsigned index, const qw_buf *buf, size_t offset) {
+    if (index >= QW_MAX_BIND) { b->failed = true; set_err(b->g, "binding index %u out of range", index); return; }
+    b->buf[index].buf = buf;
+    b->buf[index].h = buf ? buf->handle : NULL;
+    b->buf[index].off = offset;
+    b->blen[index] = 0;
+}
+
+void qw_batch_bytes(qw_batch *b, unsigned index, const void *data, size_t len) {
+    if (index >= QW_MAX_BIND || len > QW_MAX_BYTES) { b->failed = true; set_err(b->g, "inline bytes: index %u / length %zu out of range", index, len); return; }
+    memcpy(b->bytes[index], data, len);
+    b->blen[index] = len;
+    b->buf[index].h = NULL;
+}
+
+void qw_batch_threadgroup_mem(qw_batch *b, unsigned index, size_t len) { (void)b; (void)index; (void)len; } // LDS sizes are fixed per kernel here
+void qw_batch_barrier(qw_batch *b) { (void)b; }
+
+static bool fail(qw_batch *b, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(b->g->err, sizeof b->g->err, fmt, ap);
+    va_end(ap);
+    if (getenv("QW_HIP_VERBOSE")) fprintf(stderr, "[qw_hip] %s\n", b->g->err);
+    b->failed = true;
+    return false;
+}
+
+// Binding `index` as a device pointer with at least `need` bytes after its offset; records the use.
+static bool bind_ptr(qw_batch *b, unsigned index, size_t need, bool out, const char *what, void **p) {
+    qw_hbuf *h = b->buf[index].h;
+    if (!h) return fail(b, "%s: nothing bound at index %u (%s)", b->k->name, index, what);
+    const size_t off = b->buf[index].off;
+    if (off > h->size || need > h->size - off) return fail(b, "%s: %s at index %u needs %zu bytes after offset %zu, buffer has %zu", b->k->name, what, index, need, off, h->size);
+    if (out && h->wrapped) return fail(b, "%s: %s at index %u is a wrapped (read-only) buffer", b->k->name, what, index);
+    *p = (char *)h->dptr + off;
+    if (b->nuse == b->capuse) {
+        b->capuse = b->capuse ? 2 * b->capuse : 64;
+        b->use = realloc(b->use, sizeof *b->use * (size_t)b->capuse);
+    }
+    b->use[b->nuse++] = (qw_use){h, out};
+    return true;
+}
+static bool bind_bytes(qw_batch *b, unsigned index, void *dst, size_t len, const char *what) {
+    if (b->blen[index] < len) return fail(b, "%s: %s at index %u needs %zu inline bytes, has %zu", b->k->name, what, index, len, b->blen[index]);
+    memcpy(dst, b->bytes[index], len);
+    return true;
+}
+
+static bool add_launch(qw_batch *b, const char *fname, unsigned gx, unsigned bx, const void *args, size_t argsz) {
+    hipFunction_t f = get_func(b->g, fname);
+    if (!f) return fail(b, "%s: entry point %s missing from the code object", b->k->name, fname);
+    if (gx == 0) return true; // nothing to do
+    if (b->nl == b->capl) {
+        b->capl = b->capl ? 2 * b->capl : 64;
+        b->l = realloc(b->l, sizeof *b->l * (size_t)b->capl);
+    }
+    qw_launch *l = &b->l[b->nl++];
+    memset(l, 0, sizeof *l);
+    l->f = f;
+    l->fname = fname;
+    l->gx = gx; l->gy = 1; l->gz = 1; l->bx = bx;
+    memcpy(l->args, args, argsz);
+    l->argsz = argsz;
+    l->kname = b->k->name;
+    return true;
+}
+
+static unsigned umin(unsigned a, unsigned b) { return a < b ? a : b; }
+static unsigned cdiv(unsigned a, unsigned b) { return (a + b - 1) / b; }
+// Persistent grids: one 512-thread workgroup per compute unit (the LDS tables leave room for one), fewer if the
+// work is smaller. tasks are per-wave units; 8 waves per workgroup.
+static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks) { return umin((unsigned)g->ncu, cdiv(wave_tasks, 8)); }
+
+static const char *fname_fmt(char *buf, size_t n, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, n, fmt, ap);
+    va_end(ap);
+    return buf;
+}
+// entry-point names live as long as the process: intern them
+static const char *intern(const char *s) {
+    static char *tab[256];
+    static int n;
+    for (int i = 0; i < n; i++)
+        if (!strcmp(tab[i], s)) return tab[i];
+    if (n == 256) return "?";
+    return tab[n++] = strdup(s);
+}
+
+static int nb_variant(unsigned nb) { return nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : nb <= 8 ? 8 : 16; }
+
+// ---------------------------------------------------------------- family translators
+static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W, 1 y, 2 {K, row bytes}; grid = rows
+    const qw_kparams *p = &b->k->p;
+    uint32_t a2[2];
+    if (!bind_bytes(b, 2, a2, sizeof a2, "{K, rowbytes}")) return false;
+    if (a2[0] == 0 || a2[0] % (p->F == 21 ? 256 : 32) || a2[1] < fmt_rb(p->F, (int)a2[0])) return fail(b, "dq_test: K %u / row bytes %u do not fit type %d", a2[0], a2[1], p->F);
+    qwk_dq_args a = {.K = a2[0], .rowbytes = a2[1], .rows = gx};
+    if (!bind_ptr(b, 0, (size_t)gx * a2[1], false, "W", (void **)&a.W) || !bind_ptr(b, 1, (size_t)gx * a2[0] * 4, true, "y", (void **)&a.y)) return false;
+    return add_launch(b, p->F == 21 ? "qwk_dq_test_f21" : "qwk_dq_test_f8", gx, 64, &a, sizeof a);
+}
+
+static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
+    const qw_kparams *p = &b->k->p;
+    uint32_t a4[4];
+    if (!bind_bytes(b, 5, a4, sizeof a4, "{N, xstride, ystride, pad}")) return false;
+    qwk_qmv_args a = {.N = a4[0], .K = (uint32_t)p->K, .rowbytes = (uint32_t)p->RB, .xstride = a4[1], .ystride = a4[2], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat};
+    if (a.N == 0) return true;
+    if (a.xstride < a.K || a.xstride % 8 || a.ystride < a.N) return fail(b, "qmv_gg: xstride %u (needs >= K, multiple of 8) / ystride %u (needs >= N)", a.xstride, a.ystride);
+    if (b->buf[3].h && b->buf[3].off % 16) return fail(b, "qmv_gg: x offset %zu is not 16-byte aligned", b->buf[3].off);
+    a.ntiles = cdiv(a.N, 16);
+    if (!bind_ptr(b, 0, (size_t)a.N * a.rowbytes, false, "W", (void **)&a.W) ||
+        !bind_ptr(b, 3, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x) ||
+        !bind_ptr(b, 4, ((size_t)(a.nb - 1) * a.ystride + a.N) * (a.yfloat ? 4 : 2), true, "y", &a.y)) return false;
+    char fn[48];
+    fname_fmt(fn, sizeof fn, "qwk_qmv_f%d%s", p->F, p->K <= 2560 ? "" : "_g");
+    return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles), 512, &a, sizeof a);
+}
+
+static bool launch_router(qw_batch *b, unsigned iWr, unsigned iWsg, unsigned ix, unsigned ilg, uint32_t nbr) {
+    const qw_kparams *p = &b->k->p;
+    qwk_router_args a = {.E = (uint32_t)p->E, .D = (uint32_t)p->D, .nb = nbr};
+    if (!bind_ptr(b, iWr, (size_t)p->E * p->D * 2, false, "router weights", (void **)&a.Wr) || !bind_ptr(b, iWsg, (size_t)p->D * 2, false, "shared gate vector", (void **)&a.Wsg) ||
+        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a.x) || !bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, true, "logits", (void **)&a.logits)) return false;
+    char fn[48];
+    fname_fmt(fn, sizeof fn, "qwk_router_w%d_n%d", p->rwf, nb_variant(nbr));
+    return add_launch(b, intern(fn), cdiv((unsigned)p->E + 1, 4), 256, &a, sizeof a);
+}
+
+static bool launch_select(qw_batch *b, unsigned ilg, unsigned isel, uint32_t nbr) {
+    const qw_kparams *p = &b->k->p;
+    qwk_select_args a = {.nbr = nbr, .E = (uint32_t)p->E, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
+    if (!bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, false, "logits", (void **)&a.logits) || !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.sel)) return false;
+    return add_launch(b, "qwk_select", 1, 1024, &a, sizeof a);
+}
+
+static bool nbr_ok(qw_batch *b, uint32_t nbr) {
+    if (nbr < 1 || nbr > (uint32_t)b->k->p.NB) return fail(b, "%s: %u tokens, kernel was built for at most NB = %d", b->k->name, nbr, b->k->p.NB);
+    return true;
+}
+
+// gate/up launch. shared: one expert at (iWg, iWu), all tokens, slot topk.
+static bool launch_gu(qw_batch *b, int F, unsigned iWg, unsigned iWu, unsigned ix, unsigned isel, unsigned iH, uint32_t nbr, bool shared) {
+    const qw_kparams *p = &b->k->p;
+    const size_t rb = fmt_rb(F, p->D), ne = shared ? 1 : (size_t)p->E;
+    qwk_gu_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
+                     .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
+    if (!bind_ptr(b, iWg, ne * p->I * rb, false, "gate weights", (void **)&a.Wg) || !bind_ptr(b, iWu, ne * p->I * rb, false, "up weights", (void **)&a.Wu) ||
+        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a.x) || !bind_ptr(b, iH, (size_t)a.hplane * 4, true, "H", (void **)&a.H)) return false;
+    if (!shared && !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
+    const unsigned tasks = (shared ? 1u : umin((unsigned)p->E, nbr * (unsigned)p->topk)) * (unsigned)(p->I / 8);
+    return add_launch(b, F == 21 ? "qwk_gu_f21" : "qwk_gu_f8", persistent_grid(b->g, tasks), 512, &a, sizeof a);
+}
+
+static bool launch_dn(qw_batch *b, int F, unsigned iWd, unsigned iH, unsigned isel, unsigned iP, uint32_t nbr, bool shared) {
+    const qw_kparams *p = &b->k->p;
+    const size_t rb = fmt_rb(F, p->I), ne = shared ? 1 : (size_t)p->E;
+    qwk_dn_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
+                     .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
+    if (!bind_ptr(b, iWd, ne * p->D * rb, false, "down weights", (void **)&a.Wd) || !bind_ptr(b, iH, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
+        !bind_ptr(b, iP, (size_t)nbr * (shared ? 1 : p->topk) * p->D * 4, true, shared ? "Psh" : "Pg", (void **)&a.P)) return false;
+    if (!shared && !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
+    const unsigned tasks = (shared ? 1u : umin((unsigned)p->E, nbr * (unsigned)p->topk)) * (unsigned)(p->D / 64);
+    return add_launch(b, F == 21 ? "qwk_dn_f21" : "qwk_dn_f8", persistent_grid(b->g, tasks), 512, &a, sizeof a);
+}
+
+static bool tr_router(qw_batch *b) { return launch_router(b, 0, 1, 2, 3, (uint32_t)b->k->p.NB); } // src/engine.c:546-551; NB = token count
+
+static bool tr_tab_init(qw_batch *b) { // src/engine.c:572-574
+    qwk_tab_args a;
+    if (!bind_ptr(b, 0, QW_TAB_BYTES, true, "lookup tables", (void **)&a.tab)) return false;
+    return add_launch(b, "qwk_tab_init", 32, 256, &a, sizeof a);
+}
+
+static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nbr
+    uint32_t nbr;
+    return bind_bytes(b, 2, &nbr, 4, "nbr") && nbr_ok(b, nbr) && launch_select(b, 0, 1, nbr);
+}
+
+// src/engine.c:588-607: 0 Wr, 1 shared gate vector, 2 x, 3 logits, 4 counter, 5 sel, 6/7 shared gate/up, 8 H, 13 tables, 14 nbr.
+// Here: router launch, then selection, then the shared expert's gate/up; the counter buffer is not used.
+static bool tr_pre(qw_batch *b) {
+    const qw_kparams *p = &b->k->p;
+    uint32_t nbr;
+    if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
+    if (p->rbf && (!launch_router(b, 0, 1, 2, 3, nbr) || !launch_select(b, 3, 5, nbr))) return false;
+    return launch_gu(b, p->fsg, 6, 7, 2, 5, 8, nbr, true);
+}
+
+// src/engine.c:616-629: 0 Wg, 1 Wu, 2 shared down, 3 Psh, 4 x, 5 sel, 6 H, 11 tables, 12 nbr
+static bool tr_gu(qw_batch *b) {
+    const qw_kparams *p = &b->k->p;
+    uint32_t nbr;
+    if (!bind_bytes(b, 12, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
+    return launch_gu(b, p->fgu, 0, 1, 4, 5, 6, nbr, false) && launch_dn(b, p->fsd, 2, 6, 5, 3, nbr, true);
+}
+
+// src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
+static bool tr_dn(qw_batch *b) {
+    const qw_kparams *p = &b->k->p;
+    return launch_dn(b, p->fd, 0, 2, 3, 9, (uint32_t)p->NB, false);
+}
+
+// src/engine.c:640-646: 1 Psh, 3 sel, 4 out, 8 nbr, 9 Pg
+static bool tr_cmb(qw_batch *b) {
+    const qw_kparams *p = &b->k->p;
+    uint32_t nbr;
+    if (!bind_bytes(b, 8, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
+    qwk_cmb_args a = {.D = (uint32_t)p->D, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
+    if (!bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, false, "Pg", (void **)&a.Pg) || !bind_ptr(b, 1, (size_t)nbr * p->D * 4, false, "Psh", (void **)&a.Psh) ||
+        !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel) || !bind_ptr(b, 4, (size_t)nbr * p->D * 2, true, "out", (void **)&a.out)) return false;
+    return add_launch(b, "qwk_cmb", cdiv(nbr * (unsigned)p->D, 256), 256, &a, sizeof a);
+}
+
+// helpers: 0 src, 1 dst, 2 {n16 (uint64), seed (uint64)}; grid x = workgroups of 256 threads
+static bool tr_mem(qw_batch *b, unsigned gx) {
+    uint64_t a2[2];
+    if (!bind_bytes(b, 2, a2, sizeof a2, "{n, seed}")) return false;
+    qwk_mem_args a = {.n = a2[0], .seed = a2[1]};
+    const qw_family f = b->k->fam;
+    if (f != FAM_FILL && !bind_ptr(b, 0, a.n * 16, false, "src", (void **)&a.src)) return false;
+    if (!bind_ptr(b, 1, f == FAM_BW_READ ? 16 : a.n * 16, true, "dst", &a.dst)) return false;
+    return add_launch(b, f == FAM_BW_READ ? "qwk_bw_read" : f == FAM_COPY ? "qwk_copy" : "qwk_fill_random", gx, 256, &a, sizeof a);
+}
+
+void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsigned tx, unsigned ty, unsigned tz) {
+    (void)gy; (void)gz; (void)tx; (void)ty; (void)tz;
+    if (b->failed) return;
+    if (!b->k) { fail(b, "qw_batch_dispatch without a kernel"); return; }
+    const int first = b->nl;
+    bool ok;
+    switch (b->k->fam) {
+    case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
+    case FAM_QMV_GG: ok = tr_qmv(b); break;
+    case FAM_ROUTER: ok = tr_router(b); break;
+    case FAM_TAB_INIT: ok = tr_tab_init(b); break;
+    case FAM_SEL: ok = tr_sel(b); break;
+    case FAM_PRE: ok = tr_pre(b); break;
+    case FAM_GU: ok = tr_gu(b); break;
+    case FAM_DN: ok = tr_dn(b); break;
+    case FAM_CMB: ok = tr_cmb(b); break;
+    default: ok = tr_mem(b, gx);
+    }
+    if (ok && b->nl > first) b->l[b->nl - 1].last_of_dispatch = true;
+}
+
+// ---------------------------------------------------------------- batches: submission
+static bool submit_segment(qw_batch *b) {
+    qw_gpu *g = b->g;
+    hipStream_t st = g->stream[b->stream];
+    if (b->failed) return false;
+    if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
+    // host -> device for what this segment binds
+    const unsigned mark = ++g->mark;
+    for (int i = b->done_use; i < b->nuse; i++) {
+        qw_hbuf *h = b->use[i].b;
+        if (h->mark == mark) continue;
+        h->mark = mark;
+        if (h->device_only || !h->host) continue;
+        if (h->dirty || (!h->wrapped && h->size <= QW_HIP_SMALL_BYTES)) {
+            if (!HIPOK(g, hipMemcpyAsync(h->dptr, h->host, h->size, hipMemcpyHostToDevice, st))) { b->failed = true; return false; }
+            h->dirty = false;
+        }
+    }
+    hipEvent_t *ev = &b->ev[2 * b->nseg];
+    if (!HIPOK(g, hipEventCreate(&ev[0])) || !HIPOK(g, hipEventCreate(&ev[1]))) { b->failed = true; return false; }
+    b->nseg++;
+    if (!HIPOK(g, hipEventRecord(ev[0], st))) { b->failed = true; return false; }
+    bool open = false; // profiling: an event pair brackets the launches of one dispatch
+    for (int i = b->done_l; i < b->nl; i++) {
+        qw_launch *l = &b->l[i];
+        if (b->prof && !open) {
+            b->pev = realloc(b->pev, sizeof *b->pev * (size_t)(b->npev + 2));
+            if (!HIPOK(g, hipEventCreate(&b->pev[b->npev])) || !HIPOK(g, hipEventCreate(&b->pev[b->npev + 1])) || !HIPOK(g, hipEventRecord(b->pev[b->npev], st))) { b->failed = true; return false; }
+            open = true;
+        }
+        void *params[] = {l->args}; // every kernel takes one record by value
+        if (!HIPOK(g, hipModuleLaunchKernel(l->f, l->gx, l->gy, l->gz, l->bx, 1, 1, 0, st, params, NULL))) { b->failed = true; return false; }
+        if (b->prof && (l->last_of_dispatch || i + 1 == b->nl)) {
+            if (!HIPOK(g, hipEventRecord(b->pev[b->npev + 1], st))) { b->failed = true; return false; }
+            b->npev += 2;
+            open = false;
+        }
+    }
+    if (!HIPOK(g, hipEventRecord(ev[1], st))) { b->failed = true; return false; }
+    b->done_l = b->nl;
+    b->done_use = b->nuse;
+    return true;
+}
+
+void qw_batch_flush(qw_batch *b) {
+    if (b->prof) return; // as in the reference: a profiled batch is not split
+    if (b->nseg >= 8) return;
+    submit_segment(b);
+}
+
+void qw_batch_submit(qw_batch *b) {
+    if (b->submitted) return;
+    b->submitted = true;
+    submit_segment(b);
+}
+
+bool qw_batch_poll(qw_batch *b) {
+    if (b->failed || !b->submitted) return true;
+    return hipEventQuery(b->ev[2 * b->nseg - 1]) != hipErrorNotReady;
+}
+
+static void batch_free(qw_batch *b) {
+    for (int i = 0; i < 2 * b->nseg; i++) (void)hipEventDestroy(b->ev[i]);
+    for (int i = 0; i < b->npev; i++) (void)hipEventDestroy(b->pev[i]);
+    free(b->pev);
+    free(b->l);
+    free(b->use);
+    free(b);
+}
+
+double qw_batch_wait(qw_batch *b) {
+    qw_gpu *g = b->g;
+    hipStream_t st = g->stream[b->stream];
+    if (!b->submitted) qw_batch_submit(b);
+    double secs = -1;
+    if (b->failed) {
+        (void)hipStreamSynchronize(st);
+        if (!g->err[0]) set_err(g, "batch failed");
+        if (!getenv("QW_HIP_QUIET")) fprintf(stderr, "qw_batch: %s\n", g->err);
+        batch_free(b);
+        return -1;
+    }
+    // device -> host for everything bound in an output role
+    const unsigned mark = ++g->mark;
+    bool ok = true;
+    for (int i = 0; i < b->nuse && ok; i++) {
+        qw_hbuf *h = b->use[i].b;
+        if (!b->use[i].out || h->mark == mark) continue;
+        h->mark = mark;
+        if (h->device_only || !h->host || h->wrapped || h->size > QW_HIP_BIG_OUT_BYTES) continue;
+        ok = HIPOK(g, hipMemcpyAsync(h->host, h->dptr, h->size, hipMemcpyDeviceToHost, st));
+    }
+    ok = ok && HIPOK(g, hipStreamSynchronize(st));
+    if (ok) {
+        secs = 0;
+        for (int s = 0; s < b->nseg; s++) {
+            float ms = 0;
+            if (!HIPOK(g, hipEventElapsedTime(&ms, b->ev[2 * s], b->ev[2 * s + 1]))) { ok = false; break; }
+            secs += (double)ms * 1e-3;
+        }
+    }
+    if (ok && b->prof) {
+        g->nprof = 0;
+        int e = 0;
+        for (int i = 0; i < b->nl && g->nprof < QW_PROF_MAX && e + 1 < b->npev; i++) {
+            if (!b->l[i].last_of_dispatch && i + 1 != b->nl) continue;
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, b->pev[e], b->pev[e + 1]);
+            e += 2;
+            g->prof_name[g->nprof] = b->l[i].kname;
+            g->prof_fname[g->nprof] = b->l[i].fname;
+            g->prof_us[g->nprof++] = (double)ms * 1e3;
+        }
+    }
+    if (!ok) {
+        if (!getenv("QW_HIP_QUIET")) fprintf(stderr, "qw_batch: %s\n", g->err);
+        secs = -1;
+    }
+    batch_free(b);
+    return secs;
+}
+
+double qw_batch_end(qw_batch *b) {
+    qw_batch_submit(b);
+    return qw_batch_wait(b);
+}
+
+void qw_gpu_set_stream(qw_gpu *g, int s) { g->cur_stream = s == 1 ? 1 : 0; }
+
+// ---------------------------------------------------------------- profiling and bench utilities
+void qw_profile_enable(qw_gpu *g, bool on) { g->prof = on; }
+int qw_profile_count(const qw_gpu *g) { return g->nprof; }
+const char *qw_profile_get(const qw_gpu *g, int i, double *us) {
+    if (i < 0 || i >= g->nprof) return NULL;
+    if (us) *us = g->prof_us[i];
+    return g->prof_name[i];
+}
+double qw_hip_profile_mean(const qw_gpu *g, const char *prefix, int *count) {
+    double s = 0;
+    int n = 0;
+    for (int i = 0; i < g->nprof; i++)
+        if (!strncmp(g->prof_fname[i], prefix, strlen(prefix)) || !strncmp(g->prof_name[i], prefix, strlen(prefix))) { s += g->prof_us[i]; n++; }
+    if (count) *count = n;
+    return n ? s / n * 1e-6 : 0;
+}
+
+double qw_gpu_empty_commit_latency(qw_gpu *g, qw_kernel *k, int n) {
+    (void)k;
+    if (n < 1) return 0;
+    hipStream_t st = g->stream[g->cur_stream];
+    hipEvent_t ev;
+    if (hipEventCreate(&ev) != hipSuccess) return -1;
+    const double t0 = qw_now();
+    for (int i = 0; i < n; i++) {
+        (void)hipEventRecord(ev, st);
+        (void)hipEventSynchronize(ev);
+    }
+    const double t = (qw_now() - t0) / n;
+    (void)hipEventDestroy(ev);
+    return t;
+}
+
+void qw_power_desc(char *out, size_t len) { snprintf(out, len, "power: mains (accelerator card); thermal state not reported"); }
+bool qw_on_battery(void) { return false; }

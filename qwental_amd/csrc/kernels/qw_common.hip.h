@@ -1,0 +1,200 @@
+// Device-side building blocks for the quantized decode kernels (gfx950, wave64).
+//
+// Matrix-core formulation used by every weight-streaming kernel here: one wave owns a tile of 16 weight rows
+// and up to 16 token columns and issues v_mfma_f32_16x16x32_f16 with the ACTIVATIONS as operand A (M = token)
+// and the decoded WEIGHTS as operand B (N = weight row):
+//     lane l:  n = l & 15 (weight row in the tile),  kg = l >> 4 (which 8 of the 32 k-values of a step)
+//     A: lane supplies x[token = n][8 k-values of group kg]      B: lane supplies w[row n][8 k-values of group kg]
+//     D: lane receives out[token 4*kg + i][row n], i = 0..3
+// so a lane's four results belong to the row whose bytes that lane decodes, and the per-block scale of that row
+// is already in the lane's registers. The decoded weights are small integers (exact in binary16); products and
+// sums are accumulated in binary32 by the matrix core; the binary16 block scale d multiplies the binary32
+// partial sum afterwards. A token's result never depends on the other token columns.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "qw_kargs.h"
+#define QW_CODES_QUAL __constant__ const
+#include "iq3s_codes.h"
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+// GGUF blocks are only 2-byte aligned (110- and 34-byte blocks); the hardware takes unaligned wide loads.
+typedef u4 __attribute__((aligned(2))) u4a2;
+typedef u2 __attribute__((aligned(2))) u2a2;
+
+#define QW_LUT_ENTRIES 8192
+#define QW_LUT_BYTES (QW_LUT_ENTRIES * 8)
+
+__device__ __forceinline__ float qw_h2f(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+__device__ __forceinline__ uint16_t qw_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+__device__ __forceinline__ float qw_bf2f(uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); }
+
+// One pre-signed table entry: index = codebook entry (9 bits) | sign nibble << 9; four binary16 values, value j =
+// magnitude j of the codebook entry with the sign taken from bit j of the nibble (the reference builds the same
+// table in kernels/moe_gg.metal:495-500).
+__device__ __forceinline__ u2 qw_lut_entry(uint32_t i) {
+    const uint32_t code = qw_iq3s_codes[i & 511];
+    uint32_t h[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int mag = 2 * (int)((code >> (3 * j)) & 7) + 1;
+        h[j] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)mag) | (((i >> (9 + j)) & 1) << 15);
+    }
+    u2 r;
+    r.x = h[0] | h[1] << 16;
+    r.y = h[2] | h[3] << 16;
+    return r;
+}
+
+// Fill the 64 KB table in LDS; every thread of the workgroup takes part. Caller synchronises afterwards.
+__device__ __forceinline__ void qw_lut_build(u2 *lut) {
+    for (uint32_t i = threadIdx.x; i < QW_LUT_ENTRIES; i += blockDim.x) lut[i] = qw_lut_entry(i);
+}
+
+__device__ __forceinline__ f4 qw_mfma(h8 a, h8 b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+
+// ---------------------------------------------------------------- IQ3_S (110-byte block of 256 values)
+// Bytes: d @0 (binary16), qs[64] @2, qh[8] @66, signs[32] @74, scales[4] @106 (kernels/moe_iq.metal:102-118).
+// Lane group kg decodes the 64 values [64 kg, 64 kg + 64) of a block — sub-blocks 2 kg and 2 kg + 1 — whose
+// bytes are contiguous: qs[16 kg .. +16), signs[8 kg .. +8), qh[2 kg .. +2), scales[kg]. In step j (0..7) the lane
+// supplies values 64 kg + 8 j .. + 8. The sub-block factor 1 + 2 s is multiplied into the binary16 integers
+// (|value| <= 15 * 31, exact); the block scale d multiplies the binary32 sum of the eight steps.
+struct qw_iq3_slice {
+    u4 qs;
+    u2 sg;
+    uint32_t qh, sc;
+    float d;
+};
+
+__device__ __forceinline__ qw_iq3_slice qw_iq3_load(const uint8_t *blk, uint32_t kg) {
+    qw_iq3_slice s;
+    s.qs = *(const u4a2 *)(blk + 2 + 16 * kg);
+    s.sg = *(const u2a2 *)(blk + 74 + 8 * kg);
+    s.qh = *(const uint16_t *)(blk + 66 + 2 * kg);
+    s.sc = blk[106 + kg];
+    s.d = qw_h2f(*(const uint16_t *)blk);
+    return s;
+}
+
+// The eight binary16 values of step J, already multiplied by the sub-block factor.
+template <int J> __device__ __forceinline__ h8 qw_iq3_step(const qw_iq3_slice &s, const u2 *lut) {
+    const uint32_t q = s.qs[J / 2] >> (16 * (J % 2));  // bytes 2J, 2J + 1 of the slice's qs
+    const uint32_t sg = s.sg[J / 4] >> (8 * (J % 4));  // byte J of the slice's signs
+    const uint32_t hb = s.qh >> (8 * (J / 4) + 2 * (J % 4));
+    const uint32_t i0 = (q & 255) | ((hb & 1) << 8) | ((sg & 15) << 9);
+    const uint32_t i1 = ((q >> 8) & 255) | ((hb & 2) << 7) | ((sg & 0xf0) << 5);
+    const u2 w0 = lut[i0], w1 = lut[i1];
+    const _Float16 f = (_Float16)(int)(1 + 2 * ((s.sc >> (4 * (J / 4))) & 15));
+    const h2 ff = {f, f};
+    u4 raw = {w0.x, w0.y, w1.x, w1.y};
+#pragma unroll
+    for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+    return __builtin_bit_cast(h8, raw);
+}
+
+// ---------------------------------------------------------------- Q8_0 (34-byte block of 32 values)
+// Bytes: d @0, qs[32] int8 @2 (src/ggml_dq.c:34-37). Lane group kg decodes values [8 kg, 8 kg + 8) of a block.
+// int8 -> binary16 without conversions: (q ^ 0x80) placed under the exponent byte 0x64 is 1024 + q + 128 exactly.
+__device__ __forceinline__ h8 qw_q8_cvt(u2 q) {
+    const uint32_t a = q.x ^ 0x80808080u, b = q.y ^ 0x80808080u;
+    const h2 bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    u4 raw;
+    raw[0] = __builtin_amdgcn_perm(0x64646464u, a, 0x04010400u); // bytes: a0, 0x64, a1, 0x64
+    raw[1] = __builtin_amdgcn_perm(0x64646464u, a, 0x04030402u);
+    raw[2] = __builtin_amdgcn_perm(0x64646464u, b, 0x04010400u);
+    raw[3] = __builtin_amdgcn_perm(0x64646464u, b, 0x04030402u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) - bias);
+    return __builtin_bit_cast(h8, raw);
+}
+
+// ---------------------------------------------------------------- activation fragment providers (operand A)
+// Fragment order in LDS: chunk c (8 consecutive k-values) of token m lives at xf[c * 16 + m], 16 bytes, so that the
+// 16 lanes of a k-group read 256 contiguous bytes. Tokens >= nb are stored as zeros.
+struct qw_afrag_lds {
+    const u4 *xf;
+    uint32_t m;
+    static constexpr bool has_lo = false;
+    __device__ __forceinline__ h8 hi(uint32_t koff) const { return __builtin_bit_cast(h8, xf[(koff >> 3) * 16 + m]); }
+    __device__ __forceinline__ h8 lo(uint32_t) const { return h8{}; }
+};
+
+__device__ __forceinline__ void qw_stage_x(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
+    for (uint32_t i = threadIdx.x; i < (K >> 3) * 16; i += blockDim.x) {
+        const uint32_t c = i >> 4, m = i & 15;
+        u4 v = {0, 0, 0, 0};
+        if (m < nb) v = *(const u4 *)(x + (size_t)m * xstride + 8 * c);
+        xf[i] = v;
+    }
+}
+
+// Straight from global memory: row pointers of binary16 planes; a null row contributes zeros.
+template <bool LO> struct qw_afrag_glb {
+    const uint16_t *rowhi, *rowlo;
+    static constexpr bool has_lo = LO;
+    __device__ __forceinline__ h8 hi(uint32_t koff) const { return rowhi ? *(const h8 *)(rowhi + koff) : h8{}; }
+    __device__ __forceinline__ h8 lo(uint32_t koff) const { return rowlo ? *(const h8 *)(rowlo + koff) : h8{}; }
+};
+
+// ---------------------------------------------------------------- one 16-row tile over the whole K
+template <int F> struct qw_tile;
+
+template <> struct qw_tile<21> {
+    template <int J, class AF> static __device__ __forceinline__ void step(const qw_iq3_slice &s, const u2 *lut, const AF &af, uint32_t k0, f4 &sub) {
+        const h8 b = qw_iq3_step<J>(s, lut);
+        sub = qw_mfma(af.hi(k0 + 8 * J), b, sub);
+        if (AF::has_lo) sub = qw_mfma(af.lo(k0 + 8 * J), b, sub);
+    }
+    // row: this lane's weight row; K multiple of 256.
+    template <class AF> static __device__ __forceinline__ f4 run(const uint8_t *row, uint32_t K, uint32_t kg, const u2 *lut, const AF &af) {
+        f4 acc = {0, 0, 0, 0};
+        const uint32_t nblk = K >> 8;
+        qw_iq3_slice cur = qw_iq3_load(row, kg);
+        for (uint32_t blk = 0; blk < nblk; blk++) {
+            const qw_iq3_slice s = cur;
+            if (blk + 1 < nblk) cur = qw_iq3_load(row + 110 * (blk + 1), kg); // next block's bytes are in flight while this one is decoded
+            const uint32_t k0 = 256 * blk + 64 * kg;
+            f4 sub = {0, 0, 0, 0};
+            step<0>(s, lut, af, k0, sub);
+            step<1>(s, lut, af, k0, sub);
+            step<2>(s, lut, af, k0, sub);
+            step<3>(s, lut, af, k0, sub);
+            step<4>(s, lut, af, k0, sub);
+            step<5>(s, lut, af, k0, sub);
+            step<6>(s, lut, af, k0, sub);
+            step<7>(s, lut, af, k0, sub);
+            acc += s.d * sub;
+        }
+        return acc;
+    }
+};
+
+template <> struct qw_tile<8> {
+    // K multiple of 32; lut unused.
+    template <class AF> static __device__ __forceinline__ f4 run(const uint8_t *row, uint32_t K, uint32_t kg, const u2 *, const AF &af) {
+        f4 acc = {0, 0, 0, 0};
+        const uint32_t nblk = K >> 5;
+        u2 q = *(const u2a2 *)(row + 2 + 8 * kg);
+        float d = qw_h2f(*(const uint16_t *)row);
+#pragma unroll 4
+        for (uint32_t blk = 0; blk < nblk; blk++) {
+            const u2 qc = q;
+            const float dc = d;
+            if (blk + 1 < nblk) {
+                q = *(const u2a2 *)(row + 34 * (blk + 1) + 2 + 8 * kg);
+                d = qw_h2f(*(const uint16_t *)(row + 34 * (blk + 1)));
+            }
+            const h8 b = qw_q8_cvt(qc);
+            const uint32_t k0 = 32 * blk + 8 * kg;
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(af.hi(k0), b, sub);
+            if (AF::has_lo) sub = qw_mfma(af.lo(k0), b, sub);
+            acc += dc * sub;
+        }
+        return acc;
+    }
+};

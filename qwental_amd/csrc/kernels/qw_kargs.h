@@ -1,0 +1,84 @@
+/* Kernel argument records shared by the HIP kernels (device side) and gpu_hip.c (host side, C23).
+ * Every kernel takes exactly one of these by value. Plain C: fixed-width integers and pointers only. */
+#pragma once
+#include <stdint.h>
+
+/* Selection record written by the select kernel and read by gate/up, down and combine. For gnb == 8 and
+ * topk == 10 this is byte for byte the reference's struct gg_sel (kernels/moe_gg.metal:110-116), 1636 bytes;
+ * gnb == 16 is the wide layout for up to 16 token columns (4548 bytes with topk == 10). GU = gnb * topk.
+ *   uint32 U; uint32 ue[GU]; uint32 mask[GU]; uint8 slot[GU][gnb]; float w[gnb][topk + 1] */
+#define QW_SEL_OFF_UE(gnb, topk) 4u
+#define QW_SEL_OFF_MASK(gnb, topk) (4u + 4u * (gnb) * (topk))
+#define QW_SEL_OFF_SLOT(gnb, topk) (4u + 8u * (gnb) * (topk))
+#define QW_SEL_OFF_W(gnb, topk) (4u + 8u * (gnb) * (topk) + (gnb) * (topk) * (gnb))
+#define QW_SEL_BYTES(gnb, topk) (QW_SEL_OFF_W(gnb, topk) + 4u * (gnb) * ((topk) + 1u))
+
+/* Pre-signed IQ3_S table inside the lookup-table buffer the callers allocate (kernels/moe_gg.metal:89-95):
+ * 8192 entries of four binary16 values at byte offset 49152; the whole buffer is 117760 bytes. */
+#define QW_TAB_IQ3SS 49152u
+#define QW_TAB_IQ4 114688u
+#define QW_TAB_Q20 115712u
+#define QW_TAB_BYTES 117760u
+
+typedef struct { /* dq_test: rows x K values to float */
+    const uint8_t *W;
+    float *y;
+    uint32_t K, rowbytes, rows, pad;
+} qwk_dq_args;
+
+typedef struct { /* dense matvec, y[b][row] = W[row] . x[b] */
+    const uint8_t *W;
+    const uint16_t *x; /* binary16 [nb][xstride] */
+    void *y;           /* binary16 or float [nb][ystride] */
+    uint32_t N, K, rowbytes, xstride, ystride, nb, yfloat, ntiles;
+} qwk_qmv_args;
+
+typedef struct { /* router: logits[t][r], r in [0, E] (row E = shared gate vector), row stride E + 1 */
+    const uint16_t *Wr, *Wsg, *x;
+    float *logits;
+    uint32_t E, D, nb, pad;
+} qwk_router_args;
+
+typedef struct { /* selection + dedupe */
+    const float *logits;
+    uint8_t *sel;
+    uint32_t nbr, E, topk, gnb;
+} qwk_select_args;
+
+typedef struct { /* build the lookup-table buffer */
+    uint8_t *tab;
+} qwk_tab_args;
+
+/* gate/up + SwiGLU for a list of experts. routed: experts come from sel (U, ue, mask, slot). shared != 0: one
+ * expert at Wg/Wu with every token in nbr selected, written to slot topk.
+ * H is stored as two binary16 planes (value = hi + lo): Hhi = H, Hlo = H + nb_alloc * (topk + 1) * I halves. */
+typedef struct {
+    const uint8_t *Wg, *Wu; /* [E][I][rowbytes] */
+    const uint16_t *x;      /* binary16 [nbr][D] */
+    const uint8_t *sel;
+    uint16_t *H;
+    uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane; /* hplane: halves between the hi and lo planes */
+} qwk_gu_args;
+
+/* down projection. routed: Pg[t][slot][row] for the tokens in mask[u]; shared != 0: Psh[t][row] from slot topk. */
+typedef struct {
+    const uint8_t *Wd; /* [E][D][rowbytes] */
+    const uint16_t *H;
+    const uint8_t *sel;
+    float *P; /* Pg [nbr][topk][D] or Psh [nbr][D] */
+    uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane;
+} qwk_dn_args;
+
+typedef struct { /* out[t][row] = half(sum_s w[t][s] * Pg[t][s][row] + w[t][topk] * Psh[t][row]) */
+    const float *Pg, *Psh;
+    const uint8_t *sel;
+    uint16_t *out;
+    uint32_t D, nbr, topk, gnb;
+} qwk_cmb_args;
+
+typedef struct { /* pure-read ceiling and fill helpers */
+    const void *src;
+    void *dst;
+    uint64_t n; /* 16-byte units */
+    uint64_t seed;
+} qwk_mem_args;

@@ -1,0 +1,215 @@
+// Host side of the quantized decode path over gpu.h: the call sequences of the reference's engine for this path
+// (src/engine.c:439-724), written against the interface only. See include/qw_path.h.
+#include "qw_path.h"
+#include "qw_hip_ext.h"
+#include "kernels/qw_kargs.h"
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+struct qw_path {
+    qw_gpu *g;
+    int D, I, E, topk, nbmax;
+    qw_buf tab, H, psh, pd, cnt;
+    bool tab_ready;
+};
+
+static int blk_values(int type) { return type == 8 ? 32 : type == 21 ? 256 : 0; }
+static int blk_bytes(int type) { return type == 8 ? 34 : type == 21 ? 110 : 0; } // src/gguf.c:15-25
+static int row_bytes(int type, int K) { return blk_values(type) ? K / blk_values(type) * blk_bytes(type) : 0; }
+
+int qw_path_nbv(int nb) { return nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : nb <= 8 ? 8 : 16; }
+static int gnb_of(int nb) { return qw_path_nbv(nb) <= 8 ? 8 : 16; }
+
+size_t qw_path_sel_bytes(const qw_path *p, int nb) { return QW_SEL_BYTES((size_t)gnb_of(nb), (size_t)p->topk); }
+size_t qw_path_logits_bytes(const qw_path *p, int nb) { return (size_t)nb * (size_t)(p->E + 1) * 4; }
+
+qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool device_scratch) {
+    if (!g || nbmax < 1 || nbmax > 16) return NULL;
+    qw_path *p = calloc(1, sizeof *p);
+    if (!p) return NULL;
+    *p = (qw_path){.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = nbmax};
+    const size_t nb = (size_t)qw_path_nbv(nbmax);
+    bool (*mk)(qw_gpu *, size_t, qw_buf *) = device_scratch ? qw_hip_buf_new_device : qw_buf_new;
+    // sizes as the engine allocates them: H [nb][topk + 1][I] float, Psh [nb][D] float, Pg [nb][topk][D] float (src/engine.c:157)
+    if (!mk(g, QW_TAB_BYTES, &p->tab) || !mk(g, nb * (size_t)(topk + 1) * (size_t)I * 4, &p->H) || !mk(g, nb * (size_t)D * 4, &p->psh) ||
+        !mk(g, nb * (size_t)topk * (size_t)D * 4, &p->pd) || !mk(g, 16, &p->cnt)) {
+        qw_path_close(p);
+        return NULL;
+    }
+    return p;
+}
+
+void qw_path_close(qw_path *p) {
+    if (!p) return;
+    qw_buf_free(&p->tab); qw_buf_free(&p->H); qw_buf_free(&p->psh); qw_buf_free(&p->pd); qw_buf_free(&p->cnt);
+    free(p);
+}
+
+const qw_buf *qw_path_scratch(const qw_path *p, int which) { return which == 0 ? &p->tab : which == 1 ? &p->H : which == 2 ? &p->psh : which == 3 ? &p->pd : NULL; }
+
+static qw_kernel *compile_get(qw_path *p, const char *name, const char *defs) {
+    char err[2048];
+    qw_kernel *k = qw_kernel_get(p->g, name);
+    if (k) return k;
+    if (!qw_gpu_compile(p->g, defs, strlen(defs), err, sizeof err)) {
+        fprintf(stderr, "compile %s failed: %s\n", name, err);
+        return NULL;
+    }
+    k = qw_kernel_get(p->g, name);
+    if (!k) fprintf(stderr, "kernel %s not found\n", name);
+    return k;
+}
+
+// ---------------------------------------------------------------- dense matvec (src/engine.c:689-724)
+bool qw_path_qmv_gg(qw_path *p, qw_batch *b, const qw_tensor *W, int N, int K, const qw_buf *x, size_t xoff, const qw_buf *y,
+                    size_t yoff, int nb, bool fout) {
+    char name[96], defs[512];
+    const int f = W->type;
+    snprintf(name, sizeof name, "qmv_gg_f%d_k%d_n%d%s", f, K, nb, fout ? "_f" : "");
+    snprintf(defs, sizeof defs, "#define IQ_DQ_ONLY 1\n#define qmv_gg %s\n#define GF %d\n#define KD %d\n#define RB %d\n#define NB %d\n%s", name, f, K,
+             row_bytes(f, K), nb, fout ? "#define YT float\n" : "");
+    qw_kernel *k = compile_get(p, name, defs);
+    if (!k) return false;
+    struct { uint32_t N, xs, ys, pad; } a = {(uint32_t)N, (uint32_t)K, (uint32_t)N, 0};
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, W->buf, W->offset);
+    qw_batch_buf(b, 3, x, xoff);
+    qw_batch_buf(b, 4, y, yoff);
+    qw_batch_bytes(b, 5, &a, sizeof a);
+    qw_batch_dispatch(b, ((unsigned)N + 7) / 8, 1, 1, 256, 1, 1);
+    return true;
+}
+
+// ---------------------------------------------------------------- MoE kernels by part (src/engine.c:460-517)
+static qw_kernel *gg_kernel(qw_path *p, const char *base, const qw_moe_layer *M, int nb) {
+    const int part = !strcmp(base, "moe_sel_gg") || !strcmp(base, "gg_tab_init") ? 0 : !strcmp(base, "moe_pre_gg") ? 1 : !strcmp(base, "moe_gu_gg") ? 2
+                     : !strcmp(base, "moe_dn_gg") || !strcmp(base, "moe_cmb_gg") ? 3 : 4;
+    const int nbv = part == 4 ? nb : qw_path_nbv(nb);
+    const int rwf = M->router.type;
+    char name[128], sfx[96], defs[2048];
+    switch (part) {
+    case 0: snprintf(sfx, sizeof sfx, "_n%d", nbv); break;
+    case 1: snprintf(sfx, sizeof sfx, "_%d_%d_r%d_w%d_n%d", M->sh_gate.type, M->sh_up.type, 1, rwf, nbv); break;
+    case 2: snprintf(sfx, sizeof sfx, "_%d_%d_g%d_n%d", M->gate.type, M->sh_down.type, 1, nbv); break;
+    case 3: snprintf(sfx, sizeof sfx, "_%d_s%d_n%d", M->down.type, 4, nbv); break;
+    default: snprintf(sfx, sizeof sfx, "_w%d_n%d", rwf, nbv);
+    }
+    snprintf(name, sizeof name, "%s%s", base, sfx);
+    qw_kernel *k = qw_kernel_get(p->g, name);
+    if (k) return k;
+    if (nb < 1 || nb > 16) {
+        fprintf(stderr, "%s: unsupported token count %d\n", name, nb);
+        return NULL;
+    }
+    int n = snprintf(defs, sizeof defs, "#define IQ_DQ_ONLY\n#define E %d\n#define TOPK %d\n#define D %d\n#define I %d\n#define NB %d\n#define RWF %d\n", p->E, p->topk,
+                     p->D, p->I, nbv, rwf);
+    switch (part) {
+    case 0: snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 0\n#define moe_sel_gg moe_sel_gg%s\n#define gg_tab_init gg_tab_init%s\n", sfx, sfx); break;
+    case 1:
+        snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 1\n#define FSG %d\n#define FSU %d\n#define RBF %d\n#define moe_pre_gg moe_pre_gg%s\n", M->sh_gate.type,
+                 M->sh_up.type, 1, sfx);
+        break;
+    case 2:
+        snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 2\n#define GSG %d\n#define RG %d\n#define FGU %d\n#define FSD %d\n#define moe_gu_gg moe_gu_gg%s\n", 8, 1,
+                 M->gate.type, M->sh_down.type, sfx);
+        break;
+    case 3:
+        snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 3\n#define FD %d\n#define DSGN %d\n#define moe_dn_gg moe_dn_gg%s\n#define moe_cmb_gg moe_cmb_gg%s\n",
+                 M->down.type, 4, sfx, sfx);
+        break;
+    default:
+        snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_ROUTER\n#define moe_router_bf moe_router_bf%s\n#define p_router_bf p_router_bf%s\n"
+                 "#define p_router_bf_refine p_router_bf_refine%s\n", sfx, sfx, sfx);
+    }
+    return compile_get(p, name, defs);
+}
+
+static void bind_t(qw_batch *b, unsigned index, const qw_tensor *t) { qw_batch_buf(b, index, t->buf, t->offset); }
+
+// src/engine.c:544-552
+bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg) {
+    qw_kernel *k = gg_kernel(p, "moe_router_bf", M, nb);
+    if (!k) return false;
+    qw_batch_kernel(b, k);
+    bind_t(b, 0, &M->router);
+    bind_t(b, 1, &M->sh_gate_w);
+    qw_batch_buf(b, 2, x, 0);
+    qw_batch_buf(b, 3, lg, 0);
+    qw_batch_dispatch(b, ((unsigned)p->E + 1 + 7) / 8, 1, 1, 256, 1, 1);
+    return true;
+}
+
+// src/engine.c:568-647: front part (router + shared gate/up + selection) -> routed gate/up + shared down -> routed down -> combine
+bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
+                    const qw_buf *out) {
+    if (nb < 1 || nb > p->nbmax) {
+        fprintf(stderr, "gg_moe: %d tokens, scratch was sized for %d\n", nb, p->nbmax);
+        return false;
+    }
+    qw_kernel *k;
+    if (!p->tab_ready) { // first use: build the lookup tables in the same batch, before they are needed
+        if (!(k = gg_kernel(p, "gg_tab_init", M, 1))) return false;
+        qw_batch_kernel(b, k);
+        qw_batch_buf(b, 0, &p->tab, 0);
+        qw_batch_dispatch(b, 32, 1, 1, 256, 1, 1);
+        p->tab_ready = true;
+    }
+    const uint32_t nbr = (uint32_t)nb;
+    const unsigned E = (unsigned)p->E, I = (unsigned)p->I, D = (unsigned)p->D, K = (unsigned)p->topk;
+    if (!(k = gg_kernel(p, "moe_pre_gg", M, nb))) return false;
+    qw_batch_kernel(b, k);
+    bind_t(b, 0, &M->router);
+    bind_t(b, 1, &M->sh_gate_w);
+    qw_batch_buf(b, 2, x, 0);
+    qw_batch_buf(b, 3, lg, 0);
+    qw_batch_buf(b, 4, &p->cnt, 0);
+    qw_batch_buf(b, 5, sel, 0);
+    bind_t(b, 6, &M->sh_gate);
+    bind_t(b, 7, &M->sh_up);
+    qw_batch_buf(b, 8, &p->H, 0);
+    for (unsigned i = 0; i < 2; i++) { // scale / bias slots of the MLX formats: bound to the weights as placeholders
+        bind_t(b, 9 + 2 * i, i ? &M->sh_up : &M->sh_gate);
+        bind_t(b, 10 + 2 * i, i ? &M->sh_up : &M->sh_gate);
+    }
+    qw_batch_buf(b, 13, &p->tab, 0);
+    qw_batch_bytes(b, 14, &nbr, 4);
+    qw_batch_dispatch(b, (E + 1 + 7) / 8 + I / 8, 1, 1, 256, 1, 1);
+
+    if (!(k = gg_kernel(p, "moe_gu_gg", M, nb))) return false;
+    qw_batch_kernel(b, k);
+    bind_t(b, 0, &M->gate);
+    bind_t(b, 1, &M->up);
+    bind_t(b, 2, &M->sh_down);
+    qw_batch_buf(b, 3, &p->psh, 0);
+    qw_batch_buf(b, 4, x, 0);
+    qw_batch_buf(b, 5, sel, 0);
+    qw_batch_buf(b, 6, &p->H, 0);
+    bind_t(b, 7, &M->sh_down);
+    bind_t(b, 8, &M->sh_down);
+    qw_batch_buf(b, 11, &p->tab, 0);
+    qw_batch_bytes(b, 12, &nbr, 4);
+    {
+        const unsigned a = I / 8, c = D / 32;
+        qw_batch_dispatch(b, a > c ? a : c, nbr * K + 1, 1, 256, 1, 1);
+    }
+
+    if (!(k = gg_kernel(p, "moe_dn_gg", M, nb))) return false;
+    qw_batch_kernel(b, k);
+    bind_t(b, 0, &M->down);
+    qw_batch_buf(b, 2, &p->H, 0);
+    qw_batch_buf(b, 3, sel, 0);
+    qw_batch_buf(b, 7, &p->tab, 0);
+    qw_batch_buf(b, 9, &p->pd, 0);
+    qw_batch_dispatch(b, D / 16, nbr * K, 1, 128, 1, 1);
+
+    if (!(k = gg_kernel(p, "moe_cmb_gg", M, nb))) return false;
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 1, &p->psh, 0);
+    qw_batch_buf(b, 3, sel, 0);
+    qw_batch_buf(b, 4, out, 0);
+    qw_batch_bytes(b, 8, &nbr, 4);
+    qw_batch_buf(b, 9, &p->pd, 0);
+    qw_batch_dispatch(b, D / 256, 1, 1, 256, 1, 1);
+    return true;
+}

@@ -1,0 +1,274 @@
+"""ctypes binding of libqwgpu_hip.so: the GPU interface (include/gpu.h), its HIP additions (include/qw_hip_ext.h)
+and the host side of the path (include/qw_path.h). Thin by design: one Python method per C function."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_lib = None
+
+
+def lib_path():
+    return os.path.join(HERE, "libqwgpu_hip.so")
+
+
+class QwBuf(C.Structure):
+    _fields_ = [("handle", C.c_void_p), ("ptr", C.c_void_p), ("size", C.c_size_t)]
+
+
+class QwTensor(C.Structure):
+    _fields_ = [("buf", C.POINTER(QwBuf)), ("offset", C.c_size_t), ("type", C.c_int)]
+
+
+class QwMoeLayer(C.Structure):
+    _fields_ = [(n, QwTensor) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")]
+
+
+# every symbol include/gpu.h, include/qw_hip_ext.h and include/qw_path.h declare: (name, restype, argtypes)
+_vp, _sz, _u, _i, _b, _d = C.c_void_p, C.c_size_t, C.c_uint, C.c_int, C.c_bool, C.c_double
+_pb, _pt, _pm = C.POINTER(QwBuf), C.POINTER(QwTensor), C.POINTER(QwMoeLayer)
+SYMBOLS = [
+    ("qw_gpu_open", _vp, []), ("qw_gpu_close", None, [_vp]), ("qw_gpu_name", C.c_char_p, [_vp]), ("qw_gpu_max_working_set", _sz, [_vp]),
+    ("qw_gpu_compile", _b, [_vp, C.c_char_p, _sz, C.c_char_p, _sz]), ("qw_kernel_get", _vp, [_vp, C.c_char_p]),
+    ("qw_kernel_max_threads", _u, [_vp]), ("qw_kernel_simd_width", _u, [_vp]),
+    ("qw_buf_new", _b, [_vp, _sz, _pb]), ("qw_buf_free", None, [_pb]), ("qw_pool_push", _vp, []), ("qw_pool_pop", None, [_vp]),
+    ("qw_buf_wrap", _b, [_vp, _vp, _sz, _pb]),
+    ("qw_batch_begin", _vp, [_vp, _b]), ("qw_batch_kernel", None, [_vp, _vp]), ("qw_batch_buf", None, [_vp, _u, _pb, _sz]),
+    ("qw_batch_bytes", None, [_vp, _u, _vp, _sz]), ("qw_batch_threadgroup_mem", None, [_vp, _u, _sz]),
+    ("qw_batch_dispatch", None, [_vp, _u, _u, _u, _u, _u, _u]), ("qw_batch_barrier", None, [_vp]), ("qw_batch_flush", None, [_vp]),
+    ("qw_batch_end", _d, [_vp]), ("qw_batch_submit", None, [_vp]), ("qw_batch_wait", _d, [_vp]), ("qw_batch_poll", _b, [_vp]),
+    ("qw_gpu_set_stream", None, [_vp, _i]),
+    ("qw_profile_enable", None, [_vp, _b]), ("qw_profile_count", _i, [_vp]), ("qw_profile_get", C.c_char_p, [_vp, _i, C.POINTER(_d)]),
+    ("qw_gpu_empty_commit_latency", _d, [_vp, _vp, _i]), ("qw_power_desc", None, [C.c_char_p, _sz]), ("qw_on_battery", _b, []),
+    ("qw_now", _d, []),
+    # qw_hip_ext.h
+    ("qw_hip_buf_new_device", _b, [_vp, _sz, _pb]), ("qw_hip_buf_mark_dirty", None, [_pb]),
+    ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
+    ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
+    ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),
+    ("qw_hip_profile_mean", _d, [_vp, C.c_char_p, C.POINTER(_i)]),
+    # qw_path.h
+    ("qw_path_open", _vp, [_vp, _i, _i, _i, _i, _i, _b]), ("qw_path_close", None, [_vp]),
+    ("qw_path_sel_bytes", _sz, [_vp, _i]), ("qw_path_logits_bytes", _sz, [_vp, _i]), ("qw_path_nbv", _i, [_i]),
+    ("qw_path_qmv_gg", _b, [_vp, _vp, _pt, _i, _i, _pb, _sz, _pb, _sz, _i, _b]),
+    ("qw_path_gg_router", _b, [_vp, _vp, _pm, _i, _pb, _pb]),
+    ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
+    ("qw_path_scratch", _pb, [_vp, _i]),
+]
+
+
+def load_lib():
+    """Load the built library; raises if it has not been built (python -m qwental_amd.build)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(lib_path()):
+        raise RuntimeError("libqwgpu_hip.so is not built: run `python -m qwental_amd.build` (needs hipcc and clang from ROCm)")
+    L = C.CDLL(lib_path())
+    for name, res, args in SYMBOLS:
+        f = getattr(L, name)  # AttributeError if the library lacks a declared symbol
+        f.restype = res
+        f.argtypes = args
+    _lib = L
+    return L
+
+
+class Buf:
+    """A qw_buf plus a numpy view of its host shadow."""
+
+    def __init__(self, gpu, size, device_only=False, wrap=None):
+        self.gpu, self.L = gpu, gpu.L
+        self.c = QwBuf()
+        self._keep = wrap
+        if wrap is not None:
+            ok = self.L.qw_buf_wrap(gpu.g, wrap.ctypes.data, wrap.nbytes, C.byref(self.c))
+        elif device_only:
+            ok = self.L.qw_hip_buf_new_device(gpu.g, size, C.byref(self.c))
+        else:
+            ok = self.L.qw_buf_new(gpu.g, size, C.byref(self.c))
+        if not ok:
+            raise MemoryError("qw_buf allocation of %d bytes failed: %s" % (size, gpu.last_error()))
+        self.size = self.c.size
+
+    def view(self, dtype=np.uint8):
+        if not self.c.ptr:
+            raise ValueError("device-only buffer has no host view")
+        raw = (C.c_uint8 * self.size).from_address(self.c.ptr)
+        return np.frombuffer(raw, dtype=np.uint8).view(dtype)
+
+    def fill(self, arr, offset=0):
+        """Copy a numpy array into the buffer (shadow for host-visible buffers, HBM for device-only ones)."""
+        a = np.ascontiguousarray(arr)
+        if offset + a.nbytes > self.size:
+            raise ValueError("fill beyond the buffer")
+        if self.c.ptr and self._keep is None:
+            self.view()[offset:offset + a.nbytes] = a.view(np.uint8).ravel()
+            self.L.qw_hip_buf_mark_dirty(C.byref(self.c))
+        elif not self.L.qw_hip_buf_write(C.byref(self.c), offset, a.ctypes.data, a.nbytes):
+            raise RuntimeError("qw_hip_buf_write failed")
+
+    def read(self, nbytes=None, offset=0, dtype=np.uint8):
+        """Bytes straight from HBM (independent of the shadow rules)."""
+        n = self.size - offset if nbytes is None else nbytes
+        out = np.empty(n, np.uint8)
+        if not self.L.qw_hip_buf_read(C.byref(self.c), offset, out.ctypes.data, n):
+            raise RuntimeError("qw_hip_buf_read failed")
+        return out.view(dtype)
+
+    def free(self):
+        if self.c.handle:
+            self.L.qw_buf_free(C.byref(self.c))
+
+    def ref(self):
+        return C.byref(self.c)
+
+
+class Tensor:
+    def __init__(self, buf, ftype, offset=0):
+        self.buf, self.ftype, self.offset = buf, ftype, offset
+
+    def c(self):
+        return QwTensor(C.pointer(self.buf.c), self.offset, self.ftype)
+
+
+class MoeLayer:
+    """Weights of one layer as tensors in HBM. Fields as in include/qw_path.h."""
+
+    def __init__(self, **t):
+        self.t = t
+        self.c = QwMoeLayer(*[t[n].c() for n, _ in QwMoeLayer._fields_])
+
+
+class Batch:
+    def __init__(self, gpu, concurrent=False):
+        self.gpu, self.L = gpu, gpu.L
+        self.b = self.L.qw_batch_begin(gpu.g, concurrent)
+
+    def kernel(self, k):
+        self.L.qw_batch_kernel(self.b, k)
+
+    def buf(self, index, buf, offset=0):
+        self.L.qw_batch_buf(self.b, index, buf.ref(), offset)
+
+    def bytes(self, index, arr):
+        a = np.ascontiguousarray(arr)
+        self.L.qw_batch_bytes(self.b, index, a.ctypes.data, a.nbytes)
+
+    def dispatch(self, gx, gy=1, gz=1, tx=1, ty=1, tz=1):
+        self.L.qw_batch_dispatch(self.b, gx, gy, gz, tx, ty, tz)
+
+    def flush(self):
+        self.L.qw_batch_flush(self.b)
+
+    def end(self, check=True):
+        t = self.L.qw_batch_end(self.b)
+        self.b = None
+        if check and t < 0:
+            raise RuntimeError("GPU batch failed: " + self.gpu.last_error())
+        return t
+
+
+class Gpu:
+    def __init__(self):
+        self.L = load_lib()
+        self.g = self.L.qw_gpu_open()
+        if not self.g:
+            raise RuntimeError("qw_gpu_open: no usable gfx950 device")
+
+    def close(self):
+        if self.g:
+            self.L.qw_gpu_close(self.g)
+            self.g = None
+
+    def name(self):
+        return self.L.qw_gpu_name(self.g).decode()
+
+    def cu_count(self):
+        return self.L.qw_hip_cu_count(self.g)
+
+    def last_error(self):
+        return self.L.qw_hip_last_error(self.g).decode()
+
+    def compile(self, defs):
+        err = C.create_string_buffer(8192)
+        src = defs.encode()
+        ok = self.L.qw_gpu_compile(self.g, src, len(src), err, len(err))
+        return ok, err.value.decode()
+
+    def kernel(self, name):
+        return self.L.qw_kernel_get(self.g, name.encode())
+
+    def buf(self, size, device_only=False):
+        return Buf(self, size, device_only=device_only)
+
+    def buf_from(self, arr, device_only=False):
+        a = np.ascontiguousarray(arr)
+        b = Buf(self, max(a.nbytes, 16), device_only=device_only)
+        b.fill(a)
+        return b
+
+    def wrap(self, arr):
+        return Buf(self, arr.nbytes, wrap=arr)
+
+    def batch(self, concurrent=False):
+        return Batch(self, concurrent)
+
+    def profile(self, on):
+        self.L.qw_profile_enable(self.g, on)
+
+    def profile_entries(self):
+        out = []
+        us = C.c_double()
+        for i in range(self.L.qw_profile_count(self.g)):
+            n = self.L.qw_profile_get(self.g, i, C.byref(us))
+            out.append((n.decode(), us.value))
+        return out
+
+    def profile_mean(self, prefix):
+        n = C.c_int()
+        s = self.L.qw_hip_profile_mean(self.g, prefix.encode(), C.byref(n))
+        return s, n.value
+
+
+class Path:
+    """Host side of the path (include/qw_path.h)."""
+
+    def __init__(self, gpu, D, I, E, topk, nbmax, device_scratch=False):
+        self.gpu, self.L = gpu, gpu.L
+        self.D, self.I, self.E, self.topk, self.nbmax = D, I, E, topk, nbmax
+        self.p = self.L.qw_path_open(gpu.g, D, I, E, topk, nbmax, device_scratch)
+        if not self.p:
+            raise RuntimeError("qw_path_open failed: " + gpu.last_error())
+
+    def close(self):
+        if self.p:
+            self.L.qw_path_close(self.p)
+            self.p = None
+
+    def sel_bytes(self, nb):
+        return self.L.qw_path_sel_bytes(self.p, nb)
+
+    def logits_bytes(self, nb):
+        return self.L.qw_path_logits_bytes(self.p, nb)
+
+    def qmv_gg(self, batch, W, N, K, x, y, nb, fout=True, xoff=0, yoff=0):
+        t = W.c()
+        if not self.L.qw_path_qmv_gg(self.p, batch.b, C.byref(t), N, K, x.ref(), xoff, y.ref(), yoff, nb, fout):
+            raise RuntimeError("qw_path_qmv_gg failed")
+
+    def gg_router(self, batch, layer, nb, x, lg):
+        if not self.L.qw_path_gg_router(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref()):
+            raise RuntimeError("qw_path_gg_router failed")
+
+    def gg_moe(self, batch, layer, nb, x, lg, sel, out):
+        if not self.L.qw_path_gg_moe(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
+            raise RuntimeError("qw_path_gg_moe failed")
+
+    def scratch(self, which):
+        """0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg; returns (device bytes as uint8)."""
+        pb = self.L.qw_path_scratch(self.p, which)
+        out = np.empty(pb.contents.size, np.uint8)
+        if not self.L.qw_hip_buf_read(pb, 0, out.ctypes.data, out.nbytes):
+            raise RuntimeError("qw_hip_buf_read failed")
+        return out

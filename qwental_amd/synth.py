@@ -1,0 +1,84 @@
+"""Seeded synthetic inputs of the benchmark configurations (weights as raw GGUF blocks, activations, routing).
+
+IQ3_S block, 110 bytes: d = binary16(|N(0, 0.02)|), qs[64] / qh[8] / signs[32] uniform random bytes, scales[4]
+uniform random bytes (eight 4-bit scales). Q8_0 block, 34 bytes: d = binary16(|N(0, 0.01)|), qs uniform int8 in
+[-127, 127]. Activations binary16 N(0, 1). Router weights binary16 N(0, 0.02).
+
+One deviation, for the MoE layer only: with block scales |N(0, 0.02)| the layer's output reaches about 5e5, beyond
+binary16 (65504), and the binary16 output the interface prescribes becomes +-inf. moe_layer() therefore draws the
+block scales ten times smaller (MOE_D_SCALE); every byte other than the two scale bytes per block is unchanged, and
+so is the work the kernels do.
+"""
+import numpy as np
+
+BLOCK = {8: (32, 34), 21: (256, 110)}  # ggml type -> (values, bytes) per block
+D_SIGMA = {21: 0.02, 8: 0.01}
+MOE_D_SCALE = 0.1
+
+
+def row_bytes(ftype, K):
+    qb, bb = BLOCK[ftype]
+    assert K % qb == 0
+    return K // qb * bb
+
+
+def blocks(rng, ftype, n, d_scale=1.0):
+    """n raw blocks of the given type as uint8 [n, block_bytes]."""
+    qb, bb = BLOCK[ftype]
+    out = np.empty((n, bb), np.uint8)
+    d = np.abs(rng.normal(0.0, D_SIGMA[ftype] * d_scale, n)).astype(np.float16)
+    if ftype == 21:
+        out[:, 2:] = rng.integers(0, 256, (n, bb - 2), dtype=np.uint8)
+    else:
+        out[:, 2:] = rng.integers(-127, 128, (n, 32), dtype=np.int8).view(np.uint8)
+    out[:, :2] = d.view(np.uint8).reshape(n, 2)
+    return out
+
+
+def matrix(rng, ftype, rows, K, d_scale=1.0):
+    """rows x K quantized matrix as flat uint8 [rows * row_bytes]."""
+    qb, _ = BLOCK[ftype]
+    return blocks(rng, ftype, rows * (K // qb), d_scale).reshape(-1)
+
+
+def activations(rng, nb, K):
+    return rng.normal(0.0, 1.0, (nb, K)).astype(np.float16)
+
+
+def router(rng, E, D):
+    """(Wr [E, D], shared gate vector [D]) as binary16."""
+    return rng.normal(0.0, 0.02, (E, D)).astype(np.float16), rng.normal(0.0, 0.02, D).astype(np.float16)
+
+
+def moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21, fshd=None, experts=None, d_scale=MOE_D_SCALE):
+    """One MoE layer as a dict of numpy arrays (the field names of qwo_moe_weights / MoeLayer).
+    experts: generate only this many routed experts' bytes (the others are never read when ids are < experts)."""
+    ne = E if experts is None else experts
+    fshd = fsh if fshd is None else fshd
+    Wr, wsg = router(rng, E, D)
+    return dict(D=D, I=I, E=E, fgu=fgu, fd=fd, fsg=fsh, fsu=fsh, fsd=fshd, Wr=Wr, wsg=wsg,
+                Wg=matrix(rng, fgu, ne * I, D, d_scale), Wu=matrix(rng, fgu, ne * I, D, d_scale), Wd=matrix(rng, fd, ne * D, I, d_scale),
+                Wsg=matrix(rng, fsh, I, D, d_scale), Wsu=matrix(rng, fsh, I, D, d_scale), Wsd=matrix(rng, fshd, D, I, d_scale))
+
+
+def expert_bytes(D, I, fgu=21, fd=21):
+    return 2 * I * row_bytes(fgu, D) + D * row_bytes(fd, I)
+
+
+def zipf_ids(rng, rows, E, topk, s=1.1):
+    """Per row, topk distinct expert ids drawn without replacement with P(rank r) ~ 1 / (r + 1)^s over a seeded
+    permutation of the experts."""
+    p = 1.0 / np.arange(1, E + 1) ** s
+    p /= p.sum()
+    perm = rng.permutation(E)
+    return np.stack([perm[rng.choice(E, topk, replace=False, p=p)] for _ in range(rows)]).astype(np.uint32)
+
+
+def logits_for_ids(rng, ids, E):
+    """Router logits [rows, E + 1] whose top-k (in rank order) are exactly ids: distinct descending values on the
+    chosen experts, noise well below them elsewhere."""
+    rows, topk = ids.shape
+    lg = rng.normal(0.0, 0.1, (rows, E + 1)).astype(np.float32)
+    for t in range(rows):
+        lg[t, ids[t]] = 4.0 - 0.25 * np.arange(topk, dtype=np.float32)
+    return lg
