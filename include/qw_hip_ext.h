@@ -42,6 +42,9 @@ const char *qw_hip_arch(void);
 /* Average duration in seconds of the kernel whose entry-point name starts with `prefix`, over the dispatches of
  * the last completed batch that ran with profiling enabled; count receives how many matched. */
 double qw_hip_profile_mean(const qw_gpu *g, const char *prefix, int *count);
+/* Entry i of the last profiled batch by the code object's entry-point name (qw_profile_get gives the caller's
+ * kernel name); one entry per launch, in launch order. */
+const char *qw_hip_profile_entry(const qw_gpu *g, int i, double *us);
 
 #ifdef __cplusplus
 }

@@ -56,6 +56,10 @@ bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
 /* The whole layer: x [nb][D] binary16 -> out [nb][D] binary16; lg and sel receive the logits and the selection. */
 bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
                     const qw_buf *out);
+/* nlayers layers in a row on the same input x (the FFN stack of the benchmark): layer l writes lg[l], sel[l] and,
+ * each in turn, out. Equivalent to nlayers calls of qw_path_gg_moe. */
+bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,
+                          const qw_buf *sel, const qw_buf *out);
 /* The scratch buffers, for tests: 0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg. */
 const qw_buf *qw_path_scratch(const qw_path *p, int which);
 

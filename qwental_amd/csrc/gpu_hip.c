@@ -24,12 +24,12 @@ static const unsigned char qw_code_object[] = {
 #embed "qw_kernels_gfx950.hsaco"
 };
 
-enum { QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 2048, QW_MAX_FUNCS = 96 };
+enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 8192, QW_MAX_FUNCS = 96 };
 
 // ---------------------------------------------------------------- records
 typedef enum {
     FAM_DQ_TEST, FAM_QMV_GG, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
-    FAM_BW_READ, FAM_COPY, FAM_FILL,
+    FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
 } qw_family;
 
 typedef struct { // parameters taken from the define block
@@ -59,7 +59,7 @@ typedef struct {
     hipFunction_t f;
     const char *fname;
     unsigned gx, gy, gz, bx;
-    unsigned char args[128];
+    unsigned char args[QW_MAX_ARGS];
     size_t argsz;
     const char *kname; // caller-visible kernel name (for profiling)
     bool last_of_dispatch;
@@ -91,6 +91,7 @@ struct qw_gpu {
     size_t total_mem;
     int ncu;
     hipModule_t mod;
+    void *tabs;   // this backend's own lookup tables in HBM (QW_TAB_BYTES); the pre-signed IQ3_S table sits at QW_TAB_IQ3SS
     hipStream_t stream[2];
     int cur_stream;
     struct qw_kernel *kernels;
@@ -150,6 +151,21 @@ qw_gpu *qw_gpu_open(void) {
     for (int i = 0; i < 2; i++)
         if (hipStreamCreateWithFlags(&g->stream[i], hipStreamNonBlocking) != hipSuccess) { free(g); return NULL; }
     g->kernels = calloc(QW_MAX_KERNELS, sizeof *g->kernels);
+    { // build the pre-signed table once; every weight kernel copies it into LDS
+        hipFunction_t f;
+        qwk_tab_args ta;
+        void *params[] = {&ta};
+        if (hipMalloc(&g->tabs, QW_TAB_BYTES) != hipSuccess || hipMemset(g->tabs, 0, QW_TAB_BYTES) != hipSuccess ||
+            hipModuleGetFunction(&f, g->mod, "qwk_tab_init") != hipSuccess) { free(g->kernels); free(g); return NULL; }
+        ta.tab = g->tabs;
+        if (hipDeviceSynchronize() != hipSuccess || hipModuleLaunchKernel(f, 32, 1, 1, 256, 1, 1, 0, g->stream[0], params, NULL) != hipSuccess ||
+            hipStreamSynchronize(g->stream[0]) != hipSuccess) {
+            fprintf(stderr, "qw_gpu_open: the table kernel does not run\n");
+            free(g->kernels);
+            free(g);
+            return NULL;
+        }
+    }
     return g;
 }
 
@@ -157,6 +173,7 @@ void qw_gpu_close(qw_gpu *g) {
     if (!g) return;
     (void)hipDeviceSynchronize();
     for (int i = 0; i < 2; i++) (void)hipStreamDestroy(g->stream[i]);
+    (void)hipFree(g->tabs);
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
     free(g);
@@ -300,7 +317,7 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
     if (def_get(d, n, "QW_HIP_MEM")) { // this backend's own measurement helpers
         p = (qw_kparams){0};
         if (!reg_kernel(g, d, n, "qw_bw_read", FAM_BW_READ, &p, err, errlen) || !reg_kernel(g, d, n, "qw_copy", FAM_COPY, &p, err, errlen) ||
-            !reg_kernel(g, d, n, "qw_fill_random", FAM_FILL, &p, err, errlen)) { ok = false; goto out; }
+            !reg_kernel(g, d, n, "qw_fill_random", FAM_FILL, &p, err, errlen) || !reg_kernel(g, d, n, "qw_fill_blocks", FAM_FILL_BLOCKS, &p, err, errlen)) { ok = false; goto out; }
     }
 #undef FAIL
 out:
@@ -471,7 +488,11 @@ static bool bind_bytes(qw_batch *b, unsigned index, void *dst, size_t len, const
     return true;
 }
 
+_Static_assert(sizeof(qwk_pre_args) <= QW_MAX_ARGS && sizeof(qwk_gu_args) <= QW_MAX_ARGS && sizeof(qwk_dn_args) <= QW_MAX_ARGS && sizeof(qwk_qmv_args) <= QW_MAX_ARGS,
+               "a kernel argument record is larger than the launch record's copy of it");
+
 static bool add_launch(qw_batch *b, const char *fname, unsigned gx, unsigned bx, const void *args, size_t argsz) {
+    if (argsz > QW_MAX_ARGS) return fail(b, "%s: argument record of %zu bytes", fname, argsz);
     hipFunction_t f = get_func(b->g, fname);
     if (!f) return fail(b, "%s: entry point %s missing from the code object", b->k->name, fname);
     if (gx == 0) return true; // nothing to do
@@ -513,7 +534,6 @@ static const char *intern(const char *s) {
     return tab[n++] = strdup(s);
 }
 
-static int nb_variant(unsigned nb) { return nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : nb <= 8 ? 8 : 16; }
 
 // ---------------------------------------------------------------- family translators
 static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W, 1 y, 2 {K, row bytes}; grid = rows
@@ -526,11 +546,17 @@ static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W,
     return add_launch(b, p->F == 21 ? "qwk_dq_test_f21" : "qwk_dq_test_f8", gx, 64, &a, sizeof a);
 }
 
+static const void *glut(const qw_gpu *g) { return (const char *)g->tabs + QW_TAB_IQ3SS; }
+
+// Blocks per prefetch chunk for a row of K values (the kernels are instantiated for these; 1 = any K).
+static int chunk_of(int F, int K) { return F == 21 ? (K == 512 ? 2 : K == 2048 ? 8 : K == 2560 ? 10 : 1) : (K % 512 == 0 ? 16 : 1); }
+
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
     const qw_kparams *p = &b->k->p;
     uint32_t a4[4];
     if (!bind_bytes(b, 5, a4, sizeof a4, "{N, xstride, ystride, pad}")) return false;
-    qwk_qmv_args a = {.N = a4[0], .K = (uint32_t)p->K, .rowbytes = (uint32_t)p->RB, .xstride = a4[1], .ystride = a4[2], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat};
+    qwk_qmv_args a = {.N = a4[0], .K = (uint32_t)p->K, .rowbytes = (uint32_t)p->RB, .xstride = a4[1], .ystride = a4[2], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat,
+                      .glut = glut(b->g)};
     if (a.N == 0) return true;
     if (a.xstride < a.K || a.xstride % 8 || a.ystride < a.N) return fail(b, "qmv_gg: xstride %u (needs >= K, multiple of 8) / ystride %u (needs >= N)", a.xstride, a.ystride);
     if (b->buf[3].h && b->buf[3].off % 16) return fail(b, "qmv_gg: x offset %zu is not 16-byte aligned", b->buf[3].off);
@@ -539,25 +565,23 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
         !bind_ptr(b, 3, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x) ||
         !bind_ptr(b, 4, ((size_t)(a.nb - 1) * a.ystride + a.N) * (a.yfloat ? 4 : 2), true, "y", &a.y)) return false;
     char fn[48];
-    fname_fmt(fn, sizeof fn, "qwk_qmv_f%d%s", p->F, p->K <= 2560 ? "" : "_g");
+    if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", p->F);
+    else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", p->F, chunk_of(p->F, p->K));
     return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles), 512, &a, sizeof a);
 }
 
-static bool launch_router(qw_batch *b, unsigned iWr, unsigned iWsg, unsigned ix, unsigned ilg, uint32_t nbr) {
+static bool fill_router(qw_batch *b, qwk_router_args *a, unsigned iWr, unsigned iWsg, unsigned ix, unsigned ilg, uint32_t nbr) {
     const qw_kparams *p = &b->k->p;
-    qwk_router_args a = {.E = (uint32_t)p->E, .D = (uint32_t)p->D, .nb = nbr};
-    if (!bind_ptr(b, iWr, (size_t)p->E * p->D * 2, false, "router weights", (void **)&a.Wr) || !bind_ptr(b, iWsg, (size_t)p->D * 2, false, "shared gate vector", (void **)&a.Wsg) ||
-        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a.x) || !bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, true, "logits", (void **)&a.logits)) return false;
-    char fn[48];
-    fname_fmt(fn, sizeof fn, "qwk_router_w%d_n%d", p->rwf, nb_variant(nbr));
-    return add_launch(b, intern(fn), cdiv((unsigned)p->E + 1, 4), 256, &a, sizeof a);
+    *a = (qwk_router_args){.E = (uint32_t)p->E, .D = (uint32_t)p->D, .nb = nbr};
+    return bind_ptr(b, iWr, (size_t)p->E * p->D * 2, false, "router weights", (void **)&a->Wr) && bind_ptr(b, iWsg, (size_t)p->D * 2, false, "shared gate vector", (void **)&a->Wsg) &&
+           bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a->x) && bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, true, "logits", (void **)&a->logits);
 }
 
 static bool launch_select(qw_batch *b, unsigned ilg, unsigned isel, uint32_t nbr) {
     const qw_kparams *p = &b->k->p;
     qwk_select_args a = {.nbr = nbr, .E = (uint32_t)p->E, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
     if (!bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, false, "logits", (void **)&a.logits) || !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.sel)) return false;
-    return add_launch(b, "qwk_select", 1, 1024, &a, sizeof a);
+    return add_launch(b, "qwk_select", 1, 512, &a, sizeof a);
 }
 
 static bool nbr_ok(qw_batch *b, uint32_t nbr) {
@@ -565,32 +589,23 @@ static bool nbr_ok(qw_batch *b, uint32_t nbr) {
     return true;
 }
 
-// gate/up launch. shared: one expert at (iWg, iWu), all tokens, slot topk.
-static bool launch_gu(qw_batch *b, int F, unsigned iWg, unsigned iWu, unsigned ix, unsigned isel, unsigned iH, uint32_t nbr, bool shared) {
+// gate/up arguments. shared: one expert at (iWg, iWu), all tokens, slot topk.
+static bool fill_gu(qw_batch *b, qwk_gu_args *a, int F, unsigned iWg, unsigned iWu, unsigned ix, unsigned iH, uint32_t nbr, bool shared) {
     const qw_kparams *p = &b->k->p;
     const size_t rb = fmt_rb(F, p->D), ne = shared ? 1 : (size_t)p->E;
-    qwk_gu_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
-                     .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
-    if (!bind_ptr(b, iWg, ne * p->I * rb, false, "gate weights", (void **)&a.Wg) || !bind_ptr(b, iWu, ne * p->I * rb, false, "up weights", (void **)&a.Wu) ||
-        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a.x) || !bind_ptr(b, iH, (size_t)a.hplane * 4, true, "H", (void **)&a.H)) return false;
-    if (!shared && !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
-    const unsigned tasks = (shared ? 1u : umin((unsigned)p->E, nbr * (unsigned)p->topk)) * (unsigned)(p->I / 8);
-    return add_launch(b, F == 21 ? "qwk_gu_f21" : "qwk_gu_f8", persistent_grid(b->g, tasks), 512, &a, sizeof a);
+    *a = (qwk_gu_args){.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
+                       .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I, .glut = glut(b->g)};
+    if (!bind_ptr(b, iWg, ne * p->I * rb, false, "gate weights", (void **)&a->Wg) || !bind_ptr(b, iWu, ne * p->I * rb, false, "up weights", (void **)&a->Wu) ||
+        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a->x) || !bind_ptr(b, iH, (size_t)a->hplane * 4, true, "H", (void **)&a->H)) return false;
+    if (b->buf[ix].off % 16) return fail(b, "%s: x offset %zu is not 16-byte aligned", b->k->name, b->buf[ix].off);
+    return true;
 }
 
-static bool launch_dn(qw_batch *b, int F, unsigned iWd, unsigned iH, unsigned isel, unsigned iP, uint32_t nbr, bool shared) {
-    const qw_kparams *p = &b->k->p;
-    const size_t rb = fmt_rb(F, p->I), ne = shared ? 1 : (size_t)p->E;
-    qwk_dn_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
-                     .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
-    if (!bind_ptr(b, iWd, ne * p->D * rb, false, "down weights", (void **)&a.Wd) || !bind_ptr(b, iH, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
-        !bind_ptr(b, iP, (size_t)nbr * (shared ? 1 : p->topk) * p->D * 4, true, shared ? "Psh" : "Pg", (void **)&a.P)) return false;
-    if (!shared && !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
-    const unsigned tasks = (shared ? 1u : umin((unsigned)p->E, nbr * (unsigned)p->topk)) * (unsigned)(p->D / 64);
-    return add_launch(b, F == 21 ? "qwk_dn_f21" : "qwk_dn_f8", persistent_grid(b->g, tasks), 512, &a, sizeof a);
+static bool tr_router(qw_batch *b) { // src/engine.c:546-551; NB = token count
+    qwk_router_args a;
+    if (!fill_router(b, &a, 0, 1, 2, 3, (uint32_t)b->k->p.NB)) return false;
+    return add_launch(b, b->k->p.rwf == 30 ? "qwk_router_w30" : "qwk_router_w1", cdiv((unsigned)b->k->p.E + 1, 4), 256, &a, sizeof a);
 }
-
-static bool tr_router(qw_batch *b) { return launch_router(b, 0, 1, 2, 3, (uint32_t)b->k->p.NB); } // src/engine.c:546-551; NB = token count
 
 static bool tr_tab_init(qw_batch *b) { // src/engine.c:572-574
     qwk_tab_args a;
@@ -604,27 +619,67 @@ static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nb
 }
 
 // src/engine.c:588-607: 0 Wr, 1 shared gate vector, 2 x, 3 logits, 4 counter, 5 sel, 6/7 shared gate/up, 8 H, 13 tables, 14 nbr.
-// Here: router launch, then selection, then the shared expert's gate/up; the counter buffer is not used.
+// One launch: router rows and the shared expert's gate/up side by side, the selection by the last router workgroup.
 static bool tr_pre(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     uint32_t nbr;
     if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
-    if (p->rbf && (!launch_router(b, 0, 1, 2, 3, nbr) || !launch_select(b, 3, 5, nbr))) return false;
-    return launch_gu(b, p->fsg, 6, 7, 2, 5, 8, nbr, true);
+    qwk_pre_args a = {0};
+    if (!fill_gu(b, &a.g, p->fsg, 6, 7, 2, 8, nbr, true)) return false;
+    char fn[64];
+    const unsigned gu_wg = cdiv((unsigned)p->I / 8, 8);
+    if (!p->rbf) { // router and selection come as dispatches of their own: only the shared expert's gate/up here
+        fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", p->fsg, chunk_of(p->fsg, p->D));
+        return add_launch(b, intern(fn), gu_wg, 512, &a.g, sizeof a.g);
+    }
+    if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
+    if (!bind_ptr(b, 5, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.g.sel) || !bind_ptr(b, 4, 4, true, "counter", (void **)&a.cnt)) return false;
+    a.nrouter_wg = cdiv((unsigned)p->E + 1, 8);
+    a.do_select = 1;
+    fname_fmt(fn, sizeof fn, "qwk_pre_w%d_f%d_c%d", p->rwf, p->fsg, chunk_of(p->fsg, p->D));
+    return add_launch(b, intern(fn), a.nrouter_wg + gu_wg, 512, &a, sizeof a);
 }
 
-// src/engine.c:616-629: 0 Wg, 1 Wu, 2 shared down, 3 Psh, 4 x, 5 sel, 6 H, 11 tables, 12 nbr
+// src/engine.c:616-629: 0 Wg, 1 Wu, 2 shared down, 3 Psh, 4 x, 5 sel, 6 H, 11 tables, 12 nbr.
+// One launch: routed gate/up tiles for the selected experts and the shared expert's down tiles.
 static bool tr_gu(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     uint32_t nbr;
     if (!bind_bytes(b, 12, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
-    return launch_gu(b, p->fgu, 0, 1, 4, 5, 6, nbr, false) && launch_dn(b, p->fsd, 2, 6, 5, 3, nbr, true);
+    qwk_gu_args a;
+    if (!fill_gu(b, &a, p->fgu, 0, 1, 4, 6, nbr, false)) return false;
+    if (!bind_ptr(b, 5, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
+    a.sd_rowbytes = (uint32_t)fmt_rb(p->fsd, p->I);
+    if (!bind_ptr(b, 2, (size_t)p->D * a.sd_rowbytes, false, "shared down weights", (void **)&a.Wsd) || !bind_ptr(b, 3, (size_t)nbr * p->D * 4, true, "Psh", (void **)&a.Psh)) return false;
+    // the instantiated pairs: fast shapes (D 2048 / I 512), D 2560, or the any-shape build
+    const int cg = chunk_of(p->fgu, p->D);
+    const bool fast = (p->fgu == 21 ? cg == 8 : cg == 16) && chunk_of(p->fsd, p->I) == (p->fsd == 21 ? 2 : 16);
+    char fn[64];
+    if (fast) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_sd%d_c%d", p->fgu, cg, p->fsd, chunk_of(p->fsd, p->I));
+    else if (p->fgu == 21 && cg == 10) fname_fmt(fn, sizeof fn, "qwk_gu_f21_c10_sd%d_c1", p->fsd);
+    else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c1_sd%d_c1", p->fgu, p->fsd);
+    const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (unsigned)p->D / 16;
+    return add_launch(b, intern(fn), persistent_grid(b->g, tasks), 512, &a, sizeof a);
 }
 
 // src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
 static bool tr_dn(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
-    return launch_dn(b, p->fd, 0, 2, 3, 9, (uint32_t)p->NB, false);
+    const uint32_t nbr = (uint32_t)p->NB;
+    const size_t rb = fmt_rb(p->fd, p->I);
+    qwk_dn_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = 0,
+                     .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I, .glut = glut(b->g)};
+    if (!bind_ptr(b, 0, (size_t)p->E * p->D * rb, false, "down weights", (void **)&a.Wd) || !bind_ptr(b, 2, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
+        !bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, true, "Pg", (void **)&a.P) ||
+        !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
+    const unsigned umax = umin((unsigned)p->E, nbr * (unsigned)p->topk);
+    char fn[48];
+    if (p->I == 512 && p->fd == 21) { // workgroup tasks of 256 rows
+        fname_fmt(fn, sizeof fn, "qwk_dn_f%d_i512", p->fd);
+        return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, umax * (unsigned)(p->D / 256)), 512, &a, sizeof a);
+    }
+    fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any", p->fd);
+    return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16)), 512, &a, sizeof a);
 }
 
 // src/engine.c:640-646: 1 Psh, 3 sel, 4 out, 8 nbr, 9 Pg
@@ -649,6 +704,18 @@ static bool tr_mem(qw_batch *b, unsigned gx) {
     return add_launch(b, f == FAM_BW_READ ? "qwk_bw_read" : f == FAM_COPY ? "qwk_copy" : "qwk_fill_random", gx, 256, &a, sizeof a);
 }
 
+// synthetic weights: 1 dst (+ offset), 2 {nblocks (uint64), seed (uint64), type (uint32), sigma (float)}
+static bool tr_fill_blocks(qw_batch *b) {
+    struct { uint64_t nblocks, seed; uint32_t type; float sigma; } in;
+    if (!bind_bytes(b, 2, &in, sizeof in, "{nblocks, seed, type, sigma}")) return false;
+    if (!fmt_ok((int)in.type)) return fail(b, "qw_fill_blocks: type %u", in.type);
+    qwk_fill_args a = {.nblocks = in.nblocks, .seed = in.seed, .type = in.type, .sigma = in.sigma};
+    if (!bind_ptr(b, 1, (size_t)in.nblocks * (size_t)fmt_bb((int)in.type), true, "dst", (void **)&a.dst)) return false;
+    if (b->buf[1].off % 2) return fail(b, "qw_fill_blocks: odd offset");
+    const uint64_t wg = (in.nblocks + 255) / 256;
+    return add_launch(b, "qwk_fill_blocks", (unsigned)(wg < 65536 ? wg : 65536), 256, &a, sizeof a);
+}
+
 void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsigned tx, unsigned ty, unsigned tz) {
     (void)gy; (void)gz; (void)tx; (void)ty; (void)tz;
     if (b->failed) return;
@@ -665,6 +732,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     case FAM_GU: ok = tr_gu(b); break;
     case FAM_DN: ok = tr_dn(b); break;
     case FAM_CMB: ok = tr_cmb(b); break;
+    case FAM_FILL_BLOCKS: ok = tr_fill_blocks(b); break;
     default: ok = tr_mem(b, gx);
     }
     if (ok && b->nl > first) b->l[b->nl - 1].last_of_dispatch = true;
@@ -692,20 +760,17 @@ static bool submit_segment(qw_batch *b) {
     if (!HIPOK(g, hipEventCreate(&ev[0])) || !HIPOK(g, hipEventCreate(&ev[1]))) { b->failed = true; return false; }
     b->nseg++;
     if (!HIPOK(g, hipEventRecord(ev[0], st))) { b->failed = true; return false; }
-    bool open = false; // profiling: an event pair brackets the launches of one dispatch
     for (int i = b->done_l; i < b->nl; i++) {
         qw_launch *l = &b->l[i];
-        if (b->prof && !open) {
+        if (b->prof) { // an event pair brackets every launch
             b->pev = realloc(b->pev, sizeof *b->pev * (size_t)(b->npev + 2));
             if (!HIPOK(g, hipEventCreate(&b->pev[b->npev])) || !HIPOK(g, hipEventCreate(&b->pev[b->npev + 1])) || !HIPOK(g, hipEventRecord(b->pev[b->npev], st))) { b->failed = true; return false; }
-            open = true;
         }
         void *params[] = {l->args}; // every kernel takes one record by value
         if (!HIPOK(g, hipModuleLaunchKernel(l->f, l->gx, l->gy, l->gz, l->bx, 1, 1, 0, st, params, NULL))) { b->failed = true; return false; }
-        if (b->prof && (l->last_of_dispatch || i + 1 == b->nl)) {
+        if (b->prof) {
             if (!HIPOK(g, hipEventRecord(b->pev[b->npev + 1], st))) { b->failed = true; return false; }
             b->npev += 2;
-            open = false;
         }
     }
     if (!HIPOK(g, hipEventRecord(ev[1], st))) { b->failed = true; return false; }
@@ -773,12 +838,9 @@ double qw_batch_wait(qw_batch *b) {
     }
     if (ok && b->prof) {
         g->nprof = 0;
-        int e = 0;
-        for (int i = 0; i < b->nl && g->nprof < QW_PROF_MAX && e + 1 < b->npev; i++) {
-            if (!b->l[i].last_of_dispatch && i + 1 != b->nl) continue;
+        for (int i = 0; i < b->nl && g->nprof < QW_PROF_MAX && 2 * i + 1 < b->npev; i++) {
             float ms = 0;
-            (void)hipEventElapsedTime(&ms, b->pev[e], b->pev[e + 1]);
-            e += 2;
+            (void)hipEventElapsedTime(&ms, b->pev[2 * i], b->pev[2 * i + 1]);
             g->prof_name[g->nprof] = b->l[i].kname;
             g->prof_fname[g->nprof] = b->l[i].fname;
             g->prof_us[g->nprof++] = (double)ms * 1e3;
@@ -806,6 +868,11 @@ const char *qw_profile_get(const qw_gpu *g, int i, double *us) {
     if (i < 0 || i >= g->nprof) return NULL;
     if (us) *us = g->prof_us[i];
     return g->prof_name[i];
+}
+const char *qw_hip_profile_entry(const qw_gpu *g, int i, double *us) {
+    if (i < 0 || i >= g->nprof) return NULL;
+    if (us) *us = g->prof_us[i];
+    return g->prof_fname[i];
 }
 double qw_hip_profile_mean(const qw_gpu *g, const char *prefix, int *count) {
     double s = 0;

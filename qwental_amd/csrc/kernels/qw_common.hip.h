@@ -123,6 +123,15 @@ struct qw_afrag_lds {
     __device__ __forceinline__ h8 lo(uint32_t) const { return h8{}; }
 };
 
+// Two planes (hi + lo) staged the same way.
+struct qw_afrag_lds2 {
+    const u4 *hi_, *lo_;
+    uint32_t m;
+    static constexpr bool has_lo = true;
+    __device__ __forceinline__ h8 hi(uint32_t koff) const { return __builtin_bit_cast(h8, hi_[(koff >> 3) * 16 + m]); }
+    __device__ __forceinline__ h8 lo(uint32_t koff) const { return __builtin_bit_cast(h8, lo_[(koff >> 3) * 16 + m]); }
+};
+
 __device__ __forceinline__ void qw_stage_x(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
     for (uint32_t i = threadIdx.x; i < (K >> 3) * 16; i += blockDim.x) {
         const uint32_t c = i >> 4, m = i & 15;
@@ -140,61 +149,120 @@ template <bool LO> struct qw_afrag_glb {
     __device__ __forceinline__ h8 lo(uint32_t koff) const { return rowlo ? *(const h8 *)(rowlo + koff) : h8{}; }
 };
 
-// ---------------------------------------------------------------- one 16-row tile over the whole K
-template <int F> struct qw_tile;
+// ---------------------------------------------------------------- chunks: the unit of prefetch
+// A chunk is NB consecutive blocks of one weight row, held in registers by the lane that decodes them. Kernels keep
+// two chunks per wave: while one is decoded and multiplied, the loads of the next are in flight. With 8 waves per
+// compute unit and 14 KB per wave in flight (IQ3_S, 16 rows of K = 2048) this covers the HBM latency.
+template <int F, int NB> struct qw_chunk;
 
-template <> struct qw_tile<21> {
-    template <int J, class AF> static __device__ __forceinline__ void step(const qw_iq3_slice &s, const u2 *lut, const AF &af, uint32_t k0, f4 &sub) {
-        const h8 b = qw_iq3_step<J>(s, lut);
-        sub = qw_mfma(af.hi(k0 + 8 * J), b, sub);
-        if (AF::has_lo) sub = qw_mfma(af.lo(k0 + 8 * J), b, sub);
+template <int NB> struct qw_chunk<21, NB> {
+    static constexpr uint32_t BLK_K = 256, BLK_B = 110;
+    qw_iq3_slice s[NB];
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t kg) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) s[b] = qw_iq3_load(p + 110 * b, kg);
     }
-    // row: this lane's weight row; K multiple of 256.
-    template <class AF> static __device__ __forceinline__ f4 run(const uint8_t *row, uint32_t K, uint32_t kg, const u2 *lut, const AF &af) {
-        f4 acc = {0, 0, 0, 0};
-        const uint32_t nblk = K >> 8;
-        qw_iq3_slice cur = qw_iq3_load(row, kg);
-        for (uint32_t blk = 0; blk < nblk; blk++) {
-            const qw_iq3_slice s = cur;
-            if (blk + 1 < nblk) cur = qw_iq3_load(row + 110 * (blk + 1), kg); // next block's bytes are in flight while this one is decoded
-            const uint32_t k0 = 256 * blk + 64 * kg;
+    template <int J, class AF> __device__ __forceinline__ void step(int b, const u2 *lut, const AF &af, uint32_t k0, f4 &sub) const {
+        const h8 w = qw_iq3_step<J>(s[b], lut);
+        sub = qw_mfma(af.hi(k0 + 8 * J), w, sub);
+        if (AF::has_lo) sub = qw_mfma(af.lo(k0 + 8 * J), w, sub);
+    }
+    // acc += this chunk's contribution; k0 = k-offset of the chunk's first value.
+    template <class AF> __device__ __forceinline__ void mac(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
             f4 sub = {0, 0, 0, 0};
-            step<0>(s, lut, af, k0, sub);
-            step<1>(s, lut, af, k0, sub);
-            step<2>(s, lut, af, k0, sub);
-            step<3>(s, lut, af, k0, sub);
-            step<4>(s, lut, af, k0, sub);
-            step<5>(s, lut, af, k0, sub);
-            step<6>(s, lut, af, k0, sub);
-            step<7>(s, lut, af, k0, sub);
-            acc += s.d * sub;
+            step<0>(b, lut, af, kb, sub);
+            step<1>(b, lut, af, kb, sub);
+            step<2>(b, lut, af, kb, sub);
+            step<3>(b, lut, af, kb, sub);
+            step<4>(b, lut, af, kb, sub);
+            step<5>(b, lut, af, kb, sub);
+            step<6>(b, lut, af, kb, sub);
+            step<7>(b, lut, af, kb, sub);
+            acc += s[b].d * sub;
         }
-        return acc;
     }
 };
 
-template <> struct qw_tile<8> {
-    // K multiple of 32; lut unused.
-    template <class AF> static __device__ __forceinline__ f4 run(const uint8_t *row, uint32_t K, uint32_t kg, const u2 *, const AF &af) {
-        f4 acc = {0, 0, 0, 0};
-        const uint32_t nblk = K >> 5;
-        u2 q = *(const u2a2 *)(row + 2 + 8 * kg);
-        float d = qw_h2f(*(const uint16_t *)row);
-#pragma unroll 4
-        for (uint32_t blk = 0; blk < nblk; blk++) {
-            const u2 qc = q;
-            const float dc = d;
-            if (blk + 1 < nblk) {
-                q = *(const u2a2 *)(row + 34 * (blk + 1) + 2 + 8 * kg);
-                d = qw_h2f(*(const uint16_t *)(row + 34 * (blk + 1)));
-            }
-            const h8 b = qw_q8_cvt(qc);
-            const uint32_t k0 = 32 * blk + 8 * kg;
-            f4 sub = {0, 0, 0, 0};
-            sub = qw_mfma(af.hi(k0), b, sub);
-            if (AF::has_lo) sub = qw_mfma(af.lo(k0), b, sub);
-            acc += dc * sub;
+template <int NB> struct qw_chunk<8, NB> {
+    static constexpr uint32_t BLK_K = 32, BLK_B = 34;
+    u2 q[NB];
+    uint16_t d[NB];
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t kg) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            q[b] = *(const u2a2 *)(p + 34 * b + 2 + 8 * kg);
+            d[b] = *(const uint16_t *)(p + 34 * b);
         }
-        return acc;
+    }
+    template <class AF> __device__ __forceinline__ void mac(const u2 *, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const h8 w = qw_q8_cvt(q[b]);
+            const uint32_t kb = k0 + 32 * b + 8 * kg;
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(af.hi(kb), w, sub);
+            if (AF::has_lo) sub = qw_mfma(af.lo(kb), w, sub);
+            acc += qw_h2f(d[b]) * sub;
+        }
     }
 };
+
+// Blocks per chunk for a row of K values: the whole row for IQ3_S (K <= 2560), 16 blocks for Q8_0. 0 = no build.
+template <int F> __host__ __device__ constexpr int qw_chunk_blocks(int K) { return F == 21 ? (K == 512 ? 2 : K == 2048 ? 8 : K == 2560 ? 10 : 0) : (K % 512 == 0 ? 16 : 0); }
+
+// Two-chunk software pipeline over n items: load(i, chunk&) issues the loads of item i, use(i, chunk&) consumes them.
+template <class C, class L, class U> __device__ __forceinline__ void qw_pipeline(uint32_t n, L load, U use) {
+    C a, b;
+    if (n) load(0u, a);
+    uint32_t i = 0;
+    while (i < n) {
+        if (i + 1 < n) load(i + 1, b);
+        use(i, a);
+        if (++i >= n) break;
+        if (i + 1 < n) load(i + 1, a);
+        use(i, b);
+        ++i;
+    }
+}
+
+// Copy the 64 KB pre-signed table from global memory into LDS (all loads first, then the stores).
+__device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
+    const u4 *src = (const u4 *)glut;
+    u4 *dst = (u4 *)lut;
+    constexpr uint32_t N = QW_LUT_BYTES / 16;
+    for (uint32_t i = threadIdx.x; i < N; i += 8 * blockDim.x) {
+        u4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) v[j] = src[i + j * blockDim.x];
+#pragma unroll
+        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) dst[i + j * blockDim.x] = v[j];
+    }
+}
+
+// ---------------------------------------------------------------- wave-wide maximum of an unsigned key
+// DPP row shifts inside each row of 16 lanes, then the two row broadcasts of the gfx9 family; every lane receives
+// the result through a read of lane 63.
+__device__ __forceinline__ uint32_t qw_wave_max_u32(uint32_t v) {
+#define QW_DPP_MAX(ctrl, rmask, bmask) v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ctrl, rmask, bmask, false))
+    QW_DPP_MAX(0x111, 0xf, 0xf); // row_shr:1
+    QW_DPP_MAX(0x112, 0xf, 0xf); // row_shr:2
+    QW_DPP_MAX(0x114, 0xf, 0xf); // row_shr:4
+    QW_DPP_MAX(0x118, 0xf, 0xf); // row_shr:8  -> lane 15 of each row holds the row maximum
+    QW_DPP_MAX(0x142, 0xa, 0xf); // row_bcast:15 into rows 1 and 3
+    QW_DPP_MAX(0x143, 0xc, 0xf); // row_bcast:31 into rows 2 and 3 -> lane 63 holds the wave maximum
+#undef QW_DPP_MAX
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+// Order-preserving map float -> uint32 (larger float = larger key); -0.0 is taken as +0.0 so that the two tie.
+__device__ __forceinline__ uint32_t qw_fkey(float f) {
+    uint32_t b = __builtin_bit_cast(uint32_t, f);
+    if (b == 0x80000000u) b = 0;
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ __forceinline__ float qw_fkey_inv(uint32_t k) {
+    const uint32_t b = k ^ ((k >> 31) ? 0x80000000u : 0xffffffffu);
+    return __builtin_bit_cast(float, b);
+}

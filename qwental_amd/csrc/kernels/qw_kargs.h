@@ -31,6 +31,7 @@ typedef struct { /* dense matvec, y[b][row] = W[row] . x[b] */
     const uint16_t *x; /* binary16 [nb][xstride] */
     void *y;           /* binary16 or float [nb][ystride] */
     uint32_t N, K, rowbytes, xstride, ystride, nb, yfloat, ntiles;
+    const void *glut; /* the backend's pre-signed IQ3_S table in global memory (64 KB) */
 } qwk_qmv_args;
 
 typedef struct { /* router: logits[t][r], r in [0, E] (row E = shared gate vector), row stride E + 1 */
@@ -58,6 +59,11 @@ typedef struct {
     const uint8_t *sel;
     uint16_t *H;
     uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane; /* hplane: halves between the hi and lo planes */
+    const void *glut;
+    /* shared expert's down projection, done by the same launch when Wsd != NULL: Psh[t][row] from slot topk */
+    const uint8_t *Wsd;
+    float *Psh;
+    uint32_t sd_rowbytes, pad;
 } qwk_gu_args;
 
 /* down projection. routed: Pg[t][slot][row] for the tokens in mask[u]; shared != 0: Psh[t][row] from slot topk. */
@@ -67,7 +73,17 @@ typedef struct {
     const uint8_t *sel;
     float *P; /* Pg [nbr][topk][D] or Psh [nbr][D] */
     uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane;
+    const void *glut;
 } qwk_dn_args;
+
+/* front part of a layer in one launch: router rows, the shared expert's gate/up, and the selection, which the
+ * last router workgroup to finish performs (counter in cnt, left at zero). */
+typedef struct {
+    qwk_router_args r;
+    qwk_gu_args g;      /* shared == 1 */
+    uint32_t *cnt;
+    uint32_t nrouter_wg, do_select;
+} qwk_pre_args;
 
 typedef struct { /* out[t][row] = half(sum_s w[t][s] * Pg[t][s][row] + w[t][topk] * Psh[t][row]) */
     const float *Pg, *Psh;
@@ -82,3 +98,10 @@ typedef struct { /* pure-read ceiling and fill helpers */
     uint64_t n; /* 16-byte units */
     uint64_t seed;
 } qwk_mem_args;
+
+typedef struct { /* synthetic weights: nblocks GGUF blocks of one type, scale d = binary16(|N(0, sigma)|), the rest uniform */
+    uint8_t *dst;
+    uint64_t nblocks, seed;
+    uint32_t type; /* 8 or 21 */
+    float sigma;
+} qwk_fill_args;

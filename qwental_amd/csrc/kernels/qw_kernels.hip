@@ -1,5 +1,10 @@
 // HIP kernels of the quantized decode path for gfx950. One code object; gpu_hip.c loads it and launches these
 // entry points by name. Each kernel takes one argument record from qw_kargs.h by value.
+//
+// Shape of the weight-streaming kernels (dense matvec, gate/up, down): persistent workgroups of 512 threads, one
+// per compute unit (the 64 KB pre-signed table plus the staged activations fill most of the 160 KB LDS). Each wave
+// walks its own list of 16-row tiles through a two-chunk register pipeline: the loads of the next chunk are issued
+// before the current one is decoded, so every wave keeps about one tile of weight bytes in flight.
 #include "qw_common.hip.h"
 
 #define QW_WG 512          // threads per workgroup of the weight-streaming kernels (8 waves)
@@ -7,6 +12,7 @@
 
 __device__ __forceinline__ uint32_t qw_wave() { return threadIdx.x >> 6; }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
+__device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
 // ================================================================ dq_test (kernels/moe_iq.metal:208-217)
 // rows x K values to float, decoded with the same step decoders the matrix-core kernels use. Grid: rows x 64.
@@ -50,64 +56,65 @@ extern "C" __global__ void qwk_tab_init(qwk_tab_args a) {
 
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
 // y[b][row] = sum_k W[row][k] x[b][k] for up to 16 activations; the weights are streamed once for all of them.
-// Tiles of 16 rows are dealt round-robin to the waves of a persistent grid.
-template <int F, bool XLDS> __device__ __forceinline__ void qmv_body(const qwk_qmv_args &a, const u2 *lut, u4 *xf) {
+// Tiles of 16 rows are dealt round-robin to the waves of a persistent grid; a row is CPR chunks of CH blocks.
+template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(const qwk_qmv_args &a, u2 *lut, u4 *xf) {
+    typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t cpr = a.K / (C::BLK_K * CH), mytiles = w0 < a.ntiles ? (a.ntiles - w0 + nw - 1) / nw : 0;
+    auto rowp = [&](uint32_t t) {
+        const uint32_t r = 16 * t + n;
+        return a.W + (size_t)(r < a.N ? r : a.N - 1) * a.rowbytes;
+    };
+    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
     if (XLDS) qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
     __syncthreads();
-    const uint32_t nw = gridDim.x * (blockDim.x >> 6);
-    for (uint32_t t = blockIdx.x * (blockDim.x >> 6) + qw_wave(); t < a.ntiles; t += nw) {
-        const uint32_t r = 16 * t + n, rc = r < a.N ? r : a.N - 1;
-        const uint8_t *row = a.W + (size_t)rc * a.rowbytes;
-        f4 acc;
-        if (XLDS) {
-            const qw_afrag_lds af = {xf, n};
-            acc = qw_tile<F>::run(row, a.K, kg, lut, af);
-        } else {
-            const qw_afrag_glb<false> ho = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
-            acc = qw_tile<F>::run(row, a.K, kg, lut, ho);
-        }
-        if (r < a.N)
+    const qw_afrag_lds afl = {xf, n};
+    const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
+    f4 acc = {0, 0, 0, 0};
+    qw_pipeline<C>(mytiles * cpr,
+        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, const C &c) {
+            const uint32_t ci = i % cpr;
+            if (XLDS) c.mac(lut, afl, ci * CH * C::BLK_K, kg, acc);
+            else c.mac(lut, afg, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 == cpr) {
+                const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
+                if (r < a.N)
 #pragma unroll
-            for (uint32_t i = 0; i < 4; i++) {
-                const uint32_t tok = 4 * kg + i;
-                if (tok < a.nb) {
-                    if (a.yfloat) ((float *)a.y)[(size_t)tok * a.ystride + r] = acc[i];
-                    else ((uint16_t *)a.y)[(size_t)tok * a.ystride + r] = qw_f2h(acc[i]);
-                }
+                    for (uint32_t j = 0; j < 4; j++) {
+                        const uint32_t tok = 4 * kg + j;
+                        if (tok < a.nb) {
+                            if (a.yfloat) ((float *)a.y)[(size_t)tok * a.ystride + r] = acc[j];
+                            else ((uint16_t *)a.y)[(size_t)tok * a.ystride + r] = qw_f2h(acc[j]);
+                        }
+                    }
+                acc = f4{0, 0, 0, 0};
             }
+        });
+}
+#define QW_QMV(F, CH, XLDS, SFX)                                                                        \
+    extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
+        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                                                \
+        __shared__ u4 xf[XLDS ? QW_XF_MAXK * 2 : 1];                                                    \
+        qmv_body<F, CH, XLDS>(a, lut, xf);                                                              \
     }
-}
-
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f21(qwk_qmv_args a) {
-    __shared__ u2 lut[QW_LUT_ENTRIES];
-    __shared__ u4 xf[QW_XF_MAXK * 2];
-    qw_lut_build(lut);
-    qmv_body<21, true>(a, lut, xf);
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f21_g(qwk_qmv_args a) { // K too long for LDS staging
-    __shared__ u2 lut[QW_LUT_ENTRIES];
-    qw_lut_build(lut);
-    qmv_body<21, false>(a, lut, nullptr);
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f8(qwk_qmv_args a) {
-    __shared__ u4 xf[QW_XF_MAXK * 2];
-    qmv_body<8, true>(a, nullptr, xf);
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f8_g(qwk_qmv_args a) { qmv_body<8, false>(a, nullptr, nullptr); }
+QW_QMV(21, 8, true, _c8) QW_QMV(21, 2, true, _c2) QW_QMV(21, 10, true, _c10) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
+QW_QMV(8, 16, true, _c16) QW_QMV(8, 1, true, _c1) QW_QMV(8, 1, false, _c1g)
 
 // ================================================================ router (kernels/moe_gg.metal:25-41)
-// logits[t][r] = Wr[r] . x[t] in binary32, one wave per row; a token's sum order does not depend on nb.
-// WF: 1 = binary16 weights, 30 = bfloat16 weights. Grid: ceil((E + 1) / 4) x 256.
-template <int WF, int NB> __device__ __forceinline__ void router_body(const qwk_router_args &a) {
-    const uint32_t r = blockIdx.x * (blockDim.x >> 6) + qw_wave(), lane = qw_lane();
-    if (r > a.E) return;
+// logits[t][r] = Wr[r] . x[t] in binary32, one wave per row; a token's sum order does not depend on nb: explicit
+// fused multiply-adds in index order per lane, then a fixed butterfly. WF: 1 = binary16 weights, 30 = bfloat16.
+template <int WF, int NB> __device__ __forceinline__ void router_row(const qwk_router_args &a, uint32_t r, uint32_t lane) {
     const uint16_t *w = r < a.E ? a.Wr + (size_t)r * a.D : a.Wsg;
     float acc[NB];
 #pragma unroll
     for (int t = 0; t < NB; t++) acc[t] = 0;
     for (uint32_t c = lane; c < a.D / 8; c += 64) {
         const u4 wv = *(const u4 *)(w + 8 * c);
+        h8 xv[NB];
+#pragma unroll
+        for (int t = 0; t < NB; t++) xv[t] = *(const h8 *)(a.x + (size_t)((uint32_t)t < a.nb ? t : a.nb - 1) * a.D + 8 * c); // all loads first
         float wf[8];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -116,11 +123,8 @@ template <int WF, int NB> __device__ __forceinline__ void router_body(const qwk_
         }
 #pragma unroll
         for (int t = 0; t < NB; t++)
-            if ((uint32_t)t < a.nb) {
-                const h8 xv = *(const h8 *)(a.x + (size_t)t * a.D + 8 * c);
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[t] += wf[i] * (float)xv[i];
-            }
+            for (int i = 0; i < 8; i++) acc[t] = __builtin_fmaf(wf[i], (float)xv[t][i], acc[t]);
     }
 #pragma unroll
     for (int t = 0; t < NB; t++) {
@@ -130,179 +134,393 @@ template <int WF, int NB> __device__ __forceinline__ void router_body(const qwk_
         if (lane == 0 && (uint32_t)t < a.nb) a.logits[(size_t)t * (a.E + 1) + r] = v;
     }
 }
-#define QW_ROUTER(WF, NB) \
-    extern "C" __global__ __launch_bounds__(256) void qwk_router_w##WF##_n##NB(qwk_router_args a) { router_body<WF, NB>(a); }
-QW_ROUTER(1, 1) QW_ROUTER(1, 2) QW_ROUTER(1, 4) QW_ROUTER(1, 8) QW_ROUTER(1, 16)
-QW_ROUTER(30, 1) QW_ROUTER(30, 2) QW_ROUTER(30, 4) QW_ROUTER(30, 8) QW_ROUTER(30, 16)
+template <int WF> __device__ __forceinline__ void router_rows(const qwk_router_args &a, uint32_t r, uint32_t lane) {
+    if (r > a.E) return;
+    if (a.nb <= 1) router_row<WF, 1>(a, r, lane);
+    else if (a.nb <= 2) router_row<WF, 2>(a, r, lane);
+    else if (a.nb <= 4) router_row<WF, 4>(a, r, lane);
+    else if (a.nb <= 8) router_row<WF, 8>(a, r, lane);
+    else router_row<WF, 16>(a, r, lane);
+}
+extern "C" __global__ __launch_bounds__(256) void qwk_router_w1(qwk_router_args a) { router_rows<1>(a, blockIdx.x * 4 + qw_wave(), qw_lane()); }
+extern "C" __global__ __launch_bounds__(256) void qwk_router_w30(qwk_router_args a) { router_rows<30>(a, blockIdx.x * 4 + qw_wave(), qw_lane()); }
 
 // ================================================================ selection + dedupe (kernels/moe_gg.metal:123-189)
-// One workgroup of 1024 threads; wave t picks the top-k of token t (ties to the lowest expert index), computes the
-// softmax over the picked logits in rank order and the shared-expert sigmoid; then the nbr * topk picks are
-// deduplicated in order of first appearance. E <= 1024, topk <= 16, gnb in {8, 16}.
-#define QW_SEL_MAXE 1024
-extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a) {
-    __shared__ float lg[16][QW_SEL_MAXE];
-    __shared__ uint32_t ids[256], lead[256], first[QW_SEL_MAXE], um[256];
-    __shared__ uint32_t s_U;
-    const uint32_t tid = threadIdx.x, wave = qw_wave(), lane = qw_lane();
+// Per token (one wave): top-k by repeated maximum with ties to the lowest expert index, softmax over the picked logits
+// in rank order, sigmoid of the shared-expert logit; then the nbr * topk picks are deduplicated in order of first
+// appearance over the flat index. Scratch in LDS: ids[256], lead[256], um[256], first[1024], one counter.
+struct qw_sel_scratch {
+    uint32_t ids[256], lead[256], um[256], first[1024], U;
+};
+
+// PER = E / 64 values per lane, lane l holding experts l * PER .. l * PER + PER - 1 (lowest lane = lowest index).
+template <int PER> __device__ __forceinline__ void select_token(const float *lg, uint32_t E, uint32_t K, uint32_t tok, float *w, uint32_t *ids, uint32_t lane) {
+    uint32_t k[PER];
+#pragma unroll
+    for (int j = 0; j < PER; j++) k[j] = qw_fkey(lg[lane * PER + j]);
+    uint32_t pk = 0;
+    for (uint32_t r = 0; r < K; r++) {
+        uint32_t bk = k[0], bj = 0;
+#pragma unroll
+        for (int j = 1; j < PER; j++)
+            if (k[j] > bk) { bk = k[j]; bj = j; } // strict: the lowest j among equals
+        const uint32_t m = qw_wave_max_u32(bk);
+        const uint32_t L = (uint32_t)__builtin_ctzll(__ballot(bk == m)); // lowest lane among equals
+        const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)bj, (int)L);
+        if (lane == 0) ids[tok * K + r] = L * PER + j;
+        if (lane == r) pk = m;
+#pragma unroll
+        for (int jj = 0; jj < PER; jj++)
+            if (lane == L && (uint32_t)jj == j) k[jj] = 0; // below every key, -inf included
+    }
+    const float p = qw_fkey_inv(pk), mx = __shfl(p, 0), ex = __expf(p - mx);
+    float sm = 0;
+    for (uint32_t r = 0; r < K; r++) sm += __shfl(ex, r); // rank order
+    if (lane < K) w[tok * (K + 1) + lane] = ex / sm;
+    if (lane == K) w[tok * (K + 1) + K] = 1.0f / (1.0f + __expf(-lg[E]));
+}
+
+// Any E <= 1024: the values live in LDS (v, E floats); lane l scans experts l, l + 64, ...
+__device__ __forceinline__ void select_token_any(const float *lg, float *v, uint32_t E, uint32_t K, uint32_t tok, float *w, uint32_t *ids, uint32_t lane) {
+    for (uint32_t e = lane; e < E; e += 64) v[e] = lg[e];
+    float pk = 0;
+    for (uint32_t r = 0; r < K; r++) {
+        float bv = -INFINITY;
+        uint32_t bi = 0xffffffffu;
+        for (uint32_t e = lane; e < E; e += 64) {
+            const float x = v[e];
+            if (x > bv || bi == 0xffffffffu) { bv = x; bi = e; }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o);
+            const uint32_t oi = __shfl_xor(bi, o);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) ids[tok * K + r] = bi;
+        if (lane == r) pk = bv;
+        if ((bi & 63) == lane) v[bi] = -INFINITY; // only the owning lane ever reads this element again
+    }
+    const float mx = __shfl(pk, 0), ex = __expf(pk - mx);
+    float sm = 0;
+    for (uint32_t r = 0; r < K; r++) sm += __shfl(ex, r);
+    if (lane < K) w[tok * (K + 1) + lane] = ex / sm;
+    if (lane == K) w[tok * (K + 1) + K] = 1.0f / (1.0f + __expf(-lg[E]));
+}
+
+__device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 || E == 128 || E == 256 || E == 512 || E == 1024; }
+
+// The whole selection by one workgroup (any multiple of 64 threads). lgs: LDS scratch, 1024 floats per wave, used
+// only when E is not 64 * {1, 2, 4, 8, 16}.
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, float *lgs) {
+    const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     uint32_t *ue = (uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mask = (uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
     uint8_t *slot = a.sel + QW_SEL_OFF_SLOT(gnb, K);
     float *w = (float *)(a.sel + QW_SEL_OFF_W(gnb, K));
-    for (uint32_t i = tid; i < E; i += blockDim.x) first[i] = 0xffffffffu;
-    for (uint32_t i = tid; i < GU; i += blockDim.x) ue[i] = mask[i] = 0, um[i] = 0;
-    for (uint32_t i = tid; i < GU * gnb / 4; i += blockDim.x) ((uint32_t *)slot)[i] = 0;
-    if (wave < a.nbr) {
-        const float *src = a.logits + (size_t)wave * (E + 1);
-        float *v = lg[wave];
-        for (uint32_t e = lane; e < E; e += 64) v[e] = src[e];
-        float pk = 0; // lane k keeps the k-th picked logit
-        for (uint32_t k = 0; k < K; k++) {
-            float bv = -INFINITY;
-            uint32_t bi = 0xffffffffu;
-            for (uint32_t e = lane; e < E; e += 64) { // increasing e with strict '>' keeps the lowest index among equals
-                const float x = v[e];
-                if (x > bv || bi == 0xffffffffu) { bv = x; bi = e; }
-            }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float ov = __shfl_xor(bv, o);
-                const uint32_t oi = __shfl_xor(bi, o);
-                if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-            }
-            if (lane == 0) ids[wave * K + k] = bi;
-            if (lane == k) pk = bv;
-            if ((bi & 63) == lane) v[bi] = -INFINITY; // only the owning lane ever reads this element again
+    const bool fast = qw_select_fast_e(E);
+    for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
+    for (uint32_t i = tid; i < GU; i += nth) ue[i] = mask[i] = 0, s.um[i] = 0;
+    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)slot)[i] = 0;
+    for (uint32_t t = wave; t < a.nbr; t += nwv) {
+        const float *lg = a.logits + (size_t)t * (E + 1);
+        switch (fast ? E : 0u) {
+        case 64: select_token<1>(lg, E, K, t, w, s.ids, lane); break;
+        case 128: select_token<2>(lg, E, K, t, w, s.ids, lane); break;
+        case 256: select_token<4>(lg, E, K, t, w, s.ids, lane); break;
+        case 512: select_token<8>(lg, E, K, t, w, s.ids, lane); break;
+        case 1024: select_token<16>(lg, E, K, t, w, s.ids, lane); break;
+        default: select_token_any(lg, lgs + (size_t)wave * 1024, E, K, t, w, s.ids, lane);
         }
-        const float mx = __shfl(pk, 0), ex = __expf(pk - mx);
-        float sm = 0;
-        for (uint32_t k = 0; k < K; k++) sm += __shfl(ex, k); // rank order
-        if (lane < K) w[wave * (K + 1) + lane] = ex / sm;
-        if (lane == K) w[wave * (K + 1) + K] = 1.0f / (1.0f + __expf(-src[E]));
     }
     __syncthreads();
-    if (tid < UM) atomicMin(&first[ids[tid]], tid);
+    if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid);
     __syncthreads();
     uint32_t f = 0;
     if (tid < UM) {
-        f = first[ids[tid]];
-        lead[tid] = f == tid;
+        f = s.first[s.ids[tid]];
+        s.lead[tid] = f == tid;
     }
     __syncthreads();
     if (wave == 0) { // exclusive prefix count of the lead flags -> unique index (stored + 1)
         uint32_t carry = 0;
         for (uint32_t c = 0; c < UM; c += 64) {
-            const uint32_t i = c + lane, fl = i < UM ? lead[i] : 0;
+            const uint32_t i = c + lane, fl = i < UM ? s.lead[i] : 0;
             const unsigned long long bal = __ballot(fl);
             const uint32_t pre = __popcll(bal & ((1ull << lane) - 1)) + carry;
             carry += __popcll(bal);
-            if (fl) lead[i] = pre + 1;
+            if (fl) s.lead[i] = pre + 1;
         }
-        if (lane == 0) s_U = carry;
+        if (lane == 0) s.U = carry;
     }
     __syncthreads();
     if (tid < UM) {
-        const uint32_t u = lead[f] - 1, t = tid / K;
-        atomicOr(&um[u], 1u << t);
+        const uint32_t u = s.lead[f] - 1, t = tid / K;
+        atomicOr(&s.um[u], 1u << t);
         slot[u * gnb + t] = (uint8_t)(tid % K);
-        if (f == tid) ue[u] = ids[tid];
+        if (f == tid) ue[u] = s.ids[tid];
     }
     __syncthreads();
-    if (tid < s_U) mask[tid] = um[tid];
-    if (tid == 0) *(uint32_t *)a.sel = s_U;
+    if (tid < s.U) mask[tid] = s.um[tid];
+    if (tid == 0) *(uint32_t *)a.sel = s.U;
+}
+
+extern "C" __global__ __launch_bounds__(512) void qwk_select(qwk_select_args a) {
+    __shared__ qw_sel_scratch s;
+    __shared__ float lgs[8 * 1024];
+    select_all(a, s, lgs);
 }
 
 // ================================================================ gate/up + SwiGLU (kernels/moe_gg.metal:428-447, 563-573, 600-631)
 // A tile holds gate rows j0..j0+7 (n < 8) and up rows j0..j0+7 (n >= 8) of one expert; the up results move over by
 // 8 lanes, and H = g / (1 + exp(-g)) * up is stored as binary16 hi + lo planes for the tokens that picked the expert.
-template <int F> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, const u2 *lut, u4 *xf) {
-    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
-    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
-    __syncthreads();
-    const uint32_t U = a.shared ? 1 : *(const uint32_t *)a.sel;
-    const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mask = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
-    const uint8_t *slot = a.sel + QW_SEL_OFF_SLOT(gnb, K);
-    const uint32_t tpe = a.I / 8, ntasks = U * tpe, nw = gridDim.x * (blockDim.x >> 6);
-    const qw_afrag_lds af = {xf, n};
-    for (uint32_t task = blockIdx.x * (blockDim.x >> 6) + qw_wave(); task < ntasks; task += nw) {
-        const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
-        const uint32_t e = a.shared ? 0 : ue[u], m = a.shared ? (a.nbr >= 32 ? 0xffffffffu : (1u << a.nbr) - 1) : mask[u];
-        const uint8_t *row = (n < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (n & 7)) * a.rowbytes;
-        const f4 acc = qw_tile<F>::run(row, a.D, kg, lut, af);
-#pragma unroll
-        for (uint32_t i = 0; i < 4; i++) {
-            const float up = __shfl_xor(acc[i], 8), g = acc[i];
-            const uint32_t tok = 4 * kg + i;
-            if (n < 8 && tok < a.nbr && ((m >> tok) & 1)) {
-                const uint32_t s = a.shared ? K : slot[u * gnb + tok];
-                const float h = g / (1.0f + __expf(-g)) * up;
-                const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
-                const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
-                a.H[o] = __builtin_bit_cast(uint16_t, hi);
-                a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
-            }
-        }
-    }
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_gu_f21(qwk_gu_args a) {
-    __shared__ u2 lut[QW_LUT_ENTRIES];
-    __shared__ u4 xf[QW_XF_MAXK * 2];
-    qw_lut_build(lut);
-    gu_body<21>(a, lut, xf);
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_gu_f8(qwk_gu_args a) {
-    __shared__ u4 xf[QW_XF_MAXK * 2];
-    gu_body<8>(a, nullptr, xf);
+struct qw_sel_cache { // the part of the selection record a weight kernel needs, copied to LDS once
+    uint32_t U, ue[256], mask[256];
+    uint8_t slot[256 * 16];
+};
+__device__ __forceinline__ void qw_sel_load(qw_sel_cache &c, const uint8_t *sel, uint32_t K, uint32_t gnb) {
+    const uint32_t GU = gnb * K;
+    const uint32_t *ue = (const uint32_t *)(sel + QW_SEL_OFF_UE(gnb, K)), *mask = (const uint32_t *)(sel + QW_SEL_OFF_MASK(gnb, K));
+    const uint32_t *slot = (const uint32_t *)(sel + QW_SEL_OFF_SLOT(gnb, K));
+    for (uint32_t i = threadIdx.x; i < GU; i += blockDim.x) c.ue[i] = ue[i], c.mask[i] = mask[i];
+    for (uint32_t i = threadIdx.x; i < GU * gnb / 4; i += blockDim.x) ((uint32_t *)c.slot)[i] = slot[i];
+    if (threadIdx.x == 0) c.U = *(const uint32_t *)sel;
 }
 
-// ================================================================ down (kernels/moe_gg.metal:456-483, 606-617, 639-652)
-// Tile = 16 rows of one expert's down matrix; operand A is H (hi and lo planes) of the tokens that picked the expert,
-// read from global memory. A task is QW_DN_TPT consecutive tiles of one expert.
-#define QW_DN_TPT 4
-template <int F> __device__ __forceinline__ void dn_body(const qwk_dn_args &a, const u2 *lut) {
-    __syncthreads();
+template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw) {
+    typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
-    const uint32_t U = a.shared ? 1 : *(const uint32_t *)a.sel;
-    const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mask = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
-    const uint8_t *slot = a.sel + QW_SEL_OFF_SLOT(gnb, K);
-    const uint32_t tpe = a.D / (16 * QW_DN_TPT), ntasks = U * tpe, nw = gridDim.x * (blockDim.x >> 6);
-    for (uint32_t task = blockIdx.x * (blockDim.x >> 6) + qw_wave(); task < ntasks; task += nw) {
-        const uint32_t u = task / tpe, r0 = 16 * QW_DN_TPT * (task % tpe);
-        const uint32_t e = a.shared ? 0 : ue[u], m = a.shared ? (a.nbr >= 32 ? 0xffffffffu : (1u << a.nbr) - 1) : mask[u];
-        // operand A row of this lane's token (n): its H row for this expert, or nothing
-        qw_afrag_glb<true> af = {nullptr, nullptr};
-        if (n < a.nbr && ((m >> n) & 1)) {
-            const uint32_t s = a.shared ? K : slot[u * gnb + n];
-            af.rowhi = a.H + ((size_t)n * (K + 1) + s) * a.I;
-            af.rowlo = af.rowhi + a.hplane;
-        }
-        uint32_t sl[4]; // slots of the four tokens whose results this lane stores
+    const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
+    const uint32_t cpr = a.D / (C::BLK_K * CH), mine = w0 < ntasks ? (ntasks - w0 + nw - 1) / nw : 0;
+    const qw_afrag_lds af = {xf, n};
+    auto rowp = [&](uint32_t task) {
+        const uint32_t u = task / tpe, j0 = 8 * (task % tpe), e = a.shared ? 0 : sc->ue[u];
+        return (n < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (n & 7)) * a.rowbytes;
+    };
+    f4 acc = {0, 0, 0, 0};
+    qw_pipeline<C>(mine * cpr,
+        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, const C &c) {
+            const uint32_t ci = i % cpr;
+            c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 != cpr) return;
+            const uint32_t task = w0 + (i / cpr) * nw, u = task / tpe, j0 = 8 * (task % tpe);
+            const uint32_t m = a.shared ? qw_all_tokens(a.nbr) : sc->mask[u];
 #pragma unroll
-        for (uint32_t i = 0; i < 4; i++) {
-            const uint32_t tok = 4 * kg + i;
-            sl[i] = (!a.shared && tok < a.nbr && ((m >> tok) & 1)) ? slot[u * gnb + tok] : 0;
-        }
-        for (uint32_t tt = 0; tt < QW_DN_TPT; tt++) {
-            const uint32_t r = r0 + 16 * tt + n;
-            const uint8_t *row = a.Wd + ((size_t)e * a.D + r) * a.rowbytes;
-            const f4 acc = qw_tile<F>::run(row, a.I, kg, lut, af);
-#pragma unroll
-            for (uint32_t i = 0; i < 4; i++) {
-                const uint32_t tok = 4 * kg + i;
-                if (tok < a.nbr && ((m >> tok) & 1)) {
-                    if (a.shared) a.P[(size_t)tok * a.D + r] = acc[i];
-                    else a.P[((size_t)tok * K + sl[i]) * a.D + r] = acc[i];
+            for (uint32_t j = 0; j < 4; j++) {
+                const float up = __shfl_xor(acc[j], 8), g = acc[j];
+                const uint32_t tok = 4 * kg + j;
+                if (n < 8 && tok < a.nbr && ((m >> tok) & 1)) {
+                    const uint32_t s = a.shared ? K : sc->slot[u * gnb + tok];
+                    const float h = g / (1.0f + __expf(-g)) * up;
+                    const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
+                    const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
+                    a.H[o] = __builtin_bit_cast(uint16_t, hi);
+                    a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
                 }
             }
+            acc = f4{0, 0, 0, 0};
+        });
+}
+
+// The shared expert's down projection inside the gate/up launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
+// planes) of every token straight from global memory. Wave w takes tiles w, w + nw, ...
+template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const qwk_gu_args &a, const u2 *lut, uint32_t w0, uint32_t nw) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk;
+    const uint32_t ntiles = a.D / 16, cpr = a.I / (C::BLK_K * CH), mine = w0 < ntiles ? (ntiles - w0 + nw - 1) / nw : 0;
+    qw_afrag_glb<true> af = {nullptr, nullptr};
+    if (n < a.nbr) {
+        af.rowhi = a.H + ((size_t)n * (K + 1) + K) * a.I;
+        af.rowlo = af.rowhi + a.hplane;
+    }
+    f4 acc = {0, 0, 0, 0};
+    qw_pipeline<C>(mine * cpr,
+        [&](uint32_t i, C &c) { c.load(a.Wsd + (size_t)(16 * (w0 + (i / cpr) * nw) + n) * a.sd_rowbytes + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, const C &c) {
+            const uint32_t ci = i % cpr;
+            c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 != cpr) return;
+            const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++)
+                if (4 * kg + j < a.nbr) a.Psh[(size_t)(4 * kg + j) * a.D + r] = acc[j];
+            acc = f4{0, 0, 0, 0};
+        });
+}
+
+// FGU: routed gate/up format; FSD: shared down format (0 = no shared down in this launch).
+template <int FGU, int CHGU, int FSD, int CHSD> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
+    if (FGU == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+    if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+    __syncthreads();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    if (FSD != 0) {
+        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, w0, nw);
+    }
+    // the waves that did a shared-down tile come last in the routed deal, so that the work stays level
+    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw);
+}
+#define QW_GU(FGU, CHGU, FSD, CHSD, NAME)                                                                 \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_gu_args a) {                             \
+        __shared__ u2 lut[(FGU == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];                                 \
+        __shared__ u4 xf[QW_XF_MAXK * 2];                                                                 \
+        __shared__ qw_sel_cache sc;                                                                       \
+        gu_body<FGU, CHGU, FSD, CHSD>(a, lut, xf, &sc);                                                   \
+    }
+// K = D for gate/up: 2048 (8 blocks a chunk for IQ3_S, 16 for Q8_0), 2560 (10 / 16), other (1). K = I for down: 512 (2 / 16), other (1).
+QW_GU(21, 8, 0, 1, qwk_gu_f21_c8) QW_GU(21, 10, 0, 1, qwk_gu_f21_c10) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
+QW_GU(8, 16, 0, 1, qwk_gu_f8_c16) QW_GU(8, 1, 0, 1, qwk_gu_f8_c1)
+QW_GU(21, 8, 21, 2, qwk_gu_f21_c8_sd21_c2) QW_GU(21, 8, 8, 16, qwk_gu_f21_c8_sd8_c16)
+QW_GU(21, 10, 21, 1, qwk_gu_f21_c10_sd21_c1) QW_GU(21, 10, 8, 1, qwk_gu_f21_c10_sd8_c1)
+QW_GU(21, 1, 21, 1, qwk_gu_f21_c1_sd21_c1) QW_GU(21, 1, 8, 1, qwk_gu_f21_c1_sd8_c1)
+QW_GU(8, 16, 8, 16, qwk_gu_f8_c16_sd8_c16) QW_GU(8, 16, 21, 2, qwk_gu_f8_c16_sd21_c2)
+QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_sd8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_sd21_c1)
+
+// ================================================================ front part of a layer in one launch
+// (kernels/moe_gg.metal:534-590) Workgroups [0, nrouter_wg): router rows, 8 per workgroup; the rest: the shared
+// expert's gate/up tiles. The router workgroup that finishes last runs the selection (the others' logits are visible
+// to it: every thread fences its stores before the workgroup's counter increment).
+template <int WF, int F, int CH> __device__ __forceinline__ void pre_body(const qwk_pre_args &a, u2 *lut, u4 *xf) {
+    __shared__ uint32_t last;
+    if (blockIdx.x >= a.nrouter_wg) {
+        if (F == 21) qw_lut_copy(lut, (const u2 *)a.g.glut);
+        qw_stage_x(xf, a.g.x, a.g.D, a.g.D, a.g.nbr);
+        __syncthreads();
+        gu_tasks<F, CH>(a.g, lut, xf, nullptr, (blockIdx.x - a.nrouter_wg) * (blockDim.x >> 6) + qw_wave(), (gridDim.x - a.nrouter_wg) * (blockDim.x >> 6));
+        return;
+    }
+    router_rows<WF>(a.r, blockIdx.x * (blockDim.x >> 6) + qw_wave(), qw_lane());
+    if (!a.do_select) return;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) last = atomicAdd(a.cnt, 1u) == a.nrouter_wg - 1;
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    // the LDS of a router workgroup is free: the selection's scratch goes where the staged activations would be
+    qw_sel_scratch *s = (qw_sel_scratch *)xf;
+    const qwk_select_args sa = {a.r.logits, const_cast<uint8_t *>(a.g.sel), a.r.nb, a.r.E, a.g.topk, a.g.gnb};
+    select_all(sa, *s, (float *)(xf + 1024));
+    if (threadIdx.x == 0) *a.cnt = 0;
+}
+#define QW_PRE(WF, F, CH, NAME)                                                       \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {        \
+        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                              \
+        __shared__ u4 xf[QW_XF_MAXK * 2];                                             \
+        pre_body<WF, F, CH>(a, lut, xf);                                              \
+    }
+QW_PRE(1, 21, 8, qwk_pre_w1_f21_c8) QW_PRE(1, 21, 10, qwk_pre_w1_f21_c10) QW_PRE(1, 21, 1, qwk_pre_w1_f21_c1)
+QW_PRE(1, 8, 16, qwk_pre_w1_f8_c16) QW_PRE(1, 8, 1, qwk_pre_w1_f8_c1)
+QW_PRE(30, 21, 8, qwk_pre_w30_f21_c8) QW_PRE(30, 21, 10, qwk_pre_w30_f21_c10) QW_PRE(30, 21, 1, qwk_pre_w30_f21_c1)
+QW_PRE(30, 8, 16, qwk_pre_w30_f8_c16) QW_PRE(30, 8, 1, qwk_pre_w30_f8_c1)
+
+// ================================================================ down (kernels/moe_gg.metal:456-483, 639-652)
+// Workgroup task = (expert u, block of 256 rows): the H rows (hi and lo planes) of the tokens that picked u are staged
+// in LDS in fragment order, double-buffered; wave w owns rows 32 w .. 32 w + 31 of the block = two tiles.
+// One barrier per task; the weight loads of the next task are in flight across it.
+template <int F, int CH> __device__ __forceinline__ void dn_body(const qwk_dn_args &a, u2 *lut, u4 *abuf /* [2][2][I/8*16] */, qw_sel_cache *sc) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb, wave = qw_wave();
+    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_sel_load(*sc, a.sel, K, gnb);
+    __syncthreads();
+    const uint32_t U = sc->U, bpe = a.D / 256, ntasks = U * bpe, mine = blockIdx.x < ntasks ? (ntasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+    const uint32_t nfrag = (a.I / 8) * 16; // 16-byte fragments per plane
+    auto stage = [&](uint32_t it) { // operand A of this workgroup's it-th task into buffer it & 1
+        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, m = sc->mask[u];
+        u4 *dst = abuf + (size_t)(it & 1) * 2 * nfrag;
+        for (uint32_t i = threadIdx.x; i < 2 * nfrag; i += blockDim.x) {
+            const uint32_t pl = i / nfrag, f = i % nfrag, c = f >> 4, t = f & 15;
+            u4 v = {0, 0, 0, 0};
+            if (t < a.nbr && ((m >> t) & 1)) v = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + sc->slot[u * gnb + t]) * a.I + 8 * c);
+            dst[i] = v;
+        }
+    };
+    auto rowp = [&](uint32_t it, uint32_t tile) {
+        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, r = 256 * (task % bpe) + 32 * wave + 16 * tile + n;
+        return a.Wd + ((size_t)sc->ue[u] * a.D + r) * a.rowbytes;
+    };
+    auto compute = [&](uint32_t it, const C &t0, const C &t1) {
+        const u4 *base = abuf + (size_t)(it & 1) * 2 * nfrag;
+        const qw_afrag_lds2 af = {base, base + nfrag, n};
+        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, m = sc->mask[u];
+#pragma unroll
+        for (int tile = 0; tile < 2; tile++) {
+            f4 acc = {0, 0, 0, 0};
+            (tile ? t1 : t0).mac(lut, af, 0, kg, acc);
+            const uint32_t r = 256 * (task % bpe) + 32 * wave + 16 * tile + n;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++) {
+                const uint32_t tok = 4 * kg + j;
+                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc[j];
+            }
+        }
+    };
+    C a0, a1, b0, b1;
+    if (mine) {
+        a0.load(rowp(0, 0), kg);
+        a1.load(rowp(0, 1), kg);
+        stage(0);
+    }
+    __syncthreads();
+    for (uint32_t it = 0; it < mine; it += 2) {
+        if (it + 1 < mine) { b0.load(rowp(it + 1, 0), kg); b1.load(rowp(it + 1, 1), kg); stage(it + 1); }
+        compute(it, a0, a1);
+        __syncthreads();
+        if (it + 1 >= mine) break;
+        if (it + 2 < mine) { a0.load(rowp(it + 2, 0), kg); a1.load(rowp(it + 2, 1), kg); stage(it + 2); }
+        compute(it + 1, b0, b1);
+        __syncthreads();
+    }
+}
+#define QW_DN(F, CH, IMAX, NAME)                                                      \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
+        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                              \
+        __shared__ u4 abuf[2 * 2 * (IMAX / 8) * 16];                                  \
+        __shared__ qw_sel_cache sc;                                                   \
+        dn_body<F, CH>(a, lut, abuf, &sc);                                            \
+    }
+// I = 512 is the synthetic shape (whole row = one chunk of 2 IQ3_S blocks); Q8_0 down weights take the any-shape kernel
+QW_DN(21, 2, 512, qwk_dn_f21_i512)
+
+// Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
+template <int F> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+    typedef qw_chunk<F, 1> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
+    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_sel_load(*sc, a.sel, K, gnb);
+    __syncthreads();
+    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t cpr = a.I / C::BLK_K;
+    for (uint32_t task = w0; task < ntasks; task += nw) {
+        const uint32_t u = task / tpe, r = 16 * (task % tpe) + n, m = sc->mask[u];
+        qw_afrag_glb<true> af = {nullptr, nullptr};
+        if (n < a.nbr && ((m >> n) & 1)) {
+            af.rowhi = a.H + ((size_t)n * (K + 1) + sc->slot[u * gnb + n]) * a.I;
+            af.rowlo = af.rowhi + a.hplane;
+        }
+        const uint8_t *row = a.Wd + ((size_t)sc->ue[u] * a.D + r) * a.rowbytes;
+        f4 acc = {0, 0, 0, 0};
+        qw_pipeline<C>(cpr, [&](uint32_t i, C &c) { c.load(row + (size_t)i * C::BLK_B, kg); },
+                       [&](uint32_t i, const C &c) { c.mac(lut, af, i * C::BLK_K, kg, acc); });
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+            const uint32_t tok = 4 * kg + j;
+            if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc[j];
         }
     }
 }
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f21(qwk_dn_args a) {
+extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f21_any(qwk_dn_args a) {
     __shared__ u2 lut[QW_LUT_ENTRIES];
-    qw_lut_build(lut);
-    dn_body<21>(a, lut);
+    __shared__ qw_sel_cache sc;
+    dn_any_body<21>(a, lut, &sc);
 }
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f8(qwk_dn_args a) { dn_body<8>(a, nullptr); }
+extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f8_any(qwk_dn_args a) {
+    __shared__ qw_sel_cache sc;
+    dn_any_body<8>(a, nullptr, &sc);
+}
 
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).
@@ -311,9 +529,14 @@ extern "C" __global__ __launch_bounds__(256) void qwk_cmb(qwk_cmb_args a) {
     if (i >= a.nbr * a.D) return;
     const uint32_t t = i / a.D, row = i % a.D, K = a.topk;
     const float *w = (const float *)(a.sel + QW_SEL_OFF_W(a.gnb, K)) + t * (K + 1);
+    float pg[16];
+#pragma unroll
+    for (uint32_t s = 0; s < 16; s++) pg[s] = s < K ? a.Pg[((size_t)t * K + s) * a.D + row] : 0.0f; // loads first
     float o = 0;
-    for (uint32_t s = 0; s < K; s++) o += w[s] * a.Pg[((size_t)t * K + s) * a.D + row];
-    o += w[K] * a.Psh[(size_t)t * a.D + row];
+#pragma unroll
+    for (uint32_t s = 0; s < 16; s++)
+        if (s < K) o = __builtin_fmaf(w[s], pg[s], o);
+    o = __builtin_fmaf(w[K], a.Psh[(size_t)t * a.D + row], o);
     a.out[(size_t)t * a.D + row] = qw_f2h(o);
 }
 
@@ -350,5 +573,27 @@ extern "C" __global__ __launch_bounds__(256) void qwk_fill_random(qwk_mem_args a
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += step) {
         const uint64_t c = a.seed + 4 * i;
         q[i] = u4{qw_mix(c), qw_mix(c + 1), qw_mix(c + 2), qw_mix(c + 3)};
+    }
+}
+
+// Synthetic GGUF blocks, one thread per block: d = binary16(|N(0, sigma)|) by Box-Muller over two hashed uniforms,
+// every other byte uniform (IQ3_S), or int8 uniform in [-127, 127] (Q8_0). Blocks are 2-byte aligned: 16-bit stores.
+extern "C" __global__ __launch_bounds__(256) void qwk_fill_blocks(qwk_fill_args a) {
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    const uint32_t bb = a.type == 21 ? 110 : 34;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.nblocks; i += step) {
+        uint16_t *p = (uint16_t *)(a.dst + i * bb);
+        const uint64_t c = a.seed + i * 64;
+        const float u1 = ((float)(qw_mix(c) >> 8) + 1.0f) * (1.0f / 16777216.0f), u2 = (float)(qw_mix(c + 1) >> 8) * (1.0f / 16777216.0f);
+        const float z = sqrtf(-2.0f * __logf(u1)) * __cosf(6.2831853f * u2);
+        p[0] = qw_f2h(fabsf(z) * a.sigma);
+        for (uint32_t w = 1; w < bb / 2; w++) {
+            uint32_t r = qw_mix(c + 1 + w);
+            if (a.type == 8) { // two int8 in [-127, 127]
+                const uint32_t b0 = (r & 0xffff) % 255u, b1 = (r >> 16) % 255u;
+                r = ((b0 - 127u) & 255u) | (((b1 - 127u) & 255u) << 8);
+            }
+            p[w] = (uint16_t)r;
+        }
     }
 }

@@ -213,3 +213,10 @@ bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, cons
     qw_batch_dispatch(b, D / 256, 1, 1, 256, 1, 1);
     return true;
 }
+
+bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,
+                          const qw_buf *sel, const qw_buf *out) {
+    for (int l = 0; l < nlayers; l++)
+        if (!qw_path_gg_moe(p, b, &M[l], nb, x, &lg[l], &sel[l], out)) return false;
+    return true;
+}

@@ -48,12 +48,14 @@ SYMBOLS = [
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
     ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),
     ("qw_hip_profile_mean", _d, [_vp, C.c_char_p, C.POINTER(_i)]),
+    ("qw_hip_profile_entry", C.c_char_p, [_vp, _i, C.POINTER(_d)]),
     # qw_path.h
     ("qw_path_open", _vp, [_vp, _i, _i, _i, _i, _i, _b]), ("qw_path_close", None, [_vp]),
     ("qw_path_sel_bytes", _sz, [_vp, _i]), ("qw_path_logits_bytes", _sz, [_vp, _i]), ("qw_path_nbv", _i, [_i]),
     ("qw_path_qmv_gg", _b, [_vp, _vp, _pt, _i, _i, _pb, _sz, _pb, _sz, _i, _b]),
     ("qw_path_gg_router", _b, [_vp, _vp, _pm, _i, _pb, _pb]),
     ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
+    ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_scratch", _pb, [_vp, _i]),
 ]
 
@@ -217,11 +219,13 @@ class Gpu:
     def profile(self, on):
         self.L.qw_profile_enable(self.g, on)
 
-    def profile_entries(self):
+    def profile_entries(self, entry_points=True):
+        """(name, microseconds) per launch of the last profiled batch; entry-point names, or the callers' kernel names."""
         out = []
         us = C.c_double()
+        get = self.L.qw_hip_profile_entry if entry_points else self.L.qw_profile_get
         for i in range(self.L.qw_profile_count(self.g)):
-            n = self.L.qw_profile_get(self.g, i, C.byref(us))
+            n = get(self.g, i, C.byref(us))
             out.append((n.decode(), us.value))
         return out
 
@@ -264,6 +268,11 @@ class Path:
     def gg_moe(self, batch, layer, nb, x, lg, sel, out):
         if not self.L.qw_path_gg_moe(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
             raise RuntimeError("qw_path_gg_moe failed")
+
+    def gg_moe_stack(self, batch, layers_c, nlayers, nb, x, lg_c, sel_c, out):
+        """layers_c: ctypes array of QwMoeLayer; lg_c / sel_c: ctypes arrays of QwBuf, one per layer."""
+        if not self.L.qw_path_gg_moe_stack(self.p, batch.b, layers_c, nlayers, nb, x.ref(), lg_c, sel_c, out.ref()):
+            raise RuntimeError("qw_path_gg_moe_stack failed")
 
     def scratch(self, which):
         """0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg; returns (device bytes as uint8)."""

@@ -1,0 +1,100 @@
+"""The MoE FFN stack of the benchmark: L layers of the synthetic layer shape, every layer with its own weights
+resident in HBM (device-only buffers filled by the library's block generator), decoded for nb tokens per step.
+
+Mixed quantisation: with q8_every = 4, layers 3, 7, 11, ... carry their shared expert's three projections in Q8_0
+and everything else in IQ3_S — the reference's SC117 recipe puts Q8_0 on the shared / dense projections only
+(CHANGELOG.md:154), which keeps the stack near 33 GB.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import synth
+from .gpu import Buf, MoeLayer, Path, QwBuf, QwMoeLayer, Tensor
+
+MEM_DEFS = "#define QW_HIP_MEM 1\n"
+
+
+def fill_blocks(gpu, batch, buf, offset, nblocks, ftype, seed, sigma):
+    ok, err = gpu.compile(MEM_DEFS)
+    if not ok:
+        raise RuntimeError(err)
+    batch.kernel(gpu.kernel("qw_fill_blocks"))
+    batch.buf(1, buf, offset)
+    a = np.zeros(1, np.dtype([("n", "<u8"), ("seed", "<u8"), ("type", "<u4"), ("sigma", "<f4")]))
+    a["n"], a["seed"], a["type"], a["sigma"] = nblocks, seed, ftype, sigma
+    batch.bytes(2, a)
+    batch.dispatch(1)
+
+
+class MoeStack:
+    def __init__(self, gpu, layers=48, D=2048, I=512, E=512, topk=10, nbmax=16, q8_every=4, seed=1234, d_scale=synth.MOE_D_SCALE):
+        self.gpu, self.L, self.D, self.I, self.E, self.topk, self.nbmax = gpu, layers, D, I, E, topk, nbmax
+        self.path = Path(gpu, D, I, E, topk, nbmax, device_scratch=True)
+        rng = np.random.default_rng(seed)
+        rb_gu, rb_d = synth.row_bytes(21, D), synth.row_bytes(21, I)
+        self.exp_bytes = 2 * I * rb_gu + D * rb_d           # one IQ3_S expert
+        self.gu_bytes = 2 * I * rb_gu
+        self.layers, self.bufs, self.shared_fmt = [], [], []
+        self.router_bytes = (E + 1) * D * 2
+        b = gpu.batch()
+        for l in range(layers):
+            fsh = 8 if q8_every and l % q8_every == q8_every - 1 else 21
+            sz_e = E * I * rb_gu                              # gate, up and down each: E * I * rb(D) == E * D * rb(I)
+            assert sz_e == E * D * rb_d
+            sh_gu, sh_d = I * synth.row_bytes(fsh, D), D * synth.row_bytes(fsh, I)
+            w = gpu.buf(3 * sz_e, device_only=True)
+            sh = gpu.buf(2 * sh_gu + sh_d, device_only=True)
+            fill_blocks(gpu, b, w, 0, 3 * sz_e // 110, 21, seed * 1000003 + l * 7919, synth.D_SIGMA[21] * d_scale)
+            fill_blocks(gpu, b, sh, 0, (2 * sh_gu + sh_d) // synth.BLOCK[fsh][1], fsh, seed * 1000003 + l * 7919 + 1, synth.D_SIGMA[fsh] * d_scale)
+            Wr, wsg = synth.router(rng, E, D)
+            r = gpu.buf_from(np.concatenate([Wr.ravel(), wsg]).view(np.uint16), device_only=True)
+            T = Tensor
+            self.layers.append(MoeLayer(router=T(r, 1), sh_gate_w=T(r, 1, E * D * 2), gate=T(w, 21), up=T(w, 21, sz_e), down=T(w, 21, 2 * sz_e),
+                                        sh_gate=T(sh, fsh), sh_up=T(sh, fsh, sh_gu), sh_down=T(sh, fsh, 2 * sh_gu)))
+            self.bufs += [w, sh, r]
+            self.shared_fmt.append(fsh)
+        b.end()
+        self.layers_c = (QwMoeLayer * layers)(*[m.c for m in self.layers])
+        self.lg = [gpu.buf(self.path.logits_bytes(nbmax), device_only=True) for _ in range(layers)]
+        self.sel = [gpu.buf(self.path.sel_bytes(nbmax), device_only=True) for _ in range(layers)]
+        self.lg_c = (QwBuf * layers)(*[x.c for x in self.lg])
+        self.sel_c = (QwBuf * layers)(*[x.c for x in self.sel])
+        self.out = gpu.buf(nbmax * D * 2)
+        self.bufs += self.lg + self.sel + [self.out]
+        self.weight_bytes = sum(x.size for x in self.bufs[:3 * layers])
+
+    def shared_bytes(self, l):
+        f = self.shared_fmt[l]
+        return 2 * self.I * synth.row_bytes(f, self.D) + self.D * synth.row_bytes(f, self.I)
+
+    def step(self, x, nb, nlayers=None):
+        """One decode step over the stack; returns GPU seconds (events around the kernels)."""
+        b = self.gpu.batch()
+        self.path.gg_moe_stack(b, self.layers_c, self.L if nlayers is None else nlayers, nb, x, self.lg_c, self.sel_c, self.out)
+        return b.end()
+
+    def unique_experts(self, nb):
+        """U per layer, read from the selection records of the last step."""
+        return [int(s.read(4).view(np.uint32)[0]) for s in self.sel]
+
+    def algorithmic_bytes(self, nb, U):
+        """Per layer: router + (U_l + 1 shared) experts + activations in and out (the reference's accounting,
+        src/engine.c:8020-8038, with U distinct experts for the routed part)."""
+        return [self.router_bytes + U[l] * self.exp_bytes + self.shared_bytes(l) + nb * self.D * 4 for l in range(self.L)]
+
+    def layer_weights_host(self, l):
+        """The layer's weights copied back from HBM, as the dict the oracle takes (bytes exactly as resident)."""
+        w, sh, r = self.bufs[3 * l:3 * l + 3]
+        E, I, D = self.E, self.I, self.D
+        sz_e = E * I * synth.row_bytes(21, D)
+        f = self.shared_fmt[l]
+        sh_gu = I * synth.row_bytes(f, D)
+        wb, sb, rb = w.read(), sh.read(), r.read(dtype=np.uint16)
+        return dict(D=D, I=I, E=E, topk=self.topk, fgu=21, fd=21, fsg=f, fsu=f, fsd=f, Wg=wb[:sz_e], Wu=wb[sz_e:2 * sz_e], Wd=wb[2 * sz_e:],
+                    Wsg=sb[:sh_gu], Wsu=sb[sh_gu:2 * sh_gu], Wsd=sb[2 * sh_gu:], Wr=rb[:E * D].view(np.float16).reshape(E, D), wsg=rb[E * D:].view(np.float16))
+
+    def free(self):
+        for b in self.bufs:
+            b.free()
+        self.path.close()
