@@ -81,8 +81,13 @@ struct qw_batch {
     int nuse, capuse, done_use;
     hipEvent_t ev[2 * 9]; // start/stop per submitted segment (end + at most 8 flushes)
     int nseg;
-    hipEvent_t *pev;      // profiling: 2 events per dispatch
+    hipEvent_t *pev;      // profiling: 2 events per launch
     int npev;
+    // Work deferred from one dispatch of a layer to the next (the reference's front part also computes the shared
+    // expert's gate/up, and its gate/up dispatch the shared down; here they ride in the next launch, where they cost
+    // almost nothing): set by moe_pre_gg / moe_gu_gg, consumed by moe_gu_gg / moe_dn_gg of the same batch.
+    struct { bool valid; int fmt; const uint8_t *Wsg, *Wsu; uint32_t rowbytes, nbr; } pend_sg;
+    struct { bool valid; int fmt; const uint8_t *Wsd; float *Psh; uint32_t rowbytes, nbr; } pend_sd;
 };
 
 struct qw_gpu {
@@ -515,7 +520,8 @@ static unsigned umin(unsigned a, unsigned b) { return a < b ? a : b; }
 static unsigned cdiv(unsigned a, unsigned b) { return (a + b - 1) / b; }
 // Persistent grids: one 512-thread workgroup per compute unit (the LDS tables leave room for one), fewer if the
 // work is smaller. tasks are per-wave units; 8 waves per workgroup.
-static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks) { return umin((unsigned)g->ncu, cdiv(wave_tasks, 8)); }
+static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks, unsigned waves) { return umin((unsigned)g->ncu, cdiv(wave_tasks, waves)); }
+enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 }; // waves per workgroup of the gate/up + matvec kernels and of the down kernels
 
 static const char *fname_fmt(char *buf, size_t n, const char *fmt, ...) {
     va_list ap;
@@ -549,7 +555,7 @@ static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W,
 static const void *glut(const qw_gpu *g) { return (const char *)g->tabs + QW_TAB_IQ3SS; }
 
 // Blocks per prefetch chunk for a row of K values (the kernels are instantiated for these; 1 = any K).
-static int chunk_of(int F, int K) { return F == 21 ? (K == 512 ? 2 : K == 2048 ? 8 : K == 2560 ? 10 : 1) : (K % 512 == 0 ? 16 : 1); }
+static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1; }
 
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
     const qw_kparams *p = &b->k->p;
@@ -567,7 +573,7 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
     char fn[48];
     if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", p->F);
     else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", p->F, chunk_of(p->F, p->K));
-    return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles), 512, &a, sizeof a);
+    return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 
 static bool fill_router(qw_batch *b, qwk_router_args *a, unsigned iWr, unsigned iWsg, unsigned ix, unsigned ilg, uint32_t nbr) {
@@ -581,7 +587,7 @@ static bool launch_select(qw_batch *b, unsigned ilg, unsigned isel, uint32_t nbr
     const qw_kparams *p = &b->k->p;
     qwk_select_args a = {.nbr = nbr, .E = (uint32_t)p->E, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
     if (!bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, false, "logits", (void **)&a.logits) || !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.sel)) return false;
-    return add_launch(b, "qwk_select", 1, 512, &a, sizeof a);
+    return add_launch(b, "qwk_select", 1, 1024, &a, sizeof a);
 }
 
 static bool nbr_ok(qw_batch *b, uint32_t nbr) {
@@ -619,29 +625,32 @@ static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nb
 }
 
 // src/engine.c:588-607: 0 Wr, 1 shared gate vector, 2 x, 3 logits, 4 counter, 5 sel, 6/7 shared gate/up, 8 H, 13 tables, 14 nbr.
-// One launch: router rows and the shared expert's gate/up side by side, the selection by the last router workgroup.
+// Two launches: router rows, then the selection. The shared expert's gate/up is checked and remembered here and
+// runs inside the gate/up launch that follows.
 static bool tr_pre(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     uint32_t nbr;
     if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
-    qwk_pre_args a = {0};
-    if (!fill_gu(b, &a.g, p->fsg, 6, 7, 2, 8, nbr, true)) return false;
-    char fn[64];
-    const unsigned gu_wg = cdiv((unsigned)p->I / 8, 8);
-    if (!p->rbf) { // router and selection come as dispatches of their own: only the shared expert's gate/up here
-        fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", p->fsg, chunk_of(p->fsg, p->D));
-        return add_launch(b, intern(fn), gu_wg, 512, &a.g, sizeof a.g);
-    }
+    const size_t rb = fmt_rb(p->fsg, p->D);
+    void *h;
+    b->pend_sg.valid = false;
+    if (!bind_ptr(b, 6, (size_t)p->I * rb, false, "shared gate weights", (void **)&b->pend_sg.Wsg) || !bind_ptr(b, 7, (size_t)p->I * rb, false, "shared up weights", (void **)&b->pend_sg.Wsu) ||
+        !bind_ptr(b, 8, (size_t)p->NB * (p->topk + 1) * p->I * 4, true, "H", &h)) return false;
+    b->pend_sg.valid = true;
+    b->pend_sg.fmt = p->fsg;
+    b->pend_sg.rowbytes = (uint32_t)rb;
+    b->pend_sg.nbr = nbr;
+    if (!p->rbf) return true; // router and selection come as dispatches of their own
+    qwk_pre_args a = {.topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
     if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
-    if (!bind_ptr(b, 5, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.g.sel) || !bind_ptr(b, 4, 4, true, "counter", (void **)&a.cnt)) return false;
-    a.nrouter_wg = cdiv((unsigned)p->E + 1, 8);
-    a.do_select = 1;
-    fname_fmt(fn, sizeof fn, "qwk_pre_w%d_f%d_c%d", p->rwf, p->fsg, chunk_of(p->fsg, p->D));
-    return add_launch(b, intern(fn), a.nrouter_wg + gu_wg, 512, &a, sizeof a);
+    if (b->buf[2].off % 16) return fail(b, "moe_pre_gg: x offset %zu is not 16-byte aligned", b->buf[2].off);
+    // the counter buffer of the reference's hand-over (index 4) is not used: the selection is a launch of its own
+    return add_launch(b, p->rwf == 30 ? "qwk_pre_w30" : "qwk_pre_w1", cdiv((unsigned)p->E + 1, 8), 512, &a, sizeof a) && launch_select(b, 3, 5, nbr);
 }
 
 // src/engine.c:616-629: 0 Wg, 1 Wu, 2 shared down, 3 Psh, 4 x, 5 sel, 6 H, 11 tables, 12 nbr.
-// One launch: routed gate/up tiles for the selected experts and the shared expert's down tiles.
+// One launch: the shared expert's gate/up tiles (remembered from moe_pre_gg) and the routed gate/up tiles of the
+// selected experts. The shared down is checked and remembered for the down launch.
 static bool tr_gu(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     uint32_t nbr;
@@ -649,20 +658,32 @@ static bool tr_gu(qw_batch *b) {
     qwk_gu_args a;
     if (!fill_gu(b, &a, p->fgu, 0, 1, 4, 6, nbr, false)) return false;
     if (!bind_ptr(b, 5, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
-    a.sd_rowbytes = (uint32_t)fmt_rb(p->fsd, p->I);
-    if (!bind_ptr(b, 2, (size_t)p->D * a.sd_rowbytes, false, "shared down weights", (void **)&a.Wsd) || !bind_ptr(b, 3, (size_t)nbr * p->D * 4, true, "Psh", (void **)&a.Psh)) return false;
-    // the instantiated pairs: fast shapes (D 2048 / I 512), D 2560, or the any-shape build
-    const int cg = chunk_of(p->fgu, p->D);
-    const bool fast = (p->fgu == 21 ? cg == 8 : cg == 16) && chunk_of(p->fsd, p->I) == (p->fsd == 21 ? 2 : 16);
+    b->pend_sd.valid = false;
+    b->pend_sd.rowbytes = (uint32_t)fmt_rb(p->fsd, p->I);
+    if (!bind_ptr(b, 2, (size_t)p->D * b->pend_sd.rowbytes, false, "shared down weights", (void **)&b->pend_sd.Wsd) || !bind_ptr(b, 3, (size_t)nbr * p->D * 4, true, "Psh", (void **)&b->pend_sd.Psh)) return false;
+    b->pend_sd.valid = true;
+    b->pend_sd.fmt = p->fsd;
+    b->pend_sd.nbr = nbr;
+    int cg = chunk_of(p->fgu, p->D), fs = 0, cs = 1;
+    if (b->pend_sg.valid) {
+        if (b->pend_sg.nbr != nbr) return fail(b, "moe_gu_gg: %u tokens after a front part of %u", nbr, b->pend_sg.nbr);
+        fs = b->pend_sg.fmt;
+        cs = chunk_of(fs, p->D);
+        a.Wsg = b->pend_sg.Wsg;
+        a.Wsu = b->pend_sg.Wsu;
+        a.sg_rowbytes = b->pend_sg.rowbytes;
+        b->pend_sg.valid = false;
+        if (cg == 1 || cs == 1) cg = cs = 1; // any-shape builds come in pairs
+    }
     char fn[64];
-    if (fast) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_sd%d_c%d", p->fgu, cg, p->fsd, chunk_of(p->fsd, p->I));
-    else if (p->fgu == 21 && cg == 10) fname_fmt(fn, sizeof fn, "qwk_gu_f21_c10_sd%d_c1", p->fsd);
-    else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c1_sd%d_c1", p->fgu, p->fsd);
-    const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (unsigned)p->D / 16;
-    return add_launch(b, intern(fn), persistent_grid(b->g, tasks), 512, &a, sizeof a);
+    if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", p->fgu, cg, fs, cs);
+    else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", p->fgu, cg);
+    const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (fs ? (unsigned)p->I / 8 : 0);
+    return add_launch(b, intern(fn), persistent_grid(b->g, tasks, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 
 // src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
+// The shared down tiles (remembered from moe_gu_gg) run in the same launch.
 static bool tr_dn(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     const uint32_t nbr = (uint32_t)p->NB;
@@ -672,14 +693,24 @@ static bool tr_dn(qw_batch *b) {
     if (!bind_ptr(b, 0, (size_t)p->E * p->D * rb, false, "down weights", (void **)&a.Wd) || !bind_ptr(b, 2, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
         !bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, true, "Pg", (void **)&a.P) ||
         !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
+    int fs = 0;
+    if (b->pend_sd.valid) {
+        fs = b->pend_sd.fmt;
+        a.Wsd = b->pend_sd.Wsd;
+        a.Psh = b->pend_sd.Psh;
+        a.sd_rowbytes = b->pend_sd.rowbytes;
+        a.snbr = b->pend_sd.nbr;
+        b->pend_sd.valid = false;
+    }
     const unsigned umax = umin((unsigned)p->E, nbr * (unsigned)p->topk);
-    char fn[48];
+    char fn[48], sfx[16] = "";
+    if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
     if (p->I == 512 && p->fd == 21) { // workgroup tasks of 256 rows
-        fname_fmt(fn, sizeof fn, "qwk_dn_f%d_i512", p->fd);
+        fname_fmt(fn, sizeof fn, "qwk_dn_f21_i512%s", sfx);
         return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, umax * (unsigned)(p->D / 256)), 512, &a, sizeof a);
     }
-    fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any", p->fd);
-    return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16)), 512, &a, sizeof a);
+    fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any%s", p->fd, sfx);
+    return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DN), 64 * QW_WAVES_DN, &a, sizeof a);
 }
 
 // src/engine.c:640-646: 1 Psh, 3 sel, 4 out, 8 nbr, 9 Pg

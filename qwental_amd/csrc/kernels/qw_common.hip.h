@@ -7,7 +7,10 @@
 //     A: lane supplies x[token = n][8 k-values of group kg]      B: lane supplies w[row n][8 k-values of group kg]
 //     D: lane receives out[token 4*kg + i][row n], i = 0..3
 // so a lane's four results belong to the row whose bytes that lane decodes, and the per-block scale of that row
-// is already in the lane's registers. The decoded weights are small integers (exact in binary16); products and
+// is already in the lane's registers.
+// Global loads use another lane order: lane l loads the bytes of (row l >> 2, k-group l & 3), so that the four lanes
+// of a quad read adjacent addresses and the cache sees one access per quad instead of one per lane. The registers
+// are then moved to the matrix-core order above with ds_bpermute (a transpose of the 16 x 4 lane grid). The decoded weights are small integers (exact in binary16); products and
 // sums are accumulated in binary32 by the matrix core; the binary16 block scale d multiplies the binary32
 // partial sum afterwards. A token's result never depends on the other token columns.
 #pragma once
@@ -55,7 +58,11 @@ __device__ __forceinline__ void qw_lut_build(u2 *lut) {
     for (uint32_t i = threadIdx.x; i < QW_LUT_ENTRIES; i += blockDim.x) lut[i] = qw_lut_entry(i);
 }
 
+#ifdef QW_EXP_NOMFMA
+__device__ __forceinline__ f4 qw_mfma(h8 a, h8 b, f4 c) { c[0] += (float)a[0] * (float)b[0] + (float)b[3]; c[1] += (float)a[5] * (float)b[7] + (float)b[5]; return c; }
+#else
 __device__ __forceinline__ f4 qw_mfma(h8 a, h8 b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+#endif
 
 // ---------------------------------------------------------------- IQ3_S (110-byte block of 256 values)
 // Bytes: d @0 (binary16), qs[64] @2, qh[8] @66, signs[32] @74, scales[4] @106 (kernels/moe_iq.metal:102-118).
@@ -72,12 +79,33 @@ struct qw_iq3_slice {
 
 __device__ __forceinline__ qw_iq3_slice qw_iq3_load(const uint8_t *blk, uint32_t kg) {
     qw_iq3_slice s;
+#ifdef QW_EXP_NOLOAD
+    s.qs = u4{kg * 0x01010101u, 0x23456789u * kg, 0x11111111u, 0x77777777u}; s.sg = u2{0x12345678u, kg}; s.qh = 0x55aa; s.sc = 0x37; s.d = 1.0f;
+    return s;
+#endif
     s.qs = *(const u4a2 *)(blk + 2 + 16 * kg);
     s.sg = *(const u2a2 *)(blk + 74 + 8 * kg);
     s.qh = *(const uint16_t *)(blk + 66 + 2 * kg);
     s.sc = blk[106 + kg];
     s.d = qw_h2f(*(const uint16_t *)blk);
     return s;
+}
+
+// Pull a register from the lane that loaded this lane's (row, k-group): source lane = 4 * n + kg.
+__device__ __forceinline__ uint32_t qw_pull(uint32_t v, uint32_t src4) { return (uint32_t)__builtin_amdgcn_ds_bpermute((int)src4, (int)v); }
+__device__ __forceinline__ uint32_t qw_pull_addr() {
+    const uint32_t l = threadIdx.x & 63;
+    return 4 * (4 * (l & 15) + (l >> 4));
+}
+__device__ __forceinline__ void qw_iq3_transpose(qw_iq3_slice &s, uint32_t src4) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) s.qs[i] = qw_pull(s.qs[i], src4);
+    s.sg.x = qw_pull(s.sg.x, src4);
+    s.sg.y = qw_pull(s.sg.y, src4);
+    const uint32_t m = qw_pull(s.qh | (s.sc << 16), src4);
+    s.qh = m & 0xffff;
+    s.sc = m >> 16;
+    s.d = __builtin_bit_cast(float, qw_pull(__builtin_bit_cast(uint32_t, s.d), src4));
 }
 
 // The eight binary16 values of step J, already multiplied by the sub-block factor.
@@ -155,6 +183,15 @@ template <bool LO> struct qw_afrag_glb {
 // compute unit and 14 KB per wave in flight (IQ3_S, 16 rows of K = 2048) this covers the HBM latency.
 template <int F, int NB> struct qw_chunk;
 
+// The two table indices of step J of a slice (see qw_iq3_step).
+template <int J> __device__ __forceinline__ void qw_iq3_idx(const qw_iq3_slice &s, uint32_t &i0, uint32_t &i1) {
+    const uint32_t q = s.qs[J / 2] >> (16 * (J % 2));
+    const uint32_t sg = s.sg[J / 4] >> (8 * (J % 4));
+    const uint32_t hb = s.qh >> (8 * (J / 4) + 2 * (J % 4));
+    i0 = (q & 255) | ((hb & 1) << 8) | ((sg & 15) << 9);
+    i1 = ((q >> 8) & 255) | ((hb & 2) << 7) | ((sg & 0xf0) << 5);
+}
+
 template <int NB> struct qw_chunk<21, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = 110;
     qw_iq3_slice s[NB];
@@ -162,26 +199,129 @@ template <int NB> struct qw_chunk<21, NB> {
 #pragma unroll
         for (int b = 0; b < NB; b++) s[b] = qw_iq3_load(p + 110 * b, kg);
     }
-    template <int J, class AF> __device__ __forceinline__ void step(int b, const u2 *lut, const AF &af, uint32_t k0, f4 &sub) const {
-        const h8 w = qw_iq3_step<J>(s[b], lut);
-        sub = qw_mfma(af.hi(k0 + 8 * J), w, sub);
-        if (AF::has_lo) sub = qw_mfma(af.lo(k0 + 8 * J), w, sub);
+    // All sixteen table reads of one block, issued together.
+    __device__ __forceinline__ void lookups(int b, const u2 *lut, u2 (&w)[16]) const {
+        uint32_t i[16];
+        qw_iq3_idx<0>(s[b], i[0], i[1]);
+        qw_iq3_idx<1>(s[b], i[2], i[3]);
+        qw_iq3_idx<2>(s[b], i[4], i[5]);
+        qw_iq3_idx<3>(s[b], i[6], i[7]);
+        qw_iq3_idx<4>(s[b], i[8], i[9]);
+        qw_iq3_idx<5>(s[b], i[10], i[11]);
+        qw_iq3_idx<6>(s[b], i[12], i[13]);
+        qw_iq3_idx<7>(s[b], i[14], i[15]);
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+#ifdef QW_EXP_NOLUT
+            w[j] = u2{i[j] * 0x00010001u | 0x3c003c00u, 0x3c003c00u};
+#elif defined(QW_EXP_NOCONFLICT)
+            w[j] = lut[(i[j] & ~15u) | (threadIdx.x & 15)]; // distinct bank pair per lane of a 16-lane group (wrong values, timing only)
+#elif defined(QW_EXP_NOCONFLICT32)
+            w[j] = lut[(i[j] & ~31u) | (threadIdx.x & 31)];
+#else
+            w[j] = lut[i[j]];
+#endif
+        }
     }
-    // acc += this chunk's contribution; k0 = k-offset of the chunk's first value.
+    // acc += this chunk's contribution; k0 = k-offset of the chunk's first value. Software pipeline over the blocks:
+    // the table reads of block b + 1 and the activation fragments of block b are in flight while block b - 1's
+    // matrix instructions run; two accumulators keep consecutive matrix instructions independent.
+    // Loaded in quad order (load() was called with the row and k-group of lane >> 2, lane & 3): bring every block
+    // to the matrix-core lane order.
+    __device__ __forceinline__ void transpose() {
+        const uint32_t src4 = qw_pull_addr();
+#pragma unroll
+        for (int b = 0; b < NB; b++) qw_iq3_transpose(s[b], src4);
+    }
     template <class AF> __device__ __forceinline__ void mac(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+        u2 w[2][16];
+        lookups(0, lut, w[0]);
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const uint32_t kb = k0 + 256 * b + 64 * kg;
-            f4 sub = {0, 0, 0, 0};
-            step<0>(b, lut, af, kb, sub);
-            step<1>(b, lut, af, kb, sub);
-            step<2>(b, lut, af, kb, sub);
-            step<3>(b, lut, af, kb, sub);
-            step<4>(b, lut, af, kb, sub);
-            step<5>(b, lut, af, kb, sub);
-            step<6>(b, lut, af, kb, sub);
-            step<7>(b, lut, af, kb, sub);
-            acc += s[b].d * sub;
+            h8 xh[8], xl[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+#ifdef QW_EXP_NOXFRAG
+                xh[j] = __builtin_bit_cast(h8, u4{kb + j, kg, 0x3c003c00u, 0x3c003c00u});
+                if (AF::has_lo) xl[j] = xh[j];
+#else
+                xh[j] = af.hi(kb + 8 * j);
+                if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
+#endif
+            }
+            if (b + 1 < NB) lookups(b + 1, lut, w[(b + 1) & 1]);
+            const _Float16 f0 = (_Float16)(int)(1 + 2 * (s[b].sc & 15)), f1 = (_Float16)(int)(1 + 2 * ((s[b].sc >> 4) & 15));
+            f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const h2 ff = j < 4 ? h2{f0, f0} : h2{f1, f1};
+                const u2 w0 = w[b & 1][2 * j], w1 = w[b & 1][2 * j + 1];
+                u4 raw = {w0.x, w0.y, w1.x, w1.y};
+#pragma unroll
+                for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+                const h8 wv = __builtin_bit_cast(h8, raw);
+                if (AF::has_lo) {
+                    sub0 = qw_mfma(xh[j], wv, sub0);
+                    sub1 = qw_mfma(xl[j], wv, sub1);
+                } else if (j & 1) sub1 = qw_mfma(xh[j], wv, sub1);
+                else sub0 = qw_mfma(xh[j], wv, sub0);
+            }
+            acc += s[b].d * (sub0 + sub1);
+        }
+    }
+    // The same arithmetic without the cross-block pipeline (fewer registers; for kernels that run more waves).
+    template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w[16];
+            lookups(b, lut, w);
+            h8 xh[8], xl[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                xh[j] = af.hi(kb + 8 * j);
+                if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
+            }
+            block_mfma(b, w, xh, xl, AF::has_lo, acc);
+        }
+    }
+    // One block's table values times two operand-A fragment sets (hi, lo), accumulated the way mac() does.
+    __device__ __forceinline__ void block_mfma(int b, const u2 (&w)[16], const h8 (&xh)[8], const h8 (&xl)[8], bool lo, f4 &acc) const {
+        const _Float16 f0 = (_Float16)(int)(1 + 2 * (s[b].sc & 15)), f1 = (_Float16)(int)(1 + 2 * ((s[b].sc >> 4) & 15));
+        f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const h2 ff = j < 4 ? h2{f0, f0} : h2{f1, f1};
+            u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
+#pragma unroll
+            for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+            const h8 wv = __builtin_bit_cast(h8, raw);
+            if (lo) {
+                sub0 = qw_mfma(xh[j], wv, sub0);
+                sub1 = qw_mfma(xl[j], wv, sub1);
+            } else if (j & 1) sub1 = qw_mfma(xh[j], wv, sub1);
+            else sub0 = qw_mfma(xh[j], wv, sub0);
+        }
+        acc += s[b].d * (sub0 + sub1);
+    }
+    // Two tiles that share every operand-A fragment (the down projection: both tiles belong to one expert): the
+    // fragments are read once per block. Each tile's arithmetic is exactly that of mac().
+    template <class AF> static __device__ __forceinline__ void mac2(const qw_chunk &t0, const qw_chunk &t1, const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc0, f4 &acc1) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w0[16], w1[16];
+            t0.lookups(b, lut, w0);
+            t1.lookups(b, lut, w1);
+            h8 xh[8], xl[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                xh[j] = af.hi(kb + 8 * j);
+                if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
+            }
+            t0.block_mfma(b, w0, xh, xl, AF::has_lo, acc0);
+            t1.block_mfma(b, w1, xh, xl, AF::has_lo, acc1);
         }
     }
 };
@@ -197,6 +337,22 @@ template <int NB> struct qw_chunk<8, NB> {
             d[b] = *(const uint16_t *)(p + 34 * b);
         }
     }
+    __device__ __forceinline__ void transpose() {
+        const uint32_t src4 = qw_pull_addr();
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            q[b].x = qw_pull(q[b].x, src4);
+            q[b].y = qw_pull(q[b].y, src4);
+        }
+#pragma unroll
+        for (int b = 0; b + 1 < NB; b += 2) { // two scales per pull
+            const uint32_t m = qw_pull((uint32_t)d[b] | ((uint32_t)d[b + 1] << 16), src4);
+            d[b] = (uint16_t)m;
+            d[b + 1] = (uint16_t)(m >> 16);
+        }
+        if (NB & 1) d[NB - 1] = (uint16_t)qw_pull(d[NB - 1], src4);
+    }
+    template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     template <class AF> __device__ __forceinline__ void mac(const u2 *, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -210,19 +366,19 @@ template <int NB> struct qw_chunk<8, NB> {
     }
 };
 
-// Blocks per chunk for a row of K values: the whole row for IQ3_S (K <= 2560), 16 blocks for Q8_0. 0 = no build.
-template <int F> __host__ __device__ constexpr int qw_chunk_blocks(int K) { return F == 21 ? (K == 512 ? 2 : K == 2048 ? 8 : K == 2560 ? 10 : 0) : (K % 512 == 0 ? 16 : 0); }
-
-// Two-chunk software pipeline over n items: load(i, chunk&) issues the loads of item i, use(i, chunk&) consumes them.
+// Two-chunk software pipeline over n items: load(i, chunk&) issues the loads of item i (in quad lane order),
+// use(i, chunk&) consumes them after the move to matrix-core lane order.
 template <class C, class L, class U> __device__ __forceinline__ void qw_pipeline(uint32_t n, L load, U use) {
     C a, b;
     if (n) load(0u, a);
     uint32_t i = 0;
     while (i < n) {
         if (i + 1 < n) load(i + 1, b);
+        a.transpose();
         use(i, a);
         if (++i >= n) break;
         if (i + 1 < n) load(i + 1, a);
+        b.transpose();
         use(i, b);
         ++i;
     }

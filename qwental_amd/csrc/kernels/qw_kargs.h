@@ -60,10 +60,9 @@ typedef struct {
     uint16_t *H;
     uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane; /* hplane: halves between the hi and lo planes */
     const void *glut;
-    /* shared expert's down projection, done by the same launch when Wsd != NULL: Psh[t][row] from slot topk */
-    const uint8_t *Wsd;
-    float *Psh;
-    uint32_t sd_rowbytes, pad;
+    /* the shared expert's gate/up, done by the same launch when Wsg != NULL: all tokens, slot topk */
+    const uint8_t *Wsg, *Wsu;
+    uint32_t sg_rowbytes, pad;
 } qwk_gu_args;
 
 /* down projection. routed: Pg[t][slot][row] for the tokens in mask[u]; shared != 0: Psh[t][row] from slot topk. */
@@ -74,15 +73,18 @@ typedef struct {
     float *P; /* Pg [nbr][topk][D] or Psh [nbr][D] */
     uint32_t D, I, rowbytes, nbr, topk, gnb, shared, hplane;
     const void *glut;
+    /* the shared expert's down projection, done by the same launch when Wsd != NULL: Psh[t][row] from slot topk */
+    const uint8_t *Wsd;
+    float *Psh;
+    uint32_t sd_rowbytes, snbr; /* snbr: token count of the shared part */
 } qwk_dn_args;
 
-/* front part of a layer in one launch: router rows, the shared expert's gate/up, and the selection, which the
- * last router workgroup to finish performs (counter in cnt, left at zero). */
+/* front part of a layer: router rows (the selection is the launch after it). sel / cnt / topk / gnb are unused. */
 typedef struct {
     qwk_router_args r;
-    qwk_gu_args g;      /* shared == 1 */
+    uint8_t *sel;
     uint32_t *cnt;
-    uint32_t nrouter_wg, do_select;
+    uint32_t topk, gnb;
 } qwk_pre_args;
 
 typedef struct { /* out[t][row] = half(sum_s w[t][s] * Pg[t][s][row] + w[t][topk] * Psh[t][row]) */

@@ -7,7 +7,8 @@
 // before the current one is decoded, so every wave keeps about one tile of weight bytes in flight.
 #include "qw_common.hip.h"
 
-#define QW_WG 512          // threads per workgroup of the weight-streaming kernels (8 waves)
+#define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
+#define QW_WG_GU 768       // gate/up and dense matvec: 12 waves, three per SIMD (a wave issues at most one instruction in ~6 cycles)
 #define QW_XF_MAXK 2560    // largest K whose activations are staged in LDS in fragment order (K * 32 bytes)
 
 __device__ __forceinline__ uint32_t qw_wave() { return threadIdx.x >> 6; }
@@ -62,8 +63,9 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     const uint32_t cpr = a.K / (C::BLK_K * CH), mytiles = w0 < a.ntiles ? (a.ntiles - w0 + nw - 1) / nw : 0;
+    const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t t) {
-        const uint32_t r = 16 * t + n;
+        const uint32_t r = 16 * t + nl;
         return a.W + (size_t)(r < a.N ? r : a.N - 1) * a.rowbytes;
     };
     if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
@@ -73,11 +75,11 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
     f4 acc = {0, 0, 0, 0};
     qw_pipeline<C>(mytiles * cpr,
-        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kl); },
         [&](uint32_t i, const C &c) {
             const uint32_t ci = i % cpr;
-            if (XLDS) c.mac(lut, afl, ci * CH * C::BLK_K, kg, acc);
-            else c.mac(lut, afg, ci * CH * C::BLK_K, kg, acc);
+            if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
+            else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 == cpr) {
                 const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
                 if (r < a.N)
@@ -94,12 +96,12 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
         });
 }
 #define QW_QMV(F, CH, XLDS, SFX)                                                                        \
-    extern "C" __global__ __launch_bounds__(QW_WG) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
         __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                                                \
         __shared__ u4 xf[XLDS ? QW_XF_MAXK * 2 : 1];                                                    \
         qmv_body<F, CH, XLDS>(a, lut, xf);                                                              \
     }
-QW_QMV(21, 8, true, _c8) QW_QMV(21, 2, true, _c2) QW_QMV(21, 10, true, _c10) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
+QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
 QW_QMV(8, 16, true, _c16) QW_QMV(8, 1, true, _c1) QW_QMV(8, 1, false, _c1g)
 
 // ================================================================ router (kernels/moe_gg.metal:25-41)
@@ -134,6 +136,44 @@ template <int WF, int NB> __device__ __forceinline__ void router_row(const qwk_r
         if (lane == 0 && (uint32_t)t < a.nb) a.logits[(size_t)t * (a.E + 1) + r] = v;
     }
 }
+// The same arithmetic with the activations read from LDS (xs: binary16 [nb][D], copied there by the workgroup).
+template <int WF, int NB> __device__ __forceinline__ void router_row_lds(const qwk_router_args &a, const uint16_t *xs, uint32_t r, uint32_t lane) {
+    const uint16_t *w = r < a.E ? a.Wr + (size_t)r * a.D : a.Wsg;
+    float acc[NB];
+#pragma unroll
+    for (int t = 0; t < NB; t++) acc[t] = 0;
+    for (uint32_t c = lane; c < a.D / 8; c += 64) {
+        const u4 wv = *(const u4 *)(w + 8 * c);
+        float wf[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            wf[2 * i] = WF == 30 ? qw_bf2f((uint16_t)wv[i]) : qw_h2f((uint16_t)wv[i]);
+            wf[2 * i + 1] = WF == 30 ? qw_bf2f((uint16_t)(wv[i] >> 16)) : qw_h2f((uint16_t)(wv[i] >> 16));
+        }
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            const h8 xv = *(const h8 *)(xs + (size_t)((uint32_t)t < a.nb ? t : a.nb - 1) * a.D + 8 * c);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[t] = __builtin_fmaf(wf[i], (float)xv[i], acc[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NB; t++) {
+        float v = acc[t];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        if (lane == 0 && (uint32_t)t < a.nb) a.logits[(size_t)t * (a.E + 1) + r] = v;
+    }
+}
+template <int WF> __device__ __forceinline__ void router_rows_lds(const qwk_router_args &a, const uint16_t *xs, uint32_t r, uint32_t lane) {
+    if (r > a.E) return;
+    if (a.nb <= 1) router_row_lds<WF, 1>(a, xs, r, lane);
+    else if (a.nb <= 2) router_row_lds<WF, 2>(a, xs, r, lane);
+    else if (a.nb <= 4) router_row_lds<WF, 4>(a, xs, r, lane);
+    else if (a.nb <= 8) router_row_lds<WF, 8>(a, xs, r, lane);
+    else router_row_lds<WF, 16>(a, xs, r, lane);
+}
+
 template <int WF> __device__ __forceinline__ void router_rows(const qwk_router_args &a, uint32_t r, uint32_t lane) {
     if (r > a.E) return;
     if (a.nb <= 1) router_row<WF, 1>(a, r, lane);
@@ -151,6 +191,9 @@ extern "C" __global__ __launch_bounds__(256) void qwk_router_w30(qwk_router_args
 // appearance over the flat index. Scratch in LDS: ids[256], lead[256], um[256], first[1024], one counter.
 struct qw_sel_scratch {
     uint32_t ids[256], lead[256], um[256], first[1024], U;
+    uint32_t ue[256];            // results are assembled here and written to global memory in one pass at the end,
+    uint32_t slot[256 * 16 / 4]; // so that no barrier has to wait for global stores
+    float w[16 * 17];
 };
 
 // PER = E / 64 values per lane, lane l holding experts l * PER .. l * PER + PER - 1 (lowest lane = lowest index).
@@ -160,10 +203,19 @@ template <int PER> __device__ __forceinline__ void select_token(const float *lg,
     for (int j = 0; j < PER; j++) k[j] = qw_fkey(lg[lane * PER + j]);
     uint32_t pk = 0;
     for (uint32_t r = 0; r < K; r++) {
-        uint32_t bk = k[0], bj = 0;
+        // lane-local maximum by a balanced tree; among equals the lower position wins at every node
+        uint32_t tk[PER], tj[PER];
 #pragma unroll
-        for (int j = 1; j < PER; j++)
-            if (k[j] > bk) { bk = k[j]; bj = j; } // strict: the lowest j among equals
+        for (int j = 0; j < PER; j++) { tk[j] = k[j]; tj[j] = j; }
+#pragma unroll
+        for (int w = 1; w < PER; w *= 2)
+#pragma unroll
+            for (int j = 0; j + w < PER; j += 2 * w) {
+                const bool up = tk[j + w] > tk[j];
+                tk[j] = up ? tk[j + w] : tk[j];
+                tj[j] = up ? tj[j + w] : tj[j];
+            }
+        const uint32_t bk = tk[0], bj = tj[0];
         const uint32_t m = qw_wave_max_u32(bk);
         const uint32_t L = (uint32_t)__builtin_ctzll(__ballot(bk == m)); // lowest lane among equals
         const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)bj, (int)L);
@@ -215,22 +267,21 @@ __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 ||
 __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, float *lgs) {
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
-    uint32_t *ue = (uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mask = (uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
-    uint8_t *slot = a.sel + QW_SEL_OFF_SLOT(gnb, K);
-    float *w = (float *)(a.sel + QW_SEL_OFF_W(gnb, K));
     const bool fast = qw_select_fast_e(E);
     for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
-    for (uint32_t i = tid; i < GU; i += nth) ue[i] = mask[i] = 0, s.um[i] = 0;
-    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)slot)[i] = 0;
+    for (uint32_t i = tid; i < GU; i += nth) s.ue[i] = 0, s.um[i] = 0;
+    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) s.slot[i] = 0;
+    for (uint32_t i = tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
+    __syncthreads();
     for (uint32_t t = wave; t < a.nbr; t += nwv) {
         const float *lg = a.logits + (size_t)t * (E + 1);
         switch (fast ? E : 0u) {
-        case 64: select_token<1>(lg, E, K, t, w, s.ids, lane); break;
-        case 128: select_token<2>(lg, E, K, t, w, s.ids, lane); break;
-        case 256: select_token<4>(lg, E, K, t, w, s.ids, lane); break;
-        case 512: select_token<8>(lg, E, K, t, w, s.ids, lane); break;
-        case 1024: select_token<16>(lg, E, K, t, w, s.ids, lane); break;
-        default: select_token_any(lg, lgs + (size_t)wave * 1024, E, K, t, w, s.ids, lane);
+        case 64: select_token<1>(lg, E, K, t, s.w, s.ids, lane); break;
+        case 128: select_token<2>(lg, E, K, t, s.w, s.ids, lane); break;
+        case 256: select_token<4>(lg, E, K, t, s.w, s.ids, lane); break;
+        case 512: select_token<8>(lg, E, K, t, s.w, s.ids, lane); break;
+        case 1024: select_token<16>(lg, E, K, t, s.w, s.ids, lane); break;
+        default: select_token_any(lg, lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
         }
     }
     __syncthreads();
@@ -257,17 +308,27 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     if (tid < UM) {
         const uint32_t u = s.lead[f] - 1, t = tid / K;
         atomicOr(&s.um[u], 1u << t);
-        slot[u * gnb + t] = (uint8_t)(tid % K);
-        if (f == tid) ue[u] = s.ids[tid];
+        ((uint8_t *)s.slot)[u * gnb + t] = (uint8_t)(tid % K);
+        if (f == tid) s.ue[u] = s.ids[tid];
     }
     __syncthreads();
-    if (tid < s.U) mask[tid] = s.um[tid];
-    if (tid == 0) *(uint32_t *)a.sel = s.U;
+    // the record, in one pass of dword stores: U | ue[GU] | mask[GU] | slot[GU][gnb] | w[gnb][K + 1]
+    uint32_t *out = (uint32_t *)a.sel;
+    const uint32_t n_slot = GU * gnb / 4, n_w = gnb * (K + 1), total = 1 + 2 * GU + n_slot + n_w;
+    for (uint32_t i = tid; i < total; i += nth) {
+        uint32_t v;
+        if (i == 0) v = s.U;
+        else if (i < 1 + GU) v = s.ue[i - 1];
+        else if (i < 1 + 2 * GU) v = (i - 1 - GU) < s.U ? s.um[i - 1 - GU] : 0;
+        else if (i < 1 + 2 * GU + n_slot) v = s.slot[i - 1 - 2 * GU];
+        else v = __builtin_bit_cast(uint32_t, s.w[i - 1 - 2 * GU - n_slot]);
+        out[i] = v;
+    }
 }
 
-extern "C" __global__ __launch_bounds__(512) void qwk_select(qwk_select_args a) {
+extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a) {
     __shared__ qw_sel_scratch s;
-    __shared__ float lgs[8 * 1024];
+    __shared__ float lgs[16 * 1024];
     select_all(a, s, lgs);
 }
 
@@ -293,16 +354,17 @@ template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_a
     const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
     const uint32_t cpr = a.D / (C::BLK_K * CH), mine = w0 < ntasks ? (ntasks - w0 + nw - 1) / nw : 0;
     const qw_afrag_lds af = {xf, n};
+    const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t task) {
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe), e = a.shared ? 0 : sc->ue[u];
-        return (n < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (n & 7)) * a.rowbytes;
+        return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
     qw_pipeline<C>(mine * cpr,
-        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kl); },
         [&](uint32_t i, const C &c) {
             const uint32_t ci = i % cpr;
-            c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
+            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 != cpr) return;
             const uint32_t task = w0 + (i / cpr) * nw, u = task / tpe, j0 = 8 * (task % tpe);
             const uint32_t m = a.shared ? qw_all_tokens(a.nbr) : sc->mask[u];
@@ -323,20 +385,75 @@ template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_a
         });
 }
 
-// The shared expert's down projection inside the gate/up launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
+// FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
+template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
+    if (FGU == 21 || FSG == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+    if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+    __syncthreads();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    if (FSG != 0) {
+        if (a.Wsg) { // the shared expert's tiles go to the first waves
+            qwk_gu_args sa = a;
+            sa.Wg = a.Wsg;
+            sa.Wu = a.Wsu;
+            sa.rowbytes = a.sg_rowbytes;
+            sa.shared = 1;
+            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw);
+        }
+    }
+    // the waves that did a shared tile come last in the routed deal, so that the work stays level
+    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw);
+}
+#define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
+        __shared__ u2 lut[(FGU == 21 || FSG == 21) ? QW_LUT_ENTRIES : 1];                                 \
+        __shared__ u4 xf[QW_XF_MAXK * 2];                                                                 \
+        __shared__ qw_sel_cache sc;                                                                       \
+        gu_body<FGU, CHGU, FSG, CHSG>(a, lut, xf, &sc);                                                   \
+    }
+// K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
+QW_GU(21, 2, 0, 1, qwk_gu_f21_c2) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
+QW_GU(8, 16, 0, 1, qwk_gu_f8_c16) QW_GU(8, 1, 0, 1, qwk_gu_f8_c1)
+QW_GU(21, 2, 21, 2, qwk_gu_f21_c2_s21_c2) QW_GU(21, 2, 8, 16, qwk_gu_f21_c2_s8_c16)
+QW_GU(21, 1, 21, 1, qwk_gu_f21_c1_s21_c1) QW_GU(21, 1, 8, 1, qwk_gu_f21_c1_s8_c1)
+QW_GU(8, 16, 8, 16, qwk_gu_f8_c16_s8_c16) QW_GU(8, 16, 21, 2, qwk_gu_f8_c16_s21_c2)
+QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_s8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_s21_c1)
+
+// ================================================================ front part of a layer (kernels/moe_gg.metal:534-590)
+// Router rows with the activations copied into LDS once per workgroup (8 rows per workgroup). The selection is a
+// launch of its own (qwk_select): handing it to the last router workgroup through a device-wide counter was measured
+// slower than the kernel boundary. The shared expert's gate/up runs in the gate/up launch.
+template <int WF> __device__ __forceinline__ void pre_body(const qwk_pre_args &a, u4 *lds) {
+    const uint32_t nx = a.r.nb * a.r.D / 8; // 16-byte units of x
+    for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) lds[i] = ((const u4 *)a.r.x)[i];
+    __syncthreads();
+    router_rows_lds<WF>(a.r, (const uint16_t *)lds, blockIdx.x * (blockDim.x >> 6) + qw_wave(), qw_lane());
+}
+extern "C" __global__ __launch_bounds__(QW_WG) void qwk_pre_w1(qwk_pre_args a) {
+    __shared__ u4 lds[QW_XF_MAXK * 2];
+    pre_body<1>(a, lds);
+}
+extern "C" __global__ __launch_bounds__(QW_WG) void qwk_pre_w30(qwk_pre_args a) {
+    __shared__ u4 lds[QW_XF_MAXK * 2];
+    pre_body<30>(a, lds);
+}
+
+// ================================================================ down (kernels/moe_gg.metal:456-483, 606-617, 639-652)
+// The shared expert's down projection rides in the same launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
 // planes) of every token straight from global memory. Wave w takes tiles w, w + nw, ...
-template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const qwk_gu_args &a, const u2 *lut, uint32_t w0, uint32_t nw) {
+template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const qwk_dn_args &a, const u2 *lut, uint32_t w0, uint32_t nw) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk;
     const uint32_t ntiles = a.D / 16, cpr = a.I / (C::BLK_K * CH), mine = w0 < ntiles ? (ntiles - w0 + nw - 1) / nw : 0;
     qw_afrag_glb<true> af = {nullptr, nullptr};
-    if (n < a.nbr) {
+    if (n < a.snbr) {
         af.rowhi = a.H + ((size_t)n * (K + 1) + K) * a.I;
         af.rowlo = af.rowhi + a.hplane;
     }
     f4 acc = {0, 0, 0, 0};
     qw_pipeline<C>(mine * cpr,
-        [&](uint32_t i, C &c) { c.load(a.Wsd + (size_t)(16 * (w0 + (i / cpr) * nw) + n) * a.sd_rowbytes + (size_t)(i % cpr) * CH * C::BLK_B, kg); },
+        [&](uint32_t i, C &c) { c.load(a.Wsd + (size_t)(16 * (w0 + (i / cpr) * nw) + (lane >> 2)) * a.sd_rowbytes + (size_t)(i % cpr) * CH * C::BLK_B, lane & 3); },
         [&](uint32_t i, const C &c) {
             const uint32_t ci = i % cpr;
             c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
@@ -344,88 +461,23 @@ template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const
             const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++)
-                if (4 * kg + j < a.nbr) a.Psh[(size_t)(4 * kg + j) * a.D + r] = acc[j];
+                if (4 * kg + j < a.snbr) a.Psh[(size_t)(4 * kg + j) * a.D + r] = acc[j];
             acc = f4{0, 0, 0, 0};
         });
 }
 
-// FGU: routed gate/up format; FSD: shared down format (0 = no shared down in this launch).
-template <int FGU, int CHGU, int FSD, int CHSD> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
-    if (FGU == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
-    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
-    if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
-    __syncthreads();
-    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
-    if (FSD != 0) {
-        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, w0, nw);
-    }
-    // the waves that did a shared-down tile come last in the routed deal, so that the work stays level
-    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw);
-}
-#define QW_GU(FGU, CHGU, FSD, CHSD, NAME)                                                                 \
-    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_gu_args a) {                             \
-        __shared__ u2 lut[(FGU == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];                                 \
-        __shared__ u4 xf[QW_XF_MAXK * 2];                                                                 \
-        __shared__ qw_sel_cache sc;                                                                       \
-        gu_body<FGU, CHGU, FSD, CHSD>(a, lut, xf, &sc);                                                   \
-    }
-// K = D for gate/up: 2048 (8 blocks a chunk for IQ3_S, 16 for Q8_0), 2560 (10 / 16), other (1). K = I for down: 512 (2 / 16), other (1).
-QW_GU(21, 8, 0, 1, qwk_gu_f21_c8) QW_GU(21, 10, 0, 1, qwk_gu_f21_c10) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
-QW_GU(8, 16, 0, 1, qwk_gu_f8_c16) QW_GU(8, 1, 0, 1, qwk_gu_f8_c1)
-QW_GU(21, 8, 21, 2, qwk_gu_f21_c8_sd21_c2) QW_GU(21, 8, 8, 16, qwk_gu_f21_c8_sd8_c16)
-QW_GU(21, 10, 21, 1, qwk_gu_f21_c10_sd21_c1) QW_GU(21, 10, 8, 1, qwk_gu_f21_c10_sd8_c1)
-QW_GU(21, 1, 21, 1, qwk_gu_f21_c1_sd21_c1) QW_GU(21, 1, 8, 1, qwk_gu_f21_c1_sd8_c1)
-QW_GU(8, 16, 8, 16, qwk_gu_f8_c16_sd8_c16) QW_GU(8, 16, 21, 2, qwk_gu_f8_c16_sd21_c2)
-QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_sd8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_sd21_c1)
-
-// ================================================================ front part of a layer in one launch
-// (kernels/moe_gg.metal:534-590) Workgroups [0, nrouter_wg): router rows, 8 per workgroup; the rest: the shared
-// expert's gate/up tiles. The router workgroup that finishes last runs the selection (the others' logits are visible
-// to it: every thread fences its stores before the workgroup's counter increment).
-template <int WF, int F, int CH> __device__ __forceinline__ void pre_body(const qwk_pre_args &a, u2 *lut, u4 *xf) {
-    __shared__ uint32_t last;
-    if (blockIdx.x >= a.nrouter_wg) {
-        if (F == 21) qw_lut_copy(lut, (const u2 *)a.g.glut);
-        qw_stage_x(xf, a.g.x, a.g.D, a.g.D, a.g.nbr);
-        __syncthreads();
-        gu_tasks<F, CH>(a.g, lut, xf, nullptr, (blockIdx.x - a.nrouter_wg) * (blockDim.x >> 6) + qw_wave(), (gridDim.x - a.nrouter_wg) * (blockDim.x >> 6));
-        return;
-    }
-    router_rows<WF>(a.r, blockIdx.x * (blockDim.x >> 6) + qw_wave(), qw_lane());
-    if (!a.do_select) return;
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) last = atomicAdd(a.cnt, 1u) == a.nrouter_wg - 1;
-    __syncthreads();
-    if (!last) return;
-    __threadfence();
-    // the LDS of a router workgroup is free: the selection's scratch goes where the staged activations would be
-    qw_sel_scratch *s = (qw_sel_scratch *)xf;
-    const qwk_select_args sa = {a.r.logits, const_cast<uint8_t *>(a.g.sel), a.r.nb, a.r.E, a.g.topk, a.g.gnb};
-    select_all(sa, *s, (float *)(xf + 1024));
-    if (threadIdx.x == 0) *a.cnt = 0;
-}
-#define QW_PRE(WF, F, CH, NAME)                                                       \
-    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {        \
-        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                              \
-        __shared__ u4 xf[QW_XF_MAXK * 2];                                             \
-        pre_body<WF, F, CH>(a, lut, xf);                                              \
-    }
-QW_PRE(1, 21, 8, qwk_pre_w1_f21_c8) QW_PRE(1, 21, 10, qwk_pre_w1_f21_c10) QW_PRE(1, 21, 1, qwk_pre_w1_f21_c1)
-QW_PRE(1, 8, 16, qwk_pre_w1_f8_c16) QW_PRE(1, 8, 1, qwk_pre_w1_f8_c1)
-QW_PRE(30, 21, 8, qwk_pre_w30_f21_c8) QW_PRE(30, 21, 10, qwk_pre_w30_f21_c10) QW_PRE(30, 21, 1, qwk_pre_w30_f21_c1)
-QW_PRE(30, 8, 16, qwk_pre_w30_f8_c16) QW_PRE(30, 8, 1, qwk_pre_w30_f8_c1)
-
-// ================================================================ down (kernels/moe_gg.metal:456-483, 639-652)
 // Workgroup task = (expert u, block of 256 rows): the H rows (hi and lo planes) of the tokens that picked u are staged
 // in LDS in fragment order, double-buffered; wave w owns rows 32 w .. 32 w + 31 of the block = two tiles.
 // One barrier per task; the weight loads of the next task are in flight across it.
-template <int F, int CH> __device__ __forceinline__ void dn_body(const qwk_dn_args &a, u2 *lut, u4 *abuf /* [2][2][I/8*16] */, qw_sel_cache *sc) {
+template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_body(const qwk_dn_args &a, u2 *lut, u4 *abuf /* [2][2][I/8*16] */, qw_sel_cache *sc) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb, wave = qw_wave();
-    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
     qw_sel_load(*sc, a.sel, K, gnb);
     __syncthreads();
+    if (FSD != 0) {
+        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, blockIdx.x * (blockDim.x >> 6) + wave, gridDim.x * (blockDim.x >> 6));
+    }
     const uint32_t U = sc->U, bpe = a.D / 256, ntasks = U * bpe, mine = blockIdx.x < ntasks ? (ntasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
     const uint32_t nfrag = (a.I / 8) * 16; // 16-byte fragments per plane
     auto stage = [&](uint32_t it) { // operand A of this workgroup's it-th task into buffer it & 1
@@ -438,61 +490,67 @@ template <int F, int CH> __device__ __forceinline__ void dn_body(const qwk_dn_ar
             dst[i] = v;
         }
     };
+    const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t it, uint32_t tile) {
-        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, r = 256 * (task % bpe) + 32 * wave + 16 * tile + n;
+        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, r = 256 * (task % bpe) + 32 * wave + 16 * tile + nl;
         return a.Wd + ((size_t)sc->ue[u] * a.D + r) * a.rowbytes;
     };
-    auto compute = [&](uint32_t it, const C &t0, const C &t1) {
+    auto compute = [&](uint32_t it, C &t0, C &t1) {
+        t0.transpose();
+        t1.transpose();
         const u4 *base = abuf + (size_t)(it & 1) * 2 * nfrag;
         const qw_afrag_lds2 af = {base, base + nfrag, n};
         const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, m = sc->mask[u];
+        f4 acc2[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        C::mac2(t0, t1, lut, af, 0, kg, acc2[0], acc2[1]);
 #pragma unroll
         for (int tile = 0; tile < 2; tile++) {
-            f4 acc = {0, 0, 0, 0};
-            (tile ? t1 : t0).mac(lut, af, 0, kg, acc);
             const uint32_t r = 256 * (task % bpe) + 32 * wave + 16 * tile + n;
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++) {
                 const uint32_t tok = 4 * kg + j;
-                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc[j];
+                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc2[tile][j];
             }
         }
     };
     C a0, a1, b0, b1;
     if (mine) {
-        a0.load(rowp(0, 0), kg);
-        a1.load(rowp(0, 1), kg);
+        a0.load(rowp(0, 0), kl);
+        a1.load(rowp(0, 1), kl);
         stage(0);
     }
     __syncthreads();
     for (uint32_t it = 0; it < mine; it += 2) {
-        if (it + 1 < mine) { b0.load(rowp(it + 1, 0), kg); b1.load(rowp(it + 1, 1), kg); stage(it + 1); }
+        if (it + 1 < mine) { b0.load(rowp(it + 1, 0), kl); b1.load(rowp(it + 1, 1), kl); stage(it + 1); }
         compute(it, a0, a1);
         __syncthreads();
         if (it + 1 >= mine) break;
-        if (it + 2 < mine) { a0.load(rowp(it + 2, 0), kg); a1.load(rowp(it + 2, 1), kg); stage(it + 2); }
+        if (it + 2 < mine) { a0.load(rowp(it + 2, 0), kl); a1.load(rowp(it + 2, 1), kl); stage(it + 2); }
         compute(it + 1, b0, b1);
         __syncthreads();
     }
 }
-#define QW_DN(F, CH, IMAX, NAME)                                                      \
+#define QW_DN(F, CH, FSD, CHSD, IMAX, NAME)                                           \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
-        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                              \
+        __shared__ u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];               \
         __shared__ u4 abuf[2 * 2 * (IMAX / 8) * 16];                                  \
         __shared__ qw_sel_cache sc;                                                   \
-        dn_body<F, CH>(a, lut, abuf, &sc);                                            \
+        dn_body<F, CH, FSD, CHSD>(a, lut, abuf, &sc);                                 \
     }
 // I = 512 is the synthetic shape (whole row = one chunk of 2 IQ3_S blocks); Q8_0 down weights take the any-shape kernel
-QW_DN(21, 2, 512, qwk_dn_f21_i512)
+QW_DN(21, 2, 0, 1, 512, qwk_dn_f21_i512) QW_DN(21, 2, 21, 2, 512, qwk_dn_f21_i512_s21) QW_DN(21, 2, 8, 16, 512, qwk_dn_f21_i512_s8)
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
-template <int F> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
     typedef qw_chunk<F, 1> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
-    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
     qw_sel_load(*sc, a.sel, K, gnb);
     __syncthreads();
     const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    if (FSD != 0) {
+        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, 1>(a, lut, w0, nw);
+    }
     const uint32_t cpr = a.I / C::BLK_K;
     for (uint32_t task = w0; task < ntasks; task += nw) {
         const uint32_t u = task / tpe, r = 16 * (task % tpe) + n, m = sc->mask[u];
@@ -501,9 +559,9 @@ template <int F> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &
             af.rowhi = a.H + ((size_t)n * (K + 1) + sc->slot[u * gnb + n]) * a.I;
             af.rowlo = af.rowhi + a.hplane;
         }
-        const uint8_t *row = a.Wd + ((size_t)sc->ue[u] * a.D + r) * a.rowbytes;
+        const uint8_t *row = a.Wd + ((size_t)sc->ue[u] * a.D + 16 * (task % tpe) + (lane >> 2)) * a.rowbytes; // quad order
         f4 acc = {0, 0, 0, 0};
-        qw_pipeline<C>(cpr, [&](uint32_t i, C &c) { c.load(row + (size_t)i * C::BLK_B, kg); },
+        qw_pipeline<C>(cpr, [&](uint32_t i, C &c) { c.load(row + (size_t)i * C::BLK_B, lane & 3); },
                        [&](uint32_t i, const C &c) { c.mac(lut, af, i * C::BLK_K, kg, acc); });
 #pragma unroll
         for (uint32_t j = 0; j < 4; j++) {
@@ -512,15 +570,14 @@ template <int F> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &
         }
     }
 }
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f21_any(qwk_dn_args a) {
-    __shared__ u2 lut[QW_LUT_ENTRIES];
-    __shared__ qw_sel_cache sc;
-    dn_any_body<21>(a, lut, &sc);
-}
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_f8_any(qwk_dn_args a) {
-    __shared__ qw_sel_cache sc;
-    dn_any_body<8>(a, nullptr, &sc);
-}
+#define QW_DN_ANY(F, FSD, NAME)                                                       \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
+        __shared__ u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];               \
+        __shared__ qw_sel_cache sc;                                                   \
+        dn_any_body<F, FSD>(a, lut, &sc);                                             \
+    }
+QW_DN_ANY(21, 0, qwk_dn_f21_any) QW_DN_ANY(21, 21, qwk_dn_f21_any_s21) QW_DN_ANY(21, 8, qwk_dn_f21_any_s8)
+QW_DN_ANY(8, 0, qwk_dn_f8_any) QW_DN_ANY(8, 21, qwk_dn_f8_any_s21) QW_DN_ANY(8, 8, qwk_dn_f8_any_s8)
 
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).

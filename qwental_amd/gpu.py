@@ -10,7 +10,8 @@ _lib = None
 
 
 def lib_path():
-    return os.path.join(HERE, "libqwgpu_hip.so")
+    """The built library; QW_HIP_LIB selects another build of it (experiments)."""
+    return os.environ.get("QW_HIP_LIB") or os.path.join(HERE, "libqwgpu_hip.so")
 
 
 class QwBuf(C.Structure):
