@@ -45,7 +45,7 @@ def cpu_baseline(stack, x, nb, lg_dev, budget_s=20.0):
     from oracle import oracle as o
     cores = o.max_threads()
     t_used, n, worst = 0.0, 0, 0.0
-    while t_used < budget_s and n < stack.L and n < 8:
+    while t_used < budget_s and n < stack.L and n < len(lg_dev):
         m = stack.layer_weights_host(n)
         lg = lg_dev[n]
         t0 = time.perf_counter()
@@ -118,7 +118,7 @@ def main():
             "kernel_us_mean": {k: float(np.mean(v)) for k, v in per_kernel.items()},
             "setup_s": setup_s}
     if not a.no_cpu:
-        lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(min(8, stack.L))]
+        lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)
     print(json.dumps(line))
     stack.free()

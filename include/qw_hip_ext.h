@@ -33,6 +33,10 @@ bool qw_hip_buf_read(const qw_buf *b, size_t offset, void *dst, size_t len);
 /* Device address of a buffer (for tools that pass it to their own code). */
 void *qw_hip_buf_devptr(const qw_buf *b);
 
+/* The define-block front end of qw_gpu_compile() without a device: parses src as qw_gpu_compile would, and on
+ * success writes the names of the kernels it would register to names (comma separated). For host-side tests. */
+bool qw_hip_compile_check(const char *src, size_t len, char *err, size_t errlen, char *names, size_t nameslen);
+
 /* Last error text of this device (empty string if none); cleared by qw_batch_begin. */
 const char *qw_hip_last_error(const qw_gpu *g);
 /* Number of compute units and the name of the code-object architecture the library was built for. */

@@ -140,7 +140,7 @@ qw_gpu *qw_gpu_open(void) {
     if (!g) return NULL;
     hipDeviceProp_t pr;
     if (hipSetDevice(0) != hipSuccess || hipGetDeviceProperties(&pr, 0) != hipSuccess) { free(g); return NULL; }
-    snprintf(g->name, sizeof g->name, "%s (%s)", pr.name, pr.gcnArchName);
+    snprintf(g->name, sizeof g->name, "%s (%s, %d CUs)", pr.name[0] ? pr.name : "AMD Instinct", pr.gcnArchName, pr.multiProcessorCount);
     g->total_mem = pr.totalGlobalMem;
     g->ncu = pr.multiProcessorCount;
     if (strncmp(pr.gcnArchName, "gfx950", 6) != 0) {
@@ -327,6 +327,21 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
 #undef FAIL
 out:
     free(d);
+    return ok;
+}
+
+bool qw_hip_compile_check(const char *src, size_t len, char *err, size_t errlen, char *names, size_t nameslen) {
+    qw_gpu *g = calloc(1, sizeof *g); // no device behind it: only the kernel registry is touched
+    if (!g) return false;
+    g->kernels = calloc(QW_MAX_KERNELS, sizeof *g->kernels);
+    const bool ok = g->kernels && qw_gpu_compile(g, src, len, err, errlen);
+    if (ok && names && nameslen) {
+        size_t n = 0;
+        names[0] = 0;
+        for (int i = 0; i < g->nkernels; i++) n += (size_t)snprintf(names + n, n < nameslen ? nameslen - n : 0, "%s%s", i ? "," : "", g->kernels[i].name);
+    }
+    free(g->kernels);
+    free(g);
     return ok;
 }
 

@@ -47,6 +47,7 @@ SYMBOLS = [
     ("qw_hip_buf_new_device", _b, [_vp, _sz, _pb]), ("qw_hip_buf_mark_dirty", None, [_pb]),
     ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
+    ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
     ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),
     ("qw_hip_profile_mean", _d, [_vp, C.c_char_p, C.POINTER(_i)]),
     ("qw_hip_profile_entry", C.c_char_p, [_vp, _i, C.POINTER(_d)]),
@@ -75,6 +76,15 @@ def load_lib():
         f.argtypes = args
     _lib = L
     return L
+
+
+def compile_check(defs):
+    """(ok, error text, kernel names) of a define block, without a device."""
+    L = load_lib()
+    err, names = C.create_string_buffer(4096), C.create_string_buffer(4096)
+    src = defs.encode()
+    ok = L.qw_hip_compile_check(src, len(src), err, len(err), names, len(names))
+    return ok, err.value.decode(), [n for n in names.value.decode().split(",") if n]
 
 
 class Buf:

@@ -1,0 +1,105 @@
+"""Host logic of the HIP backend that runs without a GPU: the library loads, exports every symbol the headers
+declare, and turns the reference's define blocks into the kernels the reference's callers then ask for by name."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import qwental_amd as q
+from qwental_amd.gpu import SYMBOLS, compile_check
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    names = set()
+    for h in ("gpu.h", "qw_hip_ext.h", "qw_path.h"):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(qw_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    L = q.load_lib()
+    decl = declared_functions()
+    assert len(decl) >= 55
+    for n in decl:
+        assert hasattr(L, n), "libqwgpu_hip.so lacks %s" % n
+    assert decl == {n for n, _, _ in SYMBOLS}  # the ctypes table covers exactly what the headers declare
+
+
+def test_reference_interface_symbols_present():
+    """The 33 functions of the reference's src/gpu.h, by name."""
+    ref = """qw_gpu_open qw_gpu_close qw_gpu_name qw_gpu_max_working_set qw_gpu_compile qw_kernel_get qw_kernel_max_threads
+    qw_kernel_simd_width qw_buf_new qw_buf_free qw_pool_push qw_pool_pop qw_buf_wrap qw_batch_begin qw_batch_kernel qw_batch_buf
+    qw_batch_bytes qw_batch_threadgroup_mem qw_batch_dispatch qw_batch_barrier qw_batch_flush qw_batch_end qw_batch_submit
+    qw_batch_wait qw_batch_poll qw_gpu_set_stream qw_profile_enable qw_profile_count qw_profile_get qw_gpu_empty_commit_latency
+    qw_power_desc qw_on_battery qw_now""".split()
+    L = q.load_lib()
+    for n in ref:
+        assert hasattr(L, n)
+    L.qw_now.restype = ctypes.c_double
+    t0 = L.qw_now()
+    assert L.qw_now() >= t0 > 0
+    buf = ctypes.create_string_buffer(128)
+    L.qw_power_desc(buf, 128)
+    assert buf.value and not L.qw_on_battery()
+    assert L.qw_pool_push() is None and q.load_lib().qw_hip_arch() == b"gfx950"
+
+
+def test_no_device_is_reported_not_emulated():
+    """Without a gfx950 device qw_gpu_open returns NULL and the Python wrapper raises: there is no CPU path."""
+    L = q.load_lib()
+    if L.qw_gpu_open():
+        pytest.skip("a device is present")
+    with pytest.raises(RuntimeError):
+        q.Gpu()
+
+
+ENGINE_MOE = "#define IQ_DQ_ONLY\n#define E 512\n#define TOPK 10\n#define D 2048\n#define I 512\n#define NB %d\n"  # src/engine.c:478
+
+
+def test_define_blocks_of_the_reference_register_its_kernel_names():
+    ok, err, names = compile_check("#define IQ_DQ_ONLY 1\n#define DQ_TEST 21\n// kernel text follows\n")  # tools/dqtest.c:27
+    assert ok and names == ["dq_test"]
+    blk = "#define IQ_DQ_ONLY 1\n#define qmv_gg qmv_gg_f21_k2048_n8_f\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 8\n#define YT float\n"
+    ok, err, names = compile_check(blk + "#include <metal_stdlib>\nkernel void qmv_gg(...)")  # src/engine.c:709-710
+    assert ok and names == ["qmv_gg_f21_k2048_n8_f"]
+    ok, err, names = compile_check(ENGINE_MOE % 8 + "#define GG_PART 0\n#define moe_sel_gg moe_sel_gg_n8\n#define gg_tab_init gg_tab_init_n8\n")
+    assert ok and names == ["gg_tab_init_n8", "moe_sel_gg_n8"]
+    ok, err, names = compile_check(ENGINE_MOE % 8 + "#define GG_PART 1\n#define FSG 21\n#define FSU 21\n#define RBF 1\n#define moe_pre_gg moe_pre_gg_21_21_r1_n8\n")
+    assert ok and names == ["moe_pre_gg_21_21_r1_n8"]
+    ok, err, names = compile_check(ENGINE_MOE % 4 + "#define GG_PART 2\n#define GSG 8\n#define RG 1\n#define FGU 21\n#define FSD 8\n#define moe_gu_gg moe_gu_gg_21_8_g1_n4\n")
+    assert ok and names == ["moe_gu_gg_21_8_g1_n4"]
+    ok, err, names = compile_check(ENGINE_MOE % 1 + "#define GG_PART 3\n#define FD 21\n#define DSGN 4\n#define moe_dn_gg moe_dn_gg_21_s4_n1\n#define moe_cmb_gg moe_cmb_gg_21_s4_n1\n")
+    assert ok and names == ["moe_dn_gg_21_s4_n1", "moe_cmb_gg_21_s4_n1"]
+    ok, err, names = compile_check(ENGINE_MOE % 3 + "#define GG_ROUTER\n#define moe_router_bf moe_router_bf_n3\n#define p_router_bf p_router_bf_n3\n")
+    assert ok and names == ["moe_router_bf_n3"]  # the prefill routers have no gfx950 build: not registered, lookup gives NULL
+    ok, err, names = compile_check(ENGINE_MOE % 16 + "#define GG_PART 0\n#define moe_sel_gg s16\n#define gg_tab_init t16\n")  # beyond the reference: 16 tokens
+    assert ok and names == ["t16", "s16"]
+    ok, err, names = compile_check("#include <metal_stdlib>\nkernel void something_else() {}\n")
+    assert ok and names == []  # a source with no known block compiles to nothing; qw_kernel_get then returns NULL
+
+
+@pytest.mark.parametrize("block,needle", [
+    ("#define IQ_DQ_ONLY 1\n#define DQ_TEST 14\n", "14"),                                                    # Q6_K: no gfx950 build
+    ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 881\n#define NB 8\n", "row bytes"),
+    ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 17\n", "NB"),
+    ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 8\n#define YT bfloat\n", "YT"),
+    (ENGINE_MOE % 32 + "#define GG_PART 0\n", "NB"),
+    (ENGINE_MOE % 8 + "#define GG_PART 2\n#define FGU 23\n#define FSD 21\n", "23"),                           # IQ4_XS
+    (ENGINE_MOE % 8 + "#define GG_PART 1\n#define FSG 21\n#define FSU 8\n#define RBF 1\n", "equal"),
+    (ENGINE_MOE % 8 + "#define GG_PART 6\n", "GG_PART"),
+    ("#define E 512\n#define TOPK 10\n#define D 2000\n#define I 512\n#define NB 8\n#define GG_PART 3\n#define FD 21\n", "D 2000"),
+    ("#define E 2048\n#define TOPK 10\n#define D 2048\n#define I 512\n#define NB 8\n#define GG_PART 0\n", "E 2048"),
+])
+def test_unsupported_blocks_fail_with_a_message(block, needle):
+    ok, err, names = compile_check(block)
+    assert not ok and needle in err and names == []
+
+
+def test_later_definitions_win_and_whitespace_is_tolerated():
+    ok, err, names = compile_check("  #define   DQ_TEST   14  \n\n#define DQ_TEST\t8\r\n#define dq_test  my_dq\n")
+    assert ok and names == ["my_dq"]
