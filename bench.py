@@ -39,6 +39,35 @@ def timed_steps(stack, x, nb, steps, warmup):
     return time.perf_counter() - t0, gpu_s
 
 
+def committed_traffic():
+    """HBM bytes per launch of the dominant kernel as the committed counter summary states them (two rocprofv3
+    --pmc runs of this file with --copy-calib, FETCH_SIZE and WRITE_SIZE, scaled by the copy kernel); None without it."""
+    try:
+        for ln in open(os.path.join(ROOT, "profiles", "moe_stack_b16_hbm_traffic.txt")):
+            if ln.startswith(DOMINANT + " traffic bytes per launch ="):
+                return float(ln.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
+def copy_calibration(gpu, nbytes=1 << 30):
+    """qwk_copy over nbytes: reads nbytes and writes nbytes, a dispatch of known traffic for the counter runs."""
+    ok, err = gpu.compile("#define QW_HIP_MEM 1\n")
+    assert ok, err
+    src, dst = gpu.buf(nbytes, device_only=True), gpu.buf(nbytes, device_only=True)
+    for _ in range(3):
+        b = gpu.batch()
+        b.kernel(gpu.kernel("qw_copy"))
+        b.buf(0, src)
+        b.buf(1, dst)
+        b.bytes(2, np.array([nbytes // 16, 0], np.uint64))
+        b.dispatch(256 * 16)
+        b.end()
+    src.free()
+    dst.free()
+
+
 def cpu_baseline(stack, x, nb, lg_dev, budget_s=20.0):
     """The CPU oracle (float dot products over dequantized rows, OpenMP over all cores) on the first layers of the
     same stack with the same logits; stops after about budget_s seconds. Also the full-size parity check."""
@@ -67,6 +96,8 @@ def main():
     ap.add_argument("--nb", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--quick", action="store_true", help="B = 16 only (profiling runs)")
+    ap.add_argument("--copy-calib", action="store_true", help="also run the copy kernel over 1 GiB three times (scale for the memory counters)")
+    ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives, no sharding)" % a.gpus, file=sys.stderr)
@@ -83,6 +114,8 @@ def main():
     x = gpu.buf_from(xh, device_only=True)
     setup_s = time.perf_counter() - t0
 
+    if a.copy_calib:
+        copy_calibration(gpu)
     res = {}
     for nb in ([a.nb] if a.quick else sorted({1, 8, a.nb})):
         wall, gpu_s = timed_steps(stack, x, nb, a.steps, a.warmup)
@@ -98,13 +131,15 @@ def main():
     ent = gpu.profile_entries()
     mean_s, n_l = gpu.profile_mean(DOMINANT)
     U = stack.unique_experts(nb)
-    # gate/up of layer l reads U_l experts' gate and up rows (901,120 bytes each) and the 16 x 4 KB activations
-    gu_bytes = float(np.mean([u * stack.gu_bytes + nb * stack.D * 2 for u in U]))
+    # the gate/up launch of layer l reads U_l routed experts' gate and up rows (901,120 bytes each), the shared
+    # expert's gate and up rows (same shape, IQ3_S or Q8_0) and the nb x 4 KB activations
+    sh_gu = [2 * stack.I * synth.row_bytes(f, stack.D) for f in stack.shared_fmt]
+    gu_bytes = float(np.mean([u * stack.gu_bytes + s + nb * stack.D * 2 for u, s in zip(U, sh_gu)]))
     per_kernel = {}
     for name, us in ent:
         per_kernel.setdefault(name, []).append(us)
     roof = {"bound": "hbm", "kernel": DOMINANT, "achieved": gu_bytes / mean_s / 1e9 if mean_s > 0 else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": gu_bytes / mean_s / 1e9 / HBM_PEAK_GBS if mean_s > 0 else None, "traffic": None,
+            "frac": gu_bytes / mean_s / 1e9 / HBM_PEAK_GBS if mean_s > 0 else None, "traffic": a.traffic if a.traffic is not None else committed_traffic(),
             "launches": n_l, "mean_launch_us": mean_s * 1e6, "algorithmic_bytes_per_launch": gu_bytes}
     line = {"metric": "batched IQ3_S MoE decode tokens/s at B=16 (48-layer FFN stack); achieved HBM GB/s", "value": res[nb]["tokens_per_s"], "unit": "tokens/s",
             "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": res[nb]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
