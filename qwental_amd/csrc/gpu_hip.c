@@ -536,7 +536,12 @@ static unsigned cdiv(unsigned a, unsigned b) { return (a + b - 1) / b; }
 // Persistent grids: one 512-thread workgroup per compute unit (the LDS tables leave room for one), fewer if the
 // work is smaller. tasks are per-wave units; 8 waves per workgroup.
 static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks, unsigned waves) { return umin((unsigned)g->ncu, cdiv(wave_tasks, waves)); }
-enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 }; // waves per workgroup of the gate/up + matvec kernels and of the down kernels
+#ifdef QW_EXP_W16
+enum { QW_WAVES_GU = 16, QW_WAVES_DN = 8 };
+#else
+enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 };
+#endif
+// // waves per workgroup of the gate/up + matvec kernels and of the down kernels
 
 static const char *fname_fmt(char *buf, size_t n, const char *fmt, ...) {
     va_list ap;
@@ -570,7 +575,11 @@ static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W,
 static const void *glut(const qw_gpu *g) { return (const char *)g->tabs + QW_TAB_IQ3SS; }
 
 // Blocks per prefetch chunk for a row of K values (the kernels are instantiated for these; 1 = any K).
+#ifdef QW_EXP_W16
+static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 1 : 16) : 1; }
+#else
 static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1; }
+#endif
 
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
     const qw_kparams *p = &b->k->p;

@@ -8,7 +8,11 @@
 #include "qw_common.hip.h"
 
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
+#ifdef QW_EXP_W16
+#define QW_WG_GU 1024
+#else
 #define QW_WG_GU 768       // gate/up and dense matvec: 12 waves, three per SIMD (a wave issues at most one instruction in ~6 cycles)
+#endif
 #define QW_XF_MAXK 2560    // largest K whose activations are staged in LDS in fragment order (K * 32 bytes)
 
 __device__ __forceinline__ uint32_t qw_wave() { return threadIdx.x >> 6; }

@@ -45,6 +45,7 @@ def test_gpu_select_fixture(gpu):
     b.kernel(gpu.kernel("sel_fix"))
     b.buf(0, lb)
     b.buf(1, sb)
+    b.bytes(2, np.array([nb], np.uint32))
     b.dispatch(1, 1, 1, 1024, 1, 1)
     assert b.end() >= 0, gpu.last_error()
     rec, ref = sb.view(np.uint8).copy(), g["record"]
