@@ -162,7 +162,7 @@ qw_gpu *qw_gpu_open(void) {
         void *params[] = {&ta};
         if (hipMalloc(&g->tabs, QW_TAB_BYTES) != hipSuccess || hipMemset(g->tabs, 0, QW_TAB_BYTES) != hipSuccess ||
             hipModuleGetFunction(&f, g->mod, "qwk_tab_init") != hipSuccess) { free(g->kernels); free(g); return NULL; }
-        ta.tab = g->tabs;
+        ta = (qwk_tab_args){.tab = g->tabs, .slot_order = 1};
         if (hipDeviceSynchronize() != hipSuccess || hipModuleLaunchKernel(f, 32, 1, 1, 256, 1, 1, 0, g->stream[0], params, NULL) != hipSuccess ||
             hipStreamSynchronize(g->stream[0]) != hipSuccess) {
             fprintf(stderr, "qw_gpu_open: the table kernel does not run\n");
@@ -638,7 +638,7 @@ static bool tr_router(qw_batch *b) { // src/engine.c:546-551; NB = token count
 }
 
 static bool tr_tab_init(qw_batch *b) { // src/engine.c:572-574
-    qwk_tab_args a;
+    qwk_tab_args a = {0}; // the caller's buffer gets the reference's entry order
     if (!bind_ptr(b, 0, QW_TAB_BYTES, true, "lookup tables", (void **)&a.tab)) return false;
     return add_launch(b, "qwk_tab_init", 32, 256, &a, sizeof a);
 }

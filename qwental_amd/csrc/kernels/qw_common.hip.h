@@ -53,9 +53,15 @@ __device__ __forceinline__ u2 qw_lut_entry(uint32_t i) {
     return r;
 }
 
+// Where entry i of the reference's index order (codebook entry | sign nibble << 9) lives in this library's copy of
+// the table: slot = qs byte << 5 | ninth index bit << 4 | sign nibble. A slot's byte address is then made of two
+// whole bytes (high byte = the qs byte as loaded, low byte = (nibble | bit << 4) << 3), which one byte-permute
+// instruction assembles.
+__device__ __forceinline__ uint32_t qw_lut_slot(uint32_t i) { return ((i & 255) << 5) | (((i >> 8) & 1) << 4) | (i >> 9); }
+
 // Fill the 64 KB table in LDS; every thread of the workgroup takes part. Caller synchronises afterwards.
 __device__ __forceinline__ void qw_lut_build(u2 *lut) {
-    for (uint32_t i = threadIdx.x; i < QW_LUT_ENTRIES; i += blockDim.x) lut[i] = qw_lut_entry(i);
+    for (uint32_t i = threadIdx.x; i < QW_LUT_ENTRIES; i += blockDim.x) lut[qw_lut_slot(i)] = qw_lut_entry(i);
 }
 
 #ifdef QW_EXP_NOMFMA
@@ -108,16 +114,44 @@ __device__ __forceinline__ void qw_iq3_transpose(qw_iq3_slice &s, uint32_t src4)
     s.d = __builtin_bit_cast(float, qw_pull(__builtin_bit_cast(uint32_t, s.d), src4));
 }
 
+// Low address bytes of the sixteen table reads of a slice: p[2 t] holds, byte j, (nibble | ninth bit << 4) << 3 of
+// read 2 j of sub-block t, p[2 t + 1] the same for read 2 j + 1. The eight qh bits of a sub-block are spread to bit 4
+// of eight bytes by two 24-bit multiplications (no two partial products that can both be set meet at a kept bit).
+struct qw_iq3_keys {
+    uint32_t p[4];
+};
+__device__ __forceinline__ qw_iq3_keys qw_iq3_prep(const qw_iq3_slice &s) {
+    qw_iq3_keys k;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint32_t S = s.sg[t], H = s.qh >> (8 * t);
+        const uint32_t he = __umul24(H & 0x55u, 0x410410u); // bit 8 j + 4 = qh bit 2 j
+        const uint32_t ho = __umul24(H & 0xaau, 0x208208u); // bit 8 j + 4 = qh bit 2 j + 1
+        k.p[2 * t] = ((he & 0x10101010u) | (S & 0x0f0f0f0fu)) << 3;
+        k.p[2 * t + 1] = ((ho & 0x10101010u) | ((S >> 4) & 0x0f0f0f0fu)) << 3;
+    }
+    return k;
+}
+// Byte addresses (relative to the table) of the two reads of step J: high byte = qs byte, low byte from the keys.
+template <int J> __device__ __forceinline__ void qw_iq3_addr(const qw_iq3_slice &s, const qw_iq3_keys &k, uint32_t &a0, uint32_t &a1) {
+    constexpr uint32_t t = J / 4, j = J % 4, qb = 2 * (J % 2);
+    a0 = __builtin_amdgcn_perm(s.qs[J / 2], k.p[2 * t], 0x0c0c0000u | ((4 + qb) << 8) | j);
+    a1 = __builtin_amdgcn_perm(s.qs[J / 2], k.p[2 * t + 1], 0x0c0c0000u | ((5 + qb) << 8) | j);
+}
+__device__ __forceinline__ u2 qw_lut_at(const u2 *lut, uint32_t byteaddr) { return *(const u2 *)((const uint8_t *)lut + byteaddr); }
+// The binary16 sub-block factor 1 + 2 s of sub-block t of a slice, in both halves.
+__device__ __forceinline__ h2 qw_iq3_factor(const qw_iq3_slice &s, int t) {
+    const _Float16 f = (_Float16)(uint16_t)(1 + 2 * ((s.sc >> (4 * t)) & 15));
+    return h2{f, f};
+}
+
 // The eight binary16 values of step J, already multiplied by the sub-block factor.
 template <int J> __device__ __forceinline__ h8 qw_iq3_step(const qw_iq3_slice &s, const u2 *lut) {
-    const uint32_t q = s.qs[J / 2] >> (16 * (J % 2));  // bytes 2J, 2J + 1 of the slice's qs
-    const uint32_t sg = s.sg[J / 4] >> (8 * (J % 4));  // byte J of the slice's signs
-    const uint32_t hb = s.qh >> (8 * (J / 4) + 2 * (J % 4));
-    const uint32_t i0 = (q & 255) | ((hb & 1) << 8) | ((sg & 15) << 9);
-    const uint32_t i1 = ((q >> 8) & 255) | ((hb & 2) << 7) | ((sg & 0xf0) << 5);
-    const u2 w0 = lut[i0], w1 = lut[i1];
-    const _Float16 f = (_Float16)(int)(1 + 2 * ((s.sc >> (4 * (J / 4))) & 15));
-    const h2 ff = {f, f};
+    const qw_iq3_keys k = qw_iq3_prep(s);
+    uint32_t a0, a1;
+    qw_iq3_addr<J>(s, k, a0, a1);
+    const u2 w0 = qw_lut_at(lut, a0), w1 = qw_lut_at(lut, a1);
+    const h2 ff = qw_iq3_factor(s, J / 4);
     u4 raw = {w0.x, w0.y, w1.x, w1.y};
 #pragma unroll
     for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
@@ -183,15 +217,6 @@ template <bool LO> struct qw_afrag_glb {
 // compute unit and 14 KB per wave in flight (IQ3_S, 16 rows of K = 2048) this covers the HBM latency.
 template <int F, int NB> struct qw_chunk;
 
-// The two table indices of step J of a slice (see qw_iq3_step).
-template <int J> __device__ __forceinline__ void qw_iq3_idx(const qw_iq3_slice &s, uint32_t &i0, uint32_t &i1) {
-    const uint32_t q = s.qs[J / 2] >> (16 * (J % 2));
-    const uint32_t sg = s.sg[J / 4] >> (8 * (J % 4));
-    const uint32_t hb = s.qh >> (8 * (J / 4) + 2 * (J % 4));
-    i0 = (q & 255) | ((hb & 1) << 8) | ((sg & 15) << 9);
-    i1 = ((q >> 8) & 255) | ((hb & 2) << 7) | ((sg & 0xf0) << 5);
-}
-
 template <int NB> struct qw_chunk<21, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = 110;
     qw_iq3_slice s[NB];
@@ -201,25 +226,22 @@ template <int NB> struct qw_chunk<21, NB> {
     }
     // All sixteen table reads of one block, issued together.
     __device__ __forceinline__ void lookups(int b, const u2 *lut, u2 (&w)[16]) const {
+        const qw_iq3_keys k = qw_iq3_prep(s[b]);
         uint32_t i[16];
-        qw_iq3_idx<0>(s[b], i[0], i[1]);
-        qw_iq3_idx<1>(s[b], i[2], i[3]);
-        qw_iq3_idx<2>(s[b], i[4], i[5]);
-        qw_iq3_idx<3>(s[b], i[6], i[7]);
-        qw_iq3_idx<4>(s[b], i[8], i[9]);
-        qw_iq3_idx<5>(s[b], i[10], i[11]);
-        qw_iq3_idx<6>(s[b], i[12], i[13]);
-        qw_iq3_idx<7>(s[b], i[14], i[15]);
+        qw_iq3_addr<0>(s[b], k, i[0], i[1]);
+        qw_iq3_addr<1>(s[b], k, i[2], i[3]);
+        qw_iq3_addr<2>(s[b], k, i[4], i[5]);
+        qw_iq3_addr<3>(s[b], k, i[6], i[7]);
+        qw_iq3_addr<4>(s[b], k, i[8], i[9]);
+        qw_iq3_addr<5>(s[b], k, i[10], i[11]);
+        qw_iq3_addr<6>(s[b], k, i[12], i[13]);
+        qw_iq3_addr<7>(s[b], k, i[14], i[15]);
 #pragma unroll
         for (int j = 0; j < 16; j++) {
 #ifdef QW_EXP_NOLUT
             w[j] = u2{i[j] * 0x00010001u | 0x3c003c00u, 0x3c003c00u};
-#elif defined(QW_EXP_NOCONFLICT)
-            w[j] = lut[(i[j] & ~15u) | (threadIdx.x & 15)]; // distinct bank pair per lane of a 16-lane group (wrong values, timing only)
-#elif defined(QW_EXP_NOCONFLICT32)
-            w[j] = lut[(i[j] & ~31u) | (threadIdx.x & 31)];
 #else
-            w[j] = lut[i[j]];
+            w[j] = qw_lut_at(lut, i[j]);
 #endif
         }
     }
@@ -251,11 +273,11 @@ template <int NB> struct qw_chunk<21, NB> {
 #endif
             }
             if (b + 1 < NB) lookups(b + 1, lut, w[(b + 1) & 1]);
-            const _Float16 f0 = (_Float16)(int)(1 + 2 * (s[b].sc & 15)), f1 = (_Float16)(int)(1 + 2 * ((s[b].sc >> 4) & 15));
+            const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
             f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const h2 ff = j < 4 ? h2{f0, f0} : h2{f1, f1};
+                const h2 ff = j < 4 ? ff0 : ff1;
                 const u2 w0 = w[b & 1][2 * j], w1 = w[b & 1][2 * j + 1];
                 u4 raw = {w0.x, w0.y, w1.x, w1.y};
 #pragma unroll
@@ -288,11 +310,11 @@ template <int NB> struct qw_chunk<21, NB> {
     }
     // One block's table values times two operand-A fragment sets (hi, lo), accumulated the way mac() does.
     __device__ __forceinline__ void block_mfma(int b, const u2 (&w)[16], const h8 (&xh)[8], const h8 (&xl)[8], bool lo, f4 &acc) const {
-        const _Float16 f0 = (_Float16)(int)(1 + 2 * (s[b].sc & 15)), f1 = (_Float16)(int)(1 + 2 * ((s[b].sc >> 4) & 15));
+        const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
         f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const h2 ff = j < 4 ? h2{f0, f0} : h2{f1, f1};
+            const h2 ff = j < 4 ? ff0 : ff1;
             u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
 #pragma unroll
             for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
@@ -381,6 +403,42 @@ template <class C, class L, class U> __device__ __forceinline__ void qw_pipeline
         b.transpose();
         use(i, b);
         ++i;
+    }
+}
+
+// The same pipeline over the tasks w0, w0 + nw, ... < ntasks of one wave, cpr chunks per task, without a division
+// per chunk: two cursors step through (task, chunk). rowp(task) is the lane's byte pointer to the task's first
+// chunk (chunk c follows at c * cstride bytes); use(task, c, chunk) consumes chunk c of a task. All of ntasks, w0,
+// nw and cpr must be wave-uniform.
+template <class C, class R, class U>
+__device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use) {
+    if (w0 >= ntasks) return;
+    C a, b;
+    uint32_t lt = w0, lc = 0, ut = w0, uc = 0;
+    const uint8_t *lrow = rowp(lt);
+    auto load = [&](C &c) {
+        c.load(lrow + (size_t)lc * cstride, kl);
+        if (++lc == cpr) {
+            lc = 0;
+            lt += nw;
+            if (lt < ntasks) lrow = rowp(lt);
+        }
+    };
+    auto consume = [&](C &c) {
+        c.transpose();
+        use(ut, uc, c);
+        if (++uc == cpr) uc = 0, ut += nw;
+    };
+    load(a);
+    for (;;) {
+        const bool m1 = lt < ntasks;
+        if (m1) load(b);
+        consume(a);
+        if (!m1) break;
+        const bool m2 = lt < ntasks;
+        if (m2) load(a);
+        consume(b);
+        if (!m2) break;
     }
 }
 

@@ -48,6 +48,8 @@ typedef struct { /* selection + dedupe */
 
 typedef struct { /* build the lookup-table buffer */
     uint8_t *tab;
+    uint32_t slot_order; /* 0: the reference's entry order; 1: the order this library's kernels read from LDS */
+    uint32_t pad;
 } qwk_tab_args;
 
 /* gate/up + SwiGLU for a list of experts. routed: experts come from sel (U, ue, mask, slot). shared != 0: one

@@ -15,7 +15,8 @@
 #endif
 #define QW_XF_MAXK 2560    // largest K whose activations are staged in LDS in fragment order (K * 32 bytes)
 
-__device__ __forceinline__ uint32_t qw_wave() { return threadIdx.x >> 6; }
+// wave index in the workgroup, as a scalar (so that task indices and row bases stay in scalar registers)
+__device__ __forceinline__ uint32_t qw_wave() { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
 __device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
@@ -56,7 +57,7 @@ extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f8(qwk_dq_args a) {
 // Only the IQ3_S section is produced; the sections of formats without a gfx950 build stay zero. Grid: 32 x 256.
 extern "C" __global__ void qwk_tab_init(qwk_tab_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < QW_LUT_ENTRIES) ((u2 *)(a.tab + QW_TAB_IQ3SS))[i] = qw_lut_entry(i);
+    if (i < QW_LUT_ENTRIES) ((u2 *)(a.tab + QW_TAB_IQ3SS))[a.slot_order ? qw_lut_slot(i) : i] = qw_lut_entry(i);
 }
 
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
@@ -66,7 +67,7 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
-    const uint32_t cpr = a.K / (C::BLK_K * CH), mytiles = w0 < a.ntiles ? (a.ntiles - w0 + nw - 1) / nw : 0;
+    const uint32_t cpr = a.K / (C::BLK_K * CH);
     const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t t) {
         const uint32_t r = 16 * t + nl;
@@ -78,32 +79,27 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     const qw_afrag_lds afl = {xf, n};
     const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
     f4 acc = {0, 0, 0, 0};
-    qw_pipeline<C>(mytiles * cpr,
-        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kl); },
-        [&](uint32_t i, const C &c) {
-            const uint32_t ci = i % cpr;
-            if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
-            else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
-            if (ci + 1 == cpr) {
-                const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
-                if (r < a.N)
+    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, CH * C::BLK_B, kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
+        if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
+        else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
+        if (ci + 1 != cpr) return;
+        const uint32_t r = 16 * t + n;
+        if (r < a.N)
 #pragma unroll
-                    for (uint32_t j = 0; j < 4; j++) {
-                        const uint32_t tok = 4 * kg + j;
-                        if (tok < a.nb) {
-                            if (a.yfloat) ((float *)a.y)[(size_t)tok * a.ystride + r] = acc[j];
-                            else ((uint16_t *)a.y)[(size_t)tok * a.ystride + r] = qw_f2h(acc[j]);
-                        }
-                    }
-                acc = f4{0, 0, 0, 0};
+            for (uint32_t j = 0; j < 4; j++) {
+                const uint32_t tok = 4 * kg + j;
+                if (tok < a.nb) {
+                    if (a.yfloat) ((float *)a.y)[(size_t)tok * a.ystride + r] = acc[j];
+                    else ((uint16_t *)a.y)[(size_t)tok * a.ystride + r] = qw_f2h(acc[j]);
+                }
             }
-        });
+        acc = f4{0, 0, 0, 0};
+    });
 }
 #define QW_QMV(F, CH, XLDS, SFX)                                                                        \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
-        __shared__ u2 lut[F == 21 ? QW_LUT_ENTRIES : 1];                                                \
-        __shared__ u4 xf[XLDS ? QW_XF_MAXK * 2 : 1];                                                    \
-        qmv_body<F, CH, XLDS>(a, lut, xf);                                                              \
+        __shared__ struct { u2 lut[F == 21 ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; } L; /* table first: LDS address 0 */ \
+        qmv_body<F, CH, XLDS>(a, L.lut, L.xf);                                                          \
     }
 QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
 QW_QMV(8, 16, true, _c16) QW_QMV(8, 1, true, _c1) QW_QMV(8, 1, false, _c1g)
@@ -356,7 +352,7 @@ template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_a
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
     const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
-    const uint32_t cpr = a.D / (C::BLK_K * CH), mine = w0 < ntasks ? (ntasks - w0 + nw - 1) / nw : 0;
+    const uint32_t cpr = a.D / (C::BLK_K * CH);
     const qw_afrag_lds af = {xf, n};
     const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t task) {
@@ -364,29 +360,26 @@ template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_a
         return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
-    qw_pipeline<C>(mine * cpr,
-        [&](uint32_t i, C &c) { c.load(rowp(w0 + (i / cpr) * nw) + (size_t)(i % cpr) * CH * C::BLK_B, kl); },
-        [&](uint32_t i, const C &c) {
-            const uint32_t ci = i % cpr;
-            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
-            if (ci + 1 != cpr) return;
-            const uint32_t task = w0 + (i / cpr) * nw, u = task / tpe, j0 = 8 * (task % tpe);
-            const uint32_t m = a.shared ? qw_all_tokens(a.nbr) : sc->mask[u];
+    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, kl, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
+        c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+        if (ci + 1 != cpr) return;
+        const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
+        const uint32_t m = a.shared ? qw_all_tokens(a.nbr) : sc->mask[u];
 #pragma unroll
-            for (uint32_t j = 0; j < 4; j++) {
-                const float up = __shfl_xor(acc[j], 8), g = acc[j];
-                const uint32_t tok = 4 * kg + j;
-                if (n < 8 && tok < a.nbr && ((m >> tok) & 1)) {
-                    const uint32_t s = a.shared ? K : sc->slot[u * gnb + tok];
-                    const float h = g / (1.0f + __expf(-g)) * up;
-                    const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
-                    const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
-                    a.H[o] = __builtin_bit_cast(uint16_t, hi);
-                    a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
-                }
+        for (uint32_t j = 0; j < 4; j++) {
+            const float up = __shfl_xor(acc[j], 8), g = acc[j];
+            const uint32_t tok = 4 * kg + j;
+            if (n < 8 && tok < a.nbr && ((m >> tok) & 1)) {
+                const uint32_t s = a.shared ? K : sc->slot[u * gnb + tok];
+                const float h = g / (1.0f + __expf(-g)) * up;
+                const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
+                const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
+                a.H[o] = __builtin_bit_cast(uint16_t, hi);
+                a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
             }
-            acc = f4{0, 0, 0, 0};
-        });
+        }
+        acc = f4{0, 0, 0, 0};
+    });
 }
 
 // FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
@@ -411,10 +404,8 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
-        __shared__ u2 lut[(FGU == 21 || FSG == 21) ? QW_LUT_ENTRIES : 1];                                 \
-        __shared__ u4 xf[QW_XF_MAXK * 2];                                                                 \
-        __shared__ qw_sel_cache sc;                                                                       \
-        gu_body<FGU, CHGU, FSG, CHSG>(a, lut, xf, &sc);                                                   \
+        __shared__ struct { u2 lut[(FGU == 21 || FSG == 21) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; } L; \
+        gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc);                                             \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
 QW_GU(21, 2, 0, 1, qwk_gu_f21_c2) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
@@ -449,20 +440,19 @@ extern "C" __global__ __launch_bounds__(QW_WG) void qwk_pre_w30(qwk_pre_args a) 
 template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const qwk_dn_args &a, const u2 *lut, uint32_t w0, uint32_t nw) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk;
-    const uint32_t ntiles = a.D / 16, cpr = a.I / (C::BLK_K * CH), mine = w0 < ntiles ? (ntiles - w0 + nw - 1) / nw : 0;
+    const uint32_t ntiles = a.D / 16, cpr = a.I / (C::BLK_K * CH);
     qw_afrag_glb<true> af = {nullptr, nullptr};
     if (n < a.snbr) {
         af.rowhi = a.H + ((size_t)n * (K + 1) + K) * a.I;
         af.rowlo = af.rowhi + a.hplane;
     }
     f4 acc = {0, 0, 0, 0};
-    qw_pipeline<C>(mine * cpr,
-        [&](uint32_t i, C &c) { c.load(a.Wsd + (size_t)(16 * (w0 + (i / cpr) * nw) + (lane >> 2)) * a.sd_rowbytes + (size_t)(i % cpr) * CH * C::BLK_B, lane & 3); },
-        [&](uint32_t i, const C &c) {
-            const uint32_t ci = i % cpr;
+    qw_task_pipeline<C>(ntiles, w0, nw, cpr, CH * C::BLK_B, lane & 3,
+        [&](uint32_t t) { return a.Wsd + (size_t)(16 * t + (lane >> 2)) * a.sd_rowbytes; },
+        [&](uint32_t t, uint32_t ci, const C &c) {
             c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 != cpr) return;
-            const uint32_t r = 16 * (w0 + (i / cpr) * nw) + n;
+            const uint32_t r = 16 * t + n;
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++)
                 if (4 * kg + j < a.snbr) a.Psh[(size_t)(4 * kg + j) * a.D + r] = acc[j];
@@ -536,10 +526,8 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_b
 }
 #define QW_DN(F, CH, FSD, CHSD, IMAX, NAME)                                           \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
-        __shared__ u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];               \
-        __shared__ u4 abuf[2 * 2 * (IMAX / 8) * 16];                                  \
-        __shared__ qw_sel_cache sc;                                                   \
-        dn_body<F, CH, FSD, CHSD>(a, lut, abuf, &sc);                                 \
+        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; u4 abuf[2 * 2 * (IMAX / 8) * 16]; qw_sel_cache sc; } L; \
+        dn_body<F, CH, FSD, CHSD>(a, L.lut, L.abuf, &L.sc);                           \
     }
 // I = 512 is the synthetic shape (whole row = one chunk of 2 IQ3_S blocks); Q8_0 down weights take the any-shape kernel
 QW_DN(21, 2, 0, 1, 512, qwk_dn_f21_i512) QW_DN(21, 2, 21, 2, 512, qwk_dn_f21_i512_s21) QW_DN(21, 2, 8, 16, 512, qwk_dn_f21_i512_s8)
@@ -576,9 +564,8 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
 }
 #define QW_DN_ANY(F, FSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
-        __shared__ u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1];               \
-        __shared__ qw_sel_cache sc;                                                   \
-        dn_any_body<F, FSD>(a, lut, &sc);                                             \
+        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; qw_sel_cache sc; } L; \
+        dn_any_body<F, FSD>(a, L.lut, &L.sc);                                         \
     }
 QW_DN_ANY(21, 0, qwk_dn_f21_any) QW_DN_ANY(21, 21, qwk_dn_f21_any_s21) QW_DN_ANY(21, 8, qwk_dn_f21_any_s8)
 QW_DN_ANY(8, 0, qwk_dn_f8_any) QW_DN_ANY(8, 21, qwk_dn_f8_any_s21) QW_DN_ANY(8, 8, qwk_dn_f8_any_s8)

@@ -95,6 +95,8 @@ static qw_kernel *gg_kernel(qw_path *p, const char *base, const qw_moe_layer *M,
     case 3: snprintf(sfx, sizeof sfx, "_%d_s%d_n%d", M->down.type, 4, nbv); break;
     default: snprintf(sfx, sizeof sfx, "_w%d_n%d", rwf, nbv);
     }
+    // one model per process in the reference, so its names carry no shape; a qw_gpu here may serve several shapes
+    snprintf(sfx + strlen(sfx), sizeof sfx - strlen(sfx), "_e%dk%dd%di%d", p->E, p->topk, p->D, p->I);
     snprintf(name, sizeof name, "%s%s", base, sfx);
     qw_kernel *k = qw_kernel_get(p->g, name);
     if (k) return k;
