@@ -33,6 +33,14 @@ bool qw_hip_buf_read(const qw_buf *b, size_t offset, void *dst, size_t len);
 /* Device address of a buffer (for tools that pass it to their own code). */
 void *qw_hip_buf_devptr(const qw_buf *b);
 
+/* IQ3_S weight matrices of the MoE kernels are copied once, at their first use, into a tile-major layout that a wave
+ * reads with fully coalesced loads (the copy costs 1792 / 1760 of the matrix's bytes of HBM; the GGUF bytes stay where
+ * they are). The copy is dropped when the source buffer is freed, marked dirty, uploaded, written, or bound as a
+ * kernel's output. Buffers of at most QW_HIP_SMALL_BYTES with a host shadow are never copied. QW_HIP_REPACK=0 in the
+ * environment, or qw_hip_set_repack(g, false), turns the copies off (kernels then read the GGUF rows directly). */
+void qw_hip_set_repack(qw_gpu *g, bool on);
+size_t qw_hip_packed_bytes(const qw_gpu *g);
+
 /* The define-block front end of qw_gpu_compile() without a device: parses src as qw_gpu_compile would, and on
  * success writes the names of the kernels it would register to names (comma separated). For host-side tests. */
 bool qw_hip_compile_check(const char *src, size_t len, char *err, size_t errlen, char *names, size_t nameslen);

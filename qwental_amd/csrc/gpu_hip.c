@@ -53,7 +53,19 @@ typedef struct qw_hbuf {
     bool wrapped, device_only;
     bool dirty;      // host copy is newer than HBM (or HBM never received it)
     unsigned mark;   // scratch for de-duplication while a batch is submitted
+    struct qw_gpu *g;
+    int npack;       // packed copies made from this buffer (dropped when its contents change)
 } qw_hbuf;
+
+// A tile-major copy of IQ3_S weight rows (layout: qwk_pack_args), made at the first use of a weight matrix.
+typedef struct {
+    const void *A, *B;
+    qw_hbuf *ha, *hb;
+    uint64_t ntiles;
+    uint32_t nblk, split;
+    void *dst;
+    size_t bytes;
+} qw_pack;
 
 typedef struct {
     hipFunction_t f;
@@ -86,8 +98,8 @@ struct qw_batch {
     // Work deferred from one dispatch of a layer to the next (the reference's front part also computes the shared
     // expert's gate/up, and its gate/up dispatch the shared down; here they ride in the next launch, where they cost
     // almost nothing): set by moe_pre_gg / moe_gu_gg, consumed by moe_gu_gg / moe_dn_gg of the same batch.
-    struct { bool valid; int fmt; const uint8_t *Wsg, *Wsu; uint32_t rowbytes, nbr; } pend_sg;
-    struct { bool valid; int fmt; const uint8_t *Wsd; float *Psh; uint32_t rowbytes, nbr; } pend_sd;
+    struct { bool valid; int fmt; const uint8_t *Wsg, *Wsu; qw_hbuf *hg, *hu; uint32_t rowbytes, nbr; } pend_sg;
+    struct { bool valid; int fmt; const uint8_t *Wsd; qw_hbuf *hd; float *Psh; uint32_t rowbytes, nbr; } pend_sd;
 };
 
 struct qw_gpu {
@@ -110,6 +122,10 @@ struct qw_gpu {
     const char *prof_fname[QW_PROF_MAX];
     double prof_us[QW_PROF_MAX];
     unsigned mark;
+    qw_pack *packs;
+    int npacks, cappacks;
+    bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
+    size_t pack_bytes;
 };
 
 static void set_err(qw_gpu *g, const char *fmt, ...) {
@@ -156,6 +172,10 @@ qw_gpu *qw_gpu_open(void) {
     for (int i = 0; i < 2; i++)
         if (hipStreamCreateWithFlags(&g->stream[i], hipStreamNonBlocking) != hipSuccess) { free(g); return NULL; }
     g->kernels = calloc(QW_MAX_KERNELS, sizeof *g->kernels);
+    {
+        const char *e = getenv("QW_HIP_REPACK");
+        g->repack = !(e && e[0] == '0');
+    }
     { // build the pre-signed table once; every weight kernel copies it into LDS
         hipFunction_t f;
         qwk_tab_args ta;
@@ -178,6 +198,12 @@ void qw_gpu_close(qw_gpu *g) {
     if (!g) return;
     (void)hipDeviceSynchronize();
     for (int i = 0; i < 2; i++) (void)hipStreamDestroy(g->stream[i]);
+    for (int i = 0; i < g->npacks; i++) {
+        (void)hipFree(g->packs[i].dst);
+        if (g->packs[i].ha) g->packs[i].ha->npack = 0;
+        if (g->packs[i].hb) g->packs[i].hb->npack = 0;
+    }
+    free(g->packs);
     (void)hipFree(g->tabs);
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
@@ -330,6 +356,9 @@ out:
     return ok;
 }
 
+#ifdef QW_EXP_TRACE
+bool qw_hip_debug_tabs(qw_gpu *g, void *dst, size_t n) { return hipDeviceSynchronize() == hipSuccess && hipMemcpy(dst, g->tabs, n, hipMemcpyDeviceToHost) == hipSuccess; }
+#endif
 bool qw_hip_compile_check(const char *src, size_t len, char *err, size_t errlen, char *names, size_t nameslen) {
     qw_gpu *g = calloc(1, sizeof *g); // no device behind it: only the kernel registry is touched
     if (!g) return false;
@@ -360,6 +389,7 @@ static qw_hbuf *hbuf_new(qw_gpu *g, size_t size) {
     // the memset runs on the null stream; the batches run on non-blocking streams, so wait for it here
     if (!HIPOK(g, hipMalloc(&h->dptr, size ? size : 1)) || !HIPOK(g, hipMemset(h->dptr, 0, size)) || !HIPOK(g, hipDeviceSynchronize())) { free(h); return NULL; }
     h->size = size;
+    h->g = g;
     return h;
 }
 
@@ -405,9 +435,29 @@ bool qw_buf_wrap(qw_gpu *g, void *ptr, size_t len, qw_buf *out) {
     return true;
 }
 
+// The packed copies made from h are stale (its contents changed or it goes away): free them.
+static void packs_drop(qw_hbuf *h) {
+    if (!h || !h->npack) return;
+    qw_gpu *g = h->g;
+    (void)hipDeviceSynchronize(); // a batch in flight may still read them
+    int n = 0;
+    for (int i = 0; i < g->npacks; i++) {
+        qw_pack *p = &g->packs[i];
+        if (p->ha == h || p->hb == h) {
+            (void)hipFree(p->dst);
+            g->pack_bytes -= p->bytes;
+            if (p->ha && p->ha != h) p->ha->npack--;
+            if (p->hb && p->hb != h && p->hb != p->ha) p->hb->npack--;
+        } else g->packs[n++] = *p;
+    }
+    g->npacks = n;
+    h->npack = 0;
+}
+
 void qw_buf_free(qw_buf *b) {
     if (!b || !b->handle) return;
     qw_hbuf *h = b->handle;
+    packs_drop(h);
     (void)hipFree(h->dptr);
     if (h->own_host) {
         if (h->pinned) (void)hipHostFree(h->host);
@@ -422,11 +472,18 @@ void qw_buf_free(qw_buf *b) {
 void *qw_pool_push(void) { return NULL; }
 void qw_pool_pop(void *pool) { (void)pool; }
 
-void qw_hip_buf_mark_dirty(qw_buf *b) { if (b && b->handle) ((qw_hbuf *)b->handle)->dirty = true; }
+void qw_hip_buf_mark_dirty(qw_buf *b) {
+    if (!b || !b->handle) return;
+    ((qw_hbuf *)b->handle)->dirty = true;
+    packs_drop(b->handle);
+}
+void qw_hip_set_repack(qw_gpu *g, bool on) { g->repack = on; }
+size_t qw_hip_packed_bytes(const qw_gpu *g) { return g->pack_bytes; }
 void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle ? ((qw_hbuf *)b->handle)->dptr : NULL; }
 static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return off <= h->size && len <= h->size - off; }
 bool qw_hip_buf_upload(qw_buf *b, size_t off, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
+    packs_drop(h);
     return h && h->host && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, (char *)h->host + off, len, hipMemcpyHostToDevice) == hipSuccess;
 }
 bool qw_hip_buf_download(qw_buf *b, size_t off, size_t len) {
@@ -435,6 +492,7 @@ bool qw_hip_buf_download(qw_buf *b, size_t off, size_t len) {
 }
 bool qw_hip_buf_write(qw_buf *b, size_t off, const void *src, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
+    packs_drop(h);
     return h && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
 }
 bool qw_hip_buf_read(const qw_buf *b, size_t off, void *dst, size_t len) {
@@ -494,6 +552,7 @@ static bool bind_ptr(qw_batch *b, unsigned index, size_t need, bool out, const c
     const size_t off = b->buf[index].off;
     if (off > h->size || need > h->size - off) return fail(b, "%s: %s at index %u needs %zu bytes after offset %zu, buffer has %zu", b->k->name, what, index, need, off, h->size);
     if (out && h->wrapped) return fail(b, "%s: %s at index %u is a wrapped (read-only) buffer", b->k->name, what, index);
+    if (out) packs_drop(h); // a kernel is about to write it
     *p = (char *)h->dptr + off;
     if (b->nuse == b->capuse) {
         b->capuse = b->capuse ? 2 * b->capuse : 64;
@@ -620,6 +679,54 @@ static bool nbr_ok(qw_batch *b, uint32_t nbr) {
 }
 
 // gate/up arguments. shared: one expert at (iWg, iWu), all tokens, slot topk.
+// The packed copy of IQ3_S rows: tiles of `split` rows of A and 16 - split rows of B (B = NULL, split 16: one matrix).
+// Made at the first request, on the batch's stream, and complete when this returns; NULL when packing is off, the
+// source may change without notice (a small buffer with a host shadow is copied at every submit) or memory is short:
+// the caller then reads the GGUF rows directly.
+static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf *hb, const void *B, uint64_t ntiles, uint32_t nblk, uint32_t rowbytes, uint32_t split) {
+    qw_gpu *g = b->g;
+    if (!g->repack) return NULL;
+    for (int i = 0; i < g->npacks; i++) {
+        const qw_pack *p = &g->packs[i];
+        if (p->A == A && p->B == B && p->ntiles == ntiles && p->nblk == nblk && p->split == split) return p->dst;
+    }
+    qw_hbuf *hs[2] = {ha, hb};
+    for (int i = 0; i < 2; i++) {
+        qw_hbuf *h = hs[i];
+        if (!h) continue;
+        if (!h->device_only && !h->wrapped && h->size <= QW_HIP_SMALL_BYTES) return NULL;
+        if (h->dirty && h->host) { // what the next submit would do for this buffer
+            if (hipMemcpyAsync(h->dptr, h->host, h->size, hipMemcpyHostToDevice, g->stream[b->stream]) != hipSuccess) return NULL;
+            h->dirty = false;
+        }
+    }
+    hipFunction_t f = get_func(g, "qwk_pack_iq3");
+    if (!f) return NULL;
+    const size_t bytes = (size_t)ntiles * nblk * QW_SLAB_BYTES;
+    void *dst;
+    if (hipMalloc(&dst, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return NULL;
+    }
+    qwk_pack_args pa = {.A = A, .B = B, .dst = dst, .ntiles = ntiles, .nblk = nblk, .rowbytes = rowbytes, .split = split};
+    void *params[] = {&pa};
+    const uint64_t nslab = ntiles * nblk;
+    const unsigned gx = (unsigned)(nslab / 4 < 65536 ? (nslab + 3) / 4 : 65536);
+    if (hipModuleLaunchKernel(f, gx, 1, 1, 256, 1, 1, 0, g->stream[b->stream], params, NULL) != hipSuccess || hipStreamSynchronize(g->stream[b->stream]) != hipSuccess) {
+        (void)hipFree(dst);
+        return NULL;
+    }
+    if (g->npacks == g->cappacks) {
+        g->cappacks = g->cappacks ? 2 * g->cappacks : 64;
+        g->packs = realloc(g->packs, sizeof *g->packs * (size_t)g->cappacks);
+    }
+    g->packs[g->npacks++] = (qw_pack){.A = A, .B = B, .ha = ha, .hb = hb, .ntiles = ntiles, .nblk = nblk, .split = split, .dst = dst, .bytes = bytes};
+    g->pack_bytes += bytes;
+    if (ha) ha->npack++;
+    if (hb && hb != ha) hb->npack++;
+    return dst;
+}
+
 static bool fill_gu(qw_batch *b, qwk_gu_args *a, int F, unsigned iWg, unsigned iWu, unsigned ix, unsigned iH, uint32_t nbr, bool shared) {
     const qw_kparams *p = &b->k->p;
     const size_t rb = fmt_rb(F, p->D), ne = shared ? 1 : (size_t)p->E;
@@ -661,6 +768,8 @@ static bool tr_pre(qw_batch *b) {
     if (!bind_ptr(b, 6, (size_t)p->I * rb, false, "shared gate weights", (void **)&b->pend_sg.Wsg) || !bind_ptr(b, 7, (size_t)p->I * rb, false, "shared up weights", (void **)&b->pend_sg.Wsu) ||
         !bind_ptr(b, 8, (size_t)p->NB * (p->topk + 1) * p->I * 4, true, "H", &h)) return false;
     b->pend_sg.valid = true;
+    b->pend_sg.hg = b->buf[6].h;
+    b->pend_sg.hu = b->buf[7].h;
     b->pend_sg.fmt = p->fsg;
     b->pend_sg.rowbytes = (uint32_t)rb;
     b->pend_sg.nbr = nbr;
@@ -686,10 +795,13 @@ static bool tr_gu(qw_batch *b) {
     b->pend_sd.rowbytes = (uint32_t)fmt_rb(p->fsd, p->I);
     if (!bind_ptr(b, 2, (size_t)p->D * b->pend_sd.rowbytes, false, "shared down weights", (void **)&b->pend_sd.Wsd) || !bind_ptr(b, 3, (size_t)nbr * p->D * 4, true, "Psh", (void **)&b->pend_sd.Psh)) return false;
     b->pend_sd.valid = true;
+    b->pend_sd.hd = b->buf[2].h;
     b->pend_sd.fmt = p->fsd;
     b->pend_sd.nbr = nbr;
     int cg = chunk_of(p->fgu, p->D), fs = 0, cs = 1;
+    qw_hbuf *hsg = NULL, *hsu = NULL;
     if (b->pend_sg.valid) {
+        hsg = b->pend_sg.hg, hsu = b->pend_sg.hu;
         if (b->pend_sg.nbr != nbr) return fail(b, "moe_gu_gg: %u tokens after a front part of %u", nbr, b->pend_sg.nbr);
         fs = b->pend_sg.fmt;
         cs = chunk_of(fs, p->D);
@@ -699,9 +811,20 @@ static bool tr_gu(qw_batch *b) {
         b->pend_sg.valid = false;
         if (cg == 1 || cs == 1) cg = cs = 1; // any-shape builds come in pairs
     }
+    int fgu = p->fgu;
+    if (fgu == 21) { // tile-major copies of the IQ3_S rows, made at first use
+        const uint32_t nblk = (uint32_t)p->D / 256, tileb = nblk * QW_SLAB_BYTES;
+        const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wg, b->buf[1].h, a.Wu, (uint64_t)p->E * (uint64_t)(p->I / 8), nblk, a.rowbytes, 8);
+        const uint8_t *ps = pk && fs == 21 ? get_pack(b, hsg, a.Wsg, hsu, a.Wsu, (uint64_t)(p->I / 8), nblk, a.sg_rowbytes, 8) : NULL;
+        if (pk && (fs != 21 || ps)) {
+            fgu = QW_F_PACKED;
+            a.Wg = pk, a.Wu = NULL, a.rowbytes = tileb;
+            if (fs == 21) fs = QW_F_PACKED, a.Wsg = ps, a.Wsu = NULL, a.sg_rowbytes = tileb;
+        }
+    }
     char fn[64];
-    if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", p->fgu, cg, fs, cs);
-    else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", p->fgu, cg);
+    if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", fgu, cg, fs, cs);
+    else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", fgu, cg);
     const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (fs ? (unsigned)p->I / 8 : 0);
     return add_launch(b, intern(fn), persistent_grid(b->g, tasks, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
@@ -718,7 +841,9 @@ static bool tr_dn(qw_batch *b) {
         !bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, true, "Pg", (void **)&a.P) ||
         !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
     int fs = 0;
+    qw_hbuf *hsd = NULL;
     if (b->pend_sd.valid) {
+        hsd = b->pend_sd.hd;
         fs = b->pend_sd.fmt;
         a.Wsd = b->pend_sd.Wsd;
         a.Psh = b->pend_sd.Psh;
@@ -727,8 +852,35 @@ static bool tr_dn(qw_batch *b) {
         b->pend_sd.valid = false;
     }
     const unsigned umax = umin((unsigned)p->E, nbr * (unsigned)p->topk);
+    int fd = p->fd;
+    if (fd == 21 && p->I <= 512) {
+        const uint32_t nblk = (uint32_t)p->I / 256, tileb = nblk * QW_SLAB_BYTES;
+        const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wd, NULL, NULL, (uint64_t)p->E * (uint64_t)(p->D / 16), nblk, a.rowbytes, 16);
+        const uint8_t *ps = pk && fs == 21 ? get_pack(b, hsd, a.Wsd, NULL, NULL, (uint64_t)(p->D / 16), nblk, a.sd_rowbytes, 16) : NULL;
+        if (pk && (fs != 21 || ps)) {
+            fd = QW_F_PACKED;
+            a.Wd = pk, a.rowbytes = tileb;
+            if (fs == 21) fs = QW_F_PACKED, a.Wsd = ps, a.sd_rowbytes = tileb;
+        }
+    }
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
+#ifndef QW_EXP_DNSTREAM
+    if (p->I <= 512) { // contiguous task ranges per workgroup, operand A staged in LDS
+        const int ch = fd == 8 ? 4 : p->I / 256;
+        if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
+        else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
+        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
+    }
+#endif
+#ifndef QW_EXP_DNOLD
+    if (p->I % 512 == 0) { // independent waves, task = (expert, 16 rows)
+        const int ch = p->fd == 21 ? 2 : 4;
+        if (fs) fname_fmt(fn, sizeof fn, "qwk_dn_f%d_c%d_s%d_c%d", p->fd, ch, fs, fs == 21 ? 2 : 4);
+        else fname_fmt(fn, sizeof fn, "qwk_dn_f%d_c%d", p->fd, ch);
+        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
+    }
+#endif
     if (p->I == 512 && p->fd == 21) { // workgroup tasks of 256 rows
         fname_fmt(fn, sizeof fn, "qwk_dn_f21_i512%s", sfx);
         return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, umax * (unsigned)(p->D / 256)), 512, &a, sizeof a);

@@ -211,6 +211,35 @@ template <bool LO> struct qw_afrag_glb {
     __device__ __forceinline__ h8 lo(uint32_t koff) const { return rowlo ? *(const h8 *)(rowlo + koff) : h8{}; }
 };
 
+// One token's row of both planes staged in LDS as [hi I halves][lo I halves].
+struct qw_afrag_ldsrow {
+    const uint16_t *row;
+    uint32_t I;
+    static constexpr bool has_lo = true;
+    __device__ __forceinline__ h8 hi(uint32_t koff) const { return *(const h8 *)(row + koff); }
+    __device__ __forceinline__ h8 lo(uint32_t koff) const { return *(const h8 *)(row + I + koff); }
+};
+
+// Rows of the two H planes in global memory, read only by the lanes whose token column is in use ("on"): four
+// fragments per plane at a time inside one predicated region, into registers the caller keeps (and has zeroed once),
+// so that a lane that is off neither reads memory nor costs the address unit anything.
+struct qw_afrag_gather {
+    const uint16_t *rowhi, *rowlo;
+    bool on;
+    h8 (&hi)[4];
+    h8 (&lo)[4];
+    static constexpr bool has_lo = true;
+    __device__ __forceinline__ void fetch4(uint32_t koff, uint32_t kstep) const {
+        if (on) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                hi[i] = *(const h8 *)(rowhi + koff + i * kstep);
+                lo[i] = *(const h8 *)(rowlo + koff + i * kstep);
+            }
+        }
+    }
+};
+
 // ---------------------------------------------------------------- chunks: the unit of prefetch
 // A chunk is NB consecutive blocks of one weight row, held in registers by the lane that decodes them. Kernels keep
 // two chunks per wave: while one is decoded and multiplied, the loads of the next are in flight. With 8 waves per
@@ -219,6 +248,7 @@ template <int F, int NB> struct qw_chunk;
 
 template <int NB> struct qw_chunk<21, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = 110;
+    static constexpr int DEPTH = 3; // chunk buffers of the task pipeline (8 registers per block and buffer)
     qw_iq3_slice s[NB];
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t kg) {
 #pragma unroll
@@ -294,6 +324,10 @@ template <int NB> struct qw_chunk<21, NB> {
     }
     // The same arithmetic without the cross-block pipeline (fewer registers; for kernels that run more waves).
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#ifdef QW_EXP_NOCOMPUTE
+        for (int b = 0; b < NB; b++) acc[0] += __builtin_bit_cast(float, (s[b].qs.x ^ s[b].qs.y ^ s[b].qs.z ^ s[b].qs.w ^ s[b].sg.x ^ s[b].sg.y ^ s[b].qh ^ s[b].sc) & 0x007fffffu) + s[b].d;
+        return;
+#endif
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const uint32_t kb = k0 + 256 * b + 64 * kg;
@@ -306,6 +340,33 @@ template <int NB> struct qw_chunk<21, NB> {
                 if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
             }
             block_mfma(b, w, xh, xl, AF::has_lo, acc);
+        }
+    }
+    // The same arithmetic with operand A gathered from global memory four steps at a time (qw_afrag_gather).
+    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w[16];
+            lookups(b, lut, w);
+            const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
+            f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                af.fetch4(kb + 32 * half, 8);
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = 4 * half + jj;
+                    const h2 ff = half ? ff1 : ff0;
+                    u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+                    const h8 wv = __builtin_bit_cast(h8, raw);
+                    sub0 = qw_mfma(af.hi[jj], wv, sub0);
+                    sub1 = qw_mfma(af.lo[jj], wv, sub1);
+                }
+            }
+            acc += s[b].d * (sub0 + sub1);
         }
     }
     // One block's table values times two operand-A fragment sets (hi, lo), accumulated the way mac() does.
@@ -348,8 +409,36 @@ template <int NB> struct qw_chunk<21, NB> {
     }
 };
 
+// Packed IQ3_S (see qwk_pack_args): the slab already lies in matrix-core lane order; three coalesced loads per block
+// and no transpose. p is the (wave-uniform) address of the chunk's first slab, the second argument the lane.
+template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
+    static constexpr uint32_t BLK_K = 256, BLK_B = QW_SLAB_BYTES;
+    static constexpr int DEPTH = 3;
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t lane) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint8_t *sl = p + QW_SLAB_BYTES * b;
+            this->s[b].qs = *(const u4 *)(sl + 16 * lane);
+            this->s[b].sg = *(const u2 *)(sl + 1024 + 8 * lane);
+            this->s[b].qh = *(const uint32_t *)(sl + 1536 + 4 * lane); // qh | scales << 16 | d byte << 24: unpacked in transpose()
+        }
+    }
+    // Nothing moves between lanes except the second byte of d, which the lane 16 further holds.
+    __device__ __forceinline__ void transpose() {
+        const bool odd = (threadIdx.x >> 4) & 1;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t w = this->s[b].qh, mine = w >> 24, other = (uint32_t)__shfl_xor((int)w, 16) >> 24;
+            this->s[b].d = qw_h2f((uint16_t)(odd ? (other | mine << 8) : (mine | other << 8)));
+            this->s[b].sc = (w >> 16) & 255;
+            this->s[b].qh = w & 0xffff;
+        }
+    }
+};
+
 template <int NB> struct qw_chunk<8, NB> {
     static constexpr uint32_t BLK_K = 32, BLK_B = 34;
+    static constexpr int DEPTH = NB > 8 ? 2 : 3;
     u2 q[NB];
     uint16_t d[NB];
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t kg) {
@@ -375,6 +464,34 @@ template <int NB> struct qw_chunk<8, NB> {
         if (NB & 1) d[NB - 1] = (uint16_t)qw_pull(d[NB - 1], src4);
     }
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    // operand A gathered four blocks at a time (NB a multiple of 4)
+    __device__ __forceinline__ void mac_gather(const u2 *, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+        if constexpr (NB % 4 != 0) { // block by block
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const uint32_t kb = k0 + 32 * b + 8 * kg;
+                if (af.on) af.hi[0] = *(const h8 *)(af.rowhi + kb), af.lo[0] = *(const h8 *)(af.rowlo + kb);
+                f4 sub = {0, 0, 0, 0};
+                sub = qw_mfma(af.hi[0], qw_q8_cvt(q[b]), sub);
+                sub = qw_mfma(af.lo[0], qw_q8_cvt(q[b]), sub);
+                acc += qw_h2f(d[b]) * sub;
+            }
+            return;
+        }
+#pragma unroll
+        for (int b4 = 0; b4 + 3 < NB; b4 += 4) {
+            af.fetch4(k0 + 32 * b4 + 8 * kg, 32);
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++) {
+                const int b = b4 + bb;
+                const h8 w = qw_q8_cvt(q[b]);
+                f4 sub = {0, 0, 0, 0};
+                sub = qw_mfma(af.hi[bb], w, sub);
+                sub = qw_mfma(af.lo[bb], w, sub);
+                acc += qw_h2f(d[b]) * sub;
+            }
+        }
+    }
     template <class AF> __device__ __forceinline__ void mac(const u2 *, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -410,37 +527,49 @@ template <class C, class L, class U> __device__ __forceinline__ void qw_pipeline
 // per chunk: two cursors step through (task, chunk). rowp(task) is the lane's byte pointer to the task's first
 // chunk (chunk c follows at c * cstride bytes); use(task, c, chunk) consumes chunk c of a task. All of ntasks, w0,
 // nw and cpr must be wave-uniform.
-template <class C, class R, class U>
-__device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use) {
-    if (w0 >= ntasks) return;
-    C a, b;
-    uint32_t lt = w0, lc = 0, ut = w0, uc = 0;
+// ready() is called exactly once by every wave, after the first loads are issued and before anything is consumed:
+// the place for the workgroup's set-up and barrier, so that the first memory round trip overlaps them.
+template <class C, class R, class U, class S>
+__device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use, S ready) {
+    if (w0 >= ntasks) {
+        ready();
+        return;
+    }
+    // DEPTH chunk buffers: the loads run DEPTH - 1 chunks ahead of the arithmetic
+    constexpr int DEPTH = C::DEPTH;
+    C buf[DEPTH];
+    const uint32_t total = ((ntasks - w0 + nw - 1) / nw) * cpr;
+    uint32_t li = 0, ui = 0, lt = w0, lc = 0, ut = w0, uc = 0;
     const uint8_t *lrow = rowp(lt);
-    auto load = [&](C &c) {
-        c.load(lrow + (size_t)lc * cstride, kl);
+    auto load = [&](C &x) {
+        if (li == total) return;
+        ++li;
+        x.load(lrow + (size_t)lc * cstride, kl);
         if (++lc == cpr) {
             lc = 0;
             lt += nw;
             if (lt < ntasks) lrow = rowp(lt);
         }
     };
-    auto consume = [&](C &c) {
-        c.transpose();
-        use(ut, uc, c);
+    auto consume = [&](C &x) {
+        x.transpose();
+        use(ut, uc, x);
         if (++uc == cpr) uc = 0, ut += nw;
+        return ++ui == total;
     };
-    load(a);
-    for (;;) {
-        const bool m1 = lt < ntasks;
-        if (m1) load(b);
-        consume(a);
-        if (!m1) break;
-        const bool m2 = lt < ntasks;
-        if (m2) load(a);
-        consume(b);
-        if (!m2) break;
+#pragma unroll
+    for (int i = 0; i + 1 < DEPTH; i++) load(buf[i]);
+    ready();
+    for (bool done = false; !done;) {
+#pragma unroll
+        for (int i = 0; i < DEPTH; i++) {
+            if (done) break;
+            load(buf[(i + DEPTH - 1) % DEPTH]);
+            done = consume(buf[i]);
+        }
     }
 }
+
 
 // Copy the 64 KB pre-signed table from global memory into LDS (all loads first, then the stores).
 __device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
@@ -454,6 +583,11 @@ __device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
 #pragma unroll
         for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) dst[i + j * blockDim.x] = v[j];
     }
+}
+
+template <class C, class R, class U>
+__device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use) {
+    qw_task_pipeline<C>(ntasks, w0, nw, cpr, cstride, kl, rowp, use, [] {});
 }
 
 // ---------------------------------------------------------------- wave-wide maximum of an unsigned key

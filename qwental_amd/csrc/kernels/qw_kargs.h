@@ -103,6 +103,24 @@ typedef struct { /* pure-read ceiling and fill helpers */
     uint64_t seed;
 } qwk_mem_args;
 
+/* Tile-major copy of IQ3_S rows ("packed", format code QW_F_PACKED below): rows are taken 16 at a time (a tile) and
+ * every (tile, block) slab of 16 x 110 bytes becomes QW_SLAB_BYTES contiguous bytes in the lane order of the matrix
+ * instructions (lane l: row l & 15 of the tile, 64-value slice l >> 4 of the block):
+ *     [0, 1024)     lane l: 16 bytes qs[16 kg .. 16 kg + 16)
+ *     [1024, 1536)  lane l:  8 bytes signs[8 kg .. 8 kg + 8)
+ *     [1536, 1792)  lane l:  4 bytes qh[2 kg], qh[2 kg + 1], scales[kg], one byte of d (low byte for even kg, high for odd)
+ * so that a wave reads a slab with three fully coalesced loads. Slabs of a tile follow each other by block, tiles by
+ * index. A tile's rows n < split come from matrix A (row tile * split + n), the others from matrix B
+ * (row tile * (16 - split) + n - split): split 16 = one matrix, split 8 = gate rows and up rows side by side. */
+#define QW_SLAB_BYTES 1792u
+#define QW_F_PACKED 121
+typedef struct {
+    const uint8_t *A, *B;
+    uint8_t *dst;
+    uint64_t ntiles;
+    uint32_t nblk, rowbytes, split, pad;
+} qwk_pack_args;
+
 typedef struct { /* synthetic weights: nblocks GGUF blocks of one type, scale d = binary16(|N(0, sigma)|), the rest uniform */
     uint8_t *dst;
     uint64_t nblocks, seed;

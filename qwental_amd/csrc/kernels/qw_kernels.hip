@@ -18,6 +18,7 @@
 // wave index in the workgroup, as a scalar (so that task indices and row bases stay in scalar registers)
 __device__ __forceinline__ uint32_t qw_wave() { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
+constexpr bool qw_has_lut(int f) { return f == 21 || f == QW_F_PACKED; } // formats decoded through the LDS table
 __device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
 // ================================================================ dq_test (kernels/moe_iq.metal:208-217)
@@ -58,6 +59,24 @@ extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f8(qwk_dq_args a) {
 extern "C" __global__ void qwk_tab_init(qwk_tab_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < QW_LUT_ENTRIES) ((u2 *)(a.tab + QW_TAB_IQ3SS))[a.slot_order ? qw_lut_slot(i) : i] = qw_lut_entry(i);
+}
+
+// ================================================================ packing of IQ3_S rows (layout: qwk_pack_args)
+// One thread per (slab, lane), grid-stride over the slabs; run once per weight matrix, at its first use.
+extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) {
+    const uint64_t nslab = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
+    for (uint64_t sl = (uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); sl < nslab; sl += step) {
+        const uint64_t tile = sl / a.nblk;
+        const uint32_t blk = (uint32_t)(sl % a.nblk);
+        const uint8_t *row = n < a.split ? a.A + (tile * a.split + n) * a.rowbytes : a.B + (tile * (16 - a.split) + (n - a.split)) * a.rowbytes;
+        const uint8_t *src = row + 110 * blk;
+        uint8_t *dst = a.dst + sl * QW_SLAB_BYTES;
+        *(u4 *)(dst + 16 * lane) = *(const u4a2 *)(src + 2 + 16 * kg);
+        *(u2 *)(dst + 1024 + 8 * lane) = *(const u2a2 *)(src + 74 + 8 * kg);
+        const uint32_t qh = *(const uint16_t *)(src + 66 + 2 * kg), sc = src[106 + kg], db = src[kg & 1];
+        *(uint32_t *)(dst + 1536 + 4 * lane) = qh | sc << 16 | db << 24;
+    }
 }
 
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
@@ -348,19 +367,21 @@ __device__ __forceinline__ void qw_sel_load(qw_sel_cache &c, const uint8_t *sel,
     if (threadIdx.x == 0) c.U = *(const uint32_t *)sel;
 }
 
-template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw) {
+template <int F, int CH, class S>
+__device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw, S ready) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
     const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
     const uint32_t cpr = a.D / (C::BLK_K * CH);
     const qw_afrag_lds af = {xf, n};
-    const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
+    const uint32_t nl = lane >> 2; // (row, k-group) this lane loads from GGUF rows: (lane >> 2, lane & 3)
     auto rowp = [&](uint32_t task) {
-        const uint32_t u = task / tpe, j0 = 8 * (task % tpe), e = a.shared ? 0 : sc->ue[u];
-        return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + j0 + (nl & 7)) * a.rowbytes;
+        const uint32_t u = task / tpe, e = a.shared ? 0 : sc->ue[u];
+        if constexpr (F == QW_F_PACKED) return a.Wg + ((size_t)e * tpe + task % tpe) * a.rowbytes; // the tile's slabs; rowbytes = bytes of a tile
+        else return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + 8 * (task % tpe) + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, kl, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
+    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
         c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
@@ -379,15 +400,32 @@ template <int F, int CH> __device__ __forceinline__ void gu_tasks(const qwk_gu_a
             }
         }
         acc = f4{0, 0, 0, 0};
-    });
+    }, ready);
 }
 
 // FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
+// Order of the set-up: the selection record first (one memory round trip, one barrier: the row addresses depend on
+// it); then every wave issues its first weight loads, and only then the table copy, the activation staging and the
+// second barrier follow, overlapping that first round trip to HBM.
+#ifdef QW_EXP_TRACE
+#define QW_TRACE(slot) do { if ((threadIdx.x & 63) == 0) ((long long *)a.glut - 49152 / 8)[(blockIdx.x * 2 + (threadIdx.x >> 6) / 11) * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define QW_TRACE(slot) do { } while (0)
+#endif
 template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
-    if (FGU == 21 || FSG == 21) qw_lut_copy(lut, (const u2 *)a.glut);
-    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+    QW_TRACE(0);
     if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
     __syncthreads();
+    QW_TRACE(1);
+    bool staged = false;
+    auto ready = [&] {
+        if (staged) return;
+        staged = true;
+        if (qw_has_lut(FGU) || qw_has_lut(FSG)) qw_lut_copy(lut, (const u2 *)a.glut);
+        qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+        __syncthreads();
+        QW_TRACE(2);
+    };
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     if (FSG != 0) {
         if (a.Wsg) { // the shared expert's tiles go to the first waves
@@ -396,15 +434,17 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
             sa.Wu = a.Wsu;
             sa.rowbytes = a.sg_rowbytes;
             sa.shared = 1;
-            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw);
+            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready);
         }
     }
+    QW_TRACE(3);
     // the waves that did a shared tile come last in the routed deal, so that the work stays level
-    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw);
+    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready);
+    QW_TRACE(4);
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
-        __shared__ struct { u2 lut[(FGU == 21 || FSG == 21) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; } L; \
+        __shared__ struct { u2 lut[(qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; } L; \
         gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc);                                             \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
@@ -414,6 +454,9 @@ QW_GU(21, 2, 21, 2, qwk_gu_f21_c2_s21_c2) QW_GU(21, 2, 8, 16, qwk_gu_f21_c2_s8_c
 QW_GU(21, 1, 21, 1, qwk_gu_f21_c1_s21_c1) QW_GU(21, 1, 8, 1, qwk_gu_f21_c1_s8_c1)
 QW_GU(8, 16, 8, 16, qwk_gu_f8_c16_s8_c16) QW_GU(8, 16, 21, 2, qwk_gu_f8_c16_s21_c2)
 QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_s8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_s21_c1)
+// packed IQ3_S routed experts (and shared expert, when it is IQ3_S too)
+QW_GU(121, 2, 0, 1, qwk_gu_f121_c2) QW_GU(121, 2, 121, 2, qwk_gu_f121_c2_s121_c2) QW_GU(121, 2, 8, 16, qwk_gu_f121_c2_s8_c16)
+QW_GU(121, 1, 0, 1, qwk_gu_f121_c1) QW_GU(121, 1, 121, 1, qwk_gu_f121_c1_s121_c1) QW_GU(121, 1, 8, 1, qwk_gu_f121_c1_s8_c1)
 
 // ================================================================ front part of a layer (kernels/moe_gg.metal:534-590)
 // Router rows with the activations copied into LDS once per workgroup (8 rows per workgroup). The selection is a
@@ -441,16 +484,14 @@ template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk;
     const uint32_t ntiles = a.D / 16, cpr = a.I / (C::BLK_K * CH);
-    qw_afrag_glb<true> af = {nullptr, nullptr};
-    if (n < a.snbr) {
-        af.rowhi = a.H + ((size_t)n * (K + 1) + K) * a.I;
-        af.rowlo = af.rowhi + a.hplane;
-    }
+    h8 xhi[4] = {}, xlo[4] = {}; // token columns past the batch stay zero
+    const uint16_t *rowhi = a.H + ((size_t)(n < a.snbr ? n : 0) * (K + 1) + K) * a.I;
+    const qw_afrag_gather af = {rowhi, rowhi + a.hplane, n < a.snbr, xhi, xlo};
     f4 acc = {0, 0, 0, 0};
     qw_task_pipeline<C>(ntiles, w0, nw, cpr, CH * C::BLK_B, lane & 3,
         [&](uint32_t t) { return a.Wsd + (size_t)(16 * t + (lane >> 2)) * a.sd_rowbytes; },
         [&](uint32_t t, uint32_t ci, const C &c) {
-            c.mac(lut, af, ci * CH * C::BLK_K, kg, acc);
+            c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 != cpr) return;
             const uint32_t r = 16 * t + n;
 #pragma unroll
@@ -531,6 +572,187 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_b
     }
 // I = 512 is the synthetic shape (whole row = one chunk of 2 IQ3_S blocks); Q8_0 down weights take the any-shape kernel
 QW_DN(21, 2, 0, 1, 512, qwk_dn_f21_i512) QW_DN(21, 2, 21, 2, 512, qwk_dn_f21_i512_s21) QW_DN(21, 2, 8, 16, 512, qwk_dn_f21_i512_s8)
+
+// Range form (I <= 512). The task list is "virtual experts" x tiles of 16 rows: virtual expert 0 is the shared expert
+// when the launch carries one, then the unique routed experts in record order. Every workgroup takes one contiguous
+// range of at most D / 16 tasks, which touches at most two experts: their H rows (both planes, only the tokens
+// that picked them) are copied into LDS once, in fragment order, and the waves then stream the range's tiles with operand A read
+// from LDS. The first weight loads are issued before the table copy, the row copy and the barrier.
+struct qw_dn_seg { // one expert's part of a workgroup's range (all fields wave-uniform)
+    const uint8_t *W;  // the expert's matrix
+    float *P;          // Pg or Psh
+    uint32_t rowbytes, mask, tile0, ntile, sh; // sh: shared expert (results to P[t][row], every token < nbr)
+    uint32_t u;        // routed: index into the record
+};
+template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(const qwk_dn_args &a, const u2 *lut, const uint16_t *arows, const qw_dn_seg &g0, const qw_dn_seg &g1,
+                                                                                 bool both, const uint8_t *slots0, const uint8_t *slots1, S ready) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, nwv = blockDim.x >> 6, nl = lane >> 2;
+    const uint32_t ntask = g0.ntile + (both ? g1.ntile : 0), cpr = a.I / (C::BLK_K * CH);
+    // per lane: result slots of tokens 4 kg .. 4 kg + 3 in either segment
+    uint32_t sl0 = 0, sl1 = 0;
+    if (!g0.sh) sl0 = *(const uint32_t *)(slots0 + 4 * kg);
+    if (both && !g1.sh) sl1 = *(const uint32_t *)(slots1 + 4 * kg);
+    f4 acc = {0, 0, 0, 0};
+    qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
+        [&](uint32_t i) {
+            const bool second = i >= g0.ntile;
+            const qw_dn_seg &g = second ? g1 : g0;
+            const uint32_t tile = g.tile0 + (second ? i - g0.ntile : i);
+            if constexpr (F == QW_F_PACKED) return g.W + (size_t)tile * g.rowbytes; // rowbytes = bytes of a tile
+            else return g.W + (size_t)(16 * tile + nl) * g.rowbytes;
+        },
+        [&](uint32_t i, uint32_t ci, const C &c) {
+            const bool second = i >= g0.ntile;
+            const u4 *ab = (const u4 *)arows + (second ? 4 * a.I : 0); // fragment order: [plane][8 k-values][token], 16 bytes each
+            const qw_afrag_lds2 af = {ab, ab + 2 * a.I, n};
+            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 != cpr) return;
+            const qw_dn_seg &g = second ? g1 : g0;
+            const uint32_t r = 16 * (g.tile0 + (second ? i - g0.ntile : i)) + n, sl = second ? sl1 : sl0;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++) {
+                const uint32_t tok = 4 * kg + j;
+                if ((g.mask >> tok) & 1) g.P[(g.sh ? (size_t)tok : (size_t)tok * K + ((sl >> (8 * j)) & 255)) * a.D + r] = acc[j];
+            }
+            acc = f4{0, 0, 0, 0};
+        },
+        ready);
+}
+template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
+    const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
+    qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
+    __syncthreads();
+    const uint32_t *ue = sc->ue, *mask = sc->mask;
+    const uint8_t *slot = sc->slot;
+    uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
+    if (U > GU) U = GU;
+    // a shared-expert tile of a wider format counts as several tasks, so that ranges hold about the same bytes
+    const uint32_t tb = F == QW_F_PACKED ? a.rowbytes : 16 * a.rowbytes, stb = FSD == QW_F_PACKED ? a.sd_rowbytes : 16 * a.sd_rowbytes; // bytes of a tile
+    const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0, shw = nsh ? (stb + tb - 1) / tb : 1, vsh = nsh * shw * tpe;
+    const uint32_t V = vsh + U * tpe;
+    uint32_t per = (V + gridDim.x - 1) / gridDim.x;
+    if (per > tpe) per = tpe;
+    bool tables = false;
+    for (uint32_t base = blockIdx.x * per; base < V; base += gridDim.x * per) { // one round unless the grid is small
+        const uint32_t end = base + per < V ? base + per : V;
+        // virtual expert of a position: 0 = shared (positions below vsh), then the routed experts
+        const uint32_t v0 = base < vsh ? 0 : nsh + (base - vsh) / tpe, v1 = end - 1 < vsh ? 0 : nsh + (end - 1 - vsh) / tpe;
+        qw_dn_seg g[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t v = i ? v1 : v0;
+            g[i].sh = v < nsh;
+            if (g[i].sh) {
+                const uint32_t hi = end < vsh ? end : vsh; // positions [base, hi) -> tiles, rounded so that neighbours meet
+                g[i].tile0 = (base + shw - 1) / shw;
+                g[i].ntile = (hi + shw - 1) / shw - g[i].tile0;
+                g[i].u = 0;
+                g[i].W = a.Wsd, g[i].P = a.Psh, g[i].rowbytes = a.sd_rowbytes, g[i].mask = qw_all_tokens(a.snbr);
+            } else {
+                const uint32_t first = vsh + (v - nsh) * tpe, lo = first > base ? first : base, hi = first + tpe < end ? first + tpe : end;
+                g[i].u = v - nsh;
+                g[i].tile0 = lo - first;
+                g[i].ntile = hi - lo;
+                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ue[g[i].u]);
+                g[i].W = a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, g[i].P = a.P, g[i].rowbytes = a.rowbytes;
+                g[i].mask = (uint32_t)__builtin_amdgcn_readfirstlane((int)mask[g[i].u]) & qw_all_tokens(a.nbr);
+            }
+        }
+        const bool both = v1 != v0;
+        bool staged = false;
+        // set-up of a round, run by every wave once its first weight loads are in flight: the table (first round),
+        // the H rows of the (at most two) experts of this range, and the barrier
+        auto ready = [&] {
+            if (staged) return;
+            staged = true;
+            if (!tables && (qw_has_lut(F) || qw_has_lut(FSD))) qw_lut_copy(lut, (const u2 *)a.glut);
+            tables = true;
+            const uint32_t upr = a.I / 8; // 16-byte units per plane row
+            for (uint32_t i = threadIdx.x; i < 2 * 16 * 2 * upr; i += blockDim.x) {
+                // fragment order, so that the sixteen lanes of a k-group read 256 contiguous bytes: [segment][plane][c][token]
+                const uint32_t sg = i / (32 * upr), r = i % (32 * upr), pl = r / (16 * upr), c = (r / 16) % upr, t = r & 15;
+                if ((sg && !both) || !((g[sg].mask >> t) & 1)) continue;
+                const uint32_t s = g[sg].sh ? K : slot[g[sg].u * gnb + t];
+                ((u4 *)arows)[i] = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
+            }
+            __syncthreads();
+        };
+        // the two segments share one pipeline when their formats agree; a shared expert of another format runs first
+        if (FSD != 0 && FSD != F && g[0].sh) {
+            qw_dn_seg none = g[0];
+            none.ntile = 0;
+            dn_range_run<FSD == 0 ? F : FSD, CHSD>(a, lut, arows, g[0], none, false, slot, slot, ready);
+            if (both) dn_range_run<F, CH>(a, lut, arows + 32 * a.I, g[1], none, false, slot + g[1].u * gnb, slot, ready);
+        } else {
+            dn_range_run<F, CH>(a, lut, arows, g[0], g[1], both, slot + g[0].u * gnb, slot + g[1].u * gnb, ready);
+        }
+        __syncthreads();
+    }
+}
+#define QW_DN_RANGE(F, CH, FSD, CHSD, NAME)                                                       \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_dn_args a) {                  \
+        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; } L; \
+        dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
+    }
+// I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
+QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
+QW_DN_RANGE(21, 1, 0, 1, qwk_dnr_f21_c1) QW_DN_RANGE(21, 1, 21, 1, qwk_dnr_f21_c1_s21_c1) QW_DN_RANGE(21, 1, 8, 4, qwk_dnr_f21_c1_s8_c4)
+QW_DN_RANGE(121, 2, 0, 1, qwk_dnr_f121_c2) QW_DN_RANGE(121, 2, 121, 2, qwk_dnr_f121_c2_s121_c2) QW_DN_RANGE(121, 2, 8, 4, qwk_dnr_f121_c2_s8_c4)
+QW_DN_RANGE(121, 1, 0, 1, qwk_dnr_f121_c1) QW_DN_RANGE(121, 1, 121, 1, qwk_dnr_f121_c1_s121_c1) QW_DN_RANGE(121, 1, 8, 4, qwk_dnr_f121_c1_s8_c4)
+QW_DN_RANGE(8, 4, 0, 1, qwk_dnr_f8_c4) QW_DN_RANGE(8, 4, 8, 4, qwk_dnr_f8_c4_s8_c4) QW_DN_RANGE(8, 4, 21, 2, qwk_dnr_f8_c4_s21_c2) QW_DN_RANGE(8, 4, 21, 1, qwk_dnr_f8_c4_s21_c1)
+
+// Streaming form: independent waves, task = (unique expert, tile of 16 rows), the weights of the next task are in
+// flight while this one is multiplied (the pipeline runs across task boundaries), operand A comes straight from the
+// H planes in global memory, and only the lanes whose token picked the expert read anything. No barrier after set-up.
+template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_stream_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
+    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_sel_load(*sc, a.sel, K, gnb);
+    __syncthreads();
+    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    if (FSD != 0) {
+        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, w0, nw);
+    }
+    const uint32_t cpr = a.I / (C::BLK_K * CH);
+    f4 acc = {0, 0, 0, 0};
+    h8 xhi[4] = {}, xlo[4] = {};
+    // the waves that did a shared tile come last in the routed deal
+    qw_task_pipeline<C>(ntasks, nw - 1 - w0, nw, cpr, CH * C::BLK_B, lane & 3,
+        [&](uint32_t task) {
+            const uint32_t u = task / tpe, t = task % tpe;
+            return a.Wd + ((size_t)sc->ue[u] * a.D + 16 * t + (lane >> 2)) * a.rowbytes;
+        },
+        [&](uint32_t task, uint32_t ci, const C &c) {
+            const uint32_t u = task / tpe, m = sc->mask[u];
+            // only the lanes whose token picked the expert read H; the other columns of the result are never stored
+#ifdef QW_EXP_NOGATHER
+            const bool on = false; // timing experiment: operand A is never read
+#else
+            const bool on = n < a.nbr && ((m >> n) & 1);
+#endif
+            const uint16_t *rowhi = a.H + ((size_t)(on ? n : 0) * (K + 1) + (on ? sc->slot[u * gnb + n] : 0)) * a.I;
+            const qw_afrag_gather af = {rowhi, rowhi + a.hplane, on, xhi, xlo};
+            c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 != cpr) return;
+            const uint32_t r = 16 * (task % tpe) + n;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++) {
+                const uint32_t tok = 4 * kg + j;
+                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc[j];
+            }
+            acc = f4{0, 0, 0, 0};
+        });
+}
+#define QW_DN_STREAM(F, CH, FSD, CHSD, NAME)                                                      \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_dn_args a) {                  \
+        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; qw_sel_cache sc; } L; \
+        dn_stream_body<F, CH, FSD, CHSD>(a, L.lut, &L.sc);                                        \
+    }
+// I a multiple of 512: 2 IQ3_S blocks or 4 Q8_0 blocks a chunk (operand A of a whole chunk is in flight at once)
+QW_DN_STREAM(21, 2, 0, 1, qwk_dn_f21_c2) QW_DN_STREAM(21, 2, 21, 2, qwk_dn_f21_c2_s21_c2) QW_DN_STREAM(21, 2, 8, 4, qwk_dn_f21_c2_s8_c4)
+QW_DN_STREAM(8, 4, 0, 1, qwk_dn_f8_c4) QW_DN_STREAM(8, 4, 8, 4, qwk_dn_f8_c4_s8_c4) QW_DN_STREAM(8, 4, 21, 2, qwk_dn_f8_c4_s21_c2)
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {

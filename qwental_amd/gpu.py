@@ -47,6 +47,8 @@ SYMBOLS = [
     ("qw_hip_buf_new_device", _b, [_vp, _sz, _pb]), ("qw_hip_buf_mark_dirty", None, [_pb]),
     ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
+    ("qw_hip_set_repack", None, [_vp, _b]),
+    ("qw_hip_packed_bytes", _sz, [_vp]),
     ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
     ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),
     ("qw_hip_profile_mean", _d, [_vp, C.c_char_p, C.POINTER(_i)]),
