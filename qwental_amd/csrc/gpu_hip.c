@@ -100,6 +100,7 @@ struct qw_batch {
     // almost nothing): set by moe_pre_gg / moe_gu_gg, consumed by moe_gu_gg / moe_dn_gg of the same batch.
     struct { bool valid; int fmt; const uint8_t *Wsg, *Wsu; qw_hbuf *hg, *hu; uint32_t rowbytes, nbr; } pend_sg;
     struct { bool valid; int fmt; const uint8_t *Wsd; qw_hbuf *hd; float *Psh; uint32_t rowbytes, nbr; } pend_sd;
+    struct { bool valid; qwk_select_args a; } pend_sel; // the selection moe_pre_gg owes: made inside the gate/up launch, or by a launch of its own
 };
 
 struct qw_gpu {
@@ -666,11 +667,20 @@ static bool fill_router(qw_batch *b, qwk_router_args *a, unsigned iWr, unsigned 
            bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a->x) && bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, true, "logits", (void **)&a->logits);
 }
 
-static bool launch_select(qw_batch *b, unsigned ilg, unsigned isel, uint32_t nbr) {
+static bool fill_select(qw_batch *b, qwk_select_args *a, unsigned ilg, unsigned isel, uint32_t nbr) {
     const qw_kparams *p = &b->k->p;
-    qwk_select_args a = {.nbr = nbr, .E = (uint32_t)p->E, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
-    if (!bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, false, "logits", (void **)&a.logits) || !bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a.sel)) return false;
-    return add_launch(b, "qwk_select", 1, 1024, &a, sizeof a);
+    *a = (qwk_select_args){.nbr = nbr, .E = (uint32_t)p->E, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
+    return bind_ptr(b, ilg, (size_t)nbr * (p->E + 1) * 4, false, "logits", (void **)&a->logits) && bind_ptr(b, isel, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), true, "selection", (void **)&a->sel);
+}
+static bool launch_select(qw_batch *b, unsigned ilg, unsigned isel, uint32_t nbr) {
+    qwk_select_args a;
+    return fill_select(b, &a, ilg, isel, nbr) && add_launch(b, "qwk_select", 1, 1024, &a, sizeof a);
+}
+// The selection that a moe_pre_gg dispatch left pending and no gate/up dispatch took over: a launch of its own.
+static bool flush_select(qw_batch *b) {
+    if (!b->pend_sel.valid) return true;
+    b->pend_sel.valid = false;
+    return add_launch(b, "qwk_select", 1, 1024, &b->pend_sel.a, sizeof b->pend_sel.a);
 }
 
 static bool nbr_ok(qw_batch *b, uint32_t nbr) {
@@ -761,7 +771,7 @@ static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nb
 static bool tr_pre(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     uint32_t nbr;
-    if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr)) return false;
+    if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr) || !flush_select(b)) return false;
     const size_t rb = fmt_rb(p->fsg, p->D);
     void *h;
     b->pend_sg.valid = false;
@@ -778,7 +788,9 @@ static bool tr_pre(qw_batch *b) {
     if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
     if (b->buf[2].off % 16) return fail(b, "moe_pre_gg: x offset %zu is not 16-byte aligned", b->buf[2].off);
     // the counter buffer of the reference's hand-over (index 4) is not used: the selection is a launch of its own
-    return add_launch(b, p->rwf == 30 ? "qwk_pre_w30" : "qwk_pre_w1", cdiv((unsigned)p->E + 1, 8), 512, &a, sizeof a) && launch_select(b, 3, 5, nbr);
+    if (!add_launch(b, p->rwf == 30 ? "qwk_pre_w30" : "qwk_pre_w1", cdiv((unsigned)p->E + 1, 8), 512, &a, sizeof a) || !fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
+    b->pend_sel.valid = true; // made by the gate/up launch if one follows for the same record, else by its own launch
+    return true;
 }
 
 // src/engine.c:616-629: 0 Wg, 1 Wu, 2 shared down, 3 Psh, 4 x, 5 sel, 6 H, 11 tables, 12 nbr.
@@ -811,6 +823,12 @@ static bool tr_gu(qw_batch *b) {
         b->pend_sg.valid = false;
         if (cg == 1 || cs == 1) cg = cs = 1; // any-shape builds come in pairs
     }
+    if (b->pend_sel.valid && b->pend_sel.a.sel == a.sel && b->pend_sel.a.nbr == nbr && b->pend_sel.a.E == (uint32_t)p->E && b->pend_sel.a.topk == (uint32_t)p->topk &&
+        b->pend_sel.a.gnb == (uint32_t)p->gnb && !getenv("QW_HIP_SPLIT_SELECT")) {
+        a.logits = b->pend_sel.a.logits;
+        a.E = (uint32_t)p->E;
+        b->pend_sel.valid = false;
+    } else if (!flush_select(b)) return false;
     int fgu = p->fgu;
     if (fgu == 21) { // tile-major copies of the IQ3_S rows, made at first use
         const uint32_t nblk = (uint32_t)p->D / 256, tileb = nblk * QW_SLAB_BYTES;
@@ -929,6 +947,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     if (!b->k) { fail(b, "qw_batch_dispatch without a kernel"); return; }
     const int first = b->nl;
     bool ok;
+    if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
     case FAM_QMV_GG: ok = tr_qmv(b); break;
@@ -949,7 +968,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
-    if (b->failed) return false;
+    if (b->failed || !flush_select(b)) return false;
     if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
     // host -> device for what this segment binds
     const unsigned mark = ++g->mark;

@@ -64,7 +64,10 @@ typedef struct {
     const void *glut;
     /* the shared expert's gate/up, done by the same launch when Wsg != NULL: all tokens, slot topk */
     const uint8_t *Wsg, *Wsu;
-    uint32_t sg_rowbytes, pad;
+    uint32_t sg_rowbytes, E;
+    /* logits != NULL: the selection has not been made yet; every workgroup makes it from the logits [nbr][E + 1] for
+     * itself and workgroup 0 also writes the record to sel (the later kernels of the layer read it from there) */
+    const float *logits;
 } qwk_gu_args;
 
 /* down projection. routed: Pg[t][slot][row] for the tokens in mask[u]; shared != 0: Psh[t][row] from slot topk. */

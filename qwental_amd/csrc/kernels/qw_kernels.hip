@@ -216,39 +216,57 @@ struct qw_sel_scratch {
 };
 
 // PER = E / 64 values per lane, lane l holding experts l * PER .. l * PER + PER - 1 (lowest lane = lowest index).
-template <int PER> __device__ __forceinline__ void select_token(const float *lg, uint32_t E, uint32_t K, uint32_t tok, float *w, uint32_t *ids, uint32_t lane) {
-    uint32_t k[PER];
+// T tokens at once (tok0, tok0 + tstep, ...; those >= nbr are skipped): a round is a chain of dependent instructions,
+// so two tokens in flight cost about the time of one. Every lane keeps the maximum of its PER keys and the position
+// of that maximum; a round takes the wave maximum of those, the lowest lane that holds it, and only that lane
+// recomputes its own maximum.
+template <int PER, int T>
+__device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, uint32_t K, uint32_t tok0, uint32_t tstep, uint32_t nbr, float *w, uint32_t *ids, uint32_t lane) {
+    uint32_t k[T][PER], bk[T], bj[T], pk[T];
+    bool on[T];
 #pragma unroll
-    for (int j = 0; j < PER; j++) k[j] = qw_fkey(lg[lane * PER + j]);
-    uint32_t pk = 0;
-    for (uint32_t r = 0; r < K; r++) {
-        // lane-local maximum by a balanced tree; among equals the lower position wins at every node
-        uint32_t tk[PER], tj[PER];
+    for (int t = 0; t < T; t++) {
+        const uint32_t tok = tok0 + t * tstep;
+        on[t] = tok < nbr;
+        const float *lg = logits + (size_t)(on[t] ? tok : tok0) * (E + 1);
 #pragma unroll
-        for (int j = 0; j < PER; j++) { tk[j] = k[j]; tj[j] = j; }
-#pragma unroll
-        for (int w = 1; w < PER; w *= 2)
-#pragma unroll
-            for (int j = 0; j + w < PER; j += 2 * w) {
-                const bool up = tk[j + w] > tk[j];
-                tk[j] = up ? tk[j + w] : tk[j];
-                tj[j] = up ? tj[j + w] : tj[j];
-            }
-        const uint32_t bk = tk[0], bj = tj[0];
-        const uint32_t m = qw_wave_max_u32(bk);
-        const uint32_t L = (uint32_t)__builtin_ctzll(__ballot(bk == m)); // lowest lane among equals
-        const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)bj, (int)L);
-        if (lane == 0) ids[tok * K + r] = L * PER + j;
-        if (lane == r) pk = m;
-#pragma unroll
-        for (int jj = 0; jj < PER; jj++)
-            if (lane == L && (uint32_t)jj == j) k[jj] = 0; // below every key, -inf included
+        for (int j = 0; j < PER; j++) k[t][j] = qw_fkey(lg[lane * PER + j]);
+        pk[t] = 0;
     }
-    const float p = qw_fkey_inv(pk), mx = __shfl(p, 0), ex = __expf(p - mx);
-    float sm = 0;
-    for (uint32_t r = 0; r < K; r++) sm += __shfl(ex, r); // rank order
-    if (lane < K) w[tok * (K + 1) + lane] = ex / sm;
-    if (lane == K) w[tok * (K + 1) + K] = 1.0f / (1.0f + __expf(-lg[E]));
+    auto local_max = [&](int t) { // among equals the lower position wins
+        bk[t] = k[t][0], bj[t] = 0;
+#pragma unroll
+        for (int j = 1; j < PER; j++)
+            if (k[t][j] > bk[t]) bk[t] = k[t][j], bj[t] = j;
+    };
+#pragma unroll
+    for (int t = 0; t < T; t++) local_max(t);
+    for (uint32_t r = 0; r < K; r++) {
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            const uint32_t m = qw_wave_max_u32(bk[t]);
+            const uint32_t L = (uint32_t)__builtin_ctzll(__ballot(bk[t] == m)); // lowest lane among equals
+            const uint32_t j = (uint32_t)__builtin_amdgcn_readlane((int)bj[t], (int)L);
+            if (lane == 0 && on[t]) ids[(tok0 + t * tstep) * K + r] = L * PER + j;
+            if (lane == r) pk[t] = m;
+            if (lane == L) {
+#pragma unroll
+                for (int jj = 0; jj < PER; jj++)
+                    if ((uint32_t)jj == j) k[t][jj] = 0; // below every key, -inf included
+                local_max(t);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        const uint32_t tok = tok0 + t * tstep;
+        const float p = qw_fkey_inv(pk[t]), mx = __shfl(p, 0), ex = __expf(p - mx);
+        float sm = 0;
+        for (uint32_t r = 0; r < K; r++) sm += __shfl(ex, r); // rank order
+        if (!on[t]) continue;
+        if (lane < K) w[tok * (K + 1) + lane] = ex / sm;
+        if (lane == K) w[tok * (K + 1) + K] = 1.0f / (1.0f + __expf(-logits[(size_t)tok * (E + 1) + E]));
+    }
 }
 
 // Any E <= 1024: the values live in LDS (v, E floats); lane l scans experts l, l + 64, ...
@@ -283,7 +301,7 @@ __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 ||
 
 // The whole selection by one workgroup (any multiple of 64 threads). lgs: LDS scratch, 1024 floats per wave, used
 // only when E is not 64 * {1, 2, 4, 8, 16}.
-__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, float *lgs) {
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, float *lgs, bool store = true) {
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
@@ -292,16 +310,19 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     for (uint32_t i = tid; i < GU * gnb / 4; i += nth) s.slot[i] = 0;
     for (uint32_t i = tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
     __syncthreads();
-    for (uint32_t t = wave; t < a.nbr; t += nwv) {
-        const float *lg = a.logits + (size_t)t * (E + 1);
-        switch (fast ? E : 0u) {
-        case 64: select_token<1>(lg, E, K, t, s.w, s.ids, lane); break;
-        case 128: select_token<2>(lg, E, K, t, s.w, s.ids, lane); break;
-        case 256: select_token<4>(lg, E, K, t, s.w, s.ids, lane); break;
-        case 512: select_token<8>(lg, E, K, t, s.w, s.ids, lane); break;
-        case 1024: select_token<16>(lg, E, K, t, s.w, s.ids, lane); break;
-        default: select_token_any(lg, lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
+    if (fast) { // two tokens per wave at a time when there are more tokens than waves
+        for (uint32_t t = wave; t < a.nbr; t += 2 * nwv) {
+            const bool two = t + nwv < a.nbr;
+            switch (E) {
+            case 64: two ? select_tokens<1, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<1, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 128: two ? select_tokens<2, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<2, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 256: two ? select_tokens<4, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<4, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 512: two ? select_tokens<8, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<8, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            default: two ? select_tokens<16, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<16, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            }
         }
+    } else {
+        for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
     __syncthreads();
     if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid);
@@ -331,6 +352,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         if (f == tid) s.ue[u] = s.ids[tid];
     }
     __syncthreads();
+    if (!store) return;
     // the record, in one pass of dword stores: U | ue[GU] | mask[GU] | slot[GU][gnb] | w[gnb][K + 1]
     uint32_t *out = (uint32_t *)a.sel;
     const uint32_t n_slot = GU * gnb / 4, n_w = gnb * (K + 1), total = 1 + 2 * GU + n_slot + n_w;
@@ -414,7 +436,15 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 #endif
 template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
     QW_TRACE(0);
-    if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+    if (a.logits) { // the selection, made here by every workgroup; the scratch lies where x is staged afterwards
+        qw_sel_scratch &ss = *(qw_sel_scratch *)xf;
+        const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
+        select_all(sa, ss, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
+        const uint32_t GU = a.gnb * a.topk;
+        for (uint32_t i = threadIdx.x; i < GU; i += blockDim.x) sc->ue[i] = ss.ue[i], sc->mask[i] = i < ss.U ? ss.um[i] : 0;
+        for (uint32_t i = threadIdx.x; i < GU * a.gnb / 4; i += blockDim.x) ((uint32_t *)sc->slot)[i] = ss.slot[i];
+        if (threadIdx.x == 0) sc->U = ss.U;
+    } else if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
     __syncthreads();
     QW_TRACE(1);
     bool staged = false;
