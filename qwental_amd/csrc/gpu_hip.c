@@ -773,10 +773,10 @@ static bool tr_pre(qw_batch *b) {
     uint32_t nbr;
     if (!bind_bytes(b, 14, &nbr, 4, "nbr") || !nbr_ok(b, nbr) || !flush_select(b)) return false;
     const size_t rb = fmt_rb(p->fsg, p->D);
-    void *h;
+    uint16_t *h;
     b->pend_sg.valid = false;
     if (!bind_ptr(b, 6, (size_t)p->I * rb, false, "shared gate weights", (void **)&b->pend_sg.Wsg) || !bind_ptr(b, 7, (size_t)p->I * rb, false, "shared up weights", (void **)&b->pend_sg.Wsu) ||
-        !bind_ptr(b, 8, (size_t)p->NB * (p->topk + 1) * p->I * 4, true, "H", &h)) return false;
+        !bind_ptr(b, 8, (size_t)p->NB * (p->topk + 1) * p->I * 4, true, "H", (void **)&h)) return false;
     b->pend_sg.valid = true;
     b->pend_sg.hg = b->buf[6].h;
     b->pend_sg.hu = b->buf[7].h;
@@ -784,11 +784,30 @@ static bool tr_pre(qw_batch *b) {
     b->pend_sg.rowbytes = (uint32_t)rb;
     b->pend_sg.nbr = nbr;
     if (!p->rbf) return true; // router and selection come as dispatches of their own
-    qwk_pre_args a = {.topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
+    qwk_pre_args a = {.nrouter = cdiv((unsigned)p->E + 1, 8)};
     if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
     if (b->buf[2].off % 16) return fail(b, "moe_pre_gg: x offset %zu is not 16-byte aligned", b->buf[2].off);
-    // the counter buffer of the reference's hand-over (index 4) is not used: the selection is a launch of its own
-    if (!add_launch(b, p->rwf == 30 ? "qwk_pre_w30" : "qwk_pre_w1", cdiv((unsigned)p->E + 1, 8), 512, &a, sizeof a) || !fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
+    // The shared expert's gate/up runs on the workgroups after the router's when a tile row splits into at most 8
+    // chunks (D a multiple of 512, at most 4096) and the weights are Q8_0 or packed IQ3_S; otherwise it is left for
+    // the gate/up launch (pend_sg).
+    char fn[48];
+    fname_fmt(fn, sizeof fn, "qwk_pre_w%d", p->rwf == 30 ? 30 : 1);
+    unsigned grid = a.nrouter;
+    const unsigned cpr = (unsigned)p->D / 512;
+    if (p->D % 512 == 0 && cpr <= 8 && !getenv("QW_HIP_SHARED_IN_GU")) {
+        const uint32_t nblk = (uint32_t)p->D / 256;
+        const uint8_t *ps = p->fsg == 21 ? get_pack(b, b->pend_sg.hg, b->pend_sg.Wsg, b->pend_sg.hu, b->pend_sg.Wsu, (uint64_t)(p->I / 8), nblk, (uint32_t)rb, 8) : NULL;
+        if (p->fsg == 8 || ps) {
+            a.g = (qwk_gu_args){.Wg = ps ? ps : b->pend_sg.Wsg, .Wu = ps ? NULL : b->pend_sg.Wsu, .x = a.r.x, .H = h, .D = (uint32_t)p->D, .I = (uint32_t)p->I,
+                                .rowbytes = ps ? nblk * QW_SLAB_BYTES : (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = 1,
+                                .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I, .glut = glut(b->g)};
+            fname_fmt(fn, sizeof fn, "qwk_pre_w%d_s%d_c%d", p->rwf == 30 ? 30 : 1, ps ? QW_F_PACKED : 8, ps ? 2 : 16);
+            grid += cdiv((unsigned)p->I / 8, 8 / cpr);
+            b->pend_sg.valid = false; // done here
+        }
+    }
+    // the counter buffer of the reference's hand-over (index 4) is not used
+    if (!add_launch(b, intern(fn), grid, 512, &a, sizeof a) || !fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
     b->pend_sel.valid = true; // made by the gate/up launch if one follows for the same record, else by its own launch
     return true;
 }

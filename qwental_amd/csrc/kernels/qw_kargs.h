@@ -84,12 +84,12 @@ typedef struct {
     uint32_t sd_rowbytes, snbr; /* snbr: token count of the shared part */
 } qwk_dn_args;
 
-/* front part of a layer: router rows (the selection is the launch after it). sel / cnt / topk / gnb are unused. */
+/* front part of a layer: router rows on the first nrouter workgroups; when g.Wsg != NULL the shared expert's gate/up
+ * on the workgroups after them (g: its arguments, shared = 1), one chunk of a tile per wave, summed through LDS. */
 typedef struct {
     qwk_router_args r;
-    uint8_t *sel;
-    uint32_t *cnt;
-    uint32_t topk, gnb;
+    uint32_t nrouter, pad;
+    qwk_gu_args g;
 } qwk_pre_args;
 
 typedef struct { /* out[t][row] = half(sum_s w[t][s] * Pg[t][s][row] + w[t][topk] * Psh[t][row]) */

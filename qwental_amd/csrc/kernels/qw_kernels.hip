@@ -489,23 +489,66 @@ QW_GU(121, 2, 0, 1, qwk_gu_f121_c2) QW_GU(121, 2, 121, 2, qwk_gu_f121_c2_s121_c2
 QW_GU(121, 1, 0, 1, qwk_gu_f121_c1) QW_GU(121, 1, 121, 1, qwk_gu_f121_c1_s121_c1) QW_GU(121, 1, 8, 1, qwk_gu_f121_c1_s8_c1)
 
 // ================================================================ front part of a layer (kernels/moe_gg.metal:534-590)
-// Router rows with the activations copied into LDS once per workgroup (8 rows per workgroup). The selection is a
-// launch of its own (qwk_select): handing it to the last router workgroup through a device-wide counter was measured
-// slower than the kernel boundary. The shared expert's gate/up runs in the gate/up launch.
-template <int WF> __device__ __forceinline__ void pre_body(const qwk_pre_args &a, u4 *lds) {
+// Router rows with the activations copied into LDS once per workgroup (8 rows per workgroup) on the first
+// a.nrouter workgroups. The workgroups after them do the shared expert's gate/up (the reference computes it in the
+// same dispatch, kernels/moe_gg.metal:563-573): a tile of 8 gate + 8 up rows is split by chunk over consecutive
+// waves of one workgroup (a chunk each, so that the whole expert takes one memory round trip), the partial sums meet
+// in LDS and the wave of chunk 0 adds them in chunk order, applies SwiGLU and stores H[t][topk].
+// The selection is not made here: handing it to the last router workgroup through a device-wide counter was measured
+// slower than a kernel boundary.
+template <int WF> __device__ __forceinline__ void pre_router(const qwk_pre_args &a, u4 *lds) {
     const uint32_t nx = a.r.nb * a.r.D / 8; // 16-byte units of x
     for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) lds[i] = ((const u4 *)a.r.x)[i];
     __syncthreads();
     router_rows_lds<WF>(a.r, (const uint16_t *)lds, blockIdx.x * (blockDim.x >> 6) + qw_wave(), qw_lane());
 }
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_pre_w1(qwk_pre_args a) {
-    __shared__ u4 lds[QW_XF_MAXK * 2];
-    pre_body<1>(a, lds);
+template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pre_args &pa, u2 *lut, u4 *xf, f4 *part) {
+    typedef qw_chunk<F, CH> C;
+    const qwk_gu_args &a = pa.g;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, wave = qw_wave(), nwv = blockDim.x >> 6;
+    const uint32_t cpr = a.D / (C::BLK_K * CH), tpw = nwv / cpr; // tiles per workgroup (the host checks cpr <= waves)
+    const uint32_t tile = (blockIdx.x - pa.nrouter) * tpw + wave / cpr, ci = wave % cpr;
+    const bool on = wave < tpw * cpr && tile < a.I / 8;
+    C c;
+    if (on) {
+        if constexpr (F == QW_F_PACKED) c.load(a.Wg + (size_t)tile * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane);
+        else c.load(((lane >> 2) < 8 ? a.Wg : a.Wu) + ((size_t)8 * tile + ((lane >> 2) & 7)) * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane & 3);
+    }
+    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+    __syncthreads();
+    f4 acc = {0, 0, 0, 0};
+    if (on) {
+        c.transpose();
+        const qw_afrag_lds af = {xf, n};
+        c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+        part[wave * 64 + lane] = acc;
+    }
+    __syncthreads();
+    if (!on || ci != 0) return;
+    acc = part[wave * 64 + lane];
+    for (uint32_t i = 1; i < cpr; i++) acc += part[(wave + i) * 64 + lane]; // chunk order
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) {
+        const float up = __shfl_xor(acc[j], 8), g = acc[j];
+        const uint32_t tok = 4 * kg + j;
+        if (n < 8 && tok < a.nbr) {
+            const float h = g / (1.0f + __expf(-g)) * up;
+            const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
+            const size_t o = ((size_t)tok * (K + 1) + K) * a.I + 8 * tile + n;
+            a.H[o] = __builtin_bit_cast(uint16_t, hi);
+            a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
+        }
+    }
 }
-extern "C" __global__ __launch_bounds__(QW_WG) void qwk_pre_w30(qwk_pre_args a) {
-    __shared__ u4 lds[QW_XF_MAXK * 2];
-    pre_body<30>(a, lds);
-}
+#define QW_PRE(WF, F, CH, NAME)                                                                          \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {                           \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[F ? (QW_WG / 64) * 64 : 1]; } L; \
+        if (blockIdx.x < a.nrouter) pre_router<WF>(a, L.xf);                                            \
+        else if (F != 0) pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part);                              \
+    }
+QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
+QW_PRE(1, 121, 2, qwk_pre_w1_s121_c2) QW_PRE(30, 121, 2, qwk_pre_w30_s121_c2) QW_PRE(1, 8, 16, qwk_pre_w1_s8_c16) QW_PRE(30, 8, 16, qwk_pre_w30_s8_c16)
 
 // ================================================================ down (kernels/moe_gg.metal:456-483, 606-617, 639-652)
 // The shared expert's down projection rides in the same launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
