@@ -18,6 +18,18 @@
 // wave index in the workgroup, as a scalar (so that task indices and row bases stay in scalar registers)
 __device__ __forceinline__ uint32_t qw_wave() { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
+#ifdef QW_EXP_TRACE
+#define QW_TRACE(slot) do { if ((threadIdx.x & 63) == 0) ((long long *)a.glut - 49152 / 8)[(blockIdx.x * 2 + (threadIdx.x >> 6) / 11) * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define QW_TRACE(slot) do { } while (0)
+#endif
+#ifdef QW_EXP_TRACEDN
+#define QW_TRACEG(slot) do { } while (0)
+#define QW_TRACED(slot) QW_TRACE(slot)
+#else
+#define QW_TRACEG(slot) QW_TRACE(slot)
+#define QW_TRACED(slot) do { } while (0)
+#endif
 constexpr bool qw_has_lut(int f) { return f == 21 || f == QW_F_PACKED; } // formats decoded through the LDS table
 __device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
@@ -429,13 +441,8 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 // Order of the set-up: the selection record first (one memory round trip, one barrier: the row addresses depend on
 // it); then every wave issues its first weight loads, and only then the table copy, the activation staging and the
 // second barrier follow, overlapping that first round trip to HBM.
-#ifdef QW_EXP_TRACE
-#define QW_TRACE(slot) do { if ((threadIdx.x & 63) == 0) ((long long *)a.glut - 49152 / 8)[(blockIdx.x * 2 + (threadIdx.x >> 6) / 11) * 8 + (slot)] = wall_clock64(); } while (0)
-#else
-#define QW_TRACE(slot) do { } while (0)
-#endif
 template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
-    QW_TRACE(0);
+    QW_TRACEG(0);
     if (a.logits) { // the selection, made here by every workgroup; the scratch lies where x is staged afterwards
         qw_sel_scratch &ss = *(qw_sel_scratch *)xf;
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
@@ -446,7 +453,7 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
         if (threadIdx.x == 0) sc->U = ss.U;
     } else if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
     __syncthreads();
-    QW_TRACE(1);
+    QW_TRACEG(1);
     bool staged = false;
     auto ready = [&] {
         if (staged) return;
@@ -454,7 +461,7 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
         if (qw_has_lut(FGU) || qw_has_lut(FSG)) qw_lut_copy(lut, (const u2 *)a.glut);
         qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
         __syncthreads();
-        QW_TRACE(2);
+        QW_TRACEG(2);
     };
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     if (FSG != 0) {
@@ -467,10 +474,10 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
             gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready);
         }
     }
-    QW_TRACE(3);
+    QW_TRACEG(3);
     // the waves that did a shared tile come last in the routed deal, so that the work stays level
     gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready);
-    QW_TRACE(4);
+    QW_TRACEG(4);
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
@@ -694,8 +701,10 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
 }
 template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
+    QW_TRACED(0);
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
     __syncthreads();
+    QW_TRACED(1);
     const uint32_t *ue = sc->ue, *mask = sc->mask;
     const uint8_t *slot = sc->slot;
     uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
@@ -739,17 +748,34 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         auto ready = [&] {
             if (staged) return;
             staged = true;
+            // The H rows of the tokens that picked the range's experts, both planes: the rows in use (a few of the 32
+            // possible) are numbered through the two masks, so that one pass of the workgroup usually copies them all;
+            // the loads of that pass are in flight while the table is copied. Fragment order in LDS,
+            // [segment][plane][c][token], 16 bytes each: the sixteen lanes of a k-group read 256 contiguous bytes.
+            const uint32_t upr = a.I / 8, per = 2 * upr; // 16-byte units per plane row, per row
+            const uint32_t rows = g[0].mask | (both ? g[1].mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
+            auto item = [&](uint32_t i, uint32_t &dst) {
+                uint32_t m = rows;
+                for (uint32_t k = i / per; k; k--) m &= m - 1; // drop the rows before this one
+                const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, t = bit & 15, r = i % per, pl = r / upr, c = r % upr;
+                const uint32_t s = g[sg].sh ? K : slot[g[sg].u * gnb + t];
+                dst = ((sg * 2 + pl) * upr + c) * 16 + t;
+                return *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
+            };
+            uint32_t d0 = 0;
+            u4 v0 = {0, 0, 0, 0};
+            const bool have = threadIdx.x < nitem;
+            if (have) v0 = item(threadIdx.x, d0);
             if (!tables && (qw_has_lut(F) || qw_has_lut(FSD))) qw_lut_copy(lut, (const u2 *)a.glut);
             tables = true;
-            const uint32_t upr = a.I / 8; // 16-byte units per plane row
-            for (uint32_t i = threadIdx.x; i < 2 * 16 * 2 * upr; i += blockDim.x) {
-                // fragment order, so that the sixteen lanes of a k-group read 256 contiguous bytes: [segment][plane][c][token]
-                const uint32_t sg = i / (32 * upr), r = i % (32 * upr), pl = r / (16 * upr), c = (r / 16) % upr, t = r & 15;
-                if ((sg && !both) || !((g[sg].mask >> t) & 1)) continue;
-                const uint32_t s = g[sg].sh ? K : slot[g[sg].u * gnb + t];
-                ((u4 *)arows)[i] = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
+            if (have) ((u4 *)arows)[d0] = v0;
+            for (uint32_t i = threadIdx.x + blockDim.x; i < nitem; i += blockDim.x) {
+                uint32_t d;
+                const u4 v = item(i, d);
+                ((u4 *)arows)[d] = v;
             }
             __syncthreads();
+            QW_TRACED(2);
         };
         // the two segments share one pipeline when their formats agree; a shared expert of another format runs first
         if (FSD != 0 && FSD != F && g[0].sh) {
@@ -760,6 +786,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         } else {
             dn_range_run<F, CH>(a, lut, arows, g[0], g[1], both, slot + g[0].u * gnb, slot + g[1].u * gnb, ready);
         }
+        QW_TRACED(4);
         __syncthreads();
     }
 }
