@@ -24,7 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
-DOMINANT = "qwk_gu_f21"
+DOMINANT = "qwk_gu_f"
 
 
 def timed_steps(stack, x, nb, steps, warmup):
@@ -145,7 +145,7 @@ def main():
             "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": res[nb]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "u8 blocks -> f16 matrix-core operands, f32 accumulate", "data": "synthetic (seeded, generated on device)",
             "config": {"workload": "configs[4]: %d-layer MoE FFN stack decode, B=%d, D=2048 I=512 E=512 top-10, IQ3_S experts, shared expert Q8_0 every 4th layer" % (stack.L, nb),
-                       "resident_weight_bytes": int(stack.weight_bytes), "device": gpu.name()},
+                       "resident_weight_bytes": int(stack.weight_bytes), "packed_copy_bytes": int(gpu.L.qw_hip_packed_bytes(gpu.g)), "device": gpu.name()},
             "roofline": roof,
             "stack": {"GBps_algorithmic": res[nb]["stack_GBps"], "frac_of_peak": res[nb]["stack_GBps"] / HBM_PEAK_GBS, "gpu_ms_per_step": res[nb]["gpu_ms_per_step"],
                       "mean_unique_experts": res[nb]["mean_U"], "bytes_per_step": res[nb]["bytes_per_step"]},

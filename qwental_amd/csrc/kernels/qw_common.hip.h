@@ -335,6 +335,11 @@ template <int NB> struct qw_chunk<21, NB> {
             lookups(b, lut, w);
             h8 xh[8], xl[8];
 #pragma unroll
+#ifdef QW_EXP_NOLO
+            for (int j = 0; j < 8; j++) xh[j] = af.hi(kb + 8 * j);
+            block_mfma(b, w, xh, xl, false, acc);
+            continue;
+#endif
             for (int j = 0; j < 8; j++) {
                 xh[j] = af.hi(kb + 8 * j);
                 if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
