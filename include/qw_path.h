@@ -60,6 +60,17 @@ bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, cons
  * each in turn, out. Equivalent to nlayers calls of qw_path_gg_moe. */
 bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,
                           const qw_buf *sel, const qw_buf *out);
+/* Ragged batch through the packing path (the routed part of the reference's pf_moe(), src/engine.c:4203-4254, with
+ * the kernels of kernels/moe_prefill.metal and moe_pf_gg): T rows of x, P = T * topk (token, expert) pairs given by
+ * ids [P] (uint32) and weights w [P] (float); count -> plan -> scatter -> gate / up products -> SiLU -> down product
+ * -> gathered weighted sum into out [T][D] binary16 (routed experts only). tm = rows per tile entry (16, 32 or 64).
+ * qw_path_pf_reserve sizes the packing scratch for up to tmax rows; 0 .. 6 of qw_path_pf_scratch are counts, offsets,
+ * tile table, pos_of, packed x, H, packed down output. */
+bool qw_path_pf_reserve(qw_path *p, int tmax, int tm);
+bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const qw_buf *x, const qw_buf *ids, const qw_buf *w, const qw_buf *out);
+const qw_buf *qw_path_pf_scratch(const qw_path *p, int which);
+unsigned qw_path_pf_max_tiles(const qw_path *p);
+
 /* The scratch buffers, for tests: 0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg. */
 const qw_buf *qw_path_scratch(const qw_path *p, int which);
 

@@ -24,18 +24,20 @@ static const unsigned char qw_code_object[] = {
 #embed "qw_kernels_gfx950.hsaco"
 };
 
-enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 8192, QW_MAX_FUNCS = 96 };
+enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 8192, QW_MAX_FUNCS = 256 };
 
 // ---------------------------------------------------------------- records
 typedef enum {
     FAM_DQ_TEST, FAM_QMV_GG, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
     FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
+    FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PF, // ragged packing and the grouped product
 } qw_family;
 
 typedef struct { // parameters taken from the define block
     int F, K, RB, NB, yfloat;            // dq_test / qmv_gg
     int E, topk, D, I, gnb;              // MoE
     int fgu, fd, fsg, fsu, fsd, rbf, rwf; // formats; rbf: router inside moe_pre_gg; rwf: router weight type (1 / 30)
+    int tm;                              // packing: rows per tile entry
 } qw_kparams;
 
 struct qw_kernel {
@@ -344,7 +346,26 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             if (!def_int(d, n, "FD", &p.fd)) FAIL("moe_dn_gg: FD missing");
             if (!fmt_ok(p.fd)) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 21)", p.fd);
             if (!reg_kernel(g, d, n, "moe_dn_gg", FAM_DN, &p, err, errlen) || !reg_kernel(g, d, n, "moe_cmb_gg", FAM_CMB, &p, err, errlen)) { ok = false; goto out; }
-        } else FAIL("moe_gg: GG_PART %d has no gfx950 build (have 0..3 and GG_ROUTER)", part);
+        } else if (part != 5) FAIL("moe_gg: GG_PART %d has no gfx950 build (have 0..3, 5 and GG_ROUTER)", part);
+    }
+    if (part == 5) { // the grouped product over packed rows, src/engine.c:3244-3248
+        p = (qw_kparams){0};
+        if (!def_int(d, n, "PFF", &p.F) || !def_int(d, n, "KD", &p.K) || !def_int(d, n, "TM", &p.tm) || !def_int(d, n, "E", &p.E)) FAIL("moe_pf_gg: PFF, KD, TM and E must be integer macros");
+        if (!fmt_ok(p.F)) FAIL("moe_pf_gg: ggml type %d has no gfx950 build (have 8, 21)", p.F);
+        if (p.K <= 0 || p.K % fmt_qb(p.F) || (p.F == 8 && p.K % 128)) FAIL("moe_pf_gg: KD %d does not fit type %d", p.K, p.F);
+        if (p.tm < 1 || p.tm > 64) FAIL("moe_pf_gg: TM %d outside this build (1..64 rows per tile entry)", p.tm);
+        if (p.E < 1 || p.E > 1024) FAIL("moe_pf_gg: E %d outside this build (E <= 1024)", p.E);
+        if (!reg_kernel(g, d, n, "moe_pf_gg", FAM_PF, &p, err, errlen)) { ok = false; goto out; }
+    } else if (part < 0 && !router && !def_get(d, n, "GF") && !def_get(d, n, "BITS") && def_get(d, n, "KD") && def_get(d, n, "TM") && def_get(d, n, "TOPK")) {
+        // kernels/moe_prefill.metal: E, TOPK, KD, I, TM (bench/moe_prefill.c:86-87)
+        p = (qw_kparams){0};
+        if (!def_int(d, n, "E", &p.E) || !def_int(d, n, "TOPK", &p.topk) || !def_int(d, n, "KD", &p.K) || !def_int(d, n, "I", &p.I) || !def_int(d, n, "TM", &p.tm))
+            FAIL("moe_prefill: E, TOPK, KD, I and TM must be integer macros");
+        if (p.E < 1 || p.E > 1024 || p.topk < 1 || p.topk > 16) FAIL("moe_prefill: E %d / TOPK %d outside this build (E <= 1024, TOPK <= 16)", p.E, p.topk);
+        if (p.K < 8 || p.K % 8 || p.I < 1 || p.tm < 1) FAIL("moe_prefill: KD %d / I %d / TM %d outside this build (KD a multiple of 8)", p.K, p.I, p.tm);
+        if (!reg_kernel(g, d, n, "moe_count", FAM_PK_COUNT, &p, err, errlen) || !reg_kernel(g, d, n, "moe_plan", FAM_PK_PLAN, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "moe_plan_t", FAM_PK_PLAN_T, &p, err, errlen) || !reg_kernel(g, d, n, "moe_scatter", FAM_PK_SCATTER, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "moe_act", FAM_PK_ACT, &p, err, errlen) || !reg_kernel(g, d, n, "p_act2", FAM_PK_ACT2, &p, err, errlen) || !reg_kernel(g, d, n, "moe_combine", FAM_PK_COMBINE, &p, err, errlen)) { ok = false; goto out; }
     }
     if (def_get(d, n, "QW_HIP_MEM")) { // this backend's own measurement helpers
         p = (qw_kparams){0};
@@ -937,6 +958,74 @@ static bool tr_cmb(qw_batch *b) {
     return add_launch(b, "qwk_cmb", cdiv(nbr * (unsigned)p->D, 256), 256, &a, sizeof a);
 }
 
+// ---------------------------------------------------------------- ragged packing (kernels/moe_prefill.metal; src/engine.c:4133-4224)
+static bool tr_pk_count(qw_batch *b) { // 0 ids, 1 counts, 2 P
+    qwk_count_args a = {.E = (uint32_t)b->k->p.E};
+    if (!bind_bytes(b, 2, &a.P, 4, "P") || !bind_ptr(b, 0, (size_t)a.P * 4, false, "ids", (void **)&a.ids) || !bind_ptr(b, 1, (size_t)a.E * 4, true, "counts", (void **)&a.counts)) return false;
+    return add_launch(b, "qwk_moe_count", cdiv(a.P, 256), 256, &a, sizeof a);
+}
+static bool tr_pk_plan(qw_batch *b, bool tm_bound) { // 0 counts, 1 offs, 2 cursor, 3 tiles, 4 max_tiles (, 5 tm)
+    const qw_kparams *p = &b->k->p;
+    qwk_plan_args a = {.E = (uint32_t)p->E, .tm = (uint32_t)p->tm};
+    if (!bind_bytes(b, 4, &a.max_tiles, 4, "max_tiles") || (tm_bound && !bind_bytes(b, 5, &a.tm, 4, "tm"))) return false;
+    if (a.tm < 1) return fail(b, "%s: tm 0", b->k->name);
+    if (!bind_ptr(b, 0, (size_t)a.E * 4, false, "counts", (void **)&a.counts) || !bind_ptr(b, 1, (size_t)a.E * 4, true, "offs", (void **)&a.offs) ||
+        !bind_ptr(b, 2, (size_t)a.E * 4, true, "cursor", (void **)&a.cursor) || !bind_ptr(b, 3, (size_t)a.max_tiles * 16, true, "tiles", (void **)&a.tiles)) return false;
+    if (b->buf[3].off % 16) return fail(b, "%s: tile table offset %zu is not 16-byte aligned", b->k->name, b->buf[3].off);
+    return add_launch(b, "qwk_moe_plan", 1, 1024, &a, sizeof a);
+}
+static bool tr_pk_scatter(qw_batch *b, unsigned gx) { // 0 X, 1 ids, 2 cursor, 3 Xs, 4 pos_of; grid x = P
+    const qw_kparams *p = &b->k->p;
+    qwk_scatter_args a = {.KD = (uint32_t)p->K, .topk = (uint32_t)p->topk, .E = (uint32_t)p->E, .P = gx};
+    if (gx % (unsigned)p->topk) return fail(b, "moe_scatter: %u pairs is not a multiple of TOPK %d", gx, p->topk);
+    if (!bind_ptr(b, 0, (size_t)(gx / p->topk) * p->K * 2, false, "X", (void **)&a.X) || !bind_ptr(b, 1, (size_t)gx * 4, false, "ids", (void **)&a.ids) ||
+        !bind_ptr(b, 2, (size_t)p->E * 4, true, "cursor", (void **)&a.cursor) || !bind_ptr(b, 3, (size_t)gx * p->K * 2, true, "Xs", (void **)&a.Xs) ||
+        !bind_ptr(b, 4, (size_t)gx * 4, true, "pos_of", (void **)&a.pos_of)) return false;
+    if (b->buf[0].off % 16 || b->buf[3].off % 16) return fail(b, "moe_scatter: row buffers must be 16-byte aligned");
+    return add_launch(b, "qwk_moe_scatter", gx, 256, &a, sizeof a);
+}
+static bool tr_pk_act(qw_batch *b) { // 0 G [P][2 I], 1 H [P][I], 2 P
+    const qw_kparams *p = &b->k->p;
+    qwk_act_args a = {.I = (uint32_t)p->I};
+    if (!bind_bytes(b, 2, &a.P, 4, "P")) return false;
+    a.n = a.P * a.I;
+    if (!bind_ptr(b, 0, (size_t)a.n * 4, false, "G", (void **)&a.G) || !bind_ptr(b, 1, (size_t)a.n * 2, true, "H", (void **)&a.H)) return false;
+    return add_launch(b, "qwk_moe_act", cdiv(a.n, 256), 256, &a, sizeof a);
+}
+static bool tr_pk_act2(qw_batch *b) { // kernels/prefill.metal:485-488: 0 G, 1 U, 2 H, 3 n
+    qwk_act_args a = {0};
+    if (!bind_bytes(b, 3, &a.n, 4, "n")) return false;
+    if (!bind_ptr(b, 0, (size_t)a.n * 2, false, "G", (void **)&a.G) || !bind_ptr(b, 1, (size_t)a.n * 2, false, "U", (void **)&a.U) || !bind_ptr(b, 2, (size_t)a.n * 2, true, "H", (void **)&a.H)) return false;
+    return add_launch(b, "qwk_moe_act", cdiv(a.n, 256), 256, &a, sizeof a);
+}
+static bool tr_pk_combine(qw_batch *b, unsigned gy) { // 0 D, 1 pos_of, 2 w, 3 Y; grid = (KD / 4 / 64, T)
+    const qw_kparams *p = &b->k->p;
+    qwk_combine_args a = {.KD = (uint32_t)p->K, .topk = (uint32_t)p->topk, .T = gy, .P = gy * (uint32_t)p->topk};
+    if (!bind_ptr(b, 0, (size_t)a.P * p->K * 2, false, "D", (void **)&a.Dm) || !bind_ptr(b, 1, (size_t)a.P * 4, false, "pos_of", (void **)&a.pos_of) ||
+        !bind_ptr(b, 2, (size_t)a.P * 4, false, "w", (void **)&a.w) || !bind_ptr(b, 3, (size_t)gy * p->K * 2, true, "Y", (void **)&a.Y)) return false;
+    if (!add_launch(b, "qwk_moe_combine", cdiv((unsigned)p->K / 4, 64), 64, &a, sizeof a)) return false;
+    if (gy) b->l[b->nl - 1].gy = gy;
+    return true;
+}
+// src/engine.c:3257-3264: 0 X, 1 W, 4 Y, 5 {M, N}, 6 tiles, 7 tables; grid y = entries of the tile table
+static bool tr_pf(qw_batch *b, unsigned gy) {
+    const qw_kparams *p = &b->k->p;
+    uint32_t mn[2];
+    if (!bind_bytes(b, 5, mn, sizeof mn, "{M, N}")) return false;
+    if (mn[1] == 0 || mn[1] % 16) return fail(b, "moe_pf_gg: N %u is not a multiple of 16", mn[1]);
+    if (gy > 2048) return fail(b, "moe_pf_gg: %u tile entries, this build takes at most 2048", gy);
+    const size_t rb = fmt_rb(p->F, p->K);
+    qwk_pf_args a = {.M = mn[0], .N = mn[1], .K = (uint32_t)p->K, .rowbytes = (uint32_t)rb, .max_tiles = gy, .tm = (uint32_t)p->tm, .glut = glut(b->g)};
+    if (!bind_ptr(b, 0, (size_t)a.M * p->K * 2, false, "X", (void **)&a.X) || !bind_ptr(b, 1, (size_t)p->E * a.N * rb, false, "weights", (void **)&a.W) ||
+        !bind_ptr(b, 4, (size_t)a.M * a.N * 2, true, "Y", (void **)&a.Y) || !bind_ptr(b, 6, (size_t)gy * 16, false, "tiles", (void **)&a.tiles)) return false;
+    if (b->buf[0].off % 16 || b->buf[6].off % 16) return fail(b, "moe_pf_gg: X and the tile table must be 16-byte aligned");
+    char fn[32];
+    if (p->F == 21) fname_fmt(fn, sizeof fn, "qwk_pf_f21_c%d", p->K % 512 == 0 ? 2 : 1);
+    else fname_fmt(fn, sizeof fn, "qwk_pf_f8_c4");
+    // every entry can hold a tile: the grid covers the whole table, the kernel counts the entries in use
+    return add_launch(b, intern(fn), persistent_grid(b->g, gy * (a.N / 16), 8), 512, &a, sizeof a);
+}
+
 // helpers: 0 src, 1 dst, 2 {n16 (uint64), seed (uint64)}; grid x = workgroups of 256 threads
 static bool tr_mem(qw_batch *b, unsigned gx) {
     uint64_t a2[2];
@@ -961,7 +1050,7 @@ static bool tr_fill_blocks(qw_batch *b) {
 }
 
 void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsigned tx, unsigned ty, unsigned tz) {
-    (void)gy; (void)gz; (void)tx; (void)ty; (void)tz;
+    (void)gz; (void)tx; (void)ty; (void)tz;
     if (b->failed) return;
     if (!b->k) { fail(b, "qw_batch_dispatch without a kernel"); return; }
     const int first = b->nl;
@@ -978,6 +1067,14 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     case FAM_DN: ok = tr_dn(b); break;
     case FAM_CMB: ok = tr_cmb(b); break;
     case FAM_FILL_BLOCKS: ok = tr_fill_blocks(b); break;
+    case FAM_PK_COUNT: ok = tr_pk_count(b); break;
+    case FAM_PK_PLAN: ok = tr_pk_plan(b, false); break;
+    case FAM_PK_PLAN_T: ok = tr_pk_plan(b, true); break;
+    case FAM_PK_SCATTER: ok = tr_pk_scatter(b, gx); break;
+    case FAM_PK_ACT: ok = tr_pk_act(b); break;
+    case FAM_PK_ACT2: ok = tr_pk_act2(b); break;
+    case FAM_PK_COMBINE: ok = tr_pk_combine(b, gy); break;
+    case FAM_PF: ok = tr_pf(b, gy); break;
     default: ok = tr_mem(b, gx);
     }
     if (ok && b->nl > first) b->l[b->nl - 1].last_of_dispatch = true;

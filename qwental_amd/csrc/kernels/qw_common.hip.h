@@ -347,6 +347,32 @@ template <int NB> struct qw_chunk<21, NB> {
             block_mfma(b, w, xh, xl, AF::has_lo, acc);
         }
     }
+    // NG groups of 16 activation rows against the same decoded weights (the grouped product over packed rows):
+    // rows[g] is the lane's row of group g in global memory; every group has its own accumulator.
+    template <int NG> __device__ __forceinline__ void mac_groups(const u2 *lut, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w[16];
+            lookups(b, lut, w);
+            const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
+            f4 sub[NG];
+#pragma unroll
+            for (int g = 0; g < NG; g++) sub[g] = f4{0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const h2 ff = j < 4 ? ff0 : ff1;
+                u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
+#pragma unroll
+                for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+                const h8 wv = __builtin_bit_cast(h8, raw);
+#pragma unroll
+                for (int g = 0; g < NG; g++) sub[g] = qw_mfma(*(const h8 *)(rows[g] + kb + 8 * j), wv, sub[g]);
+            }
+#pragma unroll
+            for (int g = 0; g < NG; g++) acc[g] += s[b].d * sub[g];
+        }
+    }
     // The same arithmetic with operand A gathered from global memory four steps at a time (qw_afrag_gather).
     __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
@@ -469,6 +495,19 @@ template <int NB> struct qw_chunk<8, NB> {
         if (NB & 1) d[NB - 1] = (uint16_t)qw_pull(d[NB - 1], src4);
     }
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    template <int NG> __device__ __forceinline__ void mac_groups(const u2 *, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const h8 w = qw_q8_cvt(q[b]);
+            const uint32_t kb = k0 + 32 * b + 8 * kg;
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                f4 sub = {0, 0, 0, 0};
+                sub = qw_mfma(*(const h8 *)(rows[g] + kb), w, sub);
+                acc[g] += qw_h2f(d[b]) * sub;
+            }
+        }
+    }
     // operand A gathered four blocks at a time (NB a multiple of 4)
     __device__ __forceinline__ void mac_gather(const u2 *, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
         if constexpr (NB % 4 != 0) { // block by block

@@ -124,6 +124,48 @@ typedef struct {
     uint32_t nblk, rowbytes, split, pad;
 } qwk_pack_args;
 
+/* Ragged packing of (token, expert) pairs and the grouped product over the packed rows (kernels/moe_prefill.metal,
+ * kernels/moe_gg.metal:761-838). P pairs, flat index p = token * topk + rank. */
+typedef struct {
+    const uint32_t *ids; /* [P] expert of pair p */
+    uint32_t *counts;    /* [E] */
+    uint32_t P, E;
+} qwk_count_args;
+typedef struct {
+    const uint32_t *counts;
+    uint32_t *offs, *cursor; /* [E] first packed row of each expert; cursor starts there */
+    uint32_t *tiles;         /* [max_tiles][4] = {expert, first row, end row, 0}; unused entries are zero */
+    uint32_t E, max_tiles, tm, pad;
+} qwk_plan_args;
+typedef struct {
+    const uint16_t *X; /* [T][KD] binary16 */
+    const uint32_t *ids;
+    uint32_t *cursor;
+    uint16_t *Xs;      /* [P][KD] rows in packed order */
+    uint32_t *pos_of;  /* [P] packed row of pair p */
+    uint32_t KD, topk, E, P;
+} qwk_scatter_args;
+typedef struct {
+    const uint16_t *G, *U; /* U == NULL: G is [P][2 I] (gate then up in each row); else G, U are [n] each */
+    uint16_t *H;
+    uint32_t P, I, n, pad;
+} qwk_act_args;
+typedef struct {
+    const uint16_t *Dm; /* [P][KD] binary16, packed order */
+    const uint32_t *pos_of;
+    const float *w;     /* [P] */
+    uint16_t *Y;        /* [T][KD] */
+    uint32_t KD, topk, T, P;
+} qwk_combine_args;
+typedef struct { /* Y[m][n] = X[m] . W[expert][n] for the rows m of every tile entry; binary16 in and out */
+    const uint16_t *X;
+    const uint8_t *W;     /* [E][N][rowbytes] */
+    uint16_t *Y;          /* [M][N] */
+    const uint32_t *tiles;
+    uint32_t M, N, K, rowbytes, max_tiles, tm, pad0, pad1;
+    const void *glut;
+} qwk_pf_args;
+
 typedef struct { /* synthetic weights: nblocks GGUF blocks of one type, scale d = binary16(|N(0, sigma)|), the rest uniform */
     uint8_t *dst;
     uint64_t nblocks, seed;

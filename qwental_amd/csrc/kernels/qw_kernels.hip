@@ -892,6 +892,158 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
 QW_DN_ANY(21, 0, qwk_dn_f21_any) QW_DN_ANY(21, 21, qwk_dn_f21_any_s21) QW_DN_ANY(21, 8, qwk_dn_f21_any_s8)
 QW_DN_ANY(8, 0, qwk_dn_f8_any) QW_DN_ANY(8, 21, qwk_dn_f8_any_s21) QW_DN_ANY(8, 8, qwk_dn_f8_any_s8)
 
+// ================================================================ ragged packing (kernels/moe_prefill.metal:15-119)
+// P (token, expert) pairs -> per-expert counts -> exclusive prefix sums (first packed row of every expert, tile table)
+// -> rows copied to packed order -> grouped product -> gathered, weighted sum. Integer work; bit-exact.
+extern "C" __global__ __launch_bounds__(256) void qwk_moe_count(qwk_count_args a) {
+    const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < a.P && a.ids[p] < a.E) atomicAdd(&a.counts[a.ids[p]], 1u);
+}
+// One workgroup of 1024 threads, thread e = expert e (E <= 1024): two exclusive scans (rows, tiles) by ballot-free
+// wave scans (DPP row shifts through __shfl_up) and one pass over the sixteen wave totals.
+extern "C" __global__ __launch_bounds__(1024) void qwk_moe_plan(qwk_plan_args a) {
+    __shared__ uint32_t wr[16], wt[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t c = tid < a.E ? a.counts[tid] : 0, nt = (c + a.tm - 1) / a.tm;
+    uint32_t pr = c, pt = nt; // inclusive scans inside the wave
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t ur = __shfl_up(pr, o), ut = __shfl_up(pt, o);
+        if (lane >= (uint32_t)o) pr += ur, pt += ut;
+    }
+    if (lane == 63) wr[wave] = pr, wt[wave] = pt;
+    __syncthreads();
+    uint32_t br = 0, bt = 0, total_t = 0;
+    for (uint32_t w = 0; w < 16; w++) {
+        if (w < wave) br += wr[w], bt += wt[w];
+        total_t += wt[w];
+    }
+    const uint32_t row0 = br + pr - c, tile0 = bt + pt - nt;
+    if (tid < a.E) {
+        a.offs[tid] = row0;
+        a.cursor[tid] = row0;
+        for (uint32_t t = 0; t < nt; t++) {
+            const uint32_t r = row0 + t * a.tm;
+            if (tile0 + t < a.max_tiles) *(u4 *)(a.tiles + 4 * (tile0 + t)) = u4{tid, r, r + a.tm < row0 + c ? r + a.tm : row0 + c, 0};
+        }
+    }
+    for (uint32_t t = total_t + tid; t < a.max_tiles; t += blockDim.x) *(u4 *)(a.tiles + 4 * t) = u4{0, 0, 0, 0}; // unused entries
+}
+// One workgroup per pair: take the next row of the pair's expert, remember it, copy the token's row there.
+extern "C" __global__ __launch_bounds__(256) void qwk_moe_scatter(qwk_scatter_args a) {
+    __shared__ uint32_t pos;
+    const uint32_t p = blockIdx.x;
+    if (threadIdx.x == 0) {
+        const uint32_t e = a.ids[p];
+        pos = e < a.E ? atomicAdd(&a.cursor[e], 1u) : 0xffffffffu;
+        a.pos_of[p] = pos;
+    }
+    __syncthreads();
+    if (pos >= a.P) return; // an expert id outside the table: the pair is dropped
+    const u4 *src = (const u4 *)(a.X + (size_t)(p / a.topk) * a.KD);
+    u4 *dst = (u4 *)(a.Xs + (size_t)pos * a.KD);
+    for (uint32_t i = threadIdx.x; i < a.KD / 8; i += blockDim.x) dst[i] = src[i];
+}
+// H = SiLU(gate) * up, binary16 in and out, the product rounded once (kernels/moe_prefill.metal:95-103, kernels/prefill.metal:485-488)
+extern "C" __global__ __launch_bounds__(256) void qwk_moe_act(qwk_act_args a) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n) return;
+    float g, u;
+    if (a.U) g = qw_h2f(a.G[i]), u = qw_h2f(a.U[i]);
+    else {
+        const uint32_t r = i / a.I, j = i % a.I;
+        g = qw_h2f(a.G[(size_t)r * 2 * a.I + j]), u = qw_h2f(a.G[(size_t)r * 2 * a.I + a.I + j]);
+    }
+    a.H[i] = qw_f2h(g / (1.0f + __expf(-g)) * u);
+}
+// y[t][c] = sum_s w[t][s] * D[pos_of[t][s]][c] in rank order; one thread per (token, 4 columns).
+extern "C" __global__ __launch_bounds__(64) void qwk_moe_combine(qwk_combine_args a) {
+    const uint32_t c4 = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (c4 >= a.KD / 4 || t >= a.T) return;
+    float acc[4] = {0, 0, 0, 0};
+    for (uint32_t s = 0; s < a.topk; s++) {
+        const uint32_t p = t * a.topk + s, pos = a.pos_of[p];
+        if (pos >= a.P) continue;
+        const u2 v = *(const u2 *)(a.Dm + (size_t)pos * a.KD + 4 * c4);
+        const float w = a.w[p];
+        acc[0] += w * qw_h2f((uint16_t)v.x), acc[1] += w * qw_h2f((uint16_t)(v.x >> 16));
+        acc[2] += w * qw_h2f((uint16_t)v.y), acc[3] += w * qw_h2f((uint16_t)(v.y >> 16));
+    }
+    u2 o;
+    o.x = (uint32_t)qw_f2h(acc[0]) | (uint32_t)qw_f2h(acc[1]) << 16;
+    o.y = (uint32_t)qw_f2h(acc[2]) | (uint32_t)qw_f2h(acc[3]) << 16;
+    *(u2 *)(a.Y + (size_t)t * a.KD + 4 * c4) = o;
+}
+
+// Grouped product over the packed rows (kernels/moe_gg.metal:761-838): task = (tile entry, 16 weight rows); the
+// weights of a task are decoded once and multiplied into up to four groups of 16 packed rows of the entry
+// (tm <= 64). The non-empty entries are the first ones of the table; their number is counted here.
+template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_args &a, u2 *lut, u4 *tl /* max_tiles entries */, uint32_t *cnt) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
+    if (threadIdx.x == 0) *cnt = 0;
+    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
+    __syncthreads();
+    uint32_t mine = 0;
+    for (uint32_t t = threadIdx.x; t < a.max_tiles; t += blockDim.x) {
+        const u4 e = *(const u4 *)(a.tiles + 4 * t);
+        tl[t] = e;
+        mine += e.z > e.y;
+    }
+    if (mine) atomicAdd(cnt, mine);
+    __syncthreads();
+    const uint32_t used = *cnt, ntn = a.N / 16, ntasks = used * ntn, cpr = a.K / (C::BLK_K * CH);
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    f4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, lane & 3,
+        [&](uint32_t task) {
+            const u4 e = tl[task / ntn];
+            return a.W + ((size_t)e.x * a.N + 16 * (task % ntn) + (lane >> 2)) * a.rowbytes;
+        },
+        [&](uint32_t task, uint32_t ci, const C &c) {
+            const u4 e = tl[task / ntn];
+            const uint32_t m0 = e.y, m1 = e.z, ng = (m1 - m0 + 15) / 16;
+            const uint16_t *rows[4];
+#pragma unroll
+            for (uint32_t g = 0; g < 4; g++) {
+                const uint32_t m = m0 + 16 * g + n;
+                rows[g] = a.X + (size_t)(m < m1 ? m : m1 - 1) * a.K; // rows past the entry repeat its last row; never stored
+            }
+            const uint32_t k0 = ci * CH * C::BLK_K;
+            if (ng <= 1) {
+                const uint16_t *const r1[1] = {rows[0]};
+                f4 a1[1] = {acc[0]};
+                c.template mac_groups<1>(lut, r1, k0, kg, a1);
+                acc[0] = a1[0];
+            } else if (ng == 2) {
+                const uint16_t *const r2[2] = {rows[0], rows[1]};
+                f4 a2[2] = {acc[0], acc[1]};
+                c.template mac_groups<2>(lut, r2, k0, kg, a2);
+                acc[0] = a2[0], acc[1] = a2[1];
+            } else {
+                const uint16_t *const r4[4] = {rows[0], rows[1], rows[2], rows[3]};
+                c.template mac_groups<4>(lut, r4, k0, kg, acc);
+            }
+            if (ci + 1 != cpr) return;
+            const uint32_t col = 16 * (task % ntn) + n;
+#pragma unroll
+            for (uint32_t g = 0; g < 4; g++) {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; j++) {
+                    const uint32_t m = m0 + 16 * g + 4 * kg + j;
+                    if (m < m1) a.Y[(size_t)m * a.N + col] = qw_f2h(acc[g][j]);
+                }
+                acc[g] = f4{0, 0, 0, 0};
+            }
+        });
+}
+#define QW_PF(F, CH, NAME)                                                                       \
+    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pf_args a) {                    \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 tl[2048]; uint32_t cnt; } L; \
+        pf_body<F, CH>(a, L.lut, L.tl, &L.cnt);                                                  \
+    }
+QW_PF(21, 2, qwk_pf_f21_c2) QW_PF(21, 1, qwk_pf_f21_c1) QW_PF(8, 4, qwk_pf_f8_c4)
+
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).
 extern "C" __global__ __launch_bounds__(256) void qwk_cmb(qwk_cmb_args a) {

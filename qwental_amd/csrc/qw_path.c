@@ -12,6 +12,10 @@ struct qw_path {
     int D, I, E, topk, nbmax;
     qw_buf tab, H, psh, pd, cnt;
     bool tab_ready;
+    // packing scratch (qw_path_pf_reserve)
+    qw_buf pcnt, poffs, pcur, ptiles, ppos, pXs, pGg, pGu, pH, pDm;
+    int pf_tmax, pf_tm;
+    unsigned pf_max_tiles;
 };
 
 static int blk_values(int type) { return type == 8 ? 32 : type == 21 ? 256 : 0; }
@@ -43,6 +47,8 @@ qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool 
 void qw_path_close(qw_path *p) {
     if (!p) return;
     qw_buf_free(&p->tab); qw_buf_free(&p->H); qw_buf_free(&p->psh); qw_buf_free(&p->pd); qw_buf_free(&p->cnt);
+    qw_buf *pf[] = {&p->pcnt, &p->poffs, &p->pcur, &p->ptiles, &p->ppos, &p->pXs, &p->pGg, &p->pGu, &p->pH, &p->pDm};
+    for (size_t i = 0; i < sizeof pf / sizeof *pf; i++) qw_buf_free(pf[i]);
     free(p);
 }
 
@@ -220,5 +226,109 @@ bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nl
                           const qw_buf *sel, const qw_buf *out) {
     for (int l = 0; l < nlayers; l++)
         if (!qw_path_gg_moe(p, b, &M[l], nb, x, &lg[l], &sel[l], out)) return false;
+    return true;
+}
+
+// ---------------------------------------------------------------- ragged batch through the packing path (src/engine.c:4133-4254)
+bool qw_path_pf_reserve(qw_path *p, int tmax, int tm) {
+    if (tmax < 1 || (tm != 16 && tm != 32 && tm != 64)) return false;
+    if (p->pf_tmax >= tmax && p->pf_tm == tm) return true;
+    qw_buf *pf[] = {&p->pcnt, &p->poffs, &p->pcur, &p->ptiles, &p->ppos, &p->pXs, &p->pGg, &p->pGu, &p->pH, &p->pDm};
+    for (size_t i = 0; i < sizeof pf / sizeof *pf; i++) qw_buf_free(pf[i]);
+    const size_t P = (size_t)tmax * (size_t)p->topk, E = (size_t)p->E;
+    p->pf_max_tiles = (unsigned)((P + (size_t)tm - 1) / (size_t)tm + E); // src/engine.c:4135
+    p->pf_tmax = 0;
+    if (!qw_buf_new(p->g, E * 4, &p->pcnt) || !qw_buf_new(p->g, E * 4, &p->poffs) || !qw_buf_new(p->g, E * 4, &p->pcur) ||
+        !qw_buf_new(p->g, (size_t)p->pf_max_tiles * 16, &p->ptiles) || !qw_buf_new(p->g, P * 4, &p->ppos) || !qw_buf_new(p->g, P * (size_t)p->D * 2, &p->pXs) ||
+        !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pGg) || !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pGu) || !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pH) ||
+        !qw_buf_new(p->g, P * (size_t)p->D * 2, &p->pDm)) return false;
+    p->pf_tmax = tmax;
+    p->pf_tm = tm;
+    return true;
+}
+unsigned qw_path_pf_max_tiles(const qw_path *p) { return p->pf_max_tiles; }
+const qw_buf *qw_path_pf_scratch(const qw_path *p, int which) {
+    const qw_buf *pf[] = {&p->pcnt, &p->poffs, &p->ptiles, &p->ppos, &p->pXs, &p->pH, &p->pDm};
+    return which >= 0 && which < 7 ? pf[which] : NULL;
+}
+
+static qw_kernel *pk_kernel(qw_path *p, const char *base) { // bench/moe_prefill.c:84-88
+    char name[96], defs[512];
+    snprintf(name, sizeof name, "%s_e%dk%dd%di%dt%d", base, p->E, p->topk, p->D, p->I, p->pf_tm);
+    qw_kernel *k = qw_kernel_get(p->g, name);
+    if (k) return k;
+    snprintf(defs, sizeof defs, "#define %s %s\n#define E %d\n#define TOPK %d\n#define KD %d\n#define I %d\n#define TM %d\n", base, name, p->E, p->topk, p->D, p->I, p->pf_tm);
+    return compile_get(p, name, defs);
+}
+// src/engine.c:3231-3266: Y [P][N] = X [P][K] . W_e^T over the tile table
+static bool pf_qmm_moe_iq(qw_path *p, qw_batch *b, const qw_tensor *W, int N, int K, const qw_buf *X, const qw_buf *Y, uint32_t P) {
+    char name[96], defs[1024];
+    snprintf(name, sizeof name, "moe_pf_gg_%d_k%d_tm%d_e%d", W->type, K, p->pf_tm, p->E);
+    qw_kernel *k = qw_kernel_get(p->g, name);
+    if (!k) {
+        snprintf(defs, sizeof defs, "#define IQ_DQ_ONLY\n#define E %d\n#define TOPK %d\n#define D %d\n#define I %d\n#define NB 1\n#define GG_PART 5\n"
+                 "#define PFF %d\n#define KD %d\n#define TM %d\n#define TN 64\n#define SG 4\n#define KC 64\n#define PFS 1\n#define PFT 1\n#define PFDBG 0\n#define moe_pf_gg %s\n",
+                 p->E, p->topk, p->D, p->I, W->type, K, p->pf_tm, name);
+        if (!(k = compile_get(p, name, defs))) return false;
+    }
+    const uint32_t a[2] = {P, (uint32_t)N};
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, X, 0);
+    qw_batch_buf(b, 1, W->buf, W->offset);
+    qw_batch_buf(b, 4, Y, 0);
+    qw_batch_bytes(b, 5, a, sizeof a);
+    qw_batch_buf(b, 6, &p->ptiles, 0);
+    qw_batch_buf(b, 7, &p->tab, 0);
+    qw_batch_dispatch(b, (unsigned)N / 64, p->pf_max_tiles, 1, 128, 1, 1);
+    return true;
+}
+
+bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const qw_buf *x, const qw_buf *ids, const qw_buf *w, const qw_buf *out) {
+    if (T < 1 || T > p->pf_tmax) {
+        fprintf(stderr, "qw_path_pf_moe: %d rows, reserved %d\n", T, p->pf_tmax);
+        return false;
+    }
+    const uint32_t P = (uint32_t)T * (uint32_t)p->topk, tm = (uint32_t)p->pf_tm, n = P * (uint32_t)p->I;
+    qw_kernel *k;
+    memset(p->pcnt.ptr, 0, p->pcnt.size); // the engine clears the counters on the GPU (p_zero); here the host shadow is copied at submit
+    if (!(k = pk_kernel(p, "moe_count"))) return false;
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, ids, 0);
+    qw_batch_buf(b, 1, &p->pcnt, 0);
+    qw_batch_bytes(b, 2, &P, 4);
+    qw_batch_dispatch(b, (P + 255) / 256, 1, 1, 256, 1, 1);
+    if (!(k = pk_kernel(p, "moe_plan_t"))) return false; // src/engine.c:4137-4144
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, &p->pcnt, 0);
+    qw_batch_buf(b, 1, &p->poffs, 0);
+    qw_batch_buf(b, 2, &p->pcur, 0);
+    qw_batch_buf(b, 3, &p->ptiles, 0);
+    qw_batch_bytes(b, 4, &p->pf_max_tiles, 4);
+    qw_batch_bytes(b, 5, &tm, 4);
+    qw_batch_dispatch(b, 1, 1, 1, (unsigned)p->E, 1, 1);
+    if (!(k = pk_kernel(p, "moe_scatter"))) return false; // src/engine.c:4221-4227
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, x, 0);
+    qw_batch_buf(b, 1, ids, 0);
+    qw_batch_buf(b, 2, &p->pcur, 0);
+    qw_batch_buf(b, 3, &p->pXs, 0);
+    qw_batch_buf(b, 4, &p->ppos, 0);
+    qw_batch_dispatch(b, P, 1, 1, 256, 1, 1);
+    if (!pf_qmm_moe_iq(p, b, &M->gate, p->I, p->D, &p->pXs, &p->pGg, P) || !pf_qmm_moe_iq(p, b, &M->up, p->I, p->D, &p->pXs, &p->pGu, P)) return false;
+    if (!(k = pk_kernel(p, "p_act2"))) return false; // src/engine.c:4246-4251
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, &p->pGg, 0);
+    qw_batch_buf(b, 1, &p->pGu, 0);
+    qw_batch_buf(b, 2, &p->pH, 0);
+    qw_batch_bytes(b, 3, &n, 4);
+    qw_batch_dispatch(b, (n + 255) / 256, 1, 1, 256, 1, 1);
+    if (!pf_qmm_moe_iq(p, b, &M->down, p->D, p->I, &p->pH, &p->pDm, P)) return false;
+    if (!(k = pk_kernel(p, "moe_combine"))) return false; // kernels/moe_prefill.metal:105-119
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, &p->pDm, 0);
+    qw_batch_buf(b, 1, &p->ppos, 0);
+    qw_batch_buf(b, 2, w, 0);
+    qw_batch_buf(b, 3, out, 0);
+    qw_batch_dispatch(b, (unsigned)p->D / 4 / 64, (unsigned)T, 1, 64, 1, 1);
     return true;
 }

@@ -61,6 +61,8 @@ SYMBOLS = [
     ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_scratch", _pb, [_vp, _i]),
+    ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
+    ("qw_path_pf_scratch", _pb, [_vp, _i]), ("qw_path_pf_max_tiles", C.c_uint, [_vp]),
 ]
 
 
@@ -286,6 +288,26 @@ class Path:
         """layers_c: ctypes array of QwMoeLayer; lg_c / sel_c: ctypes arrays of QwBuf, one per layer."""
         if not self.L.qw_path_gg_moe_stack(self.p, batch.b, layers_c, nlayers, nb, x.ref(), lg_c, sel_c, out.ref()):
             raise RuntimeError("qw_path_gg_moe_stack failed")
+
+    def pf_reserve(self, tmax, tm):
+        if not self.L.qw_path_pf_reserve(self.p, tmax, tm):
+            raise RuntimeError("qw_path_pf_reserve failed: " + self.gpu.last_error())
+
+    def pf_moe(self, batch, layer, T, x, ids, w, out):
+        """Ragged batch through the packing path: ids / w are [T * topk] uint32 / float32 buffers."""
+        if not self.L.qw_path_pf_moe(self.p, batch.b, C.byref(layer.c), T, x.ref(), ids.ref(), w.ref(), out.ref()):
+            raise RuntimeError("qw_path_pf_moe failed")
+
+    def pf_scratch(self, which, dtype=np.uint8):
+        """0 counts, 1 offsets, 2 tile table, 3 pos_of, 4 packed x, 5 H, 6 packed down output (device bytes)."""
+        pb = self.L.qw_path_pf_scratch(self.p, which)
+        out = np.empty(pb.contents.size, np.uint8)
+        if not self.L.qw_hip_buf_read(pb, 0, out.ctypes.data, out.nbytes):
+            raise RuntimeError("qw_hip_buf_read failed")
+        return out.view(dtype)
+
+    def pf_max_tiles(self):
+        return int(self.L.qw_path_pf_max_tiles(self.p))
 
     def scratch(self, which):
         """0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg; returns (device bytes as uint8)."""

@@ -1,0 +1,91 @@
+"""Ragged batches through the packing path (count -> plan -> scatter -> grouped product -> combine): integer stages
+bit-exact against the oracle, outputs against a float64 recompute."""
+import numpy as np
+import pytest
+
+import qwental_amd as q
+from helpers import DeviceLayer, maxrel
+from qwental_amd import synth
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+
+
+def expert_ref(o, m, e, x):
+    """float64 down(SiLU(gate x) * up x) of expert e for one row x (float16)."""
+    D, I = m["D"], m["I"]
+    rg, rd = synth.row_bytes(m["fgu"], D), synth.row_bytes(m["fd"], I)
+    Wg = m["Wg"].reshape(m["E"], I * rg)[e]
+    Wu = m["Wu"].reshape(m["E"], I * rg)[e]
+    Wd = m["Wd"].reshape(m["E"], D * rd)[e]
+    g = o.qmv(m["fgu"], Wg, I, D, x[None, :], f64=True)[0]
+    u = o.qmv(m["fgu"], Wu, I, D, x[None, :], f64=True)[0]
+    h = (g / (1.0 + np.exp(-g)) * u)
+    return h, Wd
+
+
+def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed):
+    rng = np.random.default_rng(seed)
+    m = synth.moe_layer(rng, D, I, E, fgu=fmt, fd=fmt, fsh=fmt)
+    x = synth.activations(rng, T, D)
+    w = rng.uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    w /= w.sum(axis=1, keepdims=True)
+    path = q.Path(gpu, D, I, E, K, 16)
+    path.pf_reserve(T, tm)
+    dl = DeviceLayer(gpu, m)
+    xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.ravel()), gpu.buf(T * D * 2)
+    b = gpu.batch()
+    path.pf_moe(b, dl.layer, T, xb, ib, wb, ob)
+    assert b.end() >= 0, gpu.last_error()
+    P = T * K
+    # integer stages against the oracle (kernels/moe_prefill.metal:15-93)
+    mt = path.pf_max_tiles()
+    counts, offs, pos_ref, tiles, nt = oracle.moe_pack(ids.ravel(), E, tm, mt)
+    assert np.array_equal(path.pf_scratch(0, np.uint32)[:E], counts)
+    assert np.array_equal(path.pf_scratch(1, np.uint32)[:E], offs)
+    assert np.array_equal(path.pf_scratch(2, np.uint32)[:4 * mt].reshape(mt, 4), tiles.reshape(mt, 4))
+    pos = path.pf_scratch(3, np.uint32)[:P]
+    assert sorted(pos.tolist()) == list(range(P))  # a permutation of the packed rows
+    flat = ids.ravel()
+    assert all(offs[flat[p]] <= pos[p] < offs[flat[p]] + counts[flat[p]] for p in range(P))  # inside the pair's expert range
+    Xs = path.pf_scratch(4, np.float16)[:P * D].reshape(P, D)
+    assert all(np.array_equal(Xs[pos[p]].view(np.uint16), x[p // K].view(np.uint16)) for p in range(P))  # scatter copied the right rows
+    # outputs: float64 recompute with the reference's binary16 roundings of H and of the down output (kernels/prefill.metal:485-499)
+    out = ob.view(np.float16)[:T * D].reshape(T, D).astype(np.float64)
+    ref = np.zeros((T, D))
+    for t in range(T):
+        for s in range(K):
+            h, Wd = expert_ref(oracle, m, int(ids[t, s]), x[t])
+            d = oracle.qmv(m["fd"], Wd, D, I, h.astype(np.float16)[None, :], f64=True)[0]
+            ref[t] += w[t, s] * d
+    assert maxrel(out, ref) <= TOL, maxrel(out, ref)
+    for bb in (xb, ib, wb, ob):
+        bb.free()
+    dl.free()
+    path.close()
+
+
+@pytest.mark.parametrize("fmt,tm", [(21, 16), (21, 64), (8, 32)])
+def test_packing_uniform_routing(gpu, oracle, fmt, tm):
+    T, E, K, D, I = 24, 32, 4, 512, 512
+    rng = np.random.default_rng(7 + tm)
+    ids = np.stack([rng.choice(E, K, replace=False) for _ in range(T)])
+    run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, 70 + tm)
+
+
+def test_packing_zipf_hot_experts(gpu, oracle):
+    """Continuous-batching shape in small: 16 slots with 1..16 rows each (64 rows here), Zipf(1.1) routing: a few
+    experts collect far more than one tile of rows, most none."""
+    T, E, K, D, I = 64, 64, 4, 512, 256
+    rng = np.random.default_rng(4)
+    ids = synth.zipf_ids(rng, T, E, K)
+    counts = np.bincount(ids.ravel(), minlength=E)
+    assert counts.max() > 16 and (counts == 0).sum() > 0
+    run_case(gpu, oracle, T, ids, E, K, D, I, 21, 16, 44)
+
+
+def test_packing_all_pairs_one_expert(gpu, oracle):
+    """Every token's first pick is expert 3: its rows span several tile entries; the other picks are distinct."""
+    T, E, K, D, I = 40, 16, 2, 256, 256
+    ids = np.stack([np.array([3, (5 + t) % E if (5 + t) % E != 3 else 4]) for t in range(T)])
+    run_case(gpu, oracle, T, ids, E, K, D, I, 21, 32, 9)
