@@ -56,6 +56,10 @@ bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
 /* The whole layer: x [nb][D] binary16 -> out [nb][D] binary16; lg and sel receive the logits and the selection. */
 bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
                     const qw_buf *out);
+/* The same with the router's logits given by the caller in lg (the reference's RBF = 0 build of moe_pre_gg plus a
+ * moe_sel_gg dispatch): for forced routing. */
+bool qw_path_gg_moe_lg(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
+                       const qw_buf *out);
 /* nlayers layers in a row on the same input x (the FFN stack of the benchmark): layer l writes lg[l], sel[l] and,
  * each in turn, out. Equivalent to nlayers calls of qw_path_gg_moe. */
 bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,

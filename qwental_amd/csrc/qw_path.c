@@ -15,6 +15,7 @@ struct qw_path {
     // packing scratch (qw_path_pf_reserve)
     qw_buf pcnt, poffs, pcur, ptiles, ppos, pXs, pGg, pGu, pH, pDm;
     int pf_tmax, pf_tm;
+    int rbf; // 1: moe_pre_gg computes the router (src/engine.c:577); 0: the logits are given
     unsigned pf_max_tiles;
 };
 
@@ -96,7 +97,7 @@ static qw_kernel *gg_kernel(qw_path *p, const char *base, const qw_moe_layer *M,
     char name[128], sfx[96], defs[2048];
     switch (part) {
     case 0: snprintf(sfx, sizeof sfx, "_n%d", nbv); break;
-    case 1: snprintf(sfx, sizeof sfx, "_%d_%d_r%d_w%d_n%d", M->sh_gate.type, M->sh_up.type, 1, rwf, nbv); break;
+    case 1: snprintf(sfx, sizeof sfx, "_%d_%d_r%d_w%d_n%d", M->sh_gate.type, M->sh_up.type, p->rbf, rwf, nbv); break;
     case 2: snprintf(sfx, sizeof sfx, "_%d_%d_g%d_n%d", M->gate.type, M->sh_down.type, 1, nbv); break;
     case 3: snprintf(sfx, sizeof sfx, "_%d_s%d_n%d", M->down.type, 4, nbv); break;
     default: snprintf(sfx, sizeof sfx, "_w%d_n%d", rwf, nbv);
@@ -116,7 +117,7 @@ static qw_kernel *gg_kernel(qw_path *p, const char *base, const qw_moe_layer *M,
     case 0: snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 0\n#define moe_sel_gg moe_sel_gg%s\n#define gg_tab_init gg_tab_init%s\n", sfx, sfx); break;
     case 1:
         snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 1\n#define FSG %d\n#define FSU %d\n#define RBF %d\n#define moe_pre_gg moe_pre_gg%s\n", M->sh_gate.type,
-                 M->sh_up.type, 1, sfx);
+                 M->sh_up.type, p->rbf, sfx);
         break;
     case 2:
         snprintf(defs + n, sizeof defs - (size_t)n, "#define GG_PART 2\n#define GSG %d\n#define RG %d\n#define FGU %d\n#define FSD %d\n#define moe_gu_gg moe_gu_gg%s\n", 8, 1,
@@ -149,8 +150,17 @@ bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
 }
 
 // src/engine.c:568-647: front part (router + shared gate/up + selection) -> routed gate/up + shared down -> routed down -> combine
+static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, bool given);
 bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
                     const qw_buf *out) {
+    return gg_moe(p, b, M, nb, x, lg, sel, out, false);
+}
+bool qw_path_gg_moe_lg(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
+                       const qw_buf *out) {
+    return gg_moe(p, b, M, nb, x, lg, sel, out, true);
+}
+static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, bool given) {
+    p->rbf = given ? 0 : 1;
     if (nb < 1 || nb > p->nbmax) {
         fprintf(stderr, "gg_moe: %d tokens, scratch was sized for %d\n", nb, p->nbmax);
         return false;
@@ -165,6 +175,14 @@ bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, cons
     }
     const uint32_t nbr = (uint32_t)nb;
     const unsigned E = (unsigned)p->E, I = (unsigned)p->I, D = (unsigned)p->D, K = (unsigned)p->topk;
+    if (given) { // the selection from the caller's logits (src/engine.c:609-614)
+        if (!(k = gg_kernel(p, "moe_sel_gg", M, nb))) return false;
+        qw_batch_kernel(b, k);
+        qw_batch_buf(b, 0, lg, 0);
+        qw_batch_buf(b, 1, sel, 0);
+        qw_batch_bytes(b, 2, &nbr, 4);
+        qw_batch_dispatch(b, 1, 1, 1, 1024, 1, 1);
+    }
     if (!(k = gg_kernel(p, "moe_pre_gg", M, nb))) return false;
     qw_batch_kernel(b, k);
     bind_t(b, 0, &M->router);

@@ -59,6 +59,7 @@ SYMBOLS = [
     ("qw_path_qmv_gg", _b, [_vp, _vp, _pt, _i, _i, _pb, _sz, _pb, _sz, _i, _b]),
     ("qw_path_gg_router", _b, [_vp, _vp, _pm, _i, _pb, _pb]),
     ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
+    ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_scratch", _pb, [_vp, _i]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
@@ -283,6 +284,11 @@ class Path:
     def gg_moe(self, batch, layer, nb, x, lg, sel, out):
         if not self.L.qw_path_gg_moe(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
             raise RuntimeError("qw_path_gg_moe failed")
+
+    def gg_moe_lg(self, batch, layer, nb, x, lg, sel, out):
+        """The layer with the caller's logits (forced routing)."""
+        if not self.L.qw_path_gg_moe_lg(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
+            raise RuntimeError("qw_path_gg_moe_lg failed")
 
     def gg_moe_stack(self, batch, layers_c, nlayers, nb, x, lg_c, sel_c, out):
         """layers_c: ctypes array of QwMoeLayer; lg_c / sel_c: ctypes arrays of QwBuf, one per layer."""

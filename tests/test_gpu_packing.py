@@ -89,3 +89,54 @@ def test_packing_all_pairs_one_expert(gpu, oracle):
     T, E, K, D, I = 40, 16, 2, 256, 256
     ids = np.stack([np.array([3, (5 + t) % E if (5 + t) % E != 3 else 4]) for t in range(T)])
     run_case(gpu, oracle, T, ids, E, K, D, I, 21, 32, 9)
+
+
+def test_ragged_step_decode_groups_equal_packing_path(gpu, oracle):
+    """A continuous-batching step in small (BASELINE configs[3] shape: 16 slots, n[i] ~ U{1..16} rows each, Zipf(1.1)
+    routing forced through the logits): the decode path in groups of at most 16 rows and the packing path in one pass
+    give the same routed sums. The shared expert's block scales are zero here, so that the decode path's output is
+    the routed part alone."""
+    E, K, D, I = 64, 4, 512, 512
+    rng = np.random.default_rng(21)
+    n = rng.integers(1, 17, 16)
+    T = int(n.sum())
+    m = synth.moe_layer(rng, D, I, E)
+    for key in ("Wsg", "Wsu", "Wsd"):
+        m[key].reshape(-1, 110)[:, :2] = 0  # d = 0: the shared expert contributes nothing
+    m["topk"] = K
+    x = synth.activations(rng, T, D)
+    ids = synth.zipf_ids(rng, T, E, K)
+    lg = synth.logits_for_ids(rng, ids, E)
+    path = q.Path(gpu, D, I, E, K, 16)
+    dl = DeviceLayer(gpu, m)
+    out_dec = np.zeros((T, D), np.float16)
+    wts = np.zeros((T, K), np.float32)
+    for g0 in range(0, T, 16):
+        nb = min(16, T - g0)
+        xb, lb = gpu.buf_from(x[g0:g0 + nb]), gpu.buf_from(lg[g0:g0 + nb])
+        sb, ob = gpu.buf(path.sel_bytes(nb)), gpu.buf(nb * D * 2)
+        b = gpu.batch()
+        path.gg_moe_lg(b, dl.layer, nb, xb, lb, sb, ob)
+        assert b.end() >= 0, gpu.last_error()
+        out_dec[g0:g0 + nb] = ob.view(np.float16)[:nb * D].reshape(nb, D)
+        gnb = 8 if nb <= 8 else 16
+        sel = oracle.Sel(sb.view(np.uint8).copy(), gnb, K)
+        ref = oracle.select(lg[g0:g0 + nb], K, gnb)
+        assert sel.U == ref.U and np.array_equal(sel.ue[:ref.U], ref.ue[:ref.U])
+        assert np.array_equal(oracle.topk_ids(lg[g0:g0 + nb], K), ids[g0:g0 + nb])  # the forced routing took
+        wts[g0:g0 + nb] = sel.w[:nb, :K]
+        for bb in (xb, lb, sb, ob):
+            bb.free()
+    path.pf_reserve(T, 16)
+    xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(wts.ravel()), gpu.buf(T * D * 2)
+    b = gpu.batch()
+    path.pf_moe(b, dl.layer, T, xb, ib, wb, ob)
+    assert b.end() >= 0, gpu.last_error()
+    out_pk = ob.view(np.float16)[:T * D].reshape(T, D)
+    counts = path.pf_scratch(0, np.uint32)[:E]
+    assert counts.sum() == T * K and counts.max() > 16  # a hot expert spans several tile entries
+    assert maxrel(out_pk, out_dec.astype(np.float64)) <= TOL
+    for bb in (xb, ib, wb, ob):
+        bb.free()
+    dl.free()
+    path.close()
