@@ -87,6 +87,55 @@ def cpu_baseline(stack, x, nb, lg_dev, budget_s=20.0):
             "sample": "oracle moe_layer_f32 on layers 0..%d of the stack (B = %d), %.1f s; scaled to %d layers" % (n - 1, nb, t_used, stack.L)}
 
 
+def ragged_steps(gpu, stack, reps=5):
+    """BASELINE.json configs[3]: a continuous-batching step of one layer (layer 0 of the stack): 16 slots with seeded
+    uniform row counts in 1..16 redrawn until the total is near the target, Zipf(1.1) routing forced through the
+    logits. Timed two ways on the same rows: the decode path in groups of at most 16 rows (one batch), and the packing
+    path (count -> prefix sums -> scatter -> grouped product -> combine) in one pass. Routed experts' bytes are read
+    once per group on the first way and once on the second; the table gives the crossover in rows per step."""
+    from qwental_amd import synth
+    from oracle import oracle as o
+    layer, path, E, K, D = stack.layers[0], stack.path, stack.E, stack.topk, stack.D
+    out = []
+    for target in (16, 32, 64, 128):
+        rng = np.random.default_rng(1000 + target)
+        while True:
+            n = rng.integers(1, 17, 16) if target >= 48 else rng.integers(1, max(2, target // 8 + 1), 16)
+            if abs(int(n.sum()) - target) <= max(2, target // 8):
+                break
+        T = int(n.sum())
+        x = synth.activations(rng, T, D)
+        ids = synth.zipf_ids(rng, T, E, K)
+        lg = synth.logits_for_ids(rng, ids, E)
+        groups = [(g0, min(16, T - g0)) for g0 in range(0, T, 16)]
+        bufs = [(gpu.buf_from(x[g0:g0 + nb]), gpu.buf_from(lg[g0:g0 + nb]), gpu.buf(path.sel_bytes(nb)), gpu.buf(nb * D * 2)) for g0, nb in groups]
+        t_dec = 1e9
+        for _ in range(reps):
+            b = gpu.batch()
+            for (g0, nb), (xb, lb, sb, ob) in zip(groups, bufs):
+                path.gg_moe_lg(b, layer, nb, xb, lb, sb, ob)
+            t_dec = min(t_dec, b.end())
+        w = np.concatenate([o.Sel(sb.view(np.uint8).copy(), 8 if nb <= 8 else 16, K).w[:nb, :K] for (g0, nb), (xb, lb, sb, ob) in zip(groups, bufs)])
+        path.pf_reserve(T, 16)
+        xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.astype(np.float32).ravel()), gpu.buf(T * D * 2)
+        t_pk = 1e9
+        for _ in range(reps):
+            b = gpu.batch()
+            path.pf_moe(b, layer, T, xb, ib, wb, ob)
+            t_pk = min(t_pk, b.end())
+        counts = np.bincount(ids.ravel(), minlength=E)
+        U = int((counts > 0).sum())
+        U_groups = sum(len(np.unique(ids[g0:g0 + nb])) for g0, nb in groups)
+        out.append({"rows": T, "slots": n.tolist(), "unique_experts": U, "unique_experts_summed_over_groups": U_groups, "max_rows_per_expert": int(counts.max()),
+                    "experts_by_rows": {"1": int((counts == 1).sum()), "2-4": int(((counts >= 2) & (counts <= 4)).sum()), "5-16": int(((counts >= 5) & (counts <= 16)).sum()),
+                                        ">16": int((counts > 16).sum())},
+                    "decode_groups_us": t_dec * 1e6, "packing_path_us": t_pk * 1e6,
+                    "decode_groups_GBps": (U_groups * stack.exp_bytes) / t_dec / 1e9, "packing_path_GBps": (U * stack.exp_bytes) / t_pk / 1e9})
+        for bb in [xb, ib, wb, ob] + [y for t4 in bufs for y in t4]:
+            bb.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,7 +144,7 @@ def main():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--nb", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--quick", action="store_true", help="B = 16 only (profiling runs)")
+    ap.add_argument("--quick", action="store_true", help="B = 16 only, no ragged-step table (profiling runs)")
     ap.add_argument("--copy-calib", action="store_true", help="also run the copy kernel over 1 GiB three times (scale for the memory counters)")
     ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
     a = ap.parse_args()
@@ -152,6 +201,8 @@ def main():
             "by_batch": {str(k): v for k, v in res.items()},
             "kernel_us_mean": {k: float(np.mean(v)) for k, v in per_kernel.items()},
             "setup_s": setup_s}
+    if not a.quick:
+        line["ragged_step"] = ragged_steps(gpu, stack)
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)
