@@ -136,6 +136,52 @@ def ragged_steps(gpu, stack, reps=5):
     return out
 
 
+def qmv_table(gpu, reps=5, nmat=64):
+    """BASELINE.json configs[0..1]: y = W x for a 4096 x 2048 matrix, IQ3_S and Q8_0, 1..16 activations. nmat matrices
+    at different addresses go into one batch so that no cache holds the weights (the method of bench/moe_bw.c:50-89);
+    the figure is GPU time per matrix. For IQ3_S and up to 4 activations the VALU GEMV form is timed beside the
+    matrix-core form."""
+    from qwental_amd import synth
+    from qwental_amd.stack import fill_blocks
+    import qwental_amd as q
+    N, K = 4096, 2048
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    rng = np.random.default_rng(1)
+    x = gpu.buf_from(synth.activations(rng, 16, K), device_only=True)
+    y = gpu.buf(16 * N * 4, device_only=True)
+    out = {}
+    for ft in (21, 8):
+        rb = synth.row_bytes(ft, K)
+        W = gpu.buf(nmat * N * rb, device_only=True)
+        b = gpu.batch()
+        fill_blocks(gpu, b, W, 0, nmat * N * rb // synth.BLOCK[ft][1], ft, 99 + ft, synth.D_SIGMA[ft])
+        b.end()
+        for nb in (1, 2, 4, 8, 16):
+            algo = N * rb + nb * (K * 2 + N * 4)
+            for valu in ((False, True) if ft == 21 and nb <= 4 else (False,)):
+                name = "qmv_gg_bench_f%d_n%d%s" % (ft, nb, "_valu" if valu else "")
+                ok, err = gpu.compile("#define qmv_gg %s\n#define GF %d\n#define KD %d\n#define RB %d\n#define NB %d\n#define YT float\n%s" % (name, ft, K, rb, nb, "#define QW_VALU 1\n" if valu else ""))
+                assert ok, err
+                k = gpu.kernel(name)
+                best = 1e9
+                for _ in range(reps + 1):
+                    b = gpu.batch()
+                    b.kernel(k)
+                    b.buf(3, x)
+                    b.buf(4, y)
+                    b.bytes(5, np.array([N, K, N, 0], np.uint32))
+                    for i in range(nmat):
+                        b.buf(0, W, i * N * rb)
+                        b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
+                    best = min(best, b.end())
+                out["%s_B%d%s" % ("iq3_s" if ft == 21 else "q8_0", nb, "_valu" if valu else "")] = {"us_per_matvec": best / nmat * 1e6, "GBps": algo / (best / nmat) / 1e9}
+        W.free()
+    path.close()
+    x.free()
+    y.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -203,6 +249,7 @@ def main():
             "setup_s": setup_s}
     if not a.quick:
         line["ragged_step"] = ragged_steps(gpu, stack)
+        line["qmv"] = qmv_table(gpu)
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)

@@ -38,6 +38,7 @@ typedef struct { // parameters taken from the define block
     int E, topk, D, I, gnb;              // MoE
     int fgu, fd, fsg, fsu, fsd, rbf, rwf; // formats; rbf: router inside moe_pre_gg; rwf: router weight type (1 / 30)
     int tm;                              // packing: rows per tile entry
+    int valu;                            // qmv_gg: QW_VALU in the block asks for the VALU GEMV (measurement)
 } qw_kparams;
 
 struct qw_kernel {
@@ -315,6 +316,7 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
         if (p.NB < 1 || p.NB > 16) FAIL("qmv_gg: NB %d outside 1..16", p.NB);
         const char *yt = def_get(d, n, "YT");
         p.yfloat = yt && !strcmp(yt, "float");
+        p.valu = def_get(d, n, "QW_VALU") != NULL;
         if (yt && strcmp(yt, "float") && strcmp(yt, "half")) FAIL("qmv_gg: YT %s is neither half nor float", yt);
         if (!reg_kernel(g, d, n, "qmv_gg", FAM_QMV_GG, &p, err, errlen)) { ok = false; goto out; }
     }
@@ -662,6 +664,7 @@ static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 1 : 16) : 1
 static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1; }
 #endif
 
+static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf *hb, const void *B, uint64_t ntiles, uint32_t nblk, uint32_t rowbytes, uint32_t split);
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
     const qw_kparams *p = &b->k->p;
     uint32_t a4[4];
@@ -676,8 +679,17 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
         !bind_ptr(b, 3, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x) ||
         !bind_ptr(b, 4, ((size_t)(a.nb - 1) * a.ystride + a.N) * (a.yfloat ? 4 : 2), true, "y", &a.y)) return false;
     char fn[48];
-    if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", p->F);
-    else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", p->F, chunk_of(p->F, p->K));
+    int F = p->F;
+    if (F == 21 && p->K <= 2560 && a.N % 16 == 0) { // tile-major copy of the rows, made at first use
+        const uint32_t nblk = (uint32_t)p->K / 256;
+        const uint8_t *pk = get_pack(b, b->buf[0].h, a.W, NULL, NULL, a.N / 16, nblk, a.rowbytes, 16);
+        if (pk) F = QW_F_PACKED, a.W = pk, a.rowbytes = nblk * QW_SLAB_BYTES;
+    }
+    if (p->valu) { // the VALU GEMV, for measurement against the matrix-core form
+        if (F != QW_F_PACKED || p->K % 512 || p->NB > 4) return fail(b, "qmv_gg: the VALU form needs packed IQ3_S weights, K a multiple of 512 and NB <= 4");
+        fname_fmt(fn, sizeof fn, "qwk_qmv_valu_n%d", p->NB <= 1 ? 1 : p->NB <= 2 ? 2 : 4);
+    } else if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", F);
+    else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", F, chunk_of(21 == F || F == QW_F_PACKED ? 21 : F, p->K));
     return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 

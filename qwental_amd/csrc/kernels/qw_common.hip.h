@@ -347,6 +347,36 @@ template <int NB> struct qw_chunk<21, NB> {
             block_mfma(b, w, xh, xl, AF::has_lo, acc);
         }
     }
+    // The VALU form of the same product, for NT <= 4 tokens (the GEMV the matrix-core form is measured against):
+    // the lane's 64 values of a block times the same 64 activations of every token, by two-element dot
+    // instructions into one binary32 sum per token; the caller adds the four k-group lanes of a row afterwards.
+    template <int NT> __device__ __forceinline__ void dot_valu(const u2 *lut, const u4 *xf, uint32_t k0, uint32_t kg, float (&acc)[NT]) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w[16];
+            lookups(b, lut, w);
+            const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
+            float sub[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) sub[t] = 0;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const h2 ff = j < 4 ? ff0 : ff1;
+                u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
+#pragma unroll
+                for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const u4 xv = xf[((kb + 8 * j) >> 3) * 16 + t]; // token t's 8 values: the same address in all 16 row lanes (broadcast)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) sub[t] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, (uint32_t)raw[i]), __builtin_bit_cast(h2, (uint32_t)xv[i]), sub[t], false);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t] += s[b].d * sub[t];
+        }
+    }
     // NG groups of 16 activation rows against the same decoded weights (the grouped product over packed rows):
     // rows[g] is the lane's row of group g in global memory; every group has its own accumulator.
     template <int NG> __device__ __forceinline__ void mac_groups(const u2 *lut, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {

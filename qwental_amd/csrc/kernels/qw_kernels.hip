@@ -101,16 +101,19 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     const uint32_t cpr = a.K / (C::BLK_K * CH);
     const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t t) {
-        const uint32_t r = 16 * t + nl;
-        return a.W + (size_t)(r < a.N ? r : a.N - 1) * a.rowbytes;
+        if constexpr (F == QW_F_PACKED) return a.W + (size_t)t * a.rowbytes; // the tile's slabs
+        else {
+            const uint32_t r = 16 * t + nl;
+            return a.W + (size_t)(r < a.N ? r : a.N - 1) * a.rowbytes;
+        }
     };
-    if (F == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
     if (XLDS) qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
     __syncthreads();
     const qw_afrag_lds afl = {xf, n};
     const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, CH * C::BLK_B, kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
+    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
         if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
         else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
@@ -129,10 +132,51 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
 }
 #define QW_QMV(F, CH, XLDS, SFX)                                                                        \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
-        __shared__ struct { u2 lut[F == 21 ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; } L; /* table first: LDS address 0 */ \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; } L; /* table first: LDS address 0 */ \
         qmv_body<F, CH, XLDS>(a, L.lut, L.xf);                                                          \
     }
 QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
+QW_QMV(121, 2, true, _c2) QW_QMV(121, 1, true, _c1) // packed IQ3_S: a.rowbytes = bytes of a 16-row tile
+
+// The VALU GEMV the matrix-core kernels are measured against (1, 2 or 4 activations, K a multiple of 512 up to 2560,
+// packed IQ3_S): the same streaming and decoding, v_dot2_f32_f16 instead of the matrix instruction, and a sum over
+// the four k-group lanes of a row by two cross-lane adds.
+template <int NT> __device__ __forceinline__ void qmv_valu_body(const qwk_qmv_args &a, u2 *lut, u4 *xf) {
+    typedef qw_chunk<QW_F_PACKED, 2> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave(), cpr = a.K / 512;
+    float acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = 0;
+    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, 2 * C::BLK_B, lane, [&](uint32_t t) { return a.W + (size_t)t * a.rowbytes; },
+        [&](uint32_t t, uint32_t ci, const C &c) {
+            c.template dot_valu<NT>(lut, xf, ci * 512, kg, acc);
+            if (ci + 1 != cpr) return;
+            const uint32_t r = 16 * t + n;
+#pragma unroll
+            for (int tk = 0; tk < NT; tk++) {
+                float v = acc[tk];
+                v += __shfl_xor(v, 16);
+                v += __shfl_xor(v, 32);
+                if (kg == 0 && r < a.N && (uint32_t)tk < a.nb) {
+                    if (a.yfloat) ((float *)a.y)[(size_t)tk * a.ystride + r] = v;
+                    else ((uint16_t *)a.y)[(size_t)tk * a.ystride + r] = qw_f2h(v);
+                }
+                acc[tk] = 0;
+            }
+        },
+        [&] {
+            qw_lut_copy(lut, (const u2 *)a.glut);
+            qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
+            __syncthreads();
+        });
+}
+#define QW_QMV_VALU(NT)                                                                                  \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmv_valu_n##NT(qwk_qmv_args a) {          \
+        __shared__ struct { u2 lut[QW_LUT_ENTRIES]; u4 xf[QW_XF_MAXK * 2]; } L;                          \
+        qmv_valu_body<NT>(a, L.lut, L.xf);                                                               \
+    }
+QW_QMV_VALU(1) QW_QMV_VALU(2) QW_QMV_VALU(4)
 QW_QMV(8, 16, true, _c16) QW_QMV(8, 1, true, _c1) QW_QMV(8, 1, false, _c1g)
 
 // ================================================================ router (kernels/moe_gg.metal:25-41)

@@ -274,3 +274,59 @@ def test_moe_batched_equals_single(gpu):
     assert np.array_equal(out[5].view(np.uint16), out[2].view(np.uint16))
     dl.free()
     path.close()
+
+
+@pytest.mark.parametrize("nb,valu", [(1, False), (3, False), (16, False), (1, True), (2, True), (4, True)])
+def test_qmv_packed_and_valu_forms(gpu, oracle, nb, valu):
+    """Weights in a device-only buffer take the tile-major copy; with QW_VALU in the block the VALU GEMV runs instead of
+    the matrix-core kernel. Both against the float64 oracle."""
+    N, K = 1024, 2048
+    rng = np.random.default_rng(40 + nb)
+    W = synth.matrix(rng, 21, N, K)
+    x = synth.activations(rng, nb, K)
+    rb = synth.row_bytes(21, K)
+    name = "qmv_gg_t_n%d_%d" % (nb, valu)
+    ok, err = gpu.compile("#define qmv_gg %s\n#define GF 21\n#define KD %d\n#define RB %d\n#define NB %d\n#define YT float\n%s" % (name, K, rb, nb, "#define QW_VALU 1\n" if valu else ""))
+    assert ok, err
+    wb, xb, yb = gpu.buf_from(W, device_only=True), gpu.buf_from(x), gpu.buf(nb * N * 4)
+    before = gpu.L.qw_hip_packed_bytes(gpu.g)
+    b = gpu.batch()
+    b.kernel(gpu.kernel(name))
+    b.buf(0, wb)
+    b.buf(3, xb)
+    b.buf(4, yb)
+    b.bytes(5, np.array([N, K, N, 0], np.uint32))
+    b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
+    assert b.end() >= 0, gpu.last_error()
+    assert gpu.L.qw_hip_packed_bytes(gpu.g) == before + N // 16 * (K // 256) * 1792
+    y = yb.view(np.float32)[:nb * N].reshape(nb, N)
+    assert maxrel(y, oracle.qmv(21, W, N, K, x, f64=True)) <= 1e-5
+    wb.free()  # drops the copy
+    assert gpu.L.qw_hip_packed_bytes(gpu.g) == before
+    for bb in (xb, yb):
+        bb.free()
+
+
+def test_packed_copy_follows_the_source(gpu, oracle):
+    """Rewriting a weight buffer after its first use drops the tile-major copy: the next call sees the new bytes."""
+    N, K, nb = 256, 512, 2
+    rng = np.random.default_rng(77)
+    x = synth.activations(rng, nb, K)
+    rb = synth.row_bytes(21, K)
+    ok, err = gpu.compile("#define qmv_gg qmv_gg_follow\n#define GF 21\n#define KD %d\n#define RB %d\n#define NB %d\n#define YT float\n" % (K, rb, nb))
+    assert ok, err
+    W0, W1 = synth.matrix(rng, 21, N, K), synth.matrix(rng, 21, N, K)
+    wb, xb, yb = gpu.buf_from(W0, device_only=True), gpu.buf_from(x), gpu.buf(nb * N * 4)
+    for W in (W0, W1):
+        wb.fill(W)
+        b = gpu.batch()
+        b.kernel(gpu.kernel("qmv_gg_follow"))
+        b.buf(0, wb)
+        b.buf(3, xb)
+        b.buf(4, yb)
+        b.bytes(5, np.array([N, K, N, 0], np.uint32))
+        b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
+        assert b.end() >= 0, gpu.last_error()
+        assert maxrel(yb.view(np.float32)[:nb * N].reshape(nb, N), oracle.qmv(21, W, N, K, x, f64=True)) <= 1e-5
+    for bb in (wb, xb, yb):
+        bb.free()
