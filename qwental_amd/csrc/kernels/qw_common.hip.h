@@ -430,6 +430,42 @@ template <int NB> struct qw_chunk<21, NB> {
             acc += s[b].d * (sub0 + sub1);
         }
     }
+    // mac_lean with the operand-A fragments of four steps in registers at a time instead of eight (two planes cost
+    // 32 registers instead of 64): for kernels whose operand A has a lo plane.
+    template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 256 * b + 64 * kg;
+            u2 w[16];
+            lookups(b, lut, w);
+            const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
+            f4 sub0 = {0, 0, 0, 0}, sub1 = {0, 0, 0, 0};
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                h8 xh[4], xl[4];
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    xh[jj] = af.hi(kb + 32 * half + 8 * jj);
+                    if (AF::has_lo) xl[jj] = af.lo(kb + 32 * half + 8 * jj);
+                }
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = 4 * half + jj;
+                    const h2 ff = half ? ff1 : ff0;
+                    u4 raw = {w[2 * j].x, w[2 * j].y, w[2 * j + 1].x, w[2 * j + 1].y};
+#pragma unroll
+                    for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
+                    const h8 wv = __builtin_bit_cast(h8, raw);
+                    if (AF::has_lo) {
+                        sub0 = qw_mfma(xh[jj], wv, sub0);
+                        sub1 = qw_mfma(xl[jj], wv, sub1);
+                    } else if (j & 1) sub1 = qw_mfma(xh[jj], wv, sub1);
+                    else sub0 = qw_mfma(xh[jj], wv, sub0);
+                }
+            }
+            acc += s[b].d * (sub0 + sub1);
+        }
+    }
     // One block's table values times two operand-A fragment sets (hi, lo), accumulated the way mac() does.
     __device__ __forceinline__ void block_mfma(int b, const u2 (&w)[16], const h8 (&xh)[8], const h8 (&xl)[8], bool lo, f4 &acc) const {
         const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
@@ -499,7 +535,7 @@ template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
 
 template <int NB> struct qw_chunk<8, NB> {
     static constexpr uint32_t BLK_K = 32, BLK_B = 34;
-    static constexpr int DEPTH = NB > 8 ? 2 : 3;
+    static constexpr int DEPTH = 2;
     u2 q[NB];
     uint16_t d[NB];
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t kg) {
@@ -525,6 +561,7 @@ template <int NB> struct qw_chunk<8, NB> {
         if (NB & 1) d[NB - 1] = (uint16_t)qw_pull(d[NB - 1], src4);
     }
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     template <int NG> __device__ __forceinline__ void mac_groups(const u2 *, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {

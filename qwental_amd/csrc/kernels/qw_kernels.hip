@@ -720,24 +720,26 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
     f4 acc = {0, 0, 0, 0};
     qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
         [&](uint32_t i) {
+            // (field by field: a reference chosen between the two records would put them in scratch memory)
             const bool second = i >= g0.ntile;
-            const qw_dn_seg &g = second ? g1 : g0;
-            const uint32_t tile = g.tile0 + (second ? i - g0.ntile : i);
-            if constexpr (F == QW_F_PACKED) return g.W + (size_t)tile * g.rowbytes; // rowbytes = bytes of a tile
-            else return g.W + (size_t)(16 * tile + nl) * g.rowbytes;
+            const uint8_t *W = second ? g1.W : g0.W;
+            const uint32_t tile = second ? g1.tile0 + i - g0.ntile : g0.tile0 + i, rbs = second ? g1.rowbytes : g0.rowbytes;
+            if constexpr (F == QW_F_PACKED) return W + (size_t)tile * rbs; // rowbytes = bytes of a tile
+            else return W + (size_t)(16 * tile + nl) * rbs;
         },
         [&](uint32_t i, uint32_t ci, const C &c) {
             const bool second = i >= g0.ntile;
             const u4 *ab = (const u4 *)arows + (second ? 4 * a.I : 0); // fragment order: [plane][8 k-values][token], 16 bytes each
             const qw_afrag_lds2 af = {ab, ab + 2 * a.I, n};
-            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+            c.mac_half(lut, af, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 != cpr) return;
-            const qw_dn_seg &g = second ? g1 : g0;
-            const uint32_t r = 16 * (g.tile0 + (second ? i - g0.ntile : i)) + n, sl = second ? sl1 : sl0;
+            const uint32_t r = 16 * (second ? g1.tile0 + i - g0.ntile : g0.tile0 + i) + n, sl = second ? sl1 : sl0;
+            const uint32_t gm = second ? g1.mask : g0.mask, gsh = second ? g1.sh : g0.sh;
+            float *P = second ? g1.P : g0.P;
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++) {
                 const uint32_t tok = 4 * kg + j;
-                if ((g.mask >> tok) & 1) g.P[(g.sh ? (size_t)tok : (size_t)tok * K + ((sl >> (8 * j)) & 255)) * a.D + r] = acc[j];
+                if ((gm >> tok) & 1) P[(gsh ? (size_t)tok : (size_t)tok * K + ((sl >> (8 * j)) & 255)) * a.D + r] = acc[j];
             }
             acc = f4{0, 0, 0, 0};
         },
@@ -764,27 +766,27 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         const uint32_t end = base + per < V ? base + per : V;
         // virtual expert of a position: 0 = shared (positions below vsh), then the routed experts
         const uint32_t v0 = base < vsh ? 0 : nsh + (base - vsh) / tpe, v1 = end - 1 < vsh ? 0 : nsh + (end - 1 - vsh) / tpe;
-        qw_dn_seg g[2];
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const uint32_t v = i ? v1 : v0;
-            g[i].sh = v < nsh;
-            if (g[i].sh) {
+        auto seg = [&](uint32_t v) {
+            qw_dn_seg g;
+            g.sh = v < nsh;
+            if (g.sh) {
                 const uint32_t hi = end < vsh ? end : vsh; // positions [base, hi) -> tiles, rounded so that neighbours meet
-                g[i].tile0 = (base + shw - 1) / shw;
-                g[i].ntile = (hi + shw - 1) / shw - g[i].tile0;
-                g[i].u = 0;
-                g[i].W = a.Wsd, g[i].P = a.Psh, g[i].rowbytes = a.sd_rowbytes, g[i].mask = qw_all_tokens(a.snbr);
+                g.tile0 = (base + shw - 1) / shw;
+                g.ntile = (hi + shw - 1) / shw - g.tile0;
+                g.u = 0;
+                g.W = a.Wsd, g.P = a.Psh, g.rowbytes = a.sd_rowbytes, g.mask = qw_all_tokens(a.snbr);
             } else {
                 const uint32_t first = vsh + (v - nsh) * tpe, lo = first > base ? first : base, hi = first + tpe < end ? first + tpe : end;
-                g[i].u = v - nsh;
-                g[i].tile0 = lo - first;
-                g[i].ntile = hi - lo;
-                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ue[g[i].u]);
-                g[i].W = a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, g[i].P = a.P, g[i].rowbytes = a.rowbytes;
-                g[i].mask = (uint32_t)__builtin_amdgcn_readfirstlane((int)mask[g[i].u]) & qw_all_tokens(a.nbr);
+                g.u = v - nsh;
+                g.tile0 = lo - first;
+                g.ntile = hi - lo;
+                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ue[g.u]);
+                g.W = a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, g.P = a.P, g.rowbytes = a.rowbytes;
+                g.mask = (uint32_t)__builtin_amdgcn_readfirstlane((int)mask[g.u]) & qw_all_tokens(a.nbr);
             }
-        }
+            return g;
+        };
+        const qw_dn_seg g0 = seg(v0), g1 = seg(v1);
         const bool both = v1 != v0;
         bool staged = false;
         // set-up of a round, run by every wave once its first weight loads are in flight: the table (first round),
@@ -797,12 +799,12 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             // the loads of that pass are in flight while the table is copied. Fragment order in LDS,
             // [segment][plane][c][token], 16 bytes each: the sixteen lanes of a k-group read 256 contiguous bytes.
             const uint32_t upr = a.I / 8, per = 2 * upr; // 16-byte units per plane row, per row
-            const uint32_t rows = g[0].mask | (both ? g[1].mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
+            const uint32_t rows = g0.mask | (both ? g1.mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
             auto item = [&](uint32_t i, uint32_t &dst) {
                 uint32_t m = rows;
                 for (uint32_t k = i / per; k; k--) m &= m - 1; // drop the rows before this one
                 const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, t = bit & 15, r = i % per, pl = r / upr, c = r % upr;
-                const uint32_t s = g[sg].sh ? K : slot[g[sg].u * gnb + t];
+                const uint32_t s = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + t];
                 dst = ((sg * 2 + pl) * upr + c) * 16 + t;
                 return *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
             };
@@ -822,13 +824,13 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             QW_TRACED(2);
         };
         // the two segments share one pipeline when their formats agree; a shared expert of another format runs first
-        if (FSD != 0 && FSD != F && g[0].sh) {
-            qw_dn_seg none = g[0];
+        if (FSD != 0 && FSD != F && g0.sh) {
+            qw_dn_seg none = g0;
             none.ntile = 0;
-            dn_range_run<FSD == 0 ? F : FSD, CHSD>(a, lut, arows, g[0], none, false, slot, slot, ready);
-            if (both) dn_range_run<F, CH>(a, lut, arows + 32 * a.I, g[1], none, false, slot + g[1].u * gnb, slot, ready);
+            dn_range_run<FSD == 0 ? F : FSD, CHSD>(a, lut, arows, g0, none, false, slot, slot, ready);
+            if (both) dn_range_run<F, CH>(a, lut, arows + 32 * a.I, g1, none, false, slot + g1.u * gnb, slot, ready);
         } else {
-            dn_range_run<F, CH>(a, lut, arows, g[0], g[1], both, slot + g[0].u * gnb, slot + g[1].u * gnb, ready);
+            dn_range_run<F, CH>(a, lut, arows, g0, g1, both, slot + g0.u * gnb, slot + g1.u * gnb, ready);
         }
         QW_TRACED(4);
         __syncthreads();
