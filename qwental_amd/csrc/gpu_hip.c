@@ -380,9 +380,6 @@ out:
     return ok;
 }
 
-#ifdef QW_EXP_TRACE
-bool qw_hip_debug_tabs(qw_gpu *g, void *dst, size_t n) { return hipDeviceSynchronize() == hipSuccess && hipMemcpy(dst, g->tabs, n, hipMemcpyDeviceToHost) == hipSuccess; }
-#endif
 bool qw_hip_compile_check(const char *src, size_t len, char *err, size_t errlen, char *names, size_t nameslen) {
     qw_gpu *g = calloc(1, sizeof *g); // no device behind it: only the kernel registry is touched
     if (!g) return false;
@@ -619,12 +616,7 @@ static unsigned cdiv(unsigned a, unsigned b) { return (a + b - 1) / b; }
 // Persistent grids: one 512-thread workgroup per compute unit (the LDS tables leave room for one), fewer if the
 // work is smaller. tasks are per-wave units; 8 waves per workgroup.
 static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks, unsigned waves) { return umin((unsigned)g->ncu, cdiv(wave_tasks, waves)); }
-#ifdef QW_EXP_W16
-enum { QW_WAVES_GU = 16, QW_WAVES_DN = 8 };
-#else
-enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 };
-#endif
-// // waves per workgroup of the gate/up + matvec kernels and of the down kernels
+enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 }; // // waves per workgroup of the gate/up + matvec kernels and of the down kernels
 
 static const char *fname_fmt(char *buf, size_t n, const char *fmt, ...) {
     va_list ap;
@@ -658,11 +650,7 @@ static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W,
 static const void *glut(const qw_gpu *g) { return (const char *)g->tabs + QW_TAB_IQ3SS; }
 
 // Blocks per prefetch chunk for a row of K values (the kernels are instantiated for these; 1 = any K).
-#ifdef QW_EXP_W16
-static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 1 : 16) : 1; }
-#else
 static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1; }
-#endif
 
 static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf *hb, const void *B, uint64_t ntiles, uint32_t nblk, uint32_t rowbytes, uint32_t split);
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
@@ -935,26 +923,13 @@ static bool tr_dn(qw_batch *b) {
     }
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
-#ifndef QW_EXP_DNSTREAM
     if (p->I <= 512) { // contiguous task ranges per workgroup, operand A staged in LDS
         const int ch = fd == 8 ? 4 : p->I / 256;
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
         return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
     }
-#endif
-#ifndef QW_EXP_DNOLD
-    if (p->I % 512 == 0) { // independent waves, task = (expert, 16 rows)
-        const int ch = p->fd == 21 ? 2 : 4;
-        if (fs) fname_fmt(fn, sizeof fn, "qwk_dn_f%d_c%d_s%d_c%d", p->fd, ch, fs, fs == 21 ? 2 : 4);
-        else fname_fmt(fn, sizeof fn, "qwk_dn_f%d_c%d", p->fd, ch);
-        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
-    }
-#endif
-    if (p->I == 512 && p->fd == 21) { // workgroup tasks of 256 rows
-        fname_fmt(fn, sizeof fn, "qwk_dn_f21_i512%s", sfx);
-        return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, umax * (unsigned)(p->D / 256)), 512, &a, sizeof a);
-    }
+    // wider rows: one tile at a time, operand A from global memory
     fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any%s", p->fd, sfx);
     return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DN), 64 * QW_WAVES_DN, &a, sizeof a);
 }

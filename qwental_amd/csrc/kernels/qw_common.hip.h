@@ -64,11 +64,7 @@ __device__ __forceinline__ void qw_lut_build(u2 *lut) {
     for (uint32_t i = threadIdx.x; i < QW_LUT_ENTRIES; i += blockDim.x) lut[qw_lut_slot(i)] = qw_lut_entry(i);
 }
 
-#ifdef QW_EXP_NOMFMA
-__device__ __forceinline__ f4 qw_mfma(h8 a, h8 b, f4 c) { c[0] += (float)a[0] * (float)b[0] + (float)b[3]; c[1] += (float)a[5] * (float)b[7] + (float)b[5]; return c; }
-#else
 __device__ __forceinline__ f4 qw_mfma(h8 a, h8 b, f4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
-#endif
 
 // ---------------------------------------------------------------- IQ3_S (110-byte block of 256 values)
 // Bytes: d @0 (binary16), qs[64] @2, qh[8] @66, signs[32] @74, scales[4] @106 (kernels/moe_iq.metal:102-118).
@@ -85,10 +81,6 @@ struct qw_iq3_slice {
 
 __device__ __forceinline__ qw_iq3_slice qw_iq3_load(const uint8_t *blk, uint32_t kg) {
     qw_iq3_slice s;
-#ifdef QW_EXP_NOLOAD
-    s.qs = u4{kg * 0x01010101u, 0x23456789u * kg, 0x11111111u, 0x77777777u}; s.sg = u2{0x12345678u, kg}; s.qh = 0x55aa; s.sc = 0x37; s.d = 1.0f;
-    return s;
-#endif
     s.qs = *(const u4a2 *)(blk + 2 + 16 * kg);
     s.sg = *(const u2a2 *)(blk + 74 + 8 * kg);
     s.qh = *(const uint16_t *)(blk + 66 + 2 * kg);
@@ -268,11 +260,7 @@ template <int NB> struct qw_chunk<21, NB> {
         qw_iq3_addr<7>(s[b], k, i[14], i[15]);
 #pragma unroll
         for (int j = 0; j < 16; j++) {
-#ifdef QW_EXP_NOLUT
-            w[j] = u2{i[j] * 0x00010001u | 0x3c003c00u, 0x3c003c00u};
-#else
             w[j] = qw_lut_at(lut, i[j]);
-#endif
         }
     }
     // acc += this chunk's contribution; k0 = k-offset of the chunk's first value. Software pipeline over the blocks:
@@ -294,13 +282,8 @@ template <int NB> struct qw_chunk<21, NB> {
             h8 xh[8], xl[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-#ifdef QW_EXP_NOXFRAG
-                xh[j] = __builtin_bit_cast(h8, u4{kb + j, kg, 0x3c003c00u, 0x3c003c00u});
-                if (AF::has_lo) xl[j] = xh[j];
-#else
                 xh[j] = af.hi(kb + 8 * j);
                 if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
-#endif
             }
             if (b + 1 < NB) lookups(b + 1, lut, w[(b + 1) & 1]);
             const h2 ff0 = qw_iq3_factor(s[b], 0), ff1 = qw_iq3_factor(s[b], 1);
@@ -324,10 +307,6 @@ template <int NB> struct qw_chunk<21, NB> {
     }
     // The same arithmetic without the cross-block pipeline (fewer registers; for kernels that run more waves).
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
-#ifdef QW_EXP_NOCOMPUTE
-        for (int b = 0; b < NB; b++) acc[0] += __builtin_bit_cast(float, (s[b].qs.x ^ s[b].qs.y ^ s[b].qs.z ^ s[b].qs.w ^ s[b].sg.x ^ s[b].sg.y ^ s[b].qh ^ s[b].sc) & 0x007fffffu) + s[b].d;
-        return;
-#endif
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const uint32_t kb = k0 + 256 * b + 64 * kg;
@@ -335,11 +314,6 @@ template <int NB> struct qw_chunk<21, NB> {
             lookups(b, lut, w);
             h8 xh[8], xl[8];
 #pragma unroll
-#ifdef QW_EXP_NOLO
-            for (int j = 0; j < 8; j++) xh[j] = af.hi(kb + 8 * j);
-            block_mfma(b, w, xh, xl, false, acc);
-            continue;
-#endif
             for (int j = 0; j < 8; j++) {
                 xh[j] = af.hi(kb + 8 * j);
                 if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
@@ -484,25 +458,6 @@ template <int NB> struct qw_chunk<21, NB> {
             else sub0 = qw_mfma(xh[j], wv, sub0);
         }
         acc += s[b].d * (sub0 + sub1);
-    }
-    // Two tiles that share every operand-A fragment (the down projection: both tiles belong to one expert): the
-    // fragments are read once per block. Each tile's arithmetic is exactly that of mac().
-    template <class AF> static __device__ __forceinline__ void mac2(const qw_chunk &t0, const qw_chunk &t1, const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc0, f4 &acc1) {
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const uint32_t kb = k0 + 256 * b + 64 * kg;
-            u2 w0[16], w1[16];
-            t0.lookups(b, lut, w0);
-            t1.lookups(b, lut, w1);
-            h8 xh[8], xl[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                xh[j] = af.hi(kb + 8 * j);
-                if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
-            }
-            t0.block_mfma(b, w0, xh, xl, AF::has_lo, acc0);
-            t1.block_mfma(b, w1, xh, xl, AF::has_lo, acc1);
-        }
     }
 };
 

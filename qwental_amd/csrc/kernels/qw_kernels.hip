@@ -8,28 +8,12 @@
 #include "qw_common.hip.h"
 
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
-#ifdef QW_EXP_W16
-#define QW_WG_GU 1024
-#else
 #define QW_WG_GU 768       // gate/up and dense matvec: 12 waves, three per SIMD (a wave issues at most one instruction in ~6 cycles)
-#endif
 #define QW_XF_MAXK 2560    // largest K whose activations are staged in LDS in fragment order (K * 32 bytes)
 
 // wave index in the workgroup, as a scalar (so that task indices and row bases stay in scalar registers)
 __device__ __forceinline__ uint32_t qw_wave() { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
-#ifdef QW_EXP_TRACE
-#define QW_TRACE(slot) do { if ((threadIdx.x & 63) == 0) ((long long *)a.glut - 49152 / 8)[(blockIdx.x * 2 + (threadIdx.x >> 6) / 11) * 8 + (slot)] = wall_clock64(); } while (0)
-#else
-#define QW_TRACE(slot) do { } while (0)
-#endif
-#ifdef QW_EXP_TRACEDN
-#define QW_TRACEG(slot) do { } while (0)
-#define QW_TRACED(slot) QW_TRACE(slot)
-#else
-#define QW_TRACEG(slot) QW_TRACE(slot)
-#define QW_TRACED(slot) do { } while (0)
-#endif
 constexpr bool qw_has_lut(int f) { return f == 21 || f == QW_F_PACKED; } // formats decoded through the LDS table
 __device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
@@ -486,7 +470,6 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 // it); then every wave issues its first weight loads, and only then the table copy, the activation staging and the
 // second barrier follow, overlapping that first round trip to HBM.
 template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
-    QW_TRACEG(0);
     if (a.logits) { // the selection, made here by every workgroup; the scratch lies where x is staged afterwards
         qw_sel_scratch &ss = *(qw_sel_scratch *)xf;
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
@@ -497,7 +480,6 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
         if (threadIdx.x == 0) sc->U = ss.U;
     } else if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
     __syncthreads();
-    QW_TRACEG(1);
     bool staged = false;
     auto ready = [&] {
         if (staged) return;
@@ -505,7 +487,6 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
         if (qw_has_lut(FGU) || qw_has_lut(FSG)) qw_lut_copy(lut, (const u2 *)a.glut);
         qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
         __syncthreads();
-        QW_TRACEG(2);
     };
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     if (FSG != 0) {
@@ -518,10 +499,8 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
             gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready);
         }
     }
-    QW_TRACEG(3);
     // the waves that did a shared tile come last in the routed deal, so that the work stays level
     gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready);
-    QW_TRACEG(4);
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
@@ -625,78 +604,6 @@ template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const
         });
 }
 
-// Workgroup task = (expert u, block of 256 rows): the H rows (hi and lo planes) of the tokens that picked u are staged
-// in LDS in fragment order, double-buffered; wave w owns rows 32 w .. 32 w + 31 of the block = two tiles.
-// One barrier per task; the weight loads of the next task are in flight across it.
-template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_body(const qwk_dn_args &a, u2 *lut, u4 *abuf /* [2][2][I/8*16] */, qw_sel_cache *sc) {
-    typedef qw_chunk<F, CH> C;
-    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb, wave = qw_wave();
-    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
-    qw_sel_load(*sc, a.sel, K, gnb);
-    __syncthreads();
-    if (FSD != 0) {
-        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, blockIdx.x * (blockDim.x >> 6) + wave, gridDim.x * (blockDim.x >> 6));
-    }
-    const uint32_t U = sc->U, bpe = a.D / 256, ntasks = U * bpe, mine = blockIdx.x < ntasks ? (ntasks - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
-    const uint32_t nfrag = (a.I / 8) * 16; // 16-byte fragments per plane
-    auto stage = [&](uint32_t it) { // operand A of this workgroup's it-th task into buffer it & 1
-        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, m = sc->mask[u];
-        u4 *dst = abuf + (size_t)(it & 1) * 2 * nfrag;
-        for (uint32_t i = threadIdx.x; i < 2 * nfrag; i += blockDim.x) {
-            const uint32_t pl = i / nfrag, f = i % nfrag, c = f >> 4, t = f & 15;
-            u4 v = {0, 0, 0, 0};
-            if (t < a.nbr && ((m >> t) & 1)) v = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + sc->slot[u * gnb + t]) * a.I + 8 * c);
-            dst[i] = v;
-        }
-    };
-    const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
-    auto rowp = [&](uint32_t it, uint32_t tile) {
-        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, r = 256 * (task % bpe) + 32 * wave + 16 * tile + nl;
-        return a.Wd + ((size_t)sc->ue[u] * a.D + r) * a.rowbytes;
-    };
-    auto compute = [&](uint32_t it, C &t0, C &t1) {
-        t0.transpose();
-        t1.transpose();
-        const u4 *base = abuf + (size_t)(it & 1) * 2 * nfrag;
-        const qw_afrag_lds2 af = {base, base + nfrag, n};
-        const uint32_t task = blockIdx.x + it * gridDim.x, u = task / bpe, m = sc->mask[u];
-        f4 acc2[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-        C::mac2(t0, t1, lut, af, 0, kg, acc2[0], acc2[1]);
-#pragma unroll
-        for (int tile = 0; tile < 2; tile++) {
-            const uint32_t r = 256 * (task % bpe) + 32 * wave + 16 * tile + n;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; j++) {
-                const uint32_t tok = 4 * kg + j;
-                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc2[tile][j];
-            }
-        }
-    };
-    C a0, a1, b0, b1;
-    if (mine) {
-        a0.load(rowp(0, 0), kl);
-        a1.load(rowp(0, 1), kl);
-        stage(0);
-    }
-    __syncthreads();
-    for (uint32_t it = 0; it < mine; it += 2) {
-        if (it + 1 < mine) { b0.load(rowp(it + 1, 0), kl); b1.load(rowp(it + 1, 1), kl); stage(it + 1); }
-        compute(it, a0, a1);
-        __syncthreads();
-        if (it + 1 >= mine) break;
-        if (it + 2 < mine) { a0.load(rowp(it + 2, 0), kl); a1.load(rowp(it + 2, 1), kl); stage(it + 2); }
-        compute(it + 1, b0, b1);
-        __syncthreads();
-    }
-}
-#define QW_DN(F, CH, FSD, CHSD, IMAX, NAME)                                           \
-    extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
-        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; u4 abuf[2 * 2 * (IMAX / 8) * 16]; qw_sel_cache sc; } L; \
-        dn_body<F, CH, FSD, CHSD>(a, L.lut, L.abuf, &L.sc);                           \
-    }
-// I = 512 is the synthetic shape (whole row = one chunk of 2 IQ3_S blocks); Q8_0 down weights take the any-shape kernel
-QW_DN(21, 2, 0, 1, 512, qwk_dn_f21_i512) QW_DN(21, 2, 21, 2, 512, qwk_dn_f21_i512_s21) QW_DN(21, 2, 8, 16, 512, qwk_dn_f21_i512_s8)
-
 // Range form (I <= 512). The task list is "virtual experts" x tiles of 16 rows: virtual expert 0 is the shared expert
 // when the launch carries one, then the unique routed experts in record order. Every workgroup takes one contiguous
 // range of at most D / 16 tasks, which touches at most two experts: their H rows (both planes, only the tokens
@@ -747,10 +654,8 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
 }
 template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
-    QW_TRACED(0);
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
     __syncthreads();
-    QW_TRACED(1);
     const uint32_t *ue = sc->ue, *mask = sc->mask;
     const uint8_t *slot = sc->slot;
     uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
@@ -821,7 +726,6 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
                 ((u4 *)arows)[d] = v;
             }
             __syncthreads();
-            QW_TRACED(2);
         };
         // the two segments share one pipeline when their formats agree; a shared expert of another format runs first
         if (FSD != 0 && FSD != F && g0.sh) {
@@ -832,7 +736,6 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         } else {
             dn_range_run<F, CH>(a, lut, arows, g0, g1, both, slot + g0.u * gnb, slot + g1.u * gnb, ready);
         }
-        QW_TRACED(4);
         __syncthreads();
     }
 }
@@ -847,58 +750,6 @@ QW_DN_RANGE(21, 1, 0, 1, qwk_dnr_f21_c1) QW_DN_RANGE(21, 1, 21, 1, qwk_dnr_f21_c
 QW_DN_RANGE(121, 2, 0, 1, qwk_dnr_f121_c2) QW_DN_RANGE(121, 2, 121, 2, qwk_dnr_f121_c2_s121_c2) QW_DN_RANGE(121, 2, 8, 4, qwk_dnr_f121_c2_s8_c4)
 QW_DN_RANGE(121, 1, 0, 1, qwk_dnr_f121_c1) QW_DN_RANGE(121, 1, 121, 1, qwk_dnr_f121_c1_s121_c1) QW_DN_RANGE(121, 1, 8, 4, qwk_dnr_f121_c1_s8_c4)
 QW_DN_RANGE(8, 4, 0, 1, qwk_dnr_f8_c4) QW_DN_RANGE(8, 4, 8, 4, qwk_dnr_f8_c4_s8_c4) QW_DN_RANGE(8, 4, 21, 2, qwk_dnr_f8_c4_s21_c2) QW_DN_RANGE(8, 4, 21, 1, qwk_dnr_f8_c4_s21_c1)
-
-// Streaming form: independent waves, task = (unique expert, tile of 16 rows), the weights of the next task are in
-// flight while this one is multiplied (the pipeline runs across task boundaries), operand A comes straight from the
-// H planes in global memory, and only the lanes whose token picked the expert read anything. No barrier after set-up.
-template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_stream_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
-    typedef qw_chunk<F, CH> C;
-    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
-    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
-    qw_sel_load(*sc, a.sel, K, gnb);
-    __syncthreads();
-    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
-    if (FSD != 0) {
-        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, CHSD>(a, lut, w0, nw);
-    }
-    const uint32_t cpr = a.I / (C::BLK_K * CH);
-    f4 acc = {0, 0, 0, 0};
-    h8 xhi[4] = {}, xlo[4] = {};
-    // the waves that did a shared tile come last in the routed deal
-    qw_task_pipeline<C>(ntasks, nw - 1 - w0, nw, cpr, CH * C::BLK_B, lane & 3,
-        [&](uint32_t task) {
-            const uint32_t u = task / tpe, t = task % tpe;
-            return a.Wd + ((size_t)sc->ue[u] * a.D + 16 * t + (lane >> 2)) * a.rowbytes;
-        },
-        [&](uint32_t task, uint32_t ci, const C &c) {
-            const uint32_t u = task / tpe, m = sc->mask[u];
-            // only the lanes whose token picked the expert read H; the other columns of the result are never stored
-#ifdef QW_EXP_NOGATHER
-            const bool on = false; // timing experiment: operand A is never read
-#else
-            const bool on = n < a.nbr && ((m >> n) & 1);
-#endif
-            const uint16_t *rowhi = a.H + ((size_t)(on ? n : 0) * (K + 1) + (on ? sc->slot[u * gnb + n] : 0)) * a.I;
-            const qw_afrag_gather af = {rowhi, rowhi + a.hplane, on, xhi, xlo};
-            c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc);
-            if (ci + 1 != cpr) return;
-            const uint32_t r = 16 * (task % tpe) + n;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; j++) {
-                const uint32_t tok = 4 * kg + j;
-                if (tok < a.nbr && ((m >> tok) & 1)) a.P[((size_t)tok * K + sc->slot[u * gnb + tok]) * a.D + r] = acc[j];
-            }
-            acc = f4{0, 0, 0, 0};
-        });
-}
-#define QW_DN_STREAM(F, CH, FSD, CHSD, NAME)                                                      \
-    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_dn_args a) {                  \
-        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; qw_sel_cache sc; } L; \
-        dn_stream_body<F, CH, FSD, CHSD>(a, L.lut, &L.sc);                                        \
-    }
-// I a multiple of 512: 2 IQ3_S blocks or 4 Q8_0 blocks a chunk (operand A of a whole chunk is in flight at once)
-QW_DN_STREAM(21, 2, 0, 1, qwk_dn_f21_c2) QW_DN_STREAM(21, 2, 21, 2, qwk_dn_f21_c2_s21_c2) QW_DN_STREAM(21, 2, 8, 4, qwk_dn_f21_c2_s8_c4)
-QW_DN_STREAM(8, 4, 0, 1, qwk_dn_f8_c4) QW_DN_STREAM(8, 4, 8, 4, qwk_dn_f8_c4_s8_c4) QW_DN_STREAM(8, 4, 21, 2, qwk_dn_f8_c4_s21_c2)
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
