@@ -805,9 +805,11 @@ static bool tr_pre(qw_batch *b) {
     b->pend_sg.rowbytes = (uint32_t)rb;
     b->pend_sg.nbr = nbr;
     if (!p->rbf) return true; // router and selection come as dispatches of their own
-    qwk_pre_args a = {.nrouter = cdiv((unsigned)p->E + 1, 8)};
+    // router rows per workgroup: 16 on the matrix cores (binary16 router), 8 on the vector units (bf16 router)
+    qwk_pre_args a = {.nrouter = cdiv((unsigned)p->E + 1, p->rwf == 1 ? 16 : 8)};
     if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
     if (b->buf[2].off % 16) return fail(b, "moe_pre_gg: x offset %zu is not 16-byte aligned", b->buf[2].off);
+    if (p->rwf == 1 && (b->buf[0].off % 16 || b->buf[1].off % 16)) return fail(b, "moe_pre_gg: router weight offsets must be 16-byte aligned");
     // The shared expert's gate/up runs on the workgroups after the router's when a tile row splits into at most 8
     // chunks (D a multiple of 512, at most 4096) and the weights are Q8_0 or packed IQ3_S; otherwise it is left for
     // the gate/up launch (pend_sg).

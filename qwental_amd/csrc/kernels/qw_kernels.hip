@@ -532,6 +532,39 @@ template <int WF> __device__ __forceinline__ void pre_router(const qwk_pre_args 
     __syncthreads();
     router_rows_lds<WF>(a.r, (const uint16_t *)lds, blockIdx.x * (blockDim.x >> 6) + qw_wave(), qw_lane());
 }
+// Binary16 router on the matrix cores: a workgroup takes 16 router rows (row E is the shared-expert gate vector), its
+// waves split K among themselves (256 values = 8 matrix instructions a wave per pass), the partial sums meet in LDS
+// and wave 0 adds them in wave order. A token's logits do not depend on the other token columns.
+__device__ __forceinline__ void pre_router_mfma(const qwk_pre_args &pa, u4 *xf, f4 *part) {
+    const qwk_router_args &a = pa.r;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, wave = qw_wave(), nwv = blockDim.x >> 6;
+    const uint32_t row = 16 * blockIdx.x + n;
+    const uint16_t *wrow = row < a.E ? (const uint16_t *)a.Wr + (size_t)row * a.D : (const uint16_t *)a.Wsg; // rows past E repeat the gate vector; not stored
+    f4 acc = {0, 0, 0, 0};
+    // the first pass's weights are in flight while x is staged
+    u4 w[8];
+    uint32_t k0 = 256 * wave;
+    if (k0 < a.D)
+#pragma unroll
+        for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 32 * j + 8 * kg);
+    qw_stage_x(xf, a.x, a.D, a.D, a.nb);
+    __syncthreads();
+    for (; k0 < a.D; k0 += 256 * nwv) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc = qw_mfma(__builtin_bit_cast(h8, xf[((k0 + 32 * j + 8 * kg) >> 3) * 16 + n]), __builtin_bit_cast(h8, w[j]), acc);
+        if (k0 + 256 * nwv < a.D)
+#pragma unroll
+            for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 256 * nwv + 32 * j + 8 * kg);
+    }
+    part[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave != 0) return;
+    for (uint32_t i = 1; i < nwv; i++) acc += part[i * 64 + lane];
+    if (row <= a.E)
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++)
+            if (4 * kg + j < a.nb) a.logits[(size_t)(4 * kg + j) * (a.E + 1) + row] = acc[j];
+}
 template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pre_args &pa, u2 *lut, u4 *xf, f4 *part) {
     typedef qw_chunk<F, CH> C;
     const qwk_gu_args &a = pa.g;
@@ -573,8 +606,11 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
 }
 #define QW_PRE(WF, F, CH, NAME)                                                                          \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {                           \
-        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[F ? (QW_WG / 64) * 64 : 1]; } L; \
-        if (blockIdx.x < a.nrouter) pre_router<WF>(a, L.xf);                                            \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[(QW_WG / 64) * 64]; } L; \
+        if (blockIdx.x < a.nrouter) {                                                                   \
+            if (WF == 1) pre_router_mfma(a, L.xf, L.part);                                              \
+            else pre_router<WF>(a, L.xf);                                                               \
+        }                                                                                               \
         else if (F != 0) pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part);                              \
     }
 QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
