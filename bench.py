@@ -226,10 +226,9 @@ def main():
     ent = gpu.profile_entries()
     mean_s, n_l = gpu.profile_mean(DOMINANT)
     U = stack.unique_experts(nb)
-    # the gate/up launch of layer l reads U_l routed experts' gate and up rows (901,120 bytes each), the shared
-    # expert's gate and up rows (same shape, IQ3_S or Q8_0) and the nb x 4 KB activations
-    sh_gu = [2 * stack.I * synth.row_bytes(f, stack.D) for f in stack.shared_fmt]
-    gu_bytes = float(np.mean([u * stack.gu_bytes + s + nb * stack.D * 2 for u, s in zip(U, sh_gu)]))
+    # the gate/up launch of layer l reads U_l routed experts' gate and up rows (901,120 GGUF bytes each), the logits
+    # it makes the selection from and the nb x 4 KB activations (the shared expert's rows belong to the front launch)
+    gu_bytes = float(np.mean([u * stack.gu_bytes + nb * (stack.E + 1) * 4 + nb * stack.D * 2 for u in U]))
     per_kernel = {}
     for name, us in ent:
         per_kernel.setdefault(name, []).append(us)
