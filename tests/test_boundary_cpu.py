@@ -103,3 +103,26 @@ def test_unsupported_blocks_fail_with_a_message(block, needle):
 def test_later_definitions_win_and_whitespace_is_tolerated():
     ok, err, names = compile_check("  #define   DQ_TEST   14  \n\n#define DQ_TEST\t8\r\n#define dq_test  my_dq\n")
     assert ok and names == ["my_dq"]
+
+
+def test_packing_blocks_register_the_reference_names():
+    blk = "#define moe_scatter moe_scatter_x\n#define E 512\n#define TOPK 10\n#define KD 2048\n#define I 512\n#define TM 64\n"  # bench/moe_prefill.c:86-87
+    ok, err, names = compile_check(blk)
+    assert ok, err
+    assert names == ["moe_count", "moe_plan", "moe_plan_t", "moe_scatter_x", "moe_act", "p_act2", "moe_combine"]
+    pf = ("#define IQ_DQ_ONLY\n#define E 512\n#define TOPK 10\n#define D 2048\n#define I 512\n#define NB 1\n#define GG_PART 5\n#define PFF 21\n#define KD 2048\n"
+          "#define TM 64\n#define TN 64\n#define SG 4\n#define KC 64\n#define PFS 1\n#define PFT 1\n#define PFDBG 0\n#define moe_pf_gg moe_pf_gg_21_k2048_tm64\n")  # src/engine.c:3244-3248
+    ok, err, names = compile_check(pf)
+    assert ok and names == ["moe_pf_gg_21_k2048_tm64"], err
+    ok, err, names = compile_check(pf.replace("#define TM 64", "#define TM 128"))
+    assert not ok and "TM 128" in err
+    ok, err, names = compile_check(pf.replace("#define PFF 21", "#define PFF 22"))
+    assert not ok and "22" in err  # IQ2_S
+    ok, err, names = compile_check(pf.replace("GG_PART 5", "GG_PART 6"))
+    assert not ok and "GG_PART" in err
+
+
+def test_valu_gemv_is_asked_for_by_a_macro():
+    blk = "#define qmv_gg q1\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 2\n#define YT float\n#define QW_VALU 1\n"
+    ok, err, names = compile_check(blk)
+    assert ok and names == ["q1"]
