@@ -616,7 +616,8 @@ static unsigned cdiv(unsigned a, unsigned b) { return (a + b - 1) / b; }
 // Persistent grids: one 512-thread workgroup per compute unit (the LDS tables leave room for one), fewer if the
 // work is smaller. tasks are per-wave units; 8 waves per workgroup.
 static unsigned persistent_grid(const qw_gpu *g, unsigned wave_tasks, unsigned waves) { return umin((unsigned)g->ncu, cdiv(wave_tasks, waves)); }
-enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8 }; // // waves per workgroup of the gate/up + matvec kernels and of the down kernels
+// waves per workgroup: gate/up + matvec kernels, front / any-shape down kernels, down range kernels
+enum { QW_WAVES_GU = 12, QW_WAVES_DN = 8, QW_WAVES_DNR = 12 };
 
 static const char *fname_fmt(char *buf, size_t n, const char *fmt, ...) {
     va_list ap;
@@ -929,7 +930,7 @@ static bool tr_dn(qw_batch *b) {
         const int ch = fd == 8 ? 4 : p->I / 256;
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
-        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
+        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
     }
     // wider rows: one tile at a time, operand A from global memory
     fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any%s", p->fd, sfx);

@@ -595,14 +595,13 @@ template <class C, class L, class U> __device__ __forceinline__ void qw_pipeline
 // nw and cpr must be wave-uniform.
 // ready() is called exactly once by every wave, after the first loads are issued and before anything is consumed:
 // the place for the workgroup's set-up and barrier, so that the first memory round trip overlaps them.
-template <class C, class R, class U, class S>
+template <class C, int DEPTH = C::DEPTH, class R, class U, class S>
 __device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use, S ready) {
     if (w0 >= ntasks) {
         ready();
         return;
     }
     // DEPTH chunk buffers: the loads run DEPTH - 1 chunks ahead of the arithmetic
-    constexpr int DEPTH = C::DEPTH;
     C buf[DEPTH];
     const uint32_t total = ((ntasks - w0 + nw - 1) / nw) * cpr;
     uint32_t li = 0, ui = 0, lt = w0, lc = 0, ut = w0, uc = 0;

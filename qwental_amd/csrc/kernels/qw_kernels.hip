@@ -8,6 +8,7 @@
 #include "qw_common.hip.h"
 
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
+#define QW_WG_DN 768       // down range kernels: 12 waves
 #define QW_WG_GU 768       // gate/up and dense matvec: 12 waves, three per SIMD (a wave issues at most one instruction in ~6 cycles)
 #define QW_XF_MAXK 2560    // largest K whose activations are staged in LDS in fragment order (K * 32 bytes)
 
@@ -247,11 +248,14 @@ extern "C" __global__ __launch_bounds__(256) void qwk_router_w30(qwk_router_args
 // ================================================================ selection + dedupe (kernels/moe_gg.metal:123-189)
 // Per token (one wave): top-k by repeated maximum with ties to the lowest expert index, softmax over the picked logits
 // in rank order, sigmoid of the shared-expert logit; then the nbr * topk picks are deduplicated in order of first
-// appearance over the flat index. Scratch in LDS: ids[256], lead[256], um[256], first[1024], one counter.
+// appearance over the flat index. The unique list, masks and slots are assembled in LDS (qw_sel_cache: a weight kernel
+// that makes the selection itself reads them from there) and written to global memory in one pass at the end.
+struct qw_sel_cache { // the part of the selection record a weight kernel needs, in LDS
+    uint32_t U, ue[256], mask[256];
+    uint8_t slot[256 * 16];
+};
 struct qw_sel_scratch {
-    uint32_t ids[256], lead[256], um[256], first[1024], U;
-    uint32_t ue[256];            // results are assembled here and written to global memory in one pass at the end,
-    uint32_t slot[256 * 16 / 4]; // so that no barrier has to wait for global stores
+    uint32_t ids[256], lead[8], first[1024];
     float w[16 * 17];
 };
 
@@ -302,7 +306,7 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
         const uint32_t tok = tok0 + t * tstep;
         const float p = qw_fkey_inv(pk[t]), mx = __shfl(p, 0), ex = __expf(p - mx);
         float sm = 0;
-        for (uint32_t r = 0; r < K; r++) sm += __shfl(ex, r); // rank order
+        for (uint32_t r = 0; r < K; r++) sm += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), (int)r)); // rank order
         if (!on[t]) continue;
         if (lane < K) w[tok * (K + 1) + lane] = ex / sm;
         if (lane == K) w[tok * (K + 1) + K] = 1.0f / (1.0f + __expf(-logits[(size_t)tok * (E + 1) + E]));
@@ -339,17 +343,18 @@ __device__ __forceinline__ void select_token_any(const float *lg, float *v, uint
 
 __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 || E == 128 || E == 256 || E == 512 || E == 1024; }
 
-// The whole selection by one workgroup (any multiple of 64 threads). lgs: LDS scratch, 1024 floats per wave, used
-// only when E is not 64 * {1, 2, 4, 8, 16}.
-__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, float *lgs, bool store = true) {
+// The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
+// floats per wave, used only when E is not 64 * {1, 2, 4, 8, 16}. c is complete for every thread on return.
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store = true) {
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
+    // nothing the token loop writes is cleared here (rows of w past the batch only), so no barrier separates the two
     for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
-    for (uint32_t i = tid; i < GU; i += nth) s.ue[i] = 0, s.um[i] = 0;
-    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) s.slot[i] = 0;
-    for (uint32_t i = tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
-    __syncthreads();
+    for (uint32_t i = tid; i < GU; i += nth) c.ue[i] = 0, c.mask[i] = 0;
+    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
+    if (tid < 8) s.lead[tid] = 0;
+    for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
     if (fast) { // two tokens per wave at a time when there are more tokens than waves
         for (uint32_t t = wave; t < a.nbr; t += 2 * nwv) {
             const bool two = t + nwv < a.nbr;
@@ -365,31 +370,35 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
     __syncthreads();
-    if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid);
+    if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid); // first flat index of every picked expert
     __syncthreads();
+    // lead = this pair is its expert's first; every wave leaves the ballot of its leads (UM <= 256: four waves)
     uint32_t f = 0;
+    bool lead = false;
     if (tid < UM) {
         f = s.first[s.ids[tid]];
-        s.lead[tid] = f == tid;
+        lead = f == tid;
+    }
+    if (wave < 4) { // a wave index is uniform, so the ballot is taken by whole waves
+        const unsigned long long bal = __ballot(lead);
+        if (lane == 0) s.lead[2 * wave] = (uint32_t)bal, s.lead[2 * wave + 1] = (uint32_t)(bal >> 32);
     }
     __syncthreads();
-    if (wave == 0) { // exclusive prefix count of the lead flags -> unique index (stored + 1)
-        uint32_t carry = 0;
-        for (uint32_t c = 0; c < UM; c += 64) {
-            const uint32_t i = c + lane, fl = i < UM ? s.lead[i] : 0;
-            const unsigned long long bal = __ballot(fl);
-            const uint32_t pre = __popcll(bal & ((1ull << lane) - 1)) + carry;
-            carry += __popcll(bal);
-            if (fl) s.lead[i] = pre + 1;
-        }
-        if (lane == 0) s.U = carry;
-    }
-    __syncthreads();
+    // unique index of a pair = number of leads before its expert's first pair
     if (tid < UM) {
-        const uint32_t u = s.lead[f] - 1, t = tid / K;
-        atomicOr(&s.um[u], 1u << t);
-        ((uint8_t *)s.slot)[u * gnb + t] = (uint8_t)(tid % K);
-        if (f == tid) s.ue[u] = s.ids[tid];
+        uint32_t u = 0;
+        for (uint32_t w = 0; w < (f >> 6); w++) u += __popc(s.lead[2 * w]) + __popc(s.lead[2 * w + 1]);
+        const unsigned long long m = ((unsigned long long)s.lead[2 * (f >> 6) + 1] << 32 | s.lead[2 * (f >> 6)]) & ((1ull << (f & 63)) - 1);
+        u += __popcll(m);
+        const uint32_t t = tid / K;
+        atomicOr(&c.mask[u], 1u << t);
+        c.slot[u * gnb + t] = (uint8_t)(tid % K);
+        if (lead) c.ue[u] = s.ids[tid];
+    }
+    if (tid == 0) {
+        uint32_t U = 0;
+        for (uint32_t w = 0; w < 8; w++) U += __popc(s.lead[w]);
+        c.U = U;
     }
     __syncthreads();
     if (!store) return;
@@ -398,28 +407,26 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     const uint32_t n_slot = GU * gnb / 4, n_w = gnb * (K + 1), total = 1 + 2 * GU + n_slot + n_w;
     for (uint32_t i = tid; i < total; i += nth) {
         uint32_t v;
-        if (i == 0) v = s.U;
-        else if (i < 1 + GU) v = s.ue[i - 1];
-        else if (i < 1 + 2 * GU) v = (i - 1 - GU) < s.U ? s.um[i - 1 - GU] : 0;
-        else if (i < 1 + 2 * GU + n_slot) v = s.slot[i - 1 - 2 * GU];
+        if (i == 0) v = c.U;
+        else if (i < 1 + GU) v = c.ue[i - 1];
+        else if (i < 1 + 2 * GU) v = c.mask[i - 1 - GU];
+        else if (i < 1 + 2 * GU + n_slot) v = ((const uint32_t *)c.slot)[i - 1 - 2 * GU];
         else v = __builtin_bit_cast(uint32_t, s.w[i - 1 - 2 * GU - n_slot]);
         out[i] = v;
     }
+    __syncthreads(); // the caller may reuse the scratch
 }
 
 extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a) {
     __shared__ qw_sel_scratch s;
+    __shared__ qw_sel_cache c;
     __shared__ float lgs[16 * 1024];
-    select_all(a, s, lgs);
+    select_all(a, s, c, lgs);
 }
 
 // ================================================================ gate/up + SwiGLU (kernels/moe_gg.metal:428-447, 563-573, 600-631)
 // A tile holds gate rows j0..j0+7 (n < 8) and up rows j0..j0+7 (n >= 8) of one expert; the up results move over by
 // 8 lanes, and H = g / (1 + exp(-g)) * up is stored as binary16 hi + lo planes for the tokens that picked the expert.
-struct qw_sel_cache { // the part of the selection record a weight kernel needs, copied to LDS once
-    uint32_t U, ue[256], mask[256];
-    uint8_t slot[256 * 16];
-};
 __device__ __forceinline__ void qw_sel_load(qw_sel_cache &c, const uint8_t *sel, uint32_t K, uint32_t gnb) {
     const uint32_t GU = gnb * K;
     const uint32_t *ue = (const uint32_t *)(sel + QW_SEL_OFF_UE(gnb, K)), *mask = (const uint32_t *)(sel + QW_SEL_OFF_MASK(gnb, K));
@@ -473,13 +480,11 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
     if (a.logits) { // the selection, made here by every workgroup; the scratch lies where x is staged afterwards
         qw_sel_scratch &ss = *(qw_sel_scratch *)xf;
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
-        select_all(sa, ss, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
-        const uint32_t GU = a.gnb * a.topk;
-        for (uint32_t i = threadIdx.x; i < GU; i += blockDim.x) sc->ue[i] = ss.ue[i], sc->mask[i] = i < ss.U ? ss.um[i] : 0;
-        for (uint32_t i = threadIdx.x; i < GU * a.gnb / 4; i += blockDim.x) ((uint32_t *)sc->slot)[i] = ss.slot[i];
-        if (threadIdx.x == 0) sc->U = ss.U;
-    } else if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
-    __syncthreads();
+        select_all(sa, ss, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
+    } else {
+        if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+        __syncthreads();
+    }
     bool staged = false;
     auto ready = [&] {
         if (staged) return;
@@ -776,7 +781,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     }
 }
 #define QW_DN_RANGE(F, CH, FSD, CHSD, NAME)                                                       \
-    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_dn_args a) {                  \
+    extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
         __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; } L; \
         dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
     }
