@@ -56,10 +56,30 @@ float qwo_bf2f(uint16_t h) {
 static uint16_t rd16(const uint8_t *p) { return (uint16_t)(p[0] | p[1] << 8); }
 
 // ---------------------------------------------------------------- formats (src/gguf.c:15-25)
-int qwo_block_values(int type) { return type == 8 ? 32 : type == 21 ? 256 : 0; }
-int qwo_block_bytes(int type) { return type == 8 ? 34 : type == 21 ? 110 : 0; }
+int qwo_block_values(int type) {
+    switch (type) {
+    case 0: case 1: case 30: return 1;
+    case 8: case 20: return 32;
+    case 12: case 13: case 14: case 21: case 23: return 256;
+    default: return 0;
+    }
+}
+int qwo_block_bytes(int type) {
+    switch (type) {
+    case 0: return 4;
+    case 1: case 30: return 2;
+    case 8: return 34;
+    case 20: return 18;
+    case 12: return 144;
+    case 13: return 176;
+    case 14: return 210;
+    case 21: return 110;
+    case 23: return 136;
+    default: return 0;
+    }
+}
 size_t qwo_row_bytes(int type, int K) { return qwo_block_values(type) ? (size_t)K / (size_t)qwo_block_values(type) * (size_t)qwo_block_bytes(type) : 0; }
-bool qwo_dq_ok(int type) { return type == 8 || type == 21; }
+bool qwo_dq_ok(int type) { return qwo_block_values(type) != 0; }
 const uint32_t *qwo_iq3s_table(void) { return qwo_iq3s_grid; }
 
 // Q8_0, 34 bytes: d, qs[32] (src/ggml_dq.c:34-37)
@@ -87,9 +107,83 @@ static void dq_iq3_s(const uint8_t *b, float *y) {
     }
 }
 
+// The K-quant and 4-bit codebook formats, written as "value at position i of the block" (the reference walks each
+// block with running pointers, src/ggml_dq.c:39-118; the arithmetic per value is the same and in the same order).
+static const int8_t iq4nl_values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+
+// 6-bit scale and minimum of sub-block j (0..7) from the 12 packed bytes of Q4_K / Q5_K (src/ggml_dq.c:24-32):
+// j < 4: low six bits of bytes j and j + 4; j >= 4: a nibble of byte j + 4 with the top two bits of byte j - 4 / j.
+static void k4_scale_min(const uint8_t *p, int j, int *sc, int *mn) {
+    if (j < 4) {
+        *sc = p[j] & 63;
+        *mn = p[j + 4] & 63;
+    } else {
+        *sc = (p[j + 4] & 15) | (p[j - 4] >> 6 << 4);
+        *mn = (p[j + 4] >> 4) | (p[j] >> 6 << 4);
+    }
+}
+
+// Q4_K, 144 bytes: d @0, dmin @2, scales[12] @4, qs[128] @16. Values 64 g .. 64 g + 31 are the low nibbles of
+// qs[32 g ..], values 64 g + 32 .. 64 g + 63 the high nibbles (src/ggml_dq.c:39-54).
+static float q4_k_value(const uint8_t *b, int i) {
+    int sc, mn;
+    k4_scale_min(b + 4, i >> 5, &sc, &mn);
+    const uint8_t byte = b[16 + 32 * (i >> 6) + (i & 31)];
+    const int q = (i & 32) ? byte >> 4 : byte & 15;
+    const float ds = qwo_h2f(rd16(b)) * (float)sc, ms = qwo_h2f(rd16(b + 2)) * (float)mn;
+    return ds * (float)q - ms;
+}
+
+// Q5_K, 176 bytes: d, dmin, scales[12] @4, qh[32] @16, qs[128] @48. As Q4_K with a fifth bit: bit (i >> 5) of
+// qh[i & 31] (src/ggml_dq.c:56-75).
+static float q5_k_value(const uint8_t *b, int i) {
+    int sc, mn;
+    k4_scale_min(b + 4, i >> 5, &sc, &mn);
+    const uint8_t byte = b[48 + 32 * (i >> 6) + (i & 31)];
+    const int q = ((i & 32) ? byte >> 4 : byte & 15) + ((b[16 + (i & 31)] >> (i >> 5) & 1) ? 16 : 0);
+    const float ds = qwo_h2f(rd16(b)) * (float)sc, ms = qwo_h2f(rd16(b + 2)) * (float)mn;
+    return ds * (float)q - ms;
+}
+
+// Q6_K, 210 bytes: ql[128] @0, qh[64] @128, int8 scales[16] @192, d @208. Half h = i >> 7; inside a half, quarter
+// c = (i >> 5) & 3 and l = i & 31: low four bits from ql[64 h + 32 (c & 1) + l] (high nibble when c >= 2), top two
+// bits from bits 2 c, 2 c + 1 of qh[32 h + l]; scale index 8 h + 2 c + l / 16 (src/ggml_dq.c:77-98).
+static float q6_k_value(const uint8_t *b, int i) {
+    const int h = i >> 7, c = (i >> 5) & 3, l = i & 31;
+    const uint8_t lo = b[64 * h + 32 * (c & 1) + l];
+    const int q = (int)(((c & 2) ? lo >> 4 : lo & 15) | ((b[128 + 32 * h + l] >> (2 * c) & 3) << 4)) - 32;
+    const int sc = (int8_t)b[192 + 8 * h + 2 * c + l / 16];
+    return qwo_h2f(rd16(b + 208)) * (float)sc * (float)q;
+}
+
+// IQ4_NL, 18 bytes: d, qs[16]: value j < 16 from the low nibble of qs[j], value j + 16 from the high nibble,
+// through the 16-entry codebook (src/ggml_dq.c:100-107).
+static float iq4_nl_value(const uint8_t *b, int i) {
+    const uint8_t byte = b[2 + (i & 15)];
+    return qwo_h2f(rd16(b)) * (float)iq4nl_values[(i & 16) ? byte >> 4 : byte & 15];
+}
+
+// IQ4_XS, 136 bytes: d @0, scales_h (u16) @2, scales_l[4] @4, qs[128] @8. Sub-block s = i >> 5 has the six-bit
+// scale (nibble s of scales_l | two bits of scales_h << 4) - 32, and the nibble layout of IQ4_NL (src/ggml_dq.c:109-124).
+static float iq4_xs_value(const uint8_t *b, int i) {
+    const int s = i >> 5, j = i & 31;
+    const int ls = ((b[4 + s / 2] >> (4 * (s & 1))) & 15) | ((rd16(b + 2) >> (2 * s) & 3) << 4);
+    const uint8_t byte = b[8 + 16 * s + (j & 15)];
+    const float dl = qwo_h2f(rd16(b)) * (float)(ls - 32);
+    return dl * (float)iq4nl_values[(j & 16) ? byte >> 4 : byte & 15];
+}
+
 bool qwo_dq_row(int type, const void *src, float *dst, int K) {
     const uint8_t *s = src;
     switch (type) {
+    case 0: memcpy(dst, src, (size_t)K * 4); return true;
+    case 1: for (int i = 0; i < K; i++) dst[i] = qwo_h2f(rd16(s + 2 * i)); return true;
+    case 30: for (int i = 0; i < K; i++) dst[i] = qwo_bf2f(rd16(s + 2 * i)); return true;
+    case 12: for (int i = 0; i < K; i++) dst[i] = q4_k_value(s + 144 * (i >> 8), i & 255); return true;
+    case 13: for (int i = 0; i < K; i++) dst[i] = q5_k_value(s + 176 * (i >> 8), i & 255); return true;
+    case 14: for (int i = 0; i < K; i++) dst[i] = q6_k_value(s + 210 * (i >> 8), i & 255); return true;
+    case 20: for (int i = 0; i < K; i++) dst[i] = iq4_nl_value(s + 18 * (i >> 5), i & 31); return true;
+    case 23: for (int i = 0; i < K; i++) dst[i] = iq4_xs_value(s + 136 * (i >> 8), i & 255); return true;
     case 8: for (int i = 0; i < K / 32; i++) dq_q8_0(s + 34 * i, dst + 32 * i); return true;
     case 21: for (int i = 0; i < K / 256; i++) dq_iq3_s(s + 110 * i, dst + 256 * i); return true;
     default: return false;

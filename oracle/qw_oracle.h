@@ -8,6 +8,11 @@
 //   qwo_dq_row type 8 (Q8_0)  pinned: compared against the reference's own src/ggml_dq.c compiled
 //                             into oracle/_ref (when that is built), against hand-made known answers,
 //                             and against the closed form int8 * fp16.
+//   qwo_dq_row types 12, 13, 14, 20, 23 (Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS) and 0, 1, 30 (float, binary16,
+//                             bfloat16)  pinned: written per value position (the reference walks blocks with
+//                             running pointers), compared bit for bit against the reference's src/ggml_dq.c
+//                             in oracle/_ref on random blocks, against the committed values that library gave
+//                             (tests/golden/dq_formats.npz) and against one hand block per format.
 //   qwo_dq_row type 21 (IQ3_S) pinned by: hand-made known-answer blocks (all-ones, all-negative, scale
 //                             31, high-bit codebook entry 256, denormal / largest fp16 scale), the
 //                             codebook CRC-32 0xf576e4f3, the closed form +-d*(2s+1)*g, and agreement of
@@ -41,7 +46,8 @@ int qwo_block_bytes(int type);
 size_t qwo_row_bytes(int type, int K);
 
 // ---- dequantisation. Same contract as the reference's qw_ggml_dq_row (src/ggml_dq.h:8): one row of K
-// values, K a multiple of the block size; false when the type is not handled. Types: 8 (Q8_0), 21 (IQ3_S).
+// values, K a multiple of the block size; false when the type is not handled. Types: 0, 1, 30 (float, binary16,
+// bfloat16), 8 (Q8_0), 12, 13, 14 (Q4_K, Q5_K, Q6_K), 20, 23 (IQ4_NL, IQ4_XS), 21 (IQ3_S).
 bool qwo_dq_ok(int type);
 bool qwo_dq_row(int type, const void *src, float *dst, int K);
 // Second, independent formulation of the same values: 16-value units decoded through the pre-signed

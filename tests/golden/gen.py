@@ -33,6 +33,32 @@ def blocks(seed, ftype, n):
     return out
 
 
+# ggml type -> (values per block, bytes per block, byte offsets of the binary16 scale fields)
+FORMATS = {8: (32, 34, (0,)), 21: (256, 110, (0,)), 12: (256, 144, (0, 2)), 13: (256, 176, (0, 2)), 14: (256, 210, (208,)),
+           20: (32, 18, (0,)), 23: (256, 136, (0,)), 1: (1, 2, ()), 30: (1, 2, ())}
+
+
+def blocks_fmt(seed, ftype, n):
+    """n blocks of any format of FORMATS, uint8 [n, block bytes]: hashed payload, every binary16 scale field finite
+    and positive as in blocks(). Types 1 and 30 (plain binary16 / bfloat16 values): finite values of magnitude
+    up to about 4."""
+    if ftype in (8, 21):
+        return blocks(seed, ftype, n)
+    _, bb, scales = FORMATS[ftype]
+    if ftype == 1:
+        return halves(seed, n, 4.0).view(np.uint8).reshape(n, 2).copy()
+    if ftype == 30:
+        f = halves(seed, n, 4.0).astype(np.float32) * np.float32(1.0 + 2.0 ** -9)  # not all representable in binary16
+        return (f.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(n, 2).copy()
+    out = raw_bytes(seed, n * bb).reshape(n, bb)
+    for k, off in enumerate(scales):
+        h = hash64(seed ^ (0x5bd1 + 77 * k), n)
+        d = (np.uint16(5 << 10) + (h & np.uint64(0x7FF)).astype(np.uint16)).astype(np.uint16)
+        out[:, off] = (d & 0xFF).astype(np.uint8)
+        out[:, off + 1] = (d >> 8).astype(np.uint8)
+    return out
+
+
 def halves(seed, n, scale):
     """n binary16 values, roughly uniform in (-scale, scale)."""
     h = hash64(seed, n)

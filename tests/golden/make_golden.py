@@ -6,6 +6,10 @@ The reference stores no vectors for this path (its comparators recompute from mo
                 kernels/moe_iq.metal:102-118 gives (written here, independent of the C oracle; both must agree)
   dq_q8_0.npz   hashed blocks with the values of the closed form int8 * d, checked against the reference's own
                 src/ggml_dq.c (oracle/_ref) when that is built
+  dq_formats.npz  hashed blocks of Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, binary16 and bfloat16 rows (inputs rebuilt from
+                gen.py) with the values the reference's own src/ggml_dq.c gives (oracle/_ref, built from where
+                the reference lies: this file can only be remade where the reference tree is present), plus hand
+                known-answer blocks per format
   qmv.npz       y = W x in float64 for small IQ3_S and Q8_0 matrices (inputs rebuilt from gen.py)
   select.npz    logits with ties and duplicates -> ids, weights and the selection record
   moe.npz       two small layers (inputs rebuilt from gen.py) -> logits, ids, float64 outputs
@@ -65,6 +69,52 @@ def kat_blocks():
     return np.stack(cases), exp
 
 
+def kat_formats():
+    """One hand block per format whose values can be read off the layout (scale fields 1.0 = 0x3C00)."""
+    one = [0x00, 0x3C]
+    raw, exp = {}, {}
+    # Q4_K: d = 1, dmin = 1; sub-block 0: scale 2, min 3 (bytes 4 and 8); others zero. qs[l] = l & 15 | 0xF0.
+    b = np.zeros(144, np.uint8)
+    b[0:2], b[2:4], b[4], b[8] = one, one, 2, 3
+    b[16:144] = np.tile((np.arange(32) & 15) | 0xF0, 4)
+    e = np.zeros(256, np.float32)
+    e[:32] = 2.0 * (np.arange(32) & 15) - 3.0  # every other sub-block: 0 * q - 0
+    raw[12], exp[12] = b.reshape(1, -1), e.reshape(1, -1)
+    # Q5_K: as above with the fifth bit of sub-block 0 set for odd l (bit 0 of qh[l]).
+    b = np.zeros(176, np.uint8)
+    b[0:2], b[2:4], b[4], b[8] = one, one, 2, 3
+    b[16:48] = np.arange(32) & 1
+    b[48:176] = np.tile(np.arange(32) & 15, 4)
+    e = np.zeros(256, np.float32)
+    e[:32] = 2.0 * ((np.arange(32) & 15) + 16 * (np.arange(32) & 1)) - 3.0
+    raw[13], exp[13] = b.reshape(1, -1), e.reshape(1, -1)
+    # Q6_K: d = 1, scales 1..16, every six-bit value 33 (ql nibbles 1, qh pairs 2) -> q = 1: value = scale of its group.
+    b = np.zeros(210, np.uint8)
+    b[0:128], b[128:192], b[192:208], b[208:210] = 0x11, 0xAA, np.arange(1, 17), one
+    e = np.empty(256, np.float32)
+    for i in range(256):
+        e[i] = 1 + 8 * (i >> 7) + 2 * ((i >> 5) & 3) + (i & 31) // 16
+    raw[14], exp[14] = b.reshape(1, -1), e.reshape(1, -1)
+    # IQ4_NL: d = 1, qs[j] = j | (15 - j) << 4 -> codebook in order, then reversed.
+    kv = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
+    b = np.zeros(18, np.uint8)
+    b[0:2], b[2:18] = one, np.arange(16) | ((15 - np.arange(16)) << 4)
+    raw[20], exp[20] = b.reshape(1, -1), np.concatenate([kv, kv[::-1]]).reshape(1, -1)
+    # IQ4_XS: d = 1; six-bit scales 33, 34, ... 40 (low nibbles 1..8, high bits 2) -> factors 1..8; nibbles as IQ4_NL.
+    b = np.zeros(136, np.uint8)
+    b[0:2] = one
+    b[2:4] = np.array([0xAAAA], np.uint16).view(np.uint8)
+    b[4:8] = [0x21, 0x43, 0x65, 0x87]
+    b[8:136] = np.tile(np.arange(16) | ((15 - np.arange(16)) << 4), 8)
+    raw[23] = b.reshape(1, -1)
+    exp[23] = np.concatenate([np.concatenate([kv, kv[::-1]]) * (s + 1) for s in range(8)]).astype(np.float32).reshape(1, -1)
+    # bfloat16: 1.0, -2.0, 2^-126, the largest finite value
+    b = np.array([0x3F80, 0xC000, 0x0080, 0x7F7F], np.uint16)
+    raw[30] = b.view(np.uint8).reshape(1, -1)
+    exp[30] = (b.astype(np.uint32) << 16).view(np.float32).reshape(1, -1)
+    return raw, exp
+
+
 def main():
     grid = o.iq3s_table()
     assert zlib.crc32(grid.astype("<u4").tobytes()) == 0xF576E4F3
@@ -93,6 +143,23 @@ def main():
     except (OSError, FileNotFoundError) as e:
         print("Q8_0: oracle/_ref not built (%s)" % e)
     np.savez_compressed(os.path.join(HERE, "dq_q8_0.npz"), raw=raw8, expect=exp8)
+    # ---- the other formats: expected values from the reference's compiled src/ggml_dq.c
+    fm = {}
+    for ft in (12, 13, 14, 20, 23, 1, 30):
+        qb, bb, _ = gen.FORMATS[ft]
+        K = 512 if qb > 1 else 384
+        raw = gen.blocks_fmt(500 + ft, ft, 6 * (K // qb)).reshape(6, -1)
+        ref = o.ref_dq_rows(ft, raw, K)
+        if ref is None:
+            raise SystemExit("oracle/_ref is not built: dq_formats.npz needs the reference tree (the other files were written)")
+        assert np.array_equal(o.dq_rows(ft, raw, K).view(np.uint32), ref.view(np.uint32)), "oracle disagrees with the reference for type %d" % ft
+        fm["expect_f%d_k%d" % (ft, K)] = ref
+    kraw, kexp = kat_formats()
+    for ft in kraw:
+        assert np.array_equal(o.dq_rows(ft, kraw[ft], kraw[ft].shape[1] // gen.FORMATS[ft][1] * gen.FORMATS[ft][0]), kexp[ft]), "hand case, type %d" % ft
+        assert np.array_equal(o.ref_dq_rows(ft, kraw[ft], kexp[ft].shape[1]), kexp[ft]), "hand case against the reference, type %d" % ft
+        fm["hand_raw_f%d" % ft], fm["hand_expect_f%d" % ft] = kraw[ft], kexp[ft]
+    np.savez_compressed(os.path.join(HERE, "dq_formats.npz"), **fm)
     # ---- matvec (inputs from gen.py)
     qm = {}
     for ft, K, N, seed in ((21, 512, 48, 201), (21, 2048, 19, 202), (8, 512, 48, 203), (8, 96, 7, 204)):

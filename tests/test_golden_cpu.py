@@ -42,6 +42,29 @@ def test_q8_0_fixture(oracle):
     assert np.array_equal(oracle.dq_rows(8, g["raw"], 32).view(np.uint32), g["expect"].view(np.uint32))
 
 
+def test_formats_fixture(oracle):
+    """Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, binary16, bfloat16: the oracle against the values the reference's own
+    src/ggml_dq.c gave for hashed blocks, and against the hand blocks."""
+    g = load("dq_formats.npz")
+    seen = set()
+    for key in g.files:
+        if key.startswith("expect_f"):
+            ft, K = int(key.split("_")[1][1:]), int(key.split("_")[2][1:])
+            qb = gen.FORMATS[ft][0]
+            raw = gen.blocks_fmt(500 + ft, ft, 6 * (K // qb)).reshape(6, -1)
+            got = oracle.dq_rows(ft, raw, K)
+            assert np.array_equal(got.view(np.uint32), g[key].view(np.uint32)), ft
+            assert np.isfinite(got).all() and np.abs(got).max() > 0
+            seen.add(ft)
+        elif key.startswith("hand_raw_f"):
+            ft = int(key[len("hand_raw_f"):])
+            exp = g["hand_expect_f%d" % ft]
+            assert np.array_equal(oracle.dq_rows(ft, g[key], exp.shape[1]).view(np.uint32), exp.view(np.uint32)), ft
+    assert seen == {12, 13, 14, 20, 23, 1, 30}
+    assert g["hand_expect_f14"][0, 0] == 1.0 and g["hand_expect_f14"][0, 255] == 16.0  # the hand cases are in the file
+    assert g["hand_expect_f20"][0, 0] == -127.0 and g["hand_expect_f12"][0, 5] == 7.0
+
+
 def qmv_cases():
     g = load("qmv.npz")
     for key in g.files:
