@@ -3,6 +3,7 @@
  * These functions restate, against gpu.h only, what the reference's engine does for this path: build the kernel
  * name and the "#define" block, compile on a miss, bind by index, dispatch. They mirror
  *     qmv_gg()      src/engine.c:689-724      qw_path_qmv_gg()
+ *     qmv_ggm()     src/engine.c:752-771      qw_path_qmv_ggm()
  *     gg_router()   src/engine.c:544-552      qw_path_gg_router()
  *     gg_kernel()   src/engine.c:460-517      (internal)
  *     gg_moe()      src/engine.c:568-647      qw_path_gg_moe()
@@ -24,7 +25,8 @@ extern "C" {
 typedef struct {
     const qw_buf *buf;
     size_t offset;
-    int type; /* ggml type: 8 = Q8_0, 21 = IQ3_S; router: 1 = F16, 30 = BF16 */
+    int type; /* ggml type. MoE weights: 8 = Q8_0, 21 = IQ3_S; router: 1 = F16, 30 = BF16; dense matvec: also
+               * 12, 13, 14 = Q4_K, Q5_K, Q6_K, 20 = IQ4_NL, 23 = IQ4_XS, 1, 30 */
 } qw_tensor;
 
 /* One MoE layer's weights (the fields of the reference's qw_moe that this path reads, src/model.h). */
@@ -51,6 +53,10 @@ int qw_path_nbv(int nb);
 /* y[b][0..N) = W x[b], b < nb; x stride K, y stride N; fout selects float (else binary16) output. */
 bool qw_path_qmv_gg(qw_path *p, qw_batch *b, const qw_tensor *W, int N, int K, const qw_buf *x, size_t xoff, const qw_buf *y,
                     size_t yoff, int nb, bool fout);
+/* n <= 4 matrices W[i] (N[i] rows of K values, K a multiple of 256 up to 4096; types from 1, 12, 13, 14, 20, 23, 30,
+ * mixed freely) times the same x [nb][K], one launch: y[i][b][0..N[i]) with row stride N[i]; nb <= 16. The weights'
+ * first bytes must be 16-byte aligned. */
+bool qw_path_qmv_ggm(qw_path *p, qw_batch *b, const qw_tensor *W, const int *N, int n, int K, const qw_buf *x, const qw_buf *const *y, int nb, bool fout);
 /* logits[nb][E + 1] alone. */
 bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg);
 /* The whole layer: x [nb][D] binary16 -> out [nb][D] binary16; lg and sel receive the logits and the selection. */

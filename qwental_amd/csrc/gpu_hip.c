@@ -28,7 +28,7 @@ enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES 
 
 // ---------------------------------------------------------------- records
 typedef enum {
-    FAM_DQ_TEST, FAM_QMV_GG, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
+    FAM_DQ_TEST, FAM_QMV_GG, FAM_QMV_GGM, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
     FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
     FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PF, // ragged packing and the grouped product
 } qw_family;
@@ -39,6 +39,7 @@ typedef struct { // parameters taken from the define block
     int fgu, fd, fsg, fsu, fsd, rbf, rwf; // formats; rbf: router inside moe_pre_gg; rwf: router weight type (1 / 30)
     int tm;                              // packing: rows per tile entry
     int valu;                            // qmv_gg: QW_VALU in the block asks for the VALU GEMV (measurement)
+    int nmat, gf[4];                     // qmv_ggm: number of matrices and their formats
 } qw_kparams;
 
 struct qw_kernel {
@@ -275,9 +276,22 @@ static bool def_int(const qw_def *d, int n, const char *name, int *out) {
     return true;
 }
 
-static bool fmt_ok(int f) { return f == 8 || f == 21; }
-static int fmt_qb(int f) { return f == 8 ? 32 : 256; }
-static int fmt_bb(int f) { return f == 8 ? 34 : 110; }
+static bool fmt_ok(int f) { return f == 8 || f == 21; } // formats of the MoE kernels
+// formats of the multi-format dense matvec: binary16, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, bfloat16 (src/gguf.c:15-25)
+static bool kq_ok(int f) { return f == 1 || f == 12 || f == 13 || f == 14 || f == 20 || f == 23 || f == 30; }
+static int fmt_qb(int f) { return f == 1 || f == 30 || f == 8 || f == 20 ? 32 : 256; } // values per decoding unit (plain rows: 32 at a time)
+static int fmt_bb(int f) {
+    switch (f) {
+    case 1: case 30: return 64;
+    case 8: return 34;
+    case 20: return 18;
+    case 12: return 144;
+    case 13: return 176;
+    case 14: return 210;
+    case 23: return 136;
+    default: return 110;
+    }
+}
 static size_t fmt_rb(int f, int K) { return (size_t)(K / fmt_qb(f)) * (size_t)fmt_bb(f); }
 
 static bool reg_kernel(qw_gpu *g, const qw_def *d, int n, const char *base, qw_family fam, const qw_kparams *p, char *err, size_t errlen) {
@@ -304,21 +318,54 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
     bool ok = true;
 #define FAIL(...) do { snprintf(err, errlen, __VA_ARGS__); ok = false; goto out; } while (0)
     if (def_int(d, n, "DQ_TEST", &v)) { // tools/dqtest.c:27
-        if (!fmt_ok(v)) FAIL("dq_test: ggml type %d has no gfx950 build (have 8, 21)", v);
+        if (!fmt_ok(v) && !kq_ok(v)) FAIL("dq_test: ggml type %d has no gfx950 build (have 1, 8, 12, 13, 14, 20, 21, 23, 30)", v);
         p.F = v;
         if (!reg_kernel(g, d, n, "dq_test", FAM_DQ_TEST, &p, err, errlen)) { ok = false; goto out; }
     }
     if (def_get(d, n, "GF") && def_get(d, n, "KD")) { // src/engine.c:709-710
         if (!def_int(d, n, "GF", &p.F) || !def_int(d, n, "KD", &p.K) || !def_int(d, n, "RB", &p.RB) || !def_int(d, n, "NB", &p.NB))
             FAIL("qmv_gg: GF, KD, RB and NB must be integer macros");
-        if (!fmt_ok(p.F)) FAIL("qmv_gg: ggml type %d has no gfx950 build (have 8, 21)", p.F);
+        if (!fmt_ok(p.F) && !kq_ok(p.F)) FAIL("qmv_gg: ggml type %d has no gfx950 build (have 1, 8, 12, 13, 14, 20, 21, 23, 30)", p.F);
         if (p.K <= 0 || p.K % fmt_qb(p.F) || (size_t)p.RB != fmt_rb(p.F, p.K)) FAIL("qmv_gg: K %d / row bytes %d do not fit type %d", p.K, p.RB, p.F);
+        if (kq_ok(p.F) && p.K > (int)QW_KQ_MAXK) FAIL("qmv_gg: K %d beyond %u for type %d in this build", p.K, QW_KQ_MAXK, p.F);
         if (p.NB < 1 || p.NB > 16) FAIL("qmv_gg: NB %d outside 1..16", p.NB);
         const char *yt = def_get(d, n, "YT");
         p.yfloat = yt && !strcmp(yt, "float");
         p.valu = def_get(d, n, "QW_VALU") != NULL;
         if (yt && strcmp(yt, "float") && strcmp(yt, "half")) FAIL("qmv_gg: YT %s is neither half nor float", yt);
         if (!reg_kernel(g, d, n, "qmv_gg", FAM_QMV_GG, &p, err, errlen)) { ok = false; goto out; }
+    }
+    if (def_get(d, n, "NMAT") && def_get(d, n, "GF0")) { // src/engine.c:730-744: one launch for up to four matrices over the same activations
+        p = (qw_kparams){0};
+        if (!def_int(d, n, "KD", &p.K) || !def_int(d, n, "NB", &p.NB) || !def_int(d, n, "NMAT", &p.nmat) || !def_int(d, n, "GF0", &p.gf[0]))
+            FAIL("qmv_ggm: KD, NB, NMAT and GF0 must be integer macros");
+        if (p.nmat < 1 || p.nmat > 4) FAIL("qmv_ggm: NMAT %d outside 1..4", p.nmat);
+        if (p.NB < 0 || p.NB > 16) FAIL("qmv_ggm: NB %d outside 0..16", p.NB);
+        for (int j = 1; j < 4; j++) {
+            char nm[8];
+            snprintf(nm, sizeof nm, "GF%d", j);
+            if (!def_int(d, n, nm, &p.gf[j])) p.gf[j] = p.gf[0]; // kernels/qmv_ggm.metal:20-28
+        }
+        for (int j = 0; j < p.nmat; j++)
+            if (!kq_ok(p.gf[j])) FAIL("qmv_ggm: ggml type %d has no gfx950 build here (have 1, 12, 13, 14, 20, 23, 30)", p.gf[j]);
+        if (p.K <= 0 || p.K % 256 || p.K > (int)QW_KQ_MAXK) FAIL("qmv_ggm: KD %d must be a multiple of 256 up to %u", p.K, QW_KQ_MAXK);
+        const char *yt = def_get(d, n, "YT");
+        if (yt && strcmp(yt, "float") && strcmp(yt, "half")) FAIL("qmv_ggm: YT %s is neither half nor float", yt);
+        p.yfloat = yt && !strcmp(yt, "float");
+        if (p.NB > 0) {
+            if (!reg_kernel(g, d, n, "qmv_ggm", FAM_QMV_GGM, &p, err, errlen)) { ok = false; goto out; }
+        } else { // NB 0: one kernel per token count, <name>_b1 ... (kernels/qmv_ggm.metal:251-262; here up to 16)
+            const char *nm = def_get(d, n, "qmv_ggm");
+            if (!nm || !*nm) nm = "qmv_ggm";
+            for (int nb = 1; nb <= 16; nb++) {
+                char full[128];
+                snprintf(full, sizeof full, "%s_b%d", nm, nb);
+                qw_def one = {"qmv_ggm", ""};
+                snprintf(one.val, sizeof one.val, "%s", full);
+                p.NB = nb;
+                if (!reg_kernel(g, &one, 1, "qmv_ggm", FAM_QMV_GGM, &p, err, errlen)) { ok = false; goto out; }
+            }
+        }
     }
     const bool router = def_get(d, n, "GG_ROUTER") != NULL;
     int part = -1;
@@ -642,9 +689,13 @@ static bool tr_dq_test(qw_batch *b, unsigned gx) { // tools/dqtest.c:39-45: 0 W,
     const qw_kparams *p = &b->k->p;
     uint32_t a2[2];
     if (!bind_bytes(b, 2, a2, sizeof a2, "{K, rowbytes}")) return false;
-    if (a2[0] == 0 || a2[0] % (p->F == 21 ? 256 : 32) || a2[1] < fmt_rb(p->F, (int)a2[0])) return fail(b, "dq_test: K %u / row bytes %u do not fit type %d", a2[0], a2[1], p->F);
-    qwk_dq_args a = {.K = a2[0], .rowbytes = a2[1], .rows = gx};
+    if (a2[0] == 0 || a2[0] % (unsigned)fmt_qb(p->F) || a2[1] < fmt_rb(p->F, (int)a2[0])) return fail(b, "dq_test: K %u / row bytes %u do not fit type %d", a2[0], a2[1], p->F);
+    qwk_dq_args a = {.K = a2[0], .rowbytes = a2[1], .rows = gx, .fmt = (uint32_t)p->F};
     if (!bind_ptr(b, 0, (size_t)gx * a2[1], false, "W", (void **)&a.W) || !bind_ptr(b, 1, (size_t)gx * a2[0] * 4, true, "y", (void **)&a.y)) return false;
+    if (kq_ok(p->F)) {
+        if ((b->buf[0].h && b->buf[0].off % 16) || a2[1] % (p->F == 14 || p->F == 20 ? 2 : p->F == 23 ? 8 : 16)) return fail(b, "dq_test: rows of type %d must keep the alignment of its blocks (offset %zu, row bytes %u)", p->F, b->buf[0].off, a2[1]);
+        return add_launch(b, "qwk_dq_test_kq", gx, 64, &a, sizeof a);
+    }
     return add_launch(b, p->F == 21 ? "qwk_dq_test_f21" : "qwk_dq_test_f8", gx, 64, &a, sizeof a);
 }
 
@@ -654,10 +705,56 @@ static const void *glut(const qw_gpu *g) { return (const char *)g->tabs + QW_TAB
 static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1; }
 
 static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf *hb, const void *B, uint64_t ntiles, uint32_t nblk, uint32_t rowbytes, uint32_t split);
+// One launch of the multi-format matvec over nmat matrices; W / y already bound into a.
+static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a) {
+    unsigned tiles = 0;
+    a->sums = 0;
+    for (uint32_t j = 0; j < a->nmat; j++) {
+        a->ntiles[j] = cdiv(a->N[j], 16);
+        tiles += a->ntiles[j];
+        if (a->fmt[j] == 12 || a->fmt[j] == 13) a->sums = 1;
+    }
+    if (!tiles) return true;
+    return add_launch(b, "qwk_qmvm", persistent_grid(b->g, tiles, QW_WAVES_GU), 64 * QW_WAVES_GU, a, sizeof *a);
+}
+
+static bool tr_qmvm(qw_batch *b) { // src/engine.c:752-771: 0..3 W, 4 x, 5..8 y, 9 {N[4], off[4], total, xstride}; y stride = N
+    const qw_kparams *p = &b->k->p;
+    struct { uint32_t N[4], off[4], total, xstride; } in;
+    if (!bind_bytes(b, 9, &in, sizeof in, "{N[4], off[4], total, xstride}")) return false;
+    qwk_qmvm_args a = {.K = (uint32_t)p->K, .xstride = in.xstride, .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat, .nmat = (uint32_t)p->nmat};
+    if (a.xstride < a.K || a.xstride % 8) return fail(b, "qmv_ggm: xstride %u (needs >= K, multiple of 8)", a.xstride);
+    if (b->buf[4].h && b->buf[4].off % 16) return fail(b, "qmv_ggm: x offset %zu is not 16-byte aligned", b->buf[4].off);
+    if (!bind_ptr(b, 4, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x)) return false;
+    uint32_t total = 0;
+    for (int j = 0; j < p->nmat; j++) {
+        a.N[j] = in.N[j], a.fmt[j] = (uint32_t)p->gf[j], a.rowbytes[j] = (uint32_t)fmt_rb(p->gf[j], p->K), a.ystride[j] = in.N[j];
+        if (in.off[j] != total) return fail(b, "qmv_ggm: off[%d] = %u, expected %u (rows of the matrices before it)", j, in.off[j], total);
+        total += in.N[j];
+        if (!in.N[j]) return fail(b, "qmv_ggm: matrix %d has no rows", j);
+        if (b->buf[j].h && b->buf[j].off % 16) return fail(b, "qmv_ggm: offset %zu of matrix %d is not 16-byte aligned", b->buf[j].off, j);
+        if (!bind_ptr(b, (unsigned)j, (size_t)a.N[j] * a.rowbytes[j], false, "W", (void **)&a.W[j]) ||
+            !bind_ptr(b, 5u + (unsigned)j, (size_t)a.nb * a.N[j] * (a.yfloat ? 4 : 2), true, "y", &a.y[j])) return false;
+    }
+    if (in.total != total) return fail(b, "qmv_ggm: total %u, the matrices have %u rows", in.total, total);
+    return launch_qmvm(b, &a);
+}
+
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
     const qw_kparams *p = &b->k->p;
     uint32_t a4[4];
     if (!bind_bytes(b, 5, a4, sizeof a4, "{N, xstride, ystride, pad}")) return false;
+    if (kq_ok(p->F)) { // the multi-format kernel with one matrix
+        qwk_qmvm_args m = {.K = (uint32_t)p->K, .xstride = a4[1], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat, .nmat = 1,
+                           .N = {a4[0]}, .fmt = {(uint32_t)p->F}, .rowbytes = {(uint32_t)p->RB}, .ystride = {a4[2]}};
+        if (!m.N[0]) return true;
+        if (m.xstride < m.K || m.xstride % 8 || m.ystride[0] < m.N[0]) return fail(b, "qmv_gg: xstride %u (needs >= K, multiple of 8) / ystride %u (needs >= N)", m.xstride, m.ystride[0]);
+        if ((b->buf[3].h && b->buf[3].off % 16) || (b->buf[0].h && b->buf[0].off % 16)) return fail(b, "qmv_gg: x / W offsets must be 16-byte aligned");
+        if (!bind_ptr(b, 0, (size_t)m.N[0] * m.rowbytes[0], false, "W", (void **)&m.W[0]) ||
+            !bind_ptr(b, 3, ((size_t)(m.nb - 1) * m.xstride + m.K) * 2, false, "x", (void **)&m.x) ||
+            !bind_ptr(b, 4, ((size_t)(m.nb - 1) * m.ystride[0] + m.N[0]) * (m.yfloat ? 4 : 2), true, "y", &m.y[0])) return false;
+        return launch_qmvm(b, &m);
+    }
     qwk_qmv_args a = {.N = a4[0], .K = (uint32_t)p->K, .rowbytes = (uint32_t)p->RB, .xstride = a4[1], .ystride = a4[2], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat,
                       .glut = glut(b->g)};
     if (a.N == 0) return true;
@@ -1048,6 +1145,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
+    case FAM_QMV_GGM: ok = tr_qmvm(b); break;
     case FAM_QMV_GG: ok = tr_qmv(b); break;
     case FAM_ROUTER: ok = tr_router(b); break;
     case FAM_TAB_INIT: ok = tr_tab_init(b); break;

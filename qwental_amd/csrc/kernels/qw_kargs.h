@@ -23,7 +23,7 @@
 typedef struct { /* dq_test: rows x K values to float */
     const uint8_t *W;
     float *y;
-    uint32_t K, rowbytes, rows, pad;
+    uint32_t K, rowbytes, rows, fmt; /* fmt: used by the kernel that serves the formats 1, 12, 13, 14, 20, 23, 30 */
 } qwk_dq_args;
 
 typedef struct { /* dense matvec, y[b][row] = W[row] . x[b] */
@@ -33,6 +33,17 @@ typedef struct { /* dense matvec, y[b][row] = W[row] . x[b] */
     uint32_t N, K, rowbytes, xstride, ystride, nb, yfloat, ntiles;
     const void *glut; /* the backend's pre-signed IQ3_S table in global memory (64 KB) */
 } qwk_qmv_args;
+
+/* Dense matvec over up to four matrices that share the activations (kernels/qmv_ggm.metal:232-262; one matrix:
+ * kernels/qmv_gg.metal:17-39) for the formats 1, 12, 13, 14, 20, 23, 30. 16-row tiles of all matrices form one list. */
+#define QW_KQ_MAXK 4096u /* activations of up to 16 tokens staged in LDS: K * 32 bytes */
+typedef struct {
+    const uint8_t *W[4];
+    void *y[4];        /* [nb][ystride[j]] binary16 or float */
+    const uint16_t *x; /* binary16 [nb][xstride] */
+    uint32_t N[4], fmt[4], rowbytes[4], ystride[4], ntiles[4];
+    uint32_t K, xstride, nb, yfloat, nmat, sums; /* sums: some matrix is Q4_K / Q5_K (needs the 32-value sums of x) */
+} qwk_qmvm_args;
 
 typedef struct { /* router: logits[t][r], r in [0, E] (row E = shared gate vector), row stride E + 1 */
     const uint16_t *Wr, *Wsg, *x;

@@ -6,6 +6,7 @@
 // walks its own list of 16-row tiles through a two-chunk register pipeline: the loads of the next chunk are issued
 // before the current one is decoded, so every wave keeps about one tile of weight bytes in flight.
 #include "qw_common.hip.h"
+#include "qw_kquants.hip.h"
 
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
 #define QW_WG_DN 768       // down range kernels: 12 waves
@@ -50,6 +51,33 @@ extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f21(qwk_dq_args a) 
     dq_test_body<21>(a, lut);
 }
 extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f8(qwk_dq_args a) { dq_test_body<8>(a, nullptr); }
+
+// The formats of qw_kquants.hip.h: every lane decodes the slice of a block it would supply to the matrix instruction
+// and writes the values as the reference computes them (scale * integer - min in float). Grid: rows x 64.
+template <int F> __device__ __forceinline__ void dq_test_kq(const qwk_dq_args &a, const uint32_t *tab) {
+    const uint8_t *row = a.W + (size_t)blockIdx.x * a.rowbytes;
+    float *y = a.y + (size_t)blockIdx.x * a.K;
+    for (uint32_t i = threadIdx.x; i < a.K / qw_kq<F>::BLK_K * 4; i += blockDim.x) {
+        const uint32_t blk = i >> 2, kg = i & 3;
+        qw_kq<F> b;
+        b.load(row + (size_t)qw_kq<F>::BLK_B * blk, kg);
+        qw_kq_values<F>(b, tab, kg, y + (size_t)qw_kq<F>::BLK_K * blk);
+    }
+}
+extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_kq(qwk_dq_args a) {
+    __shared__ uint32_t tab[QW_KQ_TAB];
+    qw_kq_tab_build(tab);
+    __syncthreads();
+    switch (a.fmt) {
+    case 1: dq_test_kq<1>(a, tab); break;
+    case 12: dq_test_kq<12>(a, tab); break;
+    case 13: dq_test_kq<13>(a, tab); break;
+    case 14: dq_test_kq<14>(a, tab); break;
+    case 20: dq_test_kq<20>(a, tab); break;
+    case 23: dq_test_kq<23>(a, tab); break;
+    case 30: dq_test_kq<30>(a, tab); break;
+    }
+}
 
 // ================================================================ lookup-table buffer (kernels/moe_gg.metal:495-515)
 // Only the IQ3_S section is produced; the sections of formats without a gfx950 build stay zero. Grid: 32 x 256.
@@ -122,6 +150,74 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
     }
 QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
 QW_QMV(121, 2, true, _c2) QW_QMV(121, 1, true, _c1) // packed IQ3_S: a.rowbytes = bytes of a 16-row tile
+
+// ---- the other formats, one to four matrices a launch (kernels/qmv_ggm.metal:232-262): the 16-row tiles of all
+// matrices form one list dealt round-robin to the waves; a wave walks its tiles matrix by matrix, each with the
+// decoder of that matrix's format.
+template <int F, int NB> __device__ __forceinline__ void qmvm_matrix(const qwk_qmvm_args &a, uint32_t j, const uint32_t *tab, const qw_afrag_kq &af, uint32_t t0, uint32_t nw) {
+    typedef qw_chunk_kq<F, NB> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, nl = lane >> 2, kl = lane & 3;
+    const uint32_t cpr = a.K / (C::BLK_K * NB), N = a.N[j], rb = a.rowbytes[j], ys = a.ystride[j];
+    const uint8_t *W = a.W[j];
+    void *y = a.y[j];
+    auto rowp = [&](uint32_t t) {
+        const uint32_t r = 16 * t + nl;
+        return W + (size_t)(r < N ? r : N - 1) * rb;
+    };
+    f4 acc = {0, 0, 0, 0};
+    qw_task_pipeline<C>(a.ntiles[j], t0, nw, cpr, NB * C::BLK_B, kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
+        c.mac(tab, af, ci * NB * C::BLK_K, kg, acc);
+        if (ci + 1 != cpr) return;
+        const uint32_t r = 16 * t + n;
+        if (r < N)
+#pragma unroll
+            for (uint32_t i = 0; i < 4; i++) {
+                const uint32_t tok = 4 * kg + i;
+                if (tok < a.nb) {
+                    if (a.yfloat) ((float *)y)[(size_t)tok * ys + r] = acc[i];
+                    else ((uint16_t *)y)[(size_t)tok * ys + r] = qw_f2h(acc[i]);
+                }
+            }
+        acc = f4{0, 0, 0, 0};
+    });
+}
+extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmvm(qwk_qmvm_args a) {
+    __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; } L;
+    qw_kq_tab_build(L.tab);
+    qw_stage_x(L.xf, a.x, a.xstride, a.K, a.nb);
+    __syncthreads();
+    if (a.sums) { // sums of 32 activations per token, in index order
+        for (uint32_t i = threadIdx.x; i < (a.K >> 5) * 16; i += blockDim.x) {
+            const uint32_t c = i >> 4, m = i & 15;
+            float sum = 0;
+#pragma unroll
+            for (uint32_t f = 0; f < 4; f++) {
+                const h8 v = __builtin_bit_cast(h8, L.xf[(4 * c + f) * 16 + m]);
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += (float)v[e];
+            }
+            L.xs[i] = sum;
+        }
+        __syncthreads();
+    }
+    const uint32_t lane = qw_lane(), nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const qw_afrag_kq af = {L.xf, L.xs, lane & 15, lane >> 4};
+    const bool k256 = a.K % 256 == 0;
+    uint32_t toff = 0;
+    for (uint32_t j = 0; j < a.nmat; j++) {
+        const uint32_t t0 = (w0 + nw - toff % nw) % nw; // first tile of matrix j that falls to this wave
+        switch (a.fmt[j]) {
+        case 12: qmvm_matrix<12, 1>(a, j, L.tab, af, t0, nw); break;
+        case 13: qmvm_matrix<13, 1>(a, j, L.tab, af, t0, nw); break;
+        case 14: qmvm_matrix<14, 1>(a, j, L.tab, af, t0, nw); break;
+        case 23: qmvm_matrix<23, 1>(a, j, L.tab, af, t0, nw); break;
+        case 20: k256 ? qmvm_matrix<20, 8>(a, j, L.tab, af, t0, nw) : qmvm_matrix<20, 1>(a, j, L.tab, af, t0, nw); break;
+        case 1: k256 ? qmvm_matrix<1, 8>(a, j, L.tab, af, t0, nw) : qmvm_matrix<1, 1>(a, j, L.tab, af, t0, nw); break;
+        case 30: k256 ? qmvm_matrix<30, 8>(a, j, L.tab, af, t0, nw) : qmvm_matrix<30, 1>(a, j, L.tab, af, t0, nw); break;
+        }
+        toff += a.ntiles[j];
+    }
+}
 
 // The VALU GEMV the matrix-core kernels are measured against (1, 2 or 4 activations, K a multiple of 512 up to 2560,
 // packed IQ3_S): the same streaming and decoding, v_dot2_f32_f16 instead of the matrix instruction, and a sum over

@@ -19,8 +19,27 @@ struct qw_path {
     unsigned pf_max_tiles;
 };
 
-static int blk_values(int type) { return type == 8 ? 32 : type == 21 ? 256 : 0; }
-static int blk_bytes(int type) { return type == 8 ? 34 : type == 21 ? 110 : 0; } // src/gguf.c:15-25
+static int blk_values(int type) { // src/gguf.c:15-25
+    switch (type) {
+    case 1: case 30: return 1;
+    case 8: case 20: return 32;
+    case 12: case 13: case 14: case 21: case 23: return 256;
+    default: return 0;
+    }
+}
+static int blk_bytes(int type) {
+    switch (type) {
+    case 1: case 30: return 2;
+    case 8: return 34;
+    case 20: return 18;
+    case 12: return 144;
+    case 13: return 176;
+    case 14: return 210;
+    case 21: return 110;
+    case 23: return 136;
+    default: return 0;
+    }
+}
 static int row_bytes(int type, int K) { return blk_values(type) ? K / blk_values(type) * blk_bytes(type) : 0; }
 
 int qw_path_nbv(int nb) { return nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : nb <= 8 ? 8 : 16; }
@@ -85,6 +104,37 @@ bool qw_path_qmv_gg(qw_path *p, qw_batch *b, const qw_tensor *W, int N, int K, c
     qw_batch_buf(b, 4, y, yoff);
     qw_batch_bytes(b, 5, &a, sizeof a);
     qw_batch_dispatch(b, ((unsigned)N + 7) / 8, 1, 1, 256, 1, 1);
+    return true;
+}
+
+// ---------------------------------------------------------------- several matrices over one x (src/engine.c:730-771)
+bool qw_path_qmv_ggm(qw_path *p, qw_batch *b, const qw_tensor *W, const int *N, int n, int K, const qw_buf *x, const qw_buf *const *y, int nb, bool fout) {
+    if (n < 1 || n > 4 || nb < 1 || nb > 16 || K % 256) {
+        fprintf(stderr, "qmv_ggm: %d matrices / %d tokens / K %d outside 1..4 / 1..16 / multiples of 256\n", n, nb, K);
+        return false;
+    }
+    char base[128], name[140], defs[512];
+    int f[4];
+    for (int i = 0; i < 4; i++) f[i] = W[i < n ? i : 0].type;
+    snprintf(base, sizeof base, "qmv_ggm_k%d_m%d_%d_%d_%d_%d%s", K, n, f[0], f[1], f[2], f[3], fout ? "_f" : "");
+    snprintf(name, sizeof name, "%s_b%d", base, nb);
+    snprintf(defs, sizeof defs, "#define IQ_DQ_ONLY 1\n#define qmv_ggm %s\n#define KD %d\n#define NB 0\n#define NMAT %d\n#define GF0 %d\n#define GF1 %d\n#define GF2 %d\n#define GF3 %d\n%s",
+             base, K, n, f[0], f[1], f[2], f[3], fout ? "#define YT float\n" : "");
+    qw_kernel *k = compile_get(p, name, defs);
+    if (!k) return false;
+    struct { uint32_t N[4], off[4], total, xstride; } a = {{0}, {0}, 0, (uint32_t)K};
+    qw_batch_kernel(b, k);
+    for (int i = 0; i < 4; i++) {
+        const int j = i < n ? i : 0;
+        qw_batch_buf(b, (unsigned)i, W[j].buf, W[j].offset);
+        qw_batch_buf(b, 5u + (unsigned)i, y[j], 0);
+        a.N[i] = i < n ? (uint32_t)N[i] : 0;
+        a.off[i] = a.total;
+        if (i < n) a.total += (uint32_t)N[i];
+    }
+    qw_batch_buf(b, 4, x, 0);
+    qw_batch_bytes(b, 9, &a, sizeof a);
+    qw_batch_dispatch(b, (a.total + 7) / 8, 1, 1, 256, 1, 1);
     return true;
 }
 

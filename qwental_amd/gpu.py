@@ -57,6 +57,7 @@ SYMBOLS = [
     ("qw_path_open", _vp, [_vp, _i, _i, _i, _i, _i, _b]), ("qw_path_close", None, [_vp]),
     ("qw_path_sel_bytes", _sz, [_vp, _i]), ("qw_path_logits_bytes", _sz, [_vp, _i]), ("qw_path_nbv", _i, [_i]),
     ("qw_path_qmv_gg", _b, [_vp, _vp, _pt, _i, _i, _pb, _sz, _pb, _sz, _i, _b]),
+    ("qw_path_qmv_ggm", _b, [_vp, _vp, _vp, _vp, _i, _i, _pb, _vp, _i, _b]),
     ("qw_path_gg_router", _b, [_vp, _vp, _pm, _i, _pb, _pb]),
     ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
@@ -276,6 +277,15 @@ class Path:
         t = W.c()
         if not self.L.qw_path_qmv_gg(self.p, batch.b, C.byref(t), N, K, x.ref(), xoff, y.ref(), yoff, nb, fout):
             raise RuntimeError("qw_path_qmv_gg failed")
+
+    def qmv_ggm(self, batch, Ws, Ns, K, x, ys, nb, fout=True):
+        """Up to four matrices (Tensor list) over the same x in one launch; ys: one output buffer per matrix."""
+        n = len(Ws)
+        wt = (QwTensor * n)(*[w.c() for w in Ws])
+        na = (C.c_int * n)(*Ns)
+        ya = (C.POINTER(QwBuf) * n)(*[C.pointer(y.c) for y in ys])
+        if not self.L.qw_path_qmv_ggm(self.p, batch.b, wt, na, n, K, x.ref(), ya, nb, fout):
+            raise RuntimeError("qw_path_qmv_ggm failed")
 
     def gg_router(self, batch, layer, nb, x, lg):
         if not self.L.qw_path_gg_router(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref()):

@@ -11,8 +11,11 @@ so is the work the kernels do.
 """
 import numpy as np
 
-BLOCK = {8: (32, 34), 21: (256, 110)}  # ggml type -> (values, bytes) per block
+BLOCK = {8: (32, 34), 21: (256, 110), 12: (256, 144), 13: (256, 176), 14: (256, 210), 20: (32, 18), 23: (256, 136),
+         1: (1, 2), 30: (1, 2)}  # ggml type -> (values, bytes) per block
 D_SIGMA = {21: 0.02, 8: 0.01}
+# byte offsets of the binary16 scale fields of the other block formats and the sigma their |N(0, sigma)| is drawn with
+SCALE_FIELDS = {12: ((0, 2), 0.002), 13: ((0, 2), 0.001), 14: ((208,), 0.0005), 20: ((0,), 0.0005), 23: ((0,), 0.00005)}
 MOE_D_SCALE = 0.1
 
 
@@ -25,6 +28,17 @@ def row_bytes(ftype, K):
 def blocks(rng, ftype, n, d_scale=1.0):
     """n raw blocks of the given type as uint8 [n, block_bytes]."""
     qb, bb = BLOCK[ftype]
+    if ftype in (1, 30):  # plain rows: N(0, 0.02) values as binary16 / bfloat16 (truncated)
+        v = rng.normal(0.0, 0.02 * d_scale, n).astype(np.float32)
+        if ftype == 1:
+            return v.astype(np.float16).view(np.uint8).reshape(n, 2)
+        return (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(n, 2)
+    if ftype in SCALE_FIELDS:  # every byte uniform, then the scale fields
+        out = rng.integers(0, 256, (n, bb), dtype=np.uint8)
+        offs, sigma = SCALE_FIELDS[ftype]
+        for off in offs:
+            out[:, off:off + 2] = np.abs(rng.normal(0.0, sigma * d_scale, n)).astype(np.float16).view(np.uint8).reshape(n, 2)
+        return out
     out = np.empty((n, bb), np.uint8)
     d = np.abs(rng.normal(0.0, D_SIGMA[ftype] * d_scale, n)).astype(np.float16)
     if ftype == 21:

@@ -84,7 +84,11 @@ def test_define_blocks_of_the_reference_register_its_kernel_names():
 
 
 @pytest.mark.parametrize("block,needle", [
-    ("#define IQ_DQ_ONLY 1\n#define DQ_TEST 14\n", "14"),                                                    # Q6_K: no gfx950 build
+    ("#define IQ_DQ_ONLY 1\n#define DQ_TEST 10\n", "10"),                                                    # Q2_K: no gfx950 build
+    ("#define qmv_gg x\n#define GF 14\n#define KD 8192\n#define RB 6720\n#define NB 8\n", "8192"),            # K beyond the staged activations
+    ("#define qmv_ggm g\n#define KD 2048\n#define NB 0\n#define NMAT 2\n#define GF0 12\n#define GF1 21\n", "21"),  # IQ3_S is not a format of the multi-matrix kernel
+    ("#define qmv_ggm g\n#define KD 2000\n#define NB 0\n#define NMAT 1\n#define GF0 12\n", "KD 2000"),
+    ("#define qmv_ggm g\n#define KD 2048\n#define NB 0\n#define NMAT 5\n#define GF0 12\n", "NMAT"),
     ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 881\n#define NB 8\n", "row bytes"),
     ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 17\n", "NB"),
     ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 8\n#define YT bfloat\n", "YT"),
@@ -120,6 +124,21 @@ def test_packing_blocks_register_the_reference_names():
     assert not ok and "22" in err  # IQ2_S
     ok, err, names = compile_check(pf.replace("GG_PART 5", "GG_PART 6"))
     assert not ok and "GG_PART" in err
+
+
+def test_other_formats_and_the_multi_matrix_block():
+    for f, rb in ((12, 1152), (13, 1408), (14, 1680), (23, 1088), (20, 1152), (30, 4096), (1, 4096)):
+        ok, err, names = compile_check("#define qmv_gg q_%d\n#define GF %d\n#define KD 2048\n#define RB %d\n#define NB 4\n" % (f, f, rb))
+        assert ok and names == ["q_%d" % f], err
+        ok, err, names = compile_check("#define DQ_TEST %d\n" % f)
+        assert ok and names == ["dq_test"], err
+    # src/engine.c:738-739: NB 0 builds one kernel per token count, <name>_b<n>
+    blk = "#define IQ_DQ_ONLY 1\n#define qmv_ggm qmv_ggm_k2048_m4_12_12_14_30\n#define KD 2048\n#define NB 0\n#define NMAT 4\n#define GF0 12\n#define GF1 12\n#define GF2 14\n#define GF3 30\n"
+    ok, err, names = compile_check(blk)
+    assert ok, err
+    assert names == ["qmv_ggm_k2048_m4_12_12_14_30_b%d" % n for n in range(1, 17)]
+    ok, err, names = compile_check("#define qmv_ggm one\n#define KD 512\n#define NB 3\n#define NMAT 1\n#define GF0 23\n#define YT float\n")
+    assert ok and names == ["one"], err
 
 
 def test_valu_gemv_is_asked_for_by_a_macro():
