@@ -715,7 +715,17 @@ static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a) {
         if (a->fmt[j] == 12 || a->fmt[j] == 13) a->sums = 1;
     }
     if (!tiles) return true;
-    return add_launch(b, "qwk_qmvm", persistent_grid(b->g, tiles, QW_WAVES_GU), 64 * QW_WAVES_GU, a, sizeof *a);
+    // few tiles: cut every tile's K range over several waves, as far as the wave slots of the device and K allow
+    const unsigned waves = QW_WAVES_GU, slots = (unsigned)b->g->ncu * waves;
+    a->split = 1;
+    if (a->K % 256 == 0)
+        while (a->split < 4 && tiles * a->split * 2 <= slots && (a->K / 256) % (a->split * 2) == 0) a->split *= 2;
+    if (a->split > 1) {
+        unsigned groups = 0;
+        for (uint32_t j = 0; j < a->nmat; j++) groups += cdiv(a->ntiles[j], waves / a->split);
+        return add_launch(b, "qwk_qmvm", umin((unsigned)b->g->ncu, groups), 64 * waves, a, sizeof *a);
+    }
+    return add_launch(b, "qwk_qmvm", persistent_grid(b->g, tiles, waves), 64 * waves, a, sizeof *a);
 }
 
 static bool tr_qmvm(qw_batch *b) { // src/engine.c:752-771: 0..3 W, 4 x, 5..8 y, 9 {N[4], off[4], total, xstride}; y stride = N
@@ -774,8 +784,17 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
     if (p->valu) { // the VALU GEMV, for measurement against the matrix-core form
         if (F != QW_F_PACKED || p->K % 512 || p->NB > 4) return fail(b, "qmv_gg: the VALU form needs packed IQ3_S weights, K a multiple of 512 and NB <= 4");
         fname_fmt(fn, sizeof fn, "qwk_qmv_valu_n%d", p->NB <= 1 ? 1 : p->NB <= 2 ? 2 : 4);
-    } else if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", F);
-    else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", F, chunk_of(21 == F || F == QW_F_PACKED ? 21 : F, p->K));
+    } else {
+        const int base = 21 == F || F == QW_F_PACKED ? 21 : F, ch = p->K > 2560 ? 1 : chunk_of(base, p->K);
+        if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", F);
+        else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", F, ch);
+        // few tiles: cut every tile's chunks over 2 or 4 waves, as far as the wave slots of the device allow
+        const unsigned cpr = (unsigned)p->K / ((unsigned)fmt_qb(base) * (unsigned)ch), slots = (unsigned)b->g->ncu * QW_WAVES_GU;
+        a.split = 1;
+        while (a.split < 4 && a.ntiles * a.split * 2 <= slots && cpr % (a.split * 2) == 0) a.split *= 2;
+        if (a.split > 1) return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, cdiv(a.ntiles, QW_WAVES_GU / a.split)), 64 * QW_WAVES_GU, &a, sizeof a);
+    }
+    a.split = 1;
     return add_launch(b, intern(fn), persistent_grid(b->g, a.ntiles, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 

@@ -107,7 +107,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) 
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
 // y[b][row] = sum_k W[row][k] x[b][k] for up to 16 activations; the weights are streamed once for all of them.
 // Tiles of 16 rows are dealt round-robin to the waves of a persistent grid; a row is CPR chunks of CH blocks.
-template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(const qwk_qmv_args &a, u2 *lut, u4 *xf) {
+template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(const qwk_qmv_args &a, u2 *lut, u4 *xf, f4 *red) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
@@ -120,16 +120,7 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
             return a.W + (size_t)(r < a.N ? r : a.N - 1) * a.rowbytes;
         }
     };
-    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
-    if (XLDS) qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
-    __syncthreads();
-    const qw_afrag_lds afl = {xf, n};
-    const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
-    f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
-        if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
-        else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
-        if (ci + 1 != cpr) return;
+    auto store = [&](uint32_t t, const f4 &acc) {
         const uint32_t r = 16 * t + n;
         if (r < a.N)
 #pragma unroll
@@ -140,49 +131,121 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
                     else ((uint16_t *)a.y)[(size_t)tok * a.ystride + r] = qw_f2h(acc[j]);
                 }
             }
+    };
+    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (XLDS) qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
+    __syncthreads();
+    const qw_afrag_lds afl = {xf, n};
+    const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
+    f4 acc = {0, 0, 0, 0};
+    if (a.split > 1) {
+        // Few tiles (the projections of one decode step): the chunks of a tile are cut over split waves of one
+        // workgroup, so that a row is one memory round trip and not a chain of them; the partial sums are added in
+        // part order through LDS. A group is 12 / split tiles; workgroup g takes groups g, g + gridDim.x, ...
+        const uint32_t wave = qw_wave(), sp = a.split, tpg = (QW_WG_GU / 64) / sp, part = wave % sp, cpp = cpr / sp;
+        const uint32_t ngroups = (a.ntiles + tpg - 1) / tpg;
+        for (uint32_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
+            const uint32_t t = g * tpg + wave / sp;
+            acc = f4{0, 0, 0, 0};
+            if (t < a.ntiles)
+                qw_task_pipeline<C>(1, 0, 1, cpp, CH * C::BLK_B, F == QW_F_PACKED ? lane : kl, [&](uint32_t) { return rowp(t) + (size_t)part * cpp * CH * C::BLK_B; },
+                                    [&](uint32_t, uint32_t ci, const C &c) {
+                                        if (XLDS) c.mac_lean(lut, afl, (part * cpp + ci) * CH * C::BLK_K, kg, acc);
+                                        else c.mac_lean(lut, afg, (part * cpp + ci) * CH * C::BLK_K, kg, acc);
+                                    });
+            red[wave * 64 + lane] = acc;
+            __syncthreads();
+            if (part == 0 && t < a.ntiles) {
+                f4 sum = red[wave * 64 + lane];
+                for (uint32_t q = 1; q < sp; q++) sum += red[(wave + q) * 64 + lane];
+                store(t, sum);
+            }
+            __syncthreads();
+        }
+        return;
+    }
+    qw_task_pipeline<C>(a.ntiles, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
+        if (XLDS) c.mac_lean(lut, afl, ci * CH * C::BLK_K, kg, acc);
+        else c.mac_lean(lut, afg, ci * CH * C::BLK_K, kg, acc);
+        if (ci + 1 != cpr) return;
+        store(t, acc);
         acc = f4{0, 0, 0, 0};
     });
 }
 #define QW_QMV(F, CH, XLDS, SFX)                                                                        \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmv_f##F##SFX(qwk_qmv_args a) {             \
-        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; } L; /* table first: LDS address 0 */ \
-        qmv_body<F, CH, XLDS>(a, L.lut, L.xf);                                                          \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; f4 red[QW_WG_GU]; } L; /* table first: LDS address 0 */ \
+        qmv_body<F, CH, XLDS>(a, L.lut, L.xf, L.red);                                                   \
     }
 QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
 QW_QMV(121, 2, true, _c2) QW_QMV(121, 1, true, _c1) // packed IQ3_S: a.rowbytes = bytes of a 16-row tile
 
-// ---- the other formats, one to four matrices a launch (kernels/qmv_ggm.metal:232-262): the 16-row tiles of all
-// matrices form one list dealt round-robin to the waves; a wave walks its tiles matrix by matrix, each with the
-// decoder of that matrix's format.
+// ---- the other formats, one to four matrices a launch (kernels/qmv_ggm.metal:232-262).
+// split == 1: the 16-row tiles of all matrices form one list dealt round-robin to the waves of a persistent grid; a
+// wave walks its tiles matrix by matrix, each with the decoder of that matrix's format.
+// split > 1 (few tiles: the projections of one decode step): the K range of a tile is cut into split parts, one per
+// wave, so that a row is one memory round trip instead of a chain of them; the waves of a tile sit in one workgroup
+// and their partial sums are added in part order through LDS (the same order whatever else the launch holds).
+#define QW_WG_QMVM 768 // 12 waves: a tile's K range is cut over 1, 2 or 4 of them
+template <int F, int NB> struct qmvm_tile {
+    typedef qw_chunk_kq<F, NB> C;
+    const qwk_qmvm_args &a;
+    uint32_t j;
+    __device__ __forceinline__ const uint8_t *rowp(uint32_t t) const {
+        const uint32_t r = 16 * t + (qw_lane() >> 2);
+        return a.W[j] + (size_t)(r < a.N[j] ? r : a.N[j] - 1) * a.rowbytes[j];
+    }
+    __device__ __forceinline__ void store(uint32_t t, const f4 &acc) const {
+        const uint32_t lane = qw_lane(), r = 16 * t + (lane & 15), kg = lane >> 4;
+        if (r >= a.N[j]) return;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const uint32_t tok = 4 * kg + i;
+            if (tok < a.nb) {
+                if (a.yfloat) ((float *)a.y[j])[(size_t)tok * a.ystride[j] + r] = acc[i];
+                else ((uint16_t *)a.y[j])[(size_t)tok * a.ystride[j] + r] = qw_f2h(acc[i]);
+            }
+        }
+    }
+};
 template <int F, int NB> __device__ __forceinline__ void qmvm_matrix(const qwk_qmvm_args &a, uint32_t j, const uint32_t *tab, const qw_afrag_kq &af, uint32_t t0, uint32_t nw) {
     typedef qw_chunk_kq<F, NB> C;
-    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, nl = lane >> 2, kl = lane & 3;
-    const uint32_t cpr = a.K / (C::BLK_K * NB), N = a.N[j], rb = a.rowbytes[j], ys = a.ystride[j];
-    const uint8_t *W = a.W[j];
-    void *y = a.y[j];
-    auto rowp = [&](uint32_t t) {
-        const uint32_t r = 16 * t + nl;
-        return W + (size_t)(r < N ? r : N - 1) * rb;
-    };
+    const qmvm_tile<F, NB> T = {a, j};
+    const uint32_t lane = qw_lane(), kg = lane >> 4, cpr = a.K / (C::BLK_K * NB);
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(a.ntiles[j], t0, nw, cpr, NB * C::BLK_B, kl, rowp, [&](uint32_t t, uint32_t ci, const C &c) {
+    qw_task_pipeline<C>(a.ntiles[j], t0, nw, cpr, NB * C::BLK_B, lane & 3, [&](uint32_t t) { return T.rowp(t); }, [&](uint32_t t, uint32_t ci, const C &c) {
         c.mac(tab, af, ci * NB * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
-        const uint32_t r = 16 * t + n;
-        if (r < N)
-#pragma unroll
-            for (uint32_t i = 0; i < 4; i++) {
-                const uint32_t tok = 4 * kg + i;
-                if (tok < a.nb) {
-                    if (a.yfloat) ((float *)y)[(size_t)tok * ys + r] = acc[i];
-                    else ((uint16_t *)y)[(size_t)tok * ys + r] = qw_f2h(acc[i]);
-                }
-            }
+        T.store(t, acc);
         acc = f4{0, 0, 0, 0};
     });
 }
-extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmvm(qwk_qmvm_args a) {
-    __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; } L;
+// Workgroup g0, g0 + ng, ... takes the tile groups of matrix j; wave w does part
+// w % split of tile w / split of the group (12 / split tiles a group).
+template <int F, int NB> __device__ __forceinline__ void qmvm_matrix_split(const qwk_qmvm_args &a, uint32_t j, const uint32_t *tab, const qw_afrag_kq &af, f4 *red, uint32_t g0, uint32_t ng) {
+    typedef qw_chunk_kq<F, NB> C;
+    const qmvm_tile<F, NB> T = {a, j};
+    const uint32_t lane = qw_lane(), kg = lane >> 4, wave = qw_wave(), sp = a.split, tpg = (QW_WG_QMVM / 64) / sp;
+    const uint32_t cpp = a.K / (C::BLK_K * NB) / sp, part = wave % sp; // chunks per part
+    const uint32_t ngroups = (a.ntiles[j] + tpg - 1) / tpg;
+    for (uint32_t g = g0; g < ngroups; g += ng) {
+        const uint32_t t = g * tpg + wave / sp;
+        f4 acc = {0, 0, 0, 0};
+        if (t < a.ntiles[j])
+            qw_task_pipeline<C>(1, 0, 1, cpp, NB * C::BLK_B, lane & 3, [&](uint32_t) { return T.rowp(t) + (size_t)part * cpp * NB * C::BLK_B; },
+                                [&](uint32_t, uint32_t ci, const C &c) { c.mac(tab, af, (part * cpp + ci) * NB * C::BLK_K, kg, acc); });
+        red[wave * 64 + lane] = acc;
+        __syncthreads();
+        if (part == 0 && t < a.ntiles[j]) {
+            f4 sum = red[wave * 64 + lane];
+            for (uint32_t q = 1; q < sp; q++) sum += red[(wave + q) * 64 + lane];
+            T.store(t, sum);
+        }
+        __syncthreads();
+    }
+}
+extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args a) {
+    __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; } L;
     qw_kq_tab_build(L.tab);
     qw_stage_x(L.xf, a.x, a.xstride, a.K, a.nb);
     __syncthreads();
@@ -203,8 +266,22 @@ extern "C" __global__ __launch_bounds__(QW_WG_GU) void qwk_qmvm(qwk_qmvm_args a)
     const uint32_t lane = qw_lane(), nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     const qw_afrag_kq af = {L.xf, L.xs, lane & 15, lane >> 4};
     const bool k256 = a.K % 256 == 0;
-    uint32_t toff = 0;
+    uint32_t toff = 0; // tiles (split == 1) or tile groups (split > 1) of the matrices before j
     for (uint32_t j = 0; j < a.nmat; j++) {
+        if (a.split > 1) { // K is a multiple of 256 here
+            const uint32_t ng = gridDim.x, g0 = (blockIdx.x + ng - toff % ng) % ng;
+            switch (a.fmt[j]) {
+            case 12: qmvm_matrix_split<12, 1>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 13: qmvm_matrix_split<13, 1>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 14: qmvm_matrix_split<14, 1>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 23: qmvm_matrix_split<23, 1>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 20: qmvm_matrix_split<20, 8>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 1: qmvm_matrix_split<1, 8>(a, j, L.tab, af, L.red, g0, ng); break;
+            case 30: qmvm_matrix_split<30, 8>(a, j, L.tab, af, L.red, g0, ng); break;
+            }
+            toff += (a.ntiles[j] + 12 / a.split - 1) / (12 / a.split);
+            continue;
+        }
         const uint32_t t0 = (w0 + nw - toff % nw) % nw; // first tile of matrix j that falls to this wave
         switch (a.fmt[j]) {
         case 12: qmvm_matrix<12, 1>(a, j, L.tab, af, t0, nw); break;

@@ -321,7 +321,7 @@ template <int F, int S = 0> __device__ __forceinline__ void qw_kq_values(const q
 // NB blocks of one row for the task pipeline: loaded in quad order, pulled to matrix-core lane order.
 template <int F, int NB> struct qw_chunk_kq {
     static constexpr uint32_t BLK_K = qw_kq<F>::BLK_K, BLK_B = qw_kq<F>::BLK_B;
-    static constexpr int DEPTH = 2;
+    static constexpr int DEPTH = qw_kq<F>::NR * NB <= 20 ? 3 : 2; // chunks in flight ahead of the arithmetic
     qw_kq<F> b[NB];
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t kl) {
 #pragma unroll

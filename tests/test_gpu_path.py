@@ -118,8 +118,8 @@ def test_qmv_ragged_rows_and_half_output(gpu, oracle):
 
 def test_bad_calls_fail_without_launching(gpu):
     """Undersized buffers, unknown formats and unknown kernels are refused on the host."""
-    ok, err = gpu.compile("#define IQ_DQ_ONLY 1\n#define DQ_TEST 14\n")
-    assert not ok and "14" in err
+    ok, err = gpu.compile("#define IQ_DQ_ONLY 1\n#define DQ_TEST 10\n")  # Q2_K
+    assert not ok and "10" in err
     ok, err = gpu.compile("#define IQ_DQ_ONLY 1\n#define qmv_gg q_bad\n#define GF 21\n#define KD 2048\n#define RB 881\n#define NB 1\n")
     assert not ok
     assert not gpu.kernel("no_such_kernel")
