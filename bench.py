@@ -182,6 +182,74 @@ def qmv_table(gpu, reps=5, nmat=64):
     return out
 
 
+FORMAT_NAMES = {12: "q4_k", 13: "q5_k", 14: "q6_k", 20: "iq4_nl", 23: "iq4_xs", 1: "f16", 30: "bf16"}
+
+
+def formats_table(gpu, reps=4, nmat=32):
+    """The other GGUF formats of the dense matvec (4096 x 2048, 1 and 16 activations, method of qmv_table), a vocabulary
+    sized Q6_K matrix (131072 x 2048: the lm_head case) and four projections of mixed formats in one launch
+    (kernels/qmv_ggm.metal). One matrix is drawn on the host and copied to nmat addresses."""
+    from qwental_amd import synth
+    import qwental_amd as q
+    K = 2048
+    rng = np.random.default_rng(2)
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    x = gpu.buf_from(synth.activations(rng, 16, K), device_only=True)
+    out = {}
+
+    def timed(ft, N, copies, nb):
+        rb = synth.row_bytes(ft, K)
+        one = synth.matrix(rng, ft, min(N, 4096), K)
+        W = gpu.buf(copies * N * rb, device_only=True)
+        for i in range(copies * (N // min(N, 4096))):
+            W.fill(one, i * one.nbytes)
+        y = gpu.buf(16 * N * 4, device_only=True)
+        name = "qmv_gg_bench_f%d_n%d" % (ft, nb)
+        ok, err = gpu.compile("#define qmv_gg %s\n#define GF %d\n#define KD %d\n#define RB %d\n#define NB %d\n#define YT float\n" % (name, ft, K, rb, nb))
+        assert ok, err
+        k = gpu.kernel(name)
+        best = 1e9
+        for _ in range(reps):
+            b = gpu.batch()
+            b.kernel(k)
+            b.buf(3, x)
+            b.buf(4, y)
+            b.bytes(5, np.array([N, K, N, 0], np.uint32))
+            for i in range(copies):
+                b.buf(0, W, i * N * rb)
+                b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
+            best = min(best, b.end())
+        W.free()
+        y.free()
+        t = best / copies
+        return {"us_per_matvec": t * 1e6, "GBps": (N * rb + nb * (K * 2 + N * 4)) / t / 1e9}
+
+    for ft, nm in FORMAT_NAMES.items():
+        for nb in (1, 16):
+            out["%s_B%d" % (nm, nb)] = timed(ft, 4096, nmat, nb)
+    for nb in (1, 16):
+        out["q6_k_131072rows_B%d" % nb] = timed(14, 131072, 2, nb)
+    # q / k / v / indexer of one decode step: four matrices, one launch
+    fm, Ns = (12, 12, 14, 30), (4096, 512, 512, 128)
+    sets = 16
+    Ws = [gpu.buf_from(np.tile(synth.matrix(rng, f, n, K), sets), device_only=True) for f, n in zip(fm, Ns)]
+    ys = [gpu.buf(16 * n * 4, device_only=True) for n in Ns]
+    wbytes = sum(n * synth.row_bytes(f, K) for f, n in zip(fm, Ns))
+    for nb in (1, 16):
+        best = 1e9
+        for _ in range(reps):
+            b = gpu.batch()
+            for i in range(sets):
+                path.qmv_ggm(b, [q.Tensor(w, f, i * n * synth.row_bytes(f, K)) for w, f, n in zip(Ws, fm, Ns)], list(Ns), K, x, ys, nb)
+            best = min(best, b.end())
+        t = best / sets
+        out["ggm_q4k_q4k_q6k_bf16_B%d" % nb] = {"us_per_launch": t * 1e6, "GBps": wbytes / t / 1e9, "rows": list(Ns)}
+    for bb in Ws + ys + [x]:
+        bb.free()
+    path.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,6 +317,7 @@ def main():
     if not a.quick:
         line["ragged_step"] = ragged_steps(gpu, stack)
         line["qmv"] = qmv_table(gpu)
+        line["qmv_formats"] = formats_table(gpu)
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)

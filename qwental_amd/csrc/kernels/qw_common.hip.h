@@ -659,7 +659,7 @@ __device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, u
 // DPP row shifts inside each row of 16 lanes, then the two row broadcasts of the gfx9 family; every lane receives
 // the result through a read of lane 63.
 __device__ __forceinline__ uint32_t qw_wave_max_u32(uint32_t v) {
-#define QW_DPP_MAX(ctrl, rmask, bmask) v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ctrl, rmask, bmask, false))
+#define QW_DPP_MAX(ctrl, rmask, bmask) v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, ctrl, rmask, bmask, false)) /* 0: lanes without a source keep v */
     QW_DPP_MAX(0x111, 0xf, 0xf); // row_shr:1
     QW_DPP_MAX(0x112, 0xf, 0xf); // row_shr:2
     QW_DPP_MAX(0x114, 0xf, 0xf); // row_shr:4

@@ -646,23 +646,45 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 }
 
 // FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
-// Order of the set-up: the selection record first (one memory round trip, one barrier: the row addresses depend on
-// it); then every wave issues its first weight loads, and only then the table copy, the activation staging and the
-// second barrier follow, overlapping that first round trip to HBM.
-template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc) {
-    if (a.logits) { // the selection, made here by every workgroup; the scratch lies where x is staged afterwards
-        qw_sel_scratch &ss = *(qw_sel_scratch *)xf;
+// Order of the set-up when the record is given: the record first (one memory round trip, one barrier: the row
+// addresses depend on it); then every wave issues its first weight loads, and only then the table copy, the activation
+// staging and the second barrier follow, overlapping that first round trip to HBM. When the selection is made here,
+// the table is fetched under it instead.
+template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss) {
+    bool staged = false, tabled = false;
+    if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
-        select_all(sa, ss, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
+        if (qw_select_fast_e(a.E)) {
+            // The table does not depend on the selection: its loads are issued first and are in flight while the
+            // selection is made; it is written to LDS after it. (The activations follow in ready(), under the first
+            // weight loads: holding them here as well would spill registers.)
+            constexpr uint32_t NT = QW_WG_GU, NL = (QW_LUT_BYTES / 16 + NT - 1) / NT;
+            constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
+            u4 lv[NL];
+#pragma unroll
+            for (uint32_t j = 0; j < NL; j++) {
+                const uint32_t i = threadIdx.x + j * NT;
+                if (lutp && i < QW_LUT_BYTES / 16) lv[j] = ((const u4 *)a.glut)[i];
+            }
+            select_all(sa, *ss, *sc, nullptr, blockIdx.x == 0);
+#pragma unroll
+            for (uint32_t j = 0; j < NL; j++) {
+                const uint32_t i = threadIdx.x + j * NT;
+                if (lutp && i < QW_LUT_BYTES / 16) ((u4 *)lut)[i] = lv[j];
+            }
+            tabled = true; // visible to the other waves after the barrier of ready()
+        } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
+            qw_sel_scratch &so = *(qw_sel_scratch *)xf;
+            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
+        }
     } else {
         if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
         __syncthreads();
     }
-    bool staged = false;
     auto ready = [&] {
         if (staged) return;
         staged = true;
-        if (qw_has_lut(FGU) || qw_has_lut(FSG)) qw_lut_copy(lut, (const u2 *)a.glut);
+        if (!tabled && (qw_has_lut(FGU) || qw_has_lut(FSG))) qw_lut_copy(lut, (const u2 *)a.glut);
         qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
         __syncthreads();
     };
@@ -682,8 +704,8 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
-        __shared__ struct { u2 lut[(qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; } L; \
-        gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc);                                             \
+        __shared__ struct { u2 lut[(qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; qw_sel_scratch ss; } L; \
+        gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc, &L.ss);                                             \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
 QW_GU(21, 2, 0, 1, qwk_gu_f21_c2) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
@@ -868,6 +890,9 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
 }
 template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
+    const bool tp2 = (tpe & (tpe - 1)) == 0; // D = 1024, 2048: shifts instead of divisions
+    const uint32_t tsh = (uint32_t)__builtin_ctz(tpe);
+    auto div_tpe = [&](uint32_t x) { return tp2 ? x >> tsh : x / tpe; };
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
     __syncthreads();
     const uint32_t *ue = sc->ue, *mask = sc->mask;
@@ -884,14 +909,14 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     for (uint32_t base = blockIdx.x * per; base < V; base += gridDim.x * per) { // one round unless the grid is small
         const uint32_t end = base + per < V ? base + per : V;
         // virtual expert of a position: 0 = shared (positions below vsh), then the routed experts
-        const uint32_t v0 = base < vsh ? 0 : nsh + (base - vsh) / tpe, v1 = end - 1 < vsh ? 0 : nsh + (end - 1 - vsh) / tpe;
+        const uint32_t v0 = base < vsh ? 0 : nsh + div_tpe(base - vsh), v1 = end - 1 < vsh ? 0 : nsh + div_tpe(end - 1 - vsh);
         auto seg = [&](uint32_t v) {
             qw_dn_seg g;
             g.sh = v < nsh;
             if (g.sh) {
                 const uint32_t hi = end < vsh ? end : vsh; // positions [base, hi) -> tiles, rounded so that neighbours meet
-                g.tile0 = (base + shw - 1) / shw;
-                g.ntile = (hi + shw - 1) / shw - g.tile0;
+                g.tile0 = shw == 1 ? base : (base + shw - 1) / shw;
+                g.ntile = (shw == 1 ? hi : (hi + shw - 1) / shw) - g.tile0;
                 g.u = 0;
                 g.W = a.Wsd, g.P = a.Psh, g.rowbytes = a.sd_rowbytes, g.mask = qw_all_tokens(a.snbr);
             } else {
@@ -918,26 +943,43 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             // the loads of that pass are in flight while the table is copied. Fragment order in LDS,
             // [segment][plane][c][token], 16 bytes each: the sixteen lanes of a k-group read 256 contiguous bytes.
             const uint32_t upr = a.I / 8, per = 2 * upr; // 16-byte units per plane row, per row
+            const bool p2 = (upr & (upr - 1)) == 0; // I = 256, 512, 1024: shifts instead of divisions
+            const uint32_t ush = (uint32_t)__builtin_ctz(upr);
             const uint32_t rows = g0.mask | (both ? g1.mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
-            auto item = [&](uint32_t i, uint32_t &dst) {
+            // item i of the copy: (row in use, plane, 16-byte unit) -> source address and destination index
+            auto place = [&](uint32_t i, uint32_t &dst) {
                 uint32_t m = rows;
-                for (uint32_t k = i / per; k; k--) m &= m - 1; // drop the rows before this one
-                const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, t = bit & 15, r = i % per, pl = r / upr, c = r % upr;
+                for (uint32_t k = p2 ? i >> (ush + 1) : i / per; k; k--) m &= m - 1; // drop the rows before this one
+                const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, t = bit & 15, r = p2 ? i & (per - 1) : i % per;
+                const uint32_t pl = p2 ? r >> ush : r / upr, c = p2 ? r & (upr - 1) : r % upr;
                 const uint32_t s = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + t];
                 dst = ((sg * 2 + pl) * upr + c) * 16 + t;
-                return *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
+                return (const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
             };
-            uint32_t d0 = 0;
-            u4 v0 = {0, 0, 0, 0};
-            const bool have = threadIdx.x < nitem;
-            if (have) v0 = item(threadIdx.x, d0);
+            // every load of the workgroup is issued before the first store (up to 4 a thread: 24 rows of 2 x 64 units
+            // over 768 threads), with the table copy between the two; the destinations are worked out again for the
+            // stores rather than kept in registers
+            constexpr int NV = 4;
+            u4 v[NV];
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                uint32_t dd;
+                if (threadIdx.x + j * blockDim.x < nitem) v[j] = *place(threadIdx.x + j * blockDim.x, dd);
+            }
             if (!tables && (qw_has_lut(F) || qw_has_lut(FSD))) qw_lut_copy(lut, (const u2 *)a.glut);
             tables = true;
-            if (have) ((u4 *)arows)[d0] = v0;
-            for (uint32_t i = threadIdx.x + blockDim.x; i < nitem; i += blockDim.x) {
-                uint32_t d;
-                const u4 v = item(i, d);
-                ((u4 *)arows)[d] = v;
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                uint32_t dd;
+                if (threadIdx.x + j * blockDim.x < nitem) {
+                    place(threadIdx.x + j * blockDim.x, dd);
+                    ((u4 *)arows)[dd] = v[j];
+                }
+            }
+            for (uint32_t i = threadIdx.x + NV * blockDim.x; i < nitem; i += blockDim.x) { // larger I or fewer threads
+                uint32_t dd;
+                const u4 vv = *place(i, dd);
+                ((u4 *)arows)[dd] = vv;
             }
             __syncthreads();
         };
