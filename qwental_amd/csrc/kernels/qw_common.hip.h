@@ -186,8 +186,12 @@ struct qw_afrag_lds2 {
     __device__ __forceinline__ h8 lo(uint32_t koff) const { return __builtin_bit_cast(h8, lo_[(koff >> 3) * 16 + m]); }
 };
 
+// Every workgroup of a launch copies the same bytes: each starts at a different place (a rotation by its index), so
+// that at any moment the workgroups ask different memory channels instead of all the same one.
 __device__ __forceinline__ void qw_stage_x(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
-    for (uint32_t i = threadIdx.x; i < (K >> 3) * 16; i += blockDim.x) {
+    const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 272u) % n;
+    for (uint32_t i0 = threadIdx.x; i0 < n; i0 += blockDim.x) {
+        const uint32_t i = i0 + rot < n ? i0 + rot : i0 + rot - n;
         const uint32_t c = i >> 4, m = i & 15;
         u4 v = {0, 0, 0, 0};
         if (m < nb) v = *(const u4 *)(x + (size_t)m * xstride + 8 * c);
@@ -641,12 +645,13 @@ __device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
     const u4 *src = (const u4 *)glut;
     u4 *dst = (u4 *)lut;
     constexpr uint32_t N = QW_LUT_BYTES / 16;
+    const uint32_t rot = blockIdx.x * 272u; // every workgroup starts elsewhere in the table (see qw_stage_x)
     for (uint32_t i = threadIdx.x; i < N; i += 8 * blockDim.x) {
         u4 v[8];
 #pragma unroll
-        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) v[j] = src[i + j * blockDim.x];
+        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) v[j] = src[(i + j * blockDim.x + rot) & (N - 1)];
 #pragma unroll
-        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) dst[i + j * blockDim.x] = v[j];
+        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) dst[(i + j * blockDim.x + rot) & (N - 1)] = v[j];
     }
 }
 

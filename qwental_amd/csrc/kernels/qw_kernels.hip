@@ -486,6 +486,109 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
     }
 }
 
+// The same result without the chain of K dependent wave-wide maxima. Every lane finds the maximum of its PER keys;
+// a value T0 that at least K of the 64 lane maxima reach bounds the answer from below: at least K keys are >= T0, so
+// no key below T0 can be picked. The keys >= T0 (K of them, or a few more) are gathered one to a lane, each is ranked among
+// them by (key descending, expert ascending) - the order of the repeated maximum with ties to the lowest index - and
+// the ranks below K are the picks. T tokens go through together (the steps are chains of LDS and cross-lane
+// latencies, so a second token costs little). Returns a bit per token that was NOT done, with nothing written for
+// it: more than 64 keys reach T0 (many equal logits) and the caller falls back to select_tokens.
+// ws: 256 dwords of LDS scratch per token for this wave.
+// issued(): called once the loads of the logits are issued (the place for the caller's own prefetches: loads return in
+// the order of issue, and the logits are needed first).
+template <int PER, int T, class H>
+__device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, uint32_t E, uint32_t K, const uint32_t (&tok)[T], const bool (&on)[T], float *w, uint32_t *ids, uint32_t *ws,
+                                                        uint32_t lane, H issued) {
+    uint32_t k[T][PER], M[T], T0[T], c[T], pos[T][PER];
+#pragma unroll
+    for (int t = 0; t < T; t++)
+#pragma unroll
+        for (int j = 0; j < PER; j++) k[t][j] = __builtin_bit_cast(uint32_t, logits[(size_t)tok[t] * (E + 1) + lane * PER + j]);
+    issued();
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        M[t] = 0;
+#pragma unroll
+        for (int j = 0; j < PER; j++) k[t][j] = qw_fkey(__builtin_bit_cast(float, k[t][j])), M[t] = max(M[t], k[t][j]);
+        T0[t] = 0;
+    }
+    // T0: the largest value with bits [lo, 32) such that at least K lane maxima reach it, found bit by bit with a
+    // ballot each (scalar work but for the comparison). The upper 16 bits are nearly always enough to leave at most
+    // 64 keys; otherwise the lower 16 follow, which makes T0 the K-th largest lane maximum itself.
+    auto refine = [&](int t, int hi, int lo) {
+        for (int b = hi; b >= lo; b--) {
+            const uint32_t cd = T0[t] | (1u << b);
+            if ((uint32_t)__popcll(__ballot(M[t] >= cd)) >= K) T0[t] = cd;
+        }
+    };
+    // gather the keys >= T0: position = candidates of earlier j, plus those of lower lanes at this j
+    auto gather = [&](int t) {
+        c[t] = 0;
+#pragma unroll
+        for (int j = 0; j < PER; j++) {
+            const unsigned long long bal = __ballot(k[t][j] >= T0[t]);
+            pos[t][j] = c[t] + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0));
+            c[t] += (uint32_t)__popcll(bal);
+        }
+    };
+    uint32_t fail = 0;
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        refine(t, 31, 16);
+        gather(t);
+        if (c[t] > 64) {
+            refine(t, 15, 0);
+            gather(t);
+        }
+        if (c[t] > 64 || !on[t]) fail |= 1u << t;
+    }
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        if ((fail >> t) & 1) continue;
+        u2 *cand = (u2 *)(ws + 256 * t + 64); // (key, expert) of candidate p
+#pragma unroll
+        for (int j = 0; j < PER; j++)
+            if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], lane * PER + j};
+    }
+    uint32_t mk[T], me[T], rank[T];
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        const u2 mine = ((const u2 *)(ws + 256 * t + 64))[lane];
+        // one 64-bit value per candidate whose order is the ranking order; lanes without a candidate hold the least
+        mk[t] = lane < c[t] ? mine.x : 0, me[t] = lane < c[t] ? ~mine.y : 0;
+        rank[t] = 0;
+    }
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        if ((fail >> t) & 1) continue;
+        const unsigned long long mine = (unsigned long long)mk[t] << 32 | me[t];
+        for (uint32_t q0 = 0; q0 < c[t]; q0 += 16) // candidates sixteen at a time, read from their lanes
+#pragma unroll
+            for (uint32_t q = 0; q < 16; q++) {
+                if (q >= 8 && q0 + q >= c[t]) break; // uniform: ten to twelve candidates are the common case
+                const uint32_t l = q0 ? (q0 + q) & 63 : q;
+                const unsigned long long o = (unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)mk[t], (int)l) << 32 | (uint32_t)__builtin_amdgcn_readlane((int)me[t], (int)l);
+                rank[t] += o > mine;
+            }
+        uint32_t *pkr = ws + 256 * t + 192; // key of rank r
+        if (lane < c[t] && rank[t] < K) {
+            ids[tok[t] * K + rank[t]] = ~me[t];
+            pkr[rank[t]] = mk[t];
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        if ((fail >> t) & 1) continue;
+        const float p = qw_fkey_inv(ws[256 * t + 192 + (lane < K ? lane : 0)]);
+        const float mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), 0)), ex = __expf(p - mx);
+        float sm = 0;
+        for (uint32_t r = 0; r < K; r++) sm += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), (int)r)); // rank order
+        if (lane < K) w[tok[t] * (K + 1) + lane] = ex / sm;
+        if (lane == K) w[tok[t] * (K + 1) + K] = 1.0f / (1.0f + __expf(-logits[(size_t)tok[t] * (E + 1) + E]));
+    }
+    return fail;
+}
+
 // Any E <= 1024: the values live in LDS (v, E floats); lane l scans experts l, l + 64, ...
 __device__ __forceinline__ void select_token_any(const float *lg, float *v, uint32_t E, uint32_t K, uint32_t tok, float *w, uint32_t *ids, uint32_t lane) {
     for (uint32_t e = lane; e < E; e += 64) v[e] = lg[e];
@@ -517,8 +620,9 @@ __device__ __forceinline__ void select_token_any(const float *lg, float *v, uint
 __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 || E == 128 || E == 256 || E == 512 || E == 1024; }
 
 // The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
-// floats per wave, used only when E is not 64 * {1, 2, 4, 8, 16}. c is complete for every thread on return.
-__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store = true) {
+// floats per wave (512 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
+template <class H>
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued) {
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
@@ -528,20 +632,39 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
     if (tid < 8) s.lead[tid] = 0;
     for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
-    if (fast) { // two tokens per wave at a time when there are more tokens than waves
-        for (uint32_t t = wave; t < a.nbr; t += 2 * nwv) {
-            const bool two = t + nwv < a.nbr;
+    if (fast) { // two tokens per wave at a time when there are more tokens than waves; lgs gives a wave 512 dwords
+        uint32_t *ws = (uint32_t *)lgs + 512 * wave;
+        const uint32_t trot = a.nbr ? blockIdx.x % a.nbr : 0; // the workgroups of a launch read the tokens' logits in different orders
+        auto rot = [&](uint32_t tt) { return tt + trot < a.nbr ? tt + trot : tt + trot - a.nbr; };
+        const bool pairs = E <= 512; // sixteen keys a lane: one token at a time (registers)
+        for (uint32_t tt = wave; tt < a.nbr; tt += (pairs ? 2 : 1) * nwv) {
+            const bool two = pairs && tt + nwv < a.nbr;
+            const uint32_t tk[2] = {rot(tt), two ? rot(tt + nwv) : rot(tt)};
+            const bool on2[2] = {true, two}, on1[1] = {true};
+            const uint32_t t1[1] = {tk[0]};
+            uint32_t fail;
             switch (E) {
-            case 64: two ? select_tokens<1, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<1, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
-            case 128: two ? select_tokens<2, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<2, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
-            case 256: two ? select_tokens<4, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<4, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
-            case 512: two ? select_tokens<8, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<8, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
-            default: two ? select_tokens<16, 2>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane) : select_tokens<16, 1>(a.logits, E, K, t, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            }
+            for (uint32_t i = 0; i < 2; i++) { // more than 64 keys tie at the bound: the repeated maximum instead
+                if (!((fail >> i) & 1) || (i == 1 && !two)) continue;
+                switch (E) {
+                case 64: select_tokens<1, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
+                case 128: select_tokens<2, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
+                case 256: select_tokens<4, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
+                case 512: select_tokens<8, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
+                default: select_tokens<16, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
+                }
             }
         }
     } else {
         for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
+    issued(); // the waves without a token
     __syncthreads();
     if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid); // first flat index of every picked expert
     __syncthreads();
@@ -594,7 +717,7 @@ extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a)
     __shared__ qw_sel_scratch s;
     __shared__ qw_sel_cache c;
     __shared__ float lgs[16 * 1024];
-    select_all(a, s, c, lgs);
+    select_all(a, s, c, lgs, true, [] {});
 }
 
 // ================================================================ gate/up + SwiGLU (kernels/moe_gg.metal:428-447, 563-573, 600-631)
@@ -655,27 +778,32 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
     if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
         if (qw_select_fast_e(a.E)) {
-            // The table does not depend on the selection: its loads are issued first and are in flight while the
-            // selection is made; it is written to LDS after it. (The activations follow in ready(), under the first
-            // weight loads: holding them here as well would spill registers.)
+            // The table does not depend on the selection: its loads are issued right behind those of the logits and
+            // are in flight while the selection is made; it is written to LDS after it. (The activations follow in
+            // ready(), under the first weight loads: holding them here as well would spill registers.)
             constexpr uint32_t NT = QW_WG_GU, NL = (QW_LUT_BYTES / 16 + NT - 1) / NT;
             constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
+            const uint32_t lrot = blockIdx.x * 272u; // every workgroup starts elsewhere in the table
             u4 lv[NL];
+            bool fetched = false;
+            select_all(sa, *ss, *sc, (float *)xf, blockIdx.x == 0, [&] { // xf is free until ready()
+                if (fetched) return;
+                fetched = true;
+#pragma unroll
+                for (uint32_t j = 0; j < NL; j++) {
+                    const uint32_t i = threadIdx.x + j * NT;
+                    if (lutp && i < QW_LUT_BYTES / 16) lv[j] = ((const u4 *)a.glut)[(i + lrot) & (QW_LUT_BYTES / 16 - 1)];
+                }
+            });
 #pragma unroll
             for (uint32_t j = 0; j < NL; j++) {
                 const uint32_t i = threadIdx.x + j * NT;
-                if (lutp && i < QW_LUT_BYTES / 16) lv[j] = ((const u4 *)a.glut)[i];
-            }
-            select_all(sa, *ss, *sc, nullptr, blockIdx.x == 0);
-#pragma unroll
-            for (uint32_t j = 0; j < NL; j++) {
-                const uint32_t i = threadIdx.x + j * NT;
-                if (lutp && i < QW_LUT_BYTES / 16) ((u4 *)lut)[i] = lv[j];
+                if (lutp && i < QW_LUT_BYTES / 16) ((u4 *)lut)[(i + lrot) & (QW_LUT_BYTES / 16 - 1)] = lv[j];
             }
             tabled = true; // visible to the other waves after the barrier of ready()
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
             qw_sel_scratch &so = *(qw_sel_scratch *)xf;
-            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0);
+            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [] {});
         }
     } else {
         if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
