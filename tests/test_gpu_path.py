@@ -223,6 +223,28 @@ def test_selection_ties_and_duplicates(gpu, oracle):
     assert list(got.ue[:10]) == [110] + list(range(100, 109))
 
 
+@pytest.mark.parametrize("E", [64, 128, 256, 512, 1024])
+def test_selection_close_values_and_every_expert_count(gpu, oracle, E):
+    """Hundreds of logits that agree in their upper 16 bits (the selection's first bound leaves more than 64
+    candidates and has to be refined), descending and ascending runs, for every expert count with a register build."""
+    K, nb = 10, 16
+    rng = np.random.default_rng(500 + E)
+    logits = rng.normal(0, 1, (nb, E + 1)).astype(np.float32)
+    n = min(E, 200)
+    logits[:2] *= np.float32(0.1)  # the rest of rows 0 and 1 stays below the runs
+    logits[0, :n] = (1.0 + np.arange(n) * 2.0 ** -20).astype(np.float32)          # ascending by one part in 2^20
+    logits[1, :n] = (1.0 + np.arange(n)[::-1] * 2.0 ** -20).astype(np.float32)    # descending
+    logits[2, :E] = -np.float32(2.0) - rng.permutation(E).astype(np.float32) * np.float32(2.0 ** -18)  # all negative, all close
+    logits[3, :E] = np.float32(0.5)                                               # all equal
+    logits[3, E // 2:E // 2 + 3] = np.float32(0.75)
+    logits[4, :E] = np.repeat(rng.normal(0, 1, E // 8).astype(np.float32), 8)     # every value eight times
+    got = _select_on_gpu(gpu, logits, nb, E, K)
+    _check_sel(got, oracle.select(logits, K, got.gnb), nb, K)
+    ids = oracle.topk_ids(logits, K)
+    assert list(ids[0]) == list(range(n - 1, n - 11, -1)) and list(ids[1]) == list(range(10))
+    assert list(ids[3]) == [E // 2, E // 2 + 1, E // 2 + 2] + list(range(7))
+
+
 # ---------------------------------------------------------------- one MoE layer
 @pytest.mark.parametrize("nb,fmt", [(1, 21), (3, 21), (8, 21), (16, 21), (8, 8), (16, 8)])
 def test_moe_layer_parity(gpu, oracle, nb, fmt):
