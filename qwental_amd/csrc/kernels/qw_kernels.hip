@@ -1016,7 +1016,7 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
         },
         ready);
 }
-template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
+template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc, uint8_t *rowbit /* [32] */) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
     const bool tp2 = (tpe & (tpe - 1)) == 0; // D = 1024, 2048: shifts instead of divisions
     const uint32_t tsh = (uint32_t)__builtin_ctz(tpe);
@@ -1074,11 +1074,12 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             const bool p2 = (upr & (upr - 1)) == 0; // I = 256, 512, 1024: shifts instead of divisions
             const uint32_t ush = (uint32_t)__builtin_ctz(upr);
             const uint32_t rows = g0.mask | (both ? g1.mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
+            // the rows in use, in order (a table in LDS: finding the k-th set bit per item costs more than the copy)
+            if (threadIdx.x < 32 && ((rows >> threadIdx.x) & 1)) rowbit[__builtin_popcount(rows & ((1u << threadIdx.x) - 1))] = (uint8_t)threadIdx.x;
+            __syncthreads();
             // item i of the copy: (row in use, plane, 16-byte unit) -> source address and destination index
             auto place = [&](uint32_t i, uint32_t &dst) {
-                uint32_t m = rows;
-                for (uint32_t k = p2 ? i >> (ush + 1) : i / per; k; k--) m &= m - 1; // drop the rows before this one
-                const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, t = bit & 15, r = p2 ? i & (per - 1) : i % per;
+                const uint32_t bit = rowbit[p2 ? i >> (ush + 1) : i / per], sg = bit >> 4, t = bit & 15, r = p2 ? i & (per - 1) : i % per;
                 const uint32_t pl = p2 ? r >> ush : r / upr, c = p2 ? r & (upr - 1) : r % upr;
                 const uint32_t s = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + t];
                 dst = ((sg * 2 + pl) * upr + c) * 16 + t;
@@ -1125,8 +1126,8 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
 }
 #define QW_DN_RANGE(F, CH, FSD, CHSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
-        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; } L; \
-        dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
+        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; uint8_t rowbit[32]; } L; \
+        dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc, L.rowbit);                                \
     }
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
 QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
