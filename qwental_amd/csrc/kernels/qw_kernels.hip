@@ -1083,7 +1083,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
                 const uint32_t pl = p2 ? r >> ush : r / upr, c = p2 ? r & (upr - 1) : r % upr;
                 const uint32_t s = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + t];
                 dst = ((sg * 2 + pl) * upr + c) * 16 + t;
-                return (const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + s) * a.I + 8 * c);
+                return pl * a.hplane + (t * (K + 1) + s) * a.I + 8 * c; // in binary16 units from a.H (32 bits hold it)
             };
             // every load of the workgroup is issued before the first store (up to 4 a thread: 24 rows of 2 x 64 units
             // over 768 threads), with the table copy between the two; the destinations are worked out again for the
@@ -1093,7 +1093,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
 #pragma unroll
             for (int j = 0; j < NV; j++) {
                 uint32_t dd;
-                if (threadIdx.x + j * blockDim.x < nitem) v[j] = *place(threadIdx.x + j * blockDim.x, dd);
+                if (threadIdx.x + j * blockDim.x < nitem) v[j] = *(const u4 *)(a.H + place(threadIdx.x + j * blockDim.x, dd));
             }
             if (!tables && (qw_has_lut(F) || qw_has_lut(FSD))) qw_lut_copy(lut, (const u2 *)a.glut);
             tables = true;
@@ -1107,7 +1107,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             }
             for (uint32_t i = threadIdx.x + NV * blockDim.x; i < nitem; i += blockDim.x) { // larger I or fewer threads
                 uint32_t dd;
-                const u4 vv = *place(i, dd);
+                const u4 vv = *(const u4 *)(a.H + place(i, dd));
                 ((u4 *)arows)[dd] = vv;
             }
             __syncthreads();
