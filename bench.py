@@ -261,6 +261,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="B = 16 only, no ragged-step table (profiling runs)")
     ap.add_argument("--copy-calib", action="store_true", help="also run the copy kernel over 1 GiB three times (scale for the memory counters)")
     ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
+    ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives, no sharding)" % a.gpus, file=sys.stderr)
@@ -270,6 +271,9 @@ def main():
     from qwental_amd.stack import MoeStack
 
     gpu = q.Gpu()
+    if a.dense_only:
+        print(json.dumps({"qmv": qmv_table(gpu), "qmv_formats": formats_table(gpu)}))
+        return 0
     t0 = time.perf_counter()
     stack = MoeStack(gpu, layers=a.layers, nbmax=16)
     rng = np.random.default_rng(2024)

@@ -1085,10 +1085,10 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
                 dst = ((sg * 2 + pl) * upr + c) * 16 + t;
                 return pl * a.hplane + (t * (K + 1) + s) * a.I + 8 * c; // in binary16 units from a.H (32 bits hold it)
             };
-            // every load of the workgroup is issued before the first store (up to 4 a thread: 24 rows of 2 x 64 units
+            // every load of the workgroup is issued before the first store (up to 2 a thread: 12 rows of 2 x 64 units
             // over 768 threads), with the table copy between the two; the destinations are worked out again for the
             // stores rather than kept in registers
-            constexpr int NV = 4;
+            constexpr int NV = 2;
             u4 v[NV];
 #pragma unroll
             for (int j = 0; j < NV; j++) {
