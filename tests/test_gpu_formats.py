@@ -143,3 +143,53 @@ def test_matvec_rows_independent_of_batch(gpu):
         for bb in (wb, xb, yb, y1):
             bb.free()
     path.close()
+
+
+@pytest.mark.parametrize("ftype", [20, 1, 30])
+def test_matvec_short_rows_and_few_rows(gpu, oracle, ftype):
+    """K that is a multiple of 32 but not of 256 (one decoding unit per chunk), fewer rows than a tile, one row."""
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    for N, K, nb in ((5, 96, 3), (1, 32, 1), (33, 1056, 16), (16, 4064, 2)):
+        rng = np.random.default_rng(2000 + ftype + N + K)
+        W = synth.matrix(rng, ftype, N, K)
+        x = synth.activations(rng, nb, K)
+        wb, xb, yb = gpu.buf_from(W), gpu.buf_from(x), gpu.buf(nb * N * 4)
+        b = gpu.batch()
+        path.qmv_gg(b, q.Tensor(wb, ftype), N, K, xb, yb, nb, fout=True)
+        assert b.end() >= 0, gpu.last_error()
+        y = yb.view(np.float32)[:nb * N].reshape(nb, N)
+        ref = oracle.qmv(ftype, W, N, K, x, f64=True)
+        assert maxrel(y, ref) <= 1e-5, (ftype, N, K, maxrel(y, ref))
+        for bb in (wb, xb, yb):
+            bb.free()
+    path.close()
+
+
+def test_multi_matrix_largest_k_and_bad_calls(gpu, oracle):
+    """K = 4096 (the largest staged row), and the host checks of the multi-matrix launch."""
+    K, nb = 4096, 4
+    fmts, Ns = (14, 23), (48, 272)
+    rng = np.random.default_rng(31)
+    Ws = [synth.matrix(rng, f, n, K) for f, n in zip(fmts, Ns)]
+    x = synth.activations(rng, nb, K)
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    wbs, ybs, xb = [gpu.buf_from(w) for w in Ws], [gpu.buf(nb * n * 4) for n in Ns], gpu.buf_from(x)
+    b = gpu.batch()
+    path.qmv_ggm(b, [q.Tensor(wb, f) for wb, f in zip(wbs, fmts)], list(Ns), K, xb, ybs, nb)
+    assert b.end() >= 0, gpu.last_error()
+    for W, f, n, yb in zip(Ws, fmts, Ns, ybs):
+        assert maxrel(yb.view(np.float32)[:nb * n].reshape(nb, n), oracle.qmv(f, W, n, K, x, f64=True)) <= 1e-5
+    # an output buffer too small for its matrix fails the batch before anything is launched
+    small = gpu.buf(16)
+    b = gpu.batch()
+    path.qmv_ggm(b, [q.Tensor(wbs[0], fmts[0])], [Ns[0]], K, xb, [small], nb)
+    assert b.end(check=False) < 0 and "needs" in gpu.last_error()
+    # a weight buffer shorter than its rows
+    b = gpu.batch()
+    path.qmv_ggm(b, [q.Tensor(small, 14)], [Ns[0]], K, xb, [ybs[0]], nb)
+    assert b.end(check=False) < 0
+    ok, err = gpu.compile("#define qmv_ggm bad\n#define KD 8192\n#define NB 1\n#define NMAT 1\n#define GF0 12\n")
+    assert not ok and "8192" in err
+    for bb in wbs + ybs + [xb, small]:
+        bb.free()
+    path.close()
