@@ -105,6 +105,9 @@ struct qw_batch {
     struct { bool valid; int fmt; const uint8_t *Wsg, *Wsu; qw_hbuf *hg, *hu; uint32_t rowbytes, nbr; } pend_sg;
     struct { bool valid; int fmt; const uint8_t *Wsd; qw_hbuf *hd; float *Psh; uint32_t rowbytes, nbr; } pend_sd;
     struct { bool valid; qwk_select_args a; } pend_sel; // the selection moe_pre_gg owes: made inside the gate/up launch, or by a launch of its own
+    // a grouped product over IQ3_S rows that waits for its twin (gate, then up over the same packed rows: one launch
+    // over the tile-major copy that holds both); launched alone at the next other dispatch or at submit
+    struct { bool valid; qwk_pf_args a; qw_hbuf *hw, *hx, *hy; int E; } pend_pf;
 };
 
 struct qw_gpu {
@@ -1114,6 +1117,34 @@ static bool tr_pk_combine(qw_batch *b, unsigned gy) { // 0 D, 1 pos_of, 2 w, 3 Y
     return true;
 }
 // src/engine.c:3257-3264: 0 X, 1 W, 4 Y, 5 {M, N}, 6 tiles, 7 tables; grid y = entries of the tile table
+// One grouped-product launch. IQ3_S weights go through the tile-major copy when there is one: wb != NULL = the second
+// matrix of a gate / up pair (tiles of 8 + 8 rows, outputs a->Y and a->Y1), else a single matrix (tiles of 16 rows).
+static bool launch_pf(qw_batch *b, qwk_pf_args *a, int F, int E, qw_hbuf *hw, qw_hbuf *hwb, const uint8_t *wb) {
+    a->split = 16, a->ntn = a->N / 16;
+    char fn[32];
+    if (F == 21 && a->K % 256 == 0) {
+        const uint32_t nblk = a->K / 256, split = wb ? 8 : 16;
+        const uint64_t ntiles = (uint64_t)E * (a->N / split);
+        const uint8_t *pk = get_pack(b, hw, a->W, wb ? hwb : NULL, wb, ntiles, nblk, a->rowbytes, split);
+        if (pk) {
+            a->W = pk, a->rowbytes = nblk * QW_SLAB_BYTES, a->split = split, a->ntn = a->N / split;
+            fname_fmt(fn, sizeof fn, "qwk_pf_f121_c%d", a->K % 512 == 0 ? 2 : 1);
+            return add_launch(b, intern(fn), persistent_grid(b->g, a->max_tiles * a->ntn, 8), 512, a, sizeof *a);
+        }
+        if (wb) return false; // the caller launches the two matrices one by one
+    }
+    if (F == 21) fname_fmt(fn, sizeof fn, "qwk_pf_f21_c%d", a->K % 512 == 0 ? 2 : 1);
+    else fname_fmt(fn, sizeof fn, "qwk_pf_f8_c4");
+    // every entry can hold a tile: the grid covers the whole table, the kernel counts the entries in use
+    return add_launch(b, intern(fn), persistent_grid(b->g, a->max_tiles * a->ntn, 8), 512, a, sizeof *a);
+}
+
+static bool flush_pf(qw_batch *b) {
+    if (!b->pend_pf.valid) return true;
+    b->pend_pf.valid = false;
+    return launch_pf(b, &b->pend_pf.a, 21, b->pend_pf.E, b->pend_pf.hw, NULL, NULL);
+}
+
 static bool tr_pf(qw_batch *b, unsigned gy) {
     const qw_kparams *p = &b->k->p;
     uint32_t mn[2];
@@ -1125,11 +1156,30 @@ static bool tr_pf(qw_batch *b, unsigned gy) {
     if (!bind_ptr(b, 0, (size_t)a.M * p->K * 2, false, "X", (void **)&a.X) || !bind_ptr(b, 1, (size_t)p->E * a.N * rb, false, "weights", (void **)&a.W) ||
         !bind_ptr(b, 4, (size_t)a.M * a.N * 2, true, "Y", (void **)&a.Y) || !bind_ptr(b, 6, (size_t)gy * 16, false, "tiles", (void **)&a.tiles)) return false;
     if (b->buf[0].off % 16 || b->buf[6].off % 16) return fail(b, "moe_pf_gg: X and the tile table must be 16-byte aligned");
-    char fn[32];
-    if (p->F == 21) fname_fmt(fn, sizeof fn, "qwk_pf_f21_c%d", p->K % 512 == 0 ? 2 : 1);
-    else fname_fmt(fn, sizeof fn, "qwk_pf_f8_c4");
-    // every entry can hold a tile: the grid covers the whole table, the kernel counts the entries in use
-    return add_launch(b, intern(fn), persistent_grid(b->g, gy * (a.N / 16), 8), 512, &a, sizeof a);
+    qw_hbuf *hw = b->buf[1].h, *hx = b->buf[0].h, *hy = b->buf[4].h;
+    if (b->pend_pf.valid) {
+        // the twin of the waiting product: same packed rows, table and shape, other weights and output
+        const qwk_pf_args *q = &b->pend_pf.a;
+        const bool twin = p->F == 21 && q->X == a.X && q->tiles == a.tiles && q->M == a.M && q->N == a.N && q->K == a.K && q->max_tiles == a.max_tiles &&
+                          q->W != a.W && q->Y != a.Y && b->pend_pf.E == p->E && hy != b->pend_pf.hx && b->pend_pf.hy != hx && b->pend_pf.hy != hy;
+        if (twin) {
+            qwk_pf_args f = *q;
+            f.Y1 = a.Y;
+            b->pend_pf.valid = false;
+            if (launch_pf(b, &f, 21, p->E, b->pend_pf.hw, hw, a.W)) return true;
+            if (b->failed) return false;
+            qwk_pf_args first = *q; // no tile-major copy (small buffers, copies switched off): one by one
+            return launch_pf(b, &first, 21, p->E, b->pend_pf.hw, NULL, NULL) && launch_pf(b, &a, 21, p->E, hw, NULL, NULL);
+        }
+        if (!flush_pf(b)) return false;
+    }
+    if (p->F == 21 && p->K % 256 == 0 && b->g->repack) { // may be the first of a pair: wait for the next dispatch
+        b->pend_pf.valid = true;
+        b->pend_pf.a = a;
+        b->pend_pf.hw = hw, b->pend_pf.hx = hx, b->pend_pf.hy = hy, b->pend_pf.E = p->E;
+        return true;
+    }
+    return launch_pf(b, &a, p->F, p->E, hw, NULL, NULL);
 }
 
 // helpers: 0 src, 1 dst, 2 {n16 (uint64), seed (uint64)}; grid x = workgroups of 256 threads
@@ -1162,6 +1212,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     const int first = b->nl;
     bool ok;
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
+    if (b->k->fam != FAM_PF && !flush_pf(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
     case FAM_QMV_GGM: ok = tr_qmvm(b); break;
@@ -1191,7 +1242,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
-    if (b->failed || !flush_select(b)) return false;
+    if (b->failed || !flush_select(b) || !flush_pf(b)) return false;
     if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
     // host -> device for what this segment binds
     const unsigned mark = ++g->mark;

@@ -172,11 +172,14 @@ typedef struct {
 } qwk_combine_args;
 typedef struct { /* Y[m][n] = X[m] . W[expert][n] for the rows m of every tile entry; binary16 in and out */
     const uint16_t *X;
-    const uint8_t *W;     /* [E][N][rowbytes] */
+    const uint8_t *W;     /* [E][N][rowbytes]; packed (QW_F_PACKED): [E][ntn][rowbytes] tiles, rowbytes = bytes of a tile */
     uint16_t *Y;          /* [M][N] */
     const uint32_t *tiles;
-    uint32_t M, N, K, rowbytes, max_tiles, tm, pad0, pad1;
+    uint32_t M, N, K, rowbytes, max_tiles, tm;
+    uint32_t split, ntn;  /* packed: split 16 = one matrix of N rows; split 8 = a tile holds 8 rows of matrix A (-> Y) and 8 of
+                           * matrix B (-> Y1), N rows each; ntn = tiles per expert (N / 16 or N / 8) */
     const void *glut;
+    uint16_t *Y1;
 } qwk_pf_args;
 
 typedef struct { /* synthetic weights: nblocks GGUF blocks of one type, scale d = binary16(|N(0, sigma)|), the rest uniform */

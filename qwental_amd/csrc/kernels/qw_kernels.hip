@@ -1274,13 +1274,14 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
     }
     if (mine) atomicAdd(cnt, mine);
     __syncthreads();
-    const uint32_t used = *cnt, ntn = a.N / 16, ntasks = used * ntn, cpr = a.K / (C::BLK_K * CH);
+    const uint32_t used = *cnt, ntn = a.ntn, ntasks = used * ntn, cpr = a.K / (C::BLK_K * CH);
     const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
     f4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
-    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, lane & 3,
+    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
         [&](uint32_t task) {
             const u4 e = tl[task / ntn];
-            return a.W + ((size_t)e.x * a.N + 16 * (task % ntn) + (lane >> 2)) * a.rowbytes;
+            if constexpr (F == QW_F_PACKED) return a.W + ((size_t)e.x * ntn + task % ntn) * a.rowbytes; // the tile's slabs
+            else return a.W + ((size_t)e.x * a.N + 16 * (task % ntn) + (lane >> 2)) * a.rowbytes;
         },
         [&](uint32_t task, uint32_t ci, const C &c) {
             const u4 e = tl[task / ntn];
@@ -1307,13 +1308,16 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
                 c.template mac_groups<4>(lut, r4, k0, kg, acc);
             }
             if (ci + 1 != cpr) return;
-            const uint32_t col = 16 * (task % ntn) + n;
+            // a tile of two matrices: rows 0..7 are matrix A's (-> Y), rows 8..15 matrix B's (-> Y1)
+            const bool second = a.split == 8 && n >= 8;
+            const uint32_t col = a.split == 8 ? 8 * (task % ntn) + (n & 7) : 16 * (task % ntn) + n;
+            uint16_t *Y = second ? a.Y1 : a.Y;
 #pragma unroll
             for (uint32_t g = 0; g < 4; g++) {
 #pragma unroll
                 for (uint32_t j = 0; j < 4; j++) {
                     const uint32_t m = m0 + 16 * g + 4 * kg + j;
-                    if (m < m1) a.Y[(size_t)m * a.N + col] = qw_f2h(acc[g][j]);
+                    if (m < m1) Y[(size_t)m * a.N + col] = qw_f2h(acc[g][j]);
                 }
                 acc[g] = f4{0, 0, 0, 0};
             }
@@ -1325,6 +1329,7 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
         pf_body<F, CH>(a, L.lut, L.tl, &L.cnt);                                                  \
     }
 QW_PF(21, 2, qwk_pf_f21_c2) QW_PF(21, 1, qwk_pf_f21_c1) QW_PF(8, 4, qwk_pf_f8_c4)
+QW_PF(121, 2, qwk_pf_f121_c2) QW_PF(121, 1, qwk_pf_f121_c1) // tile-major IQ3_S: one matrix, or gate and up rows side by side
 
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).

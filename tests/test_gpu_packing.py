@@ -24,7 +24,7 @@ def expert_ref(o, m, e, x):
     return h, Wd
 
 
-def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed):
+def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed, device_only=False):
     rng = np.random.default_rng(seed)
     m = synth.moe_layer(rng, D, I, E, fgu=fmt, fd=fmt, fsh=fmt)
     x = synth.activations(rng, T, D)
@@ -32,11 +32,14 @@ def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed):
     w /= w.sum(axis=1, keepdims=True)
     path = q.Path(gpu, D, I, E, K, 16)
     path.pf_reserve(T, tm)
-    dl = DeviceLayer(gpu, m)
+    dl = DeviceLayer(gpu, m, device_only=device_only)
     xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.ravel()), gpu.buf(T * D * 2)
+    packed0 = gpu.L.qw_hip_packed_bytes(gpu.g)
     b = gpu.batch()
     path.pf_moe(b, dl.layer, T, xb, ib, wb, ob)
     assert b.end() >= 0, gpu.last_error()
+    if device_only and fmt == 21:  # weights that live in HBM only get the tile-major copies: gate + up as one, down
+        assert gpu.L.qw_hip_packed_bytes(gpu.g) - packed0 == (2 * E * I * (D // 256) + E * D * (I // 256)) // 16 * 1792
     P = T * K
     # integer stages against the oracle (kernels/moe_prefill.metal:15-93)
     mt = path.pf_max_tiles()
@@ -71,6 +74,16 @@ def test_packing_uniform_routing(gpu, oracle, fmt, tm):
     rng = np.random.default_rng(7 + tm)
     ids = np.stack([rng.choice(E, K, replace=False) for _ in range(T)])
     run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, 70 + tm)
+
+
+@pytest.mark.parametrize("tm", [16, 64])
+def test_packing_tile_major_weights(gpu, oracle, tm):
+    """The same through the tile-major copies (weights resident in HBM only): gate and up of a tile entry in one
+    launch, results as with the GGUF rows."""
+    T, E, K, D, I = 40, 32, 4, 512, 512
+    rng = np.random.default_rng(17 + tm)
+    ids = synth.zipf_ids(rng, T, E, K)
+    run_case(gpu, oracle, T, ids, E, K, D, I, 21, tm, 170 + tm, device_only=True)
 
 
 def test_packing_zipf_hot_experts(gpu, oracle):
