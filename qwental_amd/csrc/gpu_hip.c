@@ -1128,6 +1128,10 @@ static bool launch_pf(qw_batch *b, qwk_pf_args *a, int F, int E, qw_hbuf *hw, qw
         const uint8_t *pk = get_pack(b, hw, a->W, wb ? hwb : NULL, wb, ntiles, nblk, a->rowbytes, split);
         if (pk) {
             a->W = pk, a->rowbytes = nblk * QW_SLAB_BYTES, a->split = split, a->ntn = a->N / split;
+            if (a->tm <= 16 && a->K <= 2560) { // entries of one group of rows: the rows are staged in LDS per workgroup range
+                fname_fmt(fn, sizeof fn, "qwk_pfr_f121_c%d", a->K % 512 == 0 ? 2 : 1);
+                return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, a->max_tiles * a->ntn), 64 * QW_WAVES_GU, a, sizeof *a);
+            }
             fname_fmt(fn, sizeof fn, "qwk_pf_f121_c%d", a->K % 512 == 0 ? 2 : 1);
             return add_launch(b, intern(fn), persistent_grid(b->g, a->max_tiles * a->ntn, 8), 512, a, sizeof *a);
         }

@@ -1331,6 +1331,65 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
 QW_PF(21, 2, qwk_pf_f21_c2) QW_PF(21, 1, qwk_pf_f21_c1) QW_PF(8, 4, qwk_pf_f8_c4)
 QW_PF(121, 2, qwk_pf_f121_c2) QW_PF(121, 1, qwk_pf_f121_c1) // tile-major IQ3_S: one matrix, or gate and up rows side by side
 
+// The same product for entries of at most 16 packed rows over tile-major weights, the way the decode kernels work:
+// a workgroup takes a contiguous range of (entry, weight tile) tasks - the tiles of one entry, or the end of one and
+// the start of the next -, copies the entry's rows into LDS in fragment order once (after its first weight loads are
+// issued) and its waves walk the tiles with the activations read from LDS.
+template <int CH> __device__ __forceinline__ void pf_range_body(const qwk_pf_args &a, u2 *lut, u4 *xf, uint32_t *cnt) {
+    typedef qw_chunk<QW_F_PACKED, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, nwv = blockDim.x >> 6;
+    if (threadIdx.x == 0) *cnt = 0;
+    qw_lut_copy(lut, (const u2 *)a.glut);
+    __syncthreads();
+    uint32_t mine = 0; // the non-empty entries are the first ones of the table
+    for (uint32_t t = threadIdx.x; t < a.max_tiles; t += blockDim.x) {
+        const u4 e = *(const u4 *)(a.tiles + 4 * t);
+        mine += e.z > e.y;
+    }
+    if (mine) atomicAdd(cnt, mine);
+    __syncthreads();
+    const uint32_t used = *cnt, ntn = a.ntn, total = used * ntn, cpr = a.K / (C::BLK_K * CH);
+    const uint32_t per = (total + gridDim.x - 1) / gridDim.x;
+    const uint32_t end = (blockIdx.x + 1) * per < total ? (blockIdx.x + 1) * per : total;
+    for (uint32_t pos = blockIdx.x * per; pos < end;) {
+        const uint32_t entry = pos / ntn, t0 = pos % ntn, nt = ntn - t0 < end - pos ? ntn - t0 : end - pos;
+        const u4 e = *(const u4 *)(a.tiles + 4 * entry);
+        const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)e.y), m1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)e.z);
+        const uint8_t *W = a.W + ((size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)e.x) * ntn + t0) * a.rowbytes;
+        bool staged = false;
+        auto ready = [&] {
+            if (staged) return;
+            staged = true;
+            __syncthreads(); // the waves are done with the rows of the segment before
+            qw_stage_x(xf, a.X + (size_t)m0 * a.K, a.K, a.K, m1 - m0);
+            __syncthreads();
+        };
+        const qw_afrag_lds af = {xf, n};
+        f4 acc = {0, 0, 0, 0};
+        qw_task_pipeline<C>(nt, qw_wave(), nwv, cpr, CH * C::BLK_B, lane, [&](uint32_t i) { return W + (size_t)i * a.rowbytes; },
+            [&](uint32_t i, uint32_t ci, const C &c) {
+                c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+                if (ci + 1 != cpr) return;
+                const bool second = a.split == 8 && n >= 8; // rows 8..15 of a two-matrix tile belong to the second output
+                const uint32_t col = a.split == 8 ? 8 * (t0 + i) + (n & 7) : 16 * (t0 + i) + n;
+                uint16_t *Y = second ? a.Y1 : a.Y;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; j++) {
+                    const uint32_t m = m0 + 4 * kg + j;
+                    if (m < m1) Y[(size_t)m * a.N + col] = qw_f2h(acc[j]);
+                }
+                acc = f4{0, 0, 0, 0};
+            }, ready);
+        pos += nt;
+    }
+}
+#define QW_PFR(CH, NAME)                                                                          \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_pf_args a) {                 \
+        __shared__ struct { u2 lut[QW_LUT_ENTRIES]; u4 xf[QW_XF_MAXK * 2]; uint32_t cnt; } L;     \
+        pf_range_body<CH>(a, L.lut, L.xf, &L.cnt);                                                \
+    }
+QW_PFR(2, qwk_pfr_f121_c2) QW_PFR(1, qwk_pfr_f121_c1)
+
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).
 extern "C" __global__ __launch_bounds__(256) void qwk_cmb(qwk_cmb_args a) {
