@@ -278,6 +278,35 @@ def test_moe_layer_parity(gpu, oracle, nb, fmt):
     path.close()
 
 
+@pytest.mark.parametrize("D,I,E,K,nb,fgu,fd,fsh,fshd,dev", [
+    (2560, 512, 64, 10, 16, 21, 21, 21, 8, True),    # the widest staged activation row; shared down Q8_0; tile-major copies
+    (1024, 256, 128, 8, 5, 21, 21, 21, 21, True),    # one IQ3_S block per down row
+    (768, 768, 64, 4, 7, 21, 21, 21, 21, False),     # neither a multiple of 512: one block per chunk; I > 512: the any-shape down kernel
+    (512, 1024, 32, 6, 12, 8, 8, 8, 8, False),       # Q8_0 throughout, long down rows
+    (1536, 512, 256, 16, 16, 21, 8, 8, 21, True),    # sixteen picks per token; mixed formats per projection
+    (256, 256, 1024, 10, 3, 21, 21, 21, 21, False),  # the smallest rows, the most experts
+    (2048, 512, 48, 10, 9, 21, 21, 21, 21, True),    # an expert count without a register build of the selection
+])
+def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
+    """Shapes and format mixes off the benchmark's: every kernel variant the host can pick is reached by one of them."""
+    rng = np.random.default_rng(D + I + E + K + nb)
+    m = synth.moe_layer(rng, D, I, E, fgu=fgu, fd=fd, fsh=fsh, fshd=fshd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    path = q.Path(gpu, D, I, E, K, 16)
+    dl = DeviceLayer(gpu, m, device_only=dev)
+    out, lg, selraw, _ = run_moe(gpu, path, dl, x, nb)
+    gnb = 8 if nb <= 8 else 16
+    ref_lg = oracle.router(m["Wr"], m["wsg"], x)
+    assert maxrel(lg, ref_lg) <= 1e-5
+    _check_sel(oracle.Sel(selraw, gnb, K), oracle.select(lg, K, gnb), nb, K)
+    ref = oracle.moe_layer_f64(m, lg, x)
+    assert np.isfinite(out.astype(np.float64)).all()
+    assert maxrel(out, ref) <= TOL, maxrel(out, ref)
+    dl.free()
+    path.close()
+
+
 def test_moe_batched_equals_single(gpu):
     """Each row of a batched layer call equals the single-token call bit for bit (src/engine.c:7977-7987)."""
     D, I, E, K, nb = 2048, 512, 64, 10, 8
