@@ -641,18 +641,30 @@ __device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, u
 
 
 // Copy the 64 KB pre-signed table from global memory into LDS (all loads first, then the stores).
-__device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
+// Sixty-four 16-byte units from global memory straight into LDS, no register in between: lane l's unit lands at
+// dst + 16 l bytes (dst the same in every lane); src is per lane. Completion is counted like any other vector load:
+// qw_lds_arrive() before the barrier that publishes the data.
+__device__ __forceinline__ void qw_load_to_lds(const u4 *src_lane, u4 *dst_wave) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src_lane, (__attribute__((address_space(3))) void *)dst_wave, 16, 0, 0);
+}
+__device__ __forceinline__ void qw_lds_arrive() { __builtin_amdgcn_s_waitcnt(0); }
+
+// Issue the copy of the 64 KB table into LDS (direct loads, a wave takes 64 entries at a time). Every workgroup of a
+// launch starts at a different place of the table (a rotation by its index), so that at any moment the workgroups
+// ask different memory channels. The caller runs qw_lds_arrive() and a barrier before the table is read.
+__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut) {
     const u4 *src = (const u4 *)glut;
     u4 *dst = (u4 *)lut;
     constexpr uint32_t N = QW_LUT_BYTES / 16;
-    const uint32_t rot = blockIdx.x * 272u; // every workgroup starts elsewhere in the table (see qw_stage_x)
-    for (uint32_t i = threadIdx.x; i < N; i += 8 * blockDim.x) {
-        u4 v[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) v[j] = src[(i + j * blockDim.x + rot) & (N - 1)];
-#pragma unroll
-        for (int j = 0; j < 8; j++) if (i + j * blockDim.x < N) dst[(i + j * blockDim.x + rot) & (N - 1)] = v[j];
+    const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63;
+    for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i < N; i += blockDim.x) {
+        const uint32_t j = (i + rot) & (N - 1); // a multiple of 64, the same in every lane
+        qw_load_to_lds(src + j + lane, dst + j);
     }
+}
+__device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {
+    qw_lut_copy_issue(lut, glut);
+    qw_lds_arrive();
 }
 
 template <class C, class R, class U>
