@@ -188,15 +188,21 @@ struct qw_afrag_lds2 {
 
 // Every workgroup of a launch copies the same bytes: each starts at a different place (a rotation by its index), so
 // that at any moment the workgroups ask different memory channels instead of all the same one.
-__device__ __forceinline__ void qw_stage_x(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
-    const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 272u) % n;
-    for (uint32_t i0 = threadIdx.x; i0 < n; i0 += blockDim.x) {
-        const uint32_t i = i0 + rot < n ? i0 + rot : i0 + rot - n;
-        const uint32_t c = i >> 4, m = i & 15;
-        u4 v = {0, 0, 0, 0};
-        if (m < nb) v = *(const u4 *)(x + (size_t)m * xstride + 8 * c);
-        xf[i] = v;
+// qw_stage_x_issue: direct global-to-LDS loads of the token columns in use, plain zero stores for the others; the
+// caller runs qw_lds_arrive() and a barrier before the fragments are read.
+__device__ __forceinline__ void qw_load_to_lds(const u4 *src_lane, u4 *dst_wave);
+__device__ __forceinline__ void qw_lds_arrive();
+__device__ __forceinline__ void qw_stage_x_issue(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
+    const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 320u) % n, lane = threadIdx.x & 63; // n and rot are multiples of 64
+    for (uint32_t i0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i0 < n; i0 += blockDim.x) {
+        const uint32_t base = i0 + rot < n ? i0 + rot : i0 + rot - n, i = base + lane, c = i >> 4, m = i & 15;
+        if (m < nb) qw_load_to_lds((const u4 *)(x + (size_t)m * xstride + 8 * c), xf + base);
+        else xf[i] = u4{0, 0, 0, 0};
     }
+}
+__device__ __forceinline__ void qw_stage_x(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
+    qw_stage_x_issue(xf, x, xstride, K, nb);
+    qw_lds_arrive();
 }
 
 // Straight from global memory: row pointers of binary16 planes; a null row contributes zeros.

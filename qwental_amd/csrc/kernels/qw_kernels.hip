@@ -493,7 +493,7 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
 // the ranks below K are the picks. T tokens go through together (the steps are chains of LDS and cross-lane
 // latencies, so a second token costs little). Returns a bit per token that was NOT done, with nothing written for
 // it: more than 64 keys reach T0 (many equal logits) and the caller falls back to select_tokens.
-// ws: 256 dwords of LDS scratch per token for this wave.
+// ws: 144 dwords of LDS scratch per token for this wave.
 // issued(): called once the loads of the logits are issued (the place for the caller's own prefetches: loads return in
 // the order of issue, and the logits are needed first).
 template <int PER, int T, class H>
@@ -545,7 +545,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
 #pragma unroll
     for (int t = 0; t < T; t++) {
         if ((fail >> t) & 1) continue;
-        u2 *cand = (u2 *)(ws + 256 * t + 64); // (key, expert) of candidate p
+        u2 *cand = (u2 *)(ws + 144 * t); // (key, expert) of candidate p
 #pragma unroll
         for (int j = 0; j < PER; j++)
             if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], lane * PER + j};
@@ -553,7 +553,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
     uint32_t mk[T], me[T], rank[T];
 #pragma unroll
     for (int t = 0; t < T; t++) {
-        const u2 mine = ((const u2 *)(ws + 256 * t + 64))[lane];
+        const u2 mine = ((const u2 *)(ws + 144 * t))[lane];
         // one 64-bit value per candidate whose order is the ranking order; lanes without a candidate hold the least
         mk[t] = lane < c[t] ? mine.x : 0, me[t] = lane < c[t] ? ~mine.y : 0;
         rank[t] = 0;
@@ -570,7 +570,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
                 const unsigned long long o = (unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)mk[t], (int)l) << 32 | (uint32_t)__builtin_amdgcn_readlane((int)me[t], (int)l);
                 rank[t] += o > mine;
             }
-        uint32_t *pkr = ws + 256 * t + 192; // key of rank r
+        uint32_t *pkr = ws + 144 * t + 128; // key of rank r
         if (lane < c[t] && rank[t] < K) {
             ids[tok[t] * K + rank[t]] = ~me[t];
             pkr[rank[t]] = mk[t];
@@ -579,7 +579,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
 #pragma unroll
     for (int t = 0; t < T; t++) {
         if ((fail >> t) & 1) continue;
-        const float p = qw_fkey_inv(ws[256 * t + 192 + (lane < K ? lane : 0)]);
+        const float p = qw_fkey_inv(ws[144 * t + 128 + (lane < K ? lane : 0)]);
         const float mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, p), 0)), ex = __expf(p - mx);
         float sm = 0;
         for (uint32_t r = 0; r < K; r++) sm += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), (int)r)); // rank order
@@ -620,7 +620,7 @@ __device__ __forceinline__ void select_token_any(const float *lg, float *v, uint
 __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 || E == 128 || E == 256 || E == 512 || E == 1024; }
 
 // The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
-// floats per wave (512 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
+// floats per wave (288 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
 template <class H>
 __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued) {
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
@@ -632,8 +632,8 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
     if (tid < 8) s.lead[tid] = 0;
     for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
-    if (fast) { // two tokens per wave at a time when there are more tokens than waves; lgs gives a wave 512 dwords
-        uint32_t *ws = (uint32_t *)lgs + 512 * wave;
+    if (fast) { // two tokens per wave at a time when there are more tokens than waves; lgs gives a wave 288 dwords
+        uint32_t *ws = (uint32_t *)lgs + 288 * wave;
         const uint32_t trot = a.nbr ? blockIdx.x % a.nbr : 0; // the workgroups of a launch read the tokens' logits in different orders
         auto rot = [&](uint32_t tt) { return tt + trot < a.nbr ? tt + trot : tt + trot - a.nbr; };
         const bool pairs = E <= 512; // sixteen keys a lane: one token at a time (registers)
@@ -772,35 +772,28 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 // Order of the set-up when the record is given: the record first (one memory round trip, one barrier: the row
 // addresses depend on it); then every wave issues its first weight loads, and only then the table copy, the activation
 // staging and the second barrier follow, overlapping that first round trip to HBM. When the selection is made here,
-// the table is fetched under it instead.
+// the table and the activations are fetched under it instead (direct global-to-LDS loads: no registers are held).
 template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss) {
     bool staged = false, tabled = false;
     if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
         if (qw_select_fast_e(a.E)) {
-            // The table does not depend on the selection: its loads are issued right behind those of the logits and
-            // are in flight while the selection is made; it is written to LDS after it. (The activations follow in
-            // ready(), under the first weight loads: holding them here as well would spill registers.)
-            constexpr uint32_t NT = QW_WG_GU, NL = (QW_LUT_BYTES / 16 + NT - 1) / NT;
+            // Neither the table nor the activations depend on the selection: their direct-to-LDS loads are issued right
+            // behind those of the logits and land while the selection is made. The selection's scratch lies behind
+            // the staged activations when D leaves room there (D <= 2048), else in their place (they follow in ready()).
             constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
-            const uint32_t lrot = blockIdx.x * 272u; // every workgroup starts elsewhere in the table
-            u4 lv[NL];
+            const bool early = a.D * 2 + (QW_WG_GU / 64) * 288 / 4 <= QW_XF_MAXK * 2;
             bool fetched = false;
-            select_all(sa, *ss, *sc, (float *)xf, blockIdx.x == 0, [&] { // xf is free until ready()
+            select_all(sa, *ss, *sc, (float *)(early ? xf + a.D * 2 : xf), blockIdx.x == 0, [&] {
                 if (fetched) return;
                 fetched = true;
-#pragma unroll
-                for (uint32_t j = 0; j < NL; j++) {
-                    const uint32_t i = threadIdx.x + j * NT;
-                    if (lutp && i < QW_LUT_BYTES / 16) lv[j] = ((const u4 *)a.glut)[(i + lrot) & (QW_LUT_BYTES / 16 - 1)];
-                }
+                if (lutp) qw_lut_copy_issue(lut, (const u2 *)a.glut);
+                if (early) qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
             });
-#pragma unroll
-            for (uint32_t j = 0; j < NL; j++) {
-                const uint32_t i = threadIdx.x + j * NT;
-                if (lutp && i < QW_LUT_BYTES / 16) ((u4 *)lut)[(i + lrot) & (QW_LUT_BYTES / 16 - 1)] = lv[j];
-            }
-            tabled = true; // visible to the other waves after the barrier of ready()
+            qw_lds_arrive();
+            __syncthreads();
+            tabled = true;
+            staged = early;
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
             qw_sel_scratch &so = *(qw_sel_scratch *)xf;
             select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [] {});
