@@ -1009,12 +1009,13 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
         },
         ready);
 }
-template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc, uint8_t *rowbit /* [32] */) {
+template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
     const bool tp2 = (tpe & (tpe - 1)) == 0; // D = 1024, 2048: shifts instead of divisions
     const uint32_t tsh = (uint32_t)__builtin_ctz(tpe);
     auto div_tpe = [&](uint32_t x) { return tp2 ? x >> tsh : x / tpe; };
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
+    if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // lands in LDS meanwhile; awaited in ready()
     __syncthreads();
     const uint32_t *ue = sc->ue, *mask = sc->mask;
     const uint8_t *slot = sc->slot;
@@ -1026,7 +1027,6 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     const uint32_t V = vsh + U * tpe;
     uint32_t per = (V + gridDim.x - 1) / gridDim.x;
     if (per > tpe) per = tpe;
-    bool tables = false;
     for (uint32_t base = blockIdx.x * per; base < V; base += gridDim.x * per) { // one round unless the grid is small
         const uint32_t end = base + per < V ? base + per : V;
         // virtual expert of a position: 0 = shared (positions below vsh), then the routed experts
@@ -1054,55 +1054,37 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         const qw_dn_seg g0 = seg(v0), g1 = seg(v1);
         const bool both = v1 != v0;
         bool staged = false;
-        // set-up of a round, run by every wave once its first weight loads are in flight: the table (first round),
-        // the H rows of the (at most two) experts of this range, and the barrier
+        // Set-up of a round, run by every wave once its first weight loads are in flight: the H rows of the tokens that
+        // picked the range's (at most two) experts, both planes, by direct global-to-LDS loads, and the barrier.
+        // Fragment order in LDS, [segment][plane][c][token], 16 bytes each (the sixteen lanes of a k-group read 256
+        // contiguous bytes): one load instruction fills four c of one plane, lane = (c, token); the lanes of tokens
+        // that did not pick the expert stay off and leave their columns as they are (those results are never stored).
         auto ready = [&] {
             if (staged) return;
             staged = true;
-            // The H rows of the tokens that picked the range's experts, both planes: the rows in use (a few of the 32
-            // possible) are numbered through the two masks, so that one pass of the workgroup usually copies them all;
-            // the loads of that pass are in flight while the table is copied. Fragment order in LDS,
-            // [segment][plane][c][token], 16 bytes each: the sixteen lanes of a k-group read 256 contiguous bytes.
-            const uint32_t upr = a.I / 8, per = 2 * upr; // 16-byte units per plane row, per row
-            const bool p2 = (upr & (upr - 1)) == 0; // I = 256, 512, 1024: shifts instead of divisions
-            const uint32_t ush = (uint32_t)__builtin_ctz(upr);
-            const uint32_t rows = g0.mask | (both ? g1.mask << 16 : 0), nitem = (uint32_t)__builtin_popcount(rows) * per;
-            // the rows in use, in order (a table in LDS: finding the k-th set bit per item costs more than the copy)
-            if (threadIdx.x < 32 && ((rows >> threadIdx.x) & 1)) rowbit[__builtin_popcount(rows & ((1u << threadIdx.x) - 1))] = (uint8_t)threadIdx.x;
-            __syncthreads();
-            // item i of the copy: (row in use, plane, 16-byte unit) -> source address and destination index
-            auto place = [&](uint32_t i, uint32_t &dst) {
-                const uint32_t bit = rowbit[p2 ? i >> (ush + 1) : i / per], sg = bit >> 4, t = bit & 15, r = p2 ? i & (per - 1) : i % per;
-                const uint32_t pl = p2 ? r >> ush : r / upr, c = p2 ? r & (upr - 1) : r % upr;
-                const uint32_t s = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + t];
-                dst = ((sg * 2 + pl) * upr + c) * 16 + t;
-                return pl * a.hplane + (t * (K + 1) + s) * a.I + 8 * c; // in binary16 units from a.H (32 bits hold it)
-            };
-            // every load of the workgroup is issued before the first store (up to 2 a thread: 12 rows of 2 x 64 units
-            // over 768 threads), with the table copy between the two; the destinations are worked out again for the
-            // stores rather than kept in registers
-            constexpr int NV = 2;
-            u4 v[NV];
-#pragma unroll
-            for (int j = 0; j < NV; j++) {
-                uint32_t dd;
-                if (threadIdx.x + j * blockDim.x < nitem) v[j] = *(const u4 *)(a.H + place(threadIdx.x + j * blockDim.x, dd));
-            }
-            if (!tables && (qw_has_lut(F) || qw_has_lut(FSD))) qw_lut_copy(lut, (const u2 *)a.glut);
-            tables = true;
-#pragma unroll
-            for (int j = 0; j < NV; j++) {
-                uint32_t dd;
-                if (threadIdx.x + j * blockDim.x < nitem) {
-                    place(threadIdx.x + j * blockDim.x, dd);
-                    ((u4 *)arows)[dd] = v[j];
+            const uint32_t upr = a.I / 8, ncb = upr / 4, ninst = (both ? 2 : 1) * 2 * ncb; // 16-byte units per plane row; instructions
+            const uint32_t lane = qw_lane(), t = lane & 15, rows = g0.mask | (both ? g1.mask << 16 : 0), nrows = (uint32_t)__builtin_popcount(rows);
+            if (nrows * 2 * upr <= blockDim.x) {
+                // few rows (a token or two per expert): one 16-byte unit per thread through a register, the waves
+                // of a row finding its bit in the mask by a scalar walk
+                const uint32_t i = threadIdx.x, k = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / (2 * upr))), r = i % (2 * upr), pl = r / upr, c = r % upr;
+                if (k < nrows) {
+                    uint32_t m = rows;
+                    for (uint32_t j = 0; j < k; j++) m &= m - 1;
+                    const uint32_t bit = (uint32_t)__builtin_ctz(m), sg = bit >> 4, tk = bit & 15;
+                    const uint32_t sl = (sg ? g1.sh : g0.sh) ? K : slot[(sg ? g1.u : g0.u) * gnb + tk];
+                    ((u4 *)arows)[((sg * 2 + pl) * upr + c) * 16 + tk] = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)tk * (K + 1) + sl) * a.I + 8 * c);
+                }
+            } else {
+                const uint32_t s0 = g0.sh ? K : slot[g0.u * gnb + t], s1 = !both ? 0 : g1.sh ? K : slot[g1.u * gnb + t]; // result slot of token t
+                for (uint32_t q = qw_wave(); q < ninst; q += blockDim.x >> 6) {
+                    const uint32_t sg = q / (2 * ncb), r = q % (2 * ncb), pl = r / ncb, cb = r % ncb;
+                    const uint32_t m = sg ? g1.mask : g0.mask, sl = sg ? s1 : s0, c = 4 * cb + (lane >> 4);
+                    if ((m >> t) & 1)
+                        qw_load_to_lds((const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t * (K + 1) + sl) * a.I + 8 * c), (u4 *)arows + ((sg * 2 + pl) * upr + 4 * cb) * 16);
                 }
             }
-            for (uint32_t i = threadIdx.x + NV * blockDim.x; i < nitem; i += blockDim.x) { // larger I or fewer threads
-                uint32_t dd;
-                const u4 vv = *(const u4 *)(a.H + place(i, dd));
-                ((u4 *)arows)[dd] = vv;
-            }
+            qw_lds_arrive(); // the table's loads too (issued at the start of the kernel)
             __syncthreads();
         };
         // the two segments share one pipeline when their formats agree; a shared expert of another format runs first
@@ -1119,8 +1101,8 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
 }
 #define QW_DN_RANGE(F, CH, FSD, CHSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
-        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; uint8_t rowbit[32]; } L; \
-        dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc, L.rowbit);                                \
+        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; } L; \
+        dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
     }
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
 QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
