@@ -493,12 +493,13 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
 // the ranks below K are the picks. T tokens go through together (the steps are chains of LDS and cross-lane
 // latencies, so a second token costs little). Returns a bit per token that was NOT done, with nothing written for
 // it: more than 64 keys reach T0 (many equal logits) and the caller falls back to select_tokens.
-// ws: 144 dwords of LDS scratch per token for this wave.
+// ws: 144 dwords of LDS scratch per token for this wave. need_w: also the gating weights (softmax over the picked
+// logits in rank order, sigmoid of the shared-expert logit).
 // issued(): called once the loads of the logits are issued (the place for the caller's own prefetches: loads return in
 // the order of issue, and the logits are needed first).
 template <int PER, int T, class H>
 __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, uint32_t E, uint32_t K, const uint32_t (&tok)[T], const bool (&on)[T], float *w, uint32_t *ids, uint32_t *ws,
-                                                        uint32_t lane, H issued) {
+                                                        uint32_t lane, bool need_w, H issued) {
     uint32_t k[T][PER], M[T], T0[T], c[T], pos[T][PER];
 #pragma unroll
     for (int t = 0; t < T; t++)
@@ -576,6 +577,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
             pkr[rank[t]] = mk[t];
         }
     }
+    if (!need_w) return fail; // the gating weights are only wanted by the workgroup that writes the record
 #pragma unroll
     for (int t = 0; t < T; t++) {
         if ((fail >> t) & 1) continue;
@@ -644,11 +646,11 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
             const uint32_t t1[1] = {tk[0]};
             uint32_t fail;
             switch (E) {
-            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
-            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
-            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
-            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
-            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, issued); break;
+            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
+            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
+            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
+            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
+            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
             }
             for (uint32_t i = 0; i < 2; i++) { // more than 64 keys tie at the bound: the repeated maximum instead
                 if (!((fail >> i) & 1) || (i == 1 && !two)) continue;
