@@ -1,5 +1,7 @@
 """Ragged batches through the packing path (count -> plan -> scatter -> grouped product -> combine): integer stages
 bit-exact against the oracle, outputs against a float64 recompute."""
+import os
+
 import numpy as np
 import pytest
 
@@ -80,6 +82,8 @@ def test_packing_uniform_routing(gpu, oracle, fmt, tm):
 def test_packing_tile_major_weights(gpu, oracle, tm):
     """The same through the tile-major copies (weights resident in HBM only): gate and up of a tile entry in one
     launch, results as with the GGUF rows."""
+    if os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
     T, E, K, D, I = 40, 32, 4, 512, 512
     rng = np.random.default_rng(17 + tm)
     ids = synth.zipf_ids(rng, T, E, K)

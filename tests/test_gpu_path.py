@@ -1,6 +1,8 @@
 """GPU parity of the quantized decode path against the CPU oracle, through the C interface (include/gpu.h and
 include/qw_path.h). Bars: dequantized values bit-exact; matvec and MoE outputs max|err| / max|ref| <= 2e-3 against
 the float64 oracle; router top-k indices identical."""
+import os
+
 import numpy as np
 import pytest
 
@@ -331,6 +333,8 @@ def test_moe_batched_equals_single(gpu):
 def test_qmv_packed_and_valu_forms(gpu, oracle, nb, valu):
     """Weights in a device-only buffer take the tile-major copy; with QW_VALU in the block the VALU GEMV runs instead of
     the matrix-core kernel. Both against the float64 oracle."""
+    if os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
     N, K = 1024, 2048
     rng = np.random.default_rng(40 + nb)
     W = synth.matrix(rng, 21, N, K)
@@ -360,6 +364,8 @@ def test_qmv_packed_and_valu_forms(gpu, oracle, nb, valu):
 
 def test_packed_copy_follows_the_source(gpu, oracle):
     """Rewriting a weight buffer after its first use drops the tile-major copy: the next call sees the new bytes."""
+    if os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
     N, K, nb = 256, 512, 2
     rng = np.random.default_rng(77)
     x = synth.activations(rng, nb, K)
