@@ -262,6 +262,7 @@ def main():
     ap.add_argument("--copy-calib", action="store_true", help="also run the copy kernel over 1 GiB three times (scale for the memory counters)")
     ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
     ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
+    ap.add_argument("--ragged-only", action="store_true", help="only the continuous-batching step table (config 4) on a one-layer stack: for profiling runs")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no collectives, no sharding)" % a.gpus, file=sys.stderr)
@@ -273,6 +274,11 @@ def main():
     gpu = q.Gpu()
     if a.dense_only:
         print(json.dumps({"qmv": qmv_table(gpu), "qmv_formats": formats_table(gpu)}))
+        return 0
+    if a.ragged_only:
+        stack = MoeStack(gpu, layers=1, nbmax=16)
+        print(json.dumps({"ragged_step": ragged_steps(gpu, stack)}))
+        stack.free()
         return 0
     t0 = time.perf_counter()
     stack = MoeStack(gpu, layers=a.layers, nbmax=16)
