@@ -979,10 +979,15 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, nwv = blockDim.x >> 6, nl = lane >> 2;
     const uint32_t ntask = g0.ntile + (both ? g1.ntile : 0), cpr = a.I / (C::BLK_K * CH);
-    // per lane: result slots of tokens 4 kg .. 4 kg + 3 in either segment
-    uint32_t sl0 = 0, sl1 = 0;
-    if (!g0.sh) sl0 = *(const uint32_t *)(slots0 + 4 * kg);
-    if (both && !g1.sh) sl1 = *(const uint32_t *)(slots1 + 4 * kg);
+    // per lane: where the results of tokens 4 kg .. 4 kg + 3 go in either segment, as float offsets of row 0
+    // (token * topk + slot for a routed expert, token for the shared one; 32 bits hold them), ~0 = not picked
+    uint32_t off0[4], off1[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) {
+        const uint32_t tok = 4 * kg + j;
+        off0[j] = !((g0.mask >> tok) & 1) ? ~0u : (g0.sh ? tok : tok * K + slots0[tok]) * a.D;
+        off1[j] = !both || !((g1.mask >> tok) & 1) ? ~0u : (g1.sh ? tok : tok * K + slots1[tok]) * a.D;
+    }
     f4 acc = {0, 0, 0, 0};
     qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
         [&](uint32_t i) {
@@ -999,13 +1004,12 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
             const qw_afrag_lds2 af = {ab, ab + 2 * a.I, n};
             c.mac_half(lut, af, ci * CH * C::BLK_K, kg, acc);
             if (ci + 1 != cpr) return;
-            const uint32_t r = 16 * (second ? g1.tile0 + i - g0.ntile : g0.tile0 + i) + n, sl = second ? sl1 : sl0;
-            const uint32_t gm = second ? g1.mask : g0.mask, gsh = second ? g1.sh : g0.sh;
+            const uint32_t r = 16 * (second ? g1.tile0 + i - g0.ntile : g0.tile0 + i) + n;
             float *P = second ? g1.P : g0.P;
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++) {
-                const uint32_t tok = 4 * kg + j;
-                if ((gm >> tok) & 1) P[(gsh ? (size_t)tok : (size_t)tok * K + ((sl >> (8 * j)) & 255)) * a.D + r] = acc[j];
+                const uint32_t o = second ? off1[j] : off0[j];
+                if (o != ~0u) P[o + r] = acc[j];
             }
             acc = f4{0, 0, 0, 0};
         },
