@@ -250,6 +250,77 @@ def formats_table(gpu, reps=4, nmat=32):
     return out
 
 
+def gguf_load(gpu, layers=2, reps=3):
+    """Weight residency from GGUF files (include/qw_gguf.h): `layers` full-size MoE layers (513 experts each, IQ3_S,
+    random bytes) written to a temporary directory, then loaded into HBM by the reader; the files are in the page
+    cache (just written). Best of `reps` loads with the default worker threads, and with one thread; for scale, the
+    same bytes through one plain host-to-device copy out of the file mapping."""
+    import shutil
+    import tempfile
+
+    import qwental_amd as q
+    from qwental_amd import gguf_writer as gf
+    D, I, E = 2048, 512, 512
+    rng = np.random.default_rng(99)
+    tmp = tempfile.mkdtemp(prefix="qw_gguf_")
+    try:
+        for l in range(layers):
+            p = "blk.%d." % l
+            rb = lambda ft, dims: np.frombuffer(rng.bytes(gf.tensor_bytes(ft, dims)), np.uint8)
+            router = (rng.normal(0, 0.02, (E, D)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+            gate_v = (router[0].astype(np.uint32) << 16).view(np.float32)
+            ts = [(p + "ffn_gate_exps.weight", 21, [D, I, E], None), (p + "ffn_up_exps.weight", 21, [D, I, E], None), (p + "ffn_down_exps.weight", 21, [I, D, E], None),
+                  (p + "ffn_gate_shexp.weight", 21, [D, I], None), (p + "ffn_up_shexp.weight", 21, [D, I], None), (p + "ffn_down_shexp.weight", 21, [I, D], None)]
+            ts = [(n, ft, d, rb(ft, d)) for n, ft, d, _ in ts] + [(p + "ffn_gate_inp.weight", 30, [D, E], router), (p + "ffn_gate_inp_shexp.weight", 0, [D], gate_v)]
+            gf.write_gguf(os.path.join(tmp, "layer-%05d.gguf" % l), ts)
+            del ts
+        out = {"layers": layers, "source": "page cache (files just written)"}
+        for label, threads in (("default_threads", None), ("one_thread", "1"), ("two_threads", "2"), ("eight_threads", "8")):
+            best = None
+            for _ in range(reps):
+                if threads:
+                    os.environ["QW_HIP_LOAD_THREADS"] = threads
+                g = q.Gguf(tmp)
+                try:
+                    g.load(gpu, "moe,shared,router")
+                finally:
+                    os.environ.pop("QW_HIP_LOAD_THREADS", None)
+                n, sec = g.resident_bytes(), g.load_seconds()
+                if label == "default_threads" and best is None:  # what arrived is what the file holds
+                    t = g.find("blk.%d.ffn_down_exps.weight" % (layers - 1))
+                    tail = g.read_resident(t, t.nbytes)[-(1 << 20):]
+                    assert np.array_equal(tail, g.host(t)[-(1 << 20):]), "resident bytes differ from the file"
+                    M, d, i, e = g.moe_layer(0)
+                    assert (d, i, e) == (D, I, E)
+                g.close()
+                best = sec if best is None else min(best, sec)
+            out[label] = {"bytes": int(n), "seconds": best, "GBps": n / best / 1e9}
+        # for scale: the same bytes of one tensor by one plain copy call, out of a fresh mapping of the file (what
+        # handing a mapped file to qw_buf_wrap() amounts to) and out of ordinary process memory
+        g = q.Gguf(tmp)
+        t = g.find("blk.0.ffn_gate_exps.weight")
+        path0, off0, nb0 = g.shards()[t.shard]["path"], int(t.offset), int(t.nbytes)
+        src = g.host(t)  # a private copy in pageable memory
+        dst = gpu.buf(src.nbytes, device_only=True)
+        best = bestm = None
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            dst.fill(src)
+            best = min(best or 1e9, time.perf_counter() - t0)
+            mm = np.memmap(path0, np.uint8, "r", off0, (nb0,))
+            t0 = time.perf_counter()
+            dst.fill(mm)
+            bestm = min(bestm or 1e9, time.perf_counter() - t0)
+            del mm
+        out["plain_copy_file_mapping"] = {"bytes": nb0, "seconds": bestm, "GBps": nb0 / bestm / 1e9}
+        out["plain_copy_pageable"] = {"bytes": int(src.nbytes), "seconds": best, "GBps": src.nbytes / best / 1e9}
+        dst.free()
+        g.close()
+        return out
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -262,6 +333,7 @@ def main():
     ap.add_argument("--copy-calib", action="store_true", help="also run the copy kernel over 1 GiB three times (scale for the memory counters)")
     ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
     ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
+    ap.add_argument("--gguf-only", action="store_true", help="only the GGUF load measurement")
     ap.add_argument("--ragged-only", action="store_true", help="only the continuous-batching step table (config 4) on a one-layer stack: for profiling runs")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -274,6 +346,9 @@ def main():
     gpu = q.Gpu()
     if a.dense_only:
         print(json.dumps({"qmv": qmv_table(gpu), "qmv_formats": formats_table(gpu)}))
+        return 0
+    if a.gguf_only:
+        print(json.dumps({"gguf_load": gguf_load(gpu)}))
         return 0
     if a.ragged_only:
         stack = MoeStack(gpu, layers=1, nbmax=16)
@@ -328,6 +403,7 @@ def main():
         line["ragged_step"] = ragged_steps(gpu, stack)
         line["qmv"] = qmv_table(gpu)
         line["qmv_formats"] = formats_table(gpu)
+        line["gguf_load"] = gguf_load(gpu)
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)

@@ -11,6 +11,7 @@
  */
 #pragma once
 #include "gpu.h"
+#include <stdint.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -30,6 +31,10 @@ bool qw_hip_buf_upload(qw_buf *b, size_t offset, size_t len);
 bool qw_hip_buf_download(qw_buf *b, size_t offset, size_t len);
 bool qw_hip_buf_write(qw_buf *b, size_t offset, const void *src, size_t len);
 bool qw_hip_buf_read(const qw_buf *b, size_t offset, void *dst, size_t len);
+/* len bytes of the open file fd, from file offset file_off, into HBM at [offset, offset + len) of b: worker threads
+ * pread() into pinned staging buffers and the DMA of one chunk runs while the next is read (no page of the file is
+ * mapped). QW_HIP_LOAD_THREADS sets the number of threads (default 4, at most 16). Synchronous. */
+bool qw_hip_buf_write_fd(qw_buf *b, size_t offset, int fd, uint64_t file_off, size_t len);
 /* Device address of a buffer (for tools that pass it to their own code). */
 void *qw_hip_buf_devptr(const qw_buf *b);
 

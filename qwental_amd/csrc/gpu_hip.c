@@ -13,6 +13,7 @@
 #include "qw_hip_ext.h"
 #include "kernels/qw_kargs.h"
 #include <hip/hip_runtime_api.h>
+#include <pthread.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -110,6 +111,7 @@ struct qw_batch {
     struct { bool valid; qwk_pf_args a; qw_hbuf *hw, *hx, *hy; int E; } pend_pf;
 };
 
+#define QW_LD_MAX 16
 struct qw_gpu {
     int dev;
     char name[256];
@@ -132,6 +134,8 @@ struct qw_gpu {
     unsigned mark;
     qw_pack *packs;
     int npacks, cappacks;
+    struct qw_ldlane { void *pin[2]; hipStream_t st; hipEvent_t ev[2]; } ld[QW_LD_MAX]; // staging of qw_hip_buf_write_fd, made at first use
+    int nld;
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes;
 };
@@ -206,6 +210,13 @@ void qw_gpu_close(qw_gpu *g) {
     if (!g) return;
     (void)hipDeviceSynchronize();
     for (int i = 0; i < 2; i++) (void)hipStreamDestroy(g->stream[i]);
+    for (int i = 0; i < g->nld; i++) {
+        for (int k = 0; k < 2; k++) {
+            if (g->ld[i].ev[k]) (void)hipEventDestroy(g->ld[i].ev[k]);
+            if (g->ld[i].pin[k]) (void)hipHostFree(g->ld[i].pin[k]);
+        }
+        if (g->ld[i].st) (void)hipStreamDestroy(g->ld[i].st);
+    }
     for (int i = 0; i < g->npacks; i++) {
         (void)hipFree(g->packs[i].dst);
         if (g->packs[i].ha) g->packs[i].ha->npack = 0;
@@ -565,6 +576,87 @@ bool qw_hip_buf_write(qw_buf *b, size_t off, const void *src, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
     packs_drop(h);
     return h && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
+}
+// File -> HBM through pinned staging. Chunk c of the range belongs to lane c % nth; a lane is two pinned buffers, a
+// stream (default priority) and two events, kept by the device handle from their first use: the pread() of a lane's
+// next chunk runs while the DMA of its previous one is in flight. One thread per lane for the duration of a call.
+#define QW_FD_CHUNK ((size_t)4 << 20)
+typedef struct {
+    qw_hbuf *h;
+    struct qw_ldlane *lane;
+    size_t off, len;
+    int fd, tid, nth;
+    uint64_t foff;
+    bool ok;
+} fd_job;
+static void *fd_worker(void *arg) {
+    fd_job *j = arg;
+    struct qw_ldlane *L = j->lane;
+    bool used[2] = {false, false}, ok = hipSetDevice(j->h->g->dev) == hipSuccess;
+    int slot = 0;
+    for (size_t c = (size_t)j->tid * QW_FD_CHUNK; ok && c < j->len; c += (size_t)j->nth * QW_FD_CHUNK, slot ^= 1) {
+        const size_t n = j->len - c < QW_FD_CHUNK ? j->len - c : QW_FD_CHUNK;
+        if (used[slot]) ok = hipEventSynchronize(L->ev[slot]) == hipSuccess; // the DMA that last read this staging buffer
+        for (size_t got = 0; ok && got < n;) {
+            const ssize_t r = pread(j->fd, (char *)L->pin[slot] + got, n - got, (off_t)(j->foff + c + got));
+            if (r <= 0) ok = false; // an error, or the file ends inside the range
+            else got += (size_t)r;
+        }
+        ok = ok && hipMemcpyAsync((char *)j->h->dptr + j->off + c, L->pin[slot], n, hipMemcpyHostToDevice, L->st) == hipSuccess;
+        ok = ok && hipEventRecord(L->ev[slot], L->st) == hipSuccess;
+        used[slot] = true;
+    }
+    ok = (hipStreamSynchronize(L->st) == hipSuccess) && ok; // also when a step failed: nothing of this call stays in flight
+    j->ok = ok;
+    return NULL;
+}
+// Lanes 0 .. n-1 of the device handle, made on the calling thread.
+static bool ld_lanes(qw_gpu *g, int n) {
+    for (; g->nld < n; g->nld++) {
+        struct qw_ldlane *L = &g->ld[g->nld];
+        memset(L, 0, sizeof *L);
+        bool ok = HIPOK(g, hipHostMalloc(&L->pin[0], QW_FD_CHUNK, hipHostMallocDefault)) && HIPOK(g, hipHostMalloc(&L->pin[1], QW_FD_CHUNK, hipHostMallocDefault));
+        ok = ok && HIPOK(g, hipStreamCreateWithFlags(&L->st, hipStreamNonBlocking));
+        ok = ok && HIPOK(g, hipEventCreateWithFlags(&L->ev[0], hipEventDisableTiming)) && HIPOK(g, hipEventCreateWithFlags(&L->ev[1], hipEventDisableTiming));
+        if (!ok) {
+            for (int k = 0; k < 2; k++) {
+                if (L->ev[k]) (void)hipEventDestroy(L->ev[k]);
+                if (L->pin[k]) (void)hipHostFree(L->pin[k]);
+            }
+            if (L->st) (void)hipStreamDestroy(L->st);
+            memset(L, 0, sizeof *L);
+            return false;
+        }
+    }
+    return true;
+}
+bool qw_hip_buf_write_fd(qw_buf *b, size_t off, int fd, uint64_t foff, size_t len) {
+    qw_hbuf *h = b ? b->handle : NULL;
+    if (!h || !range_ok(h, off, len) || fd < 0) return false;
+    packs_drop(h);
+    if (!len) return true;
+    int nth = 4;
+    const char *e = getenv("QW_HIP_LOAD_THREADS");
+    if (e && atoi(e) > 0) nth = atoi(e) > QW_LD_MAX ? QW_LD_MAX : atoi(e);
+    const size_t nchunk = (len + QW_FD_CHUNK - 1) / QW_FD_CHUNK;
+    if ((size_t)nth > nchunk) nth = (int)nchunk;
+    if (!ld_lanes(h->g, nth)) return false;
+    fd_job job[QW_LD_MAX];
+    pthread_t th[QW_LD_MAX];
+    bool started[QW_LD_MAX] = {false};
+    for (int i = 0; i < nth; i++) {
+        job[i] = (fd_job){h, &h->g->ld[i], off, len, fd, i, nth, foff, false};
+        if (i + 1 < nth) started[i] = pthread_create(&th[i], NULL, fd_worker, &job[i]) == 0;
+    }
+    bool ok = true;
+    for (int i = nth - 1; i >= 0; i--) { // the calling thread takes the last lane, and any whose thread did not start
+        if (started[i]) pthread_join(th[i], NULL);
+        else fd_worker(&job[i]);
+        ok = ok && job[i].ok;
+    }
+    if (!ok) set_err(h->g, "qw_hip_buf_write_fd: read or copy failed");
+    if (h->host && !h->wrapped) h->dirty = false; // HBM is now newer than the shadow; the shadow is not refreshed
+    return ok;
 }
 bool qw_hip_buf_read(const qw_buf *b, size_t off, void *dst, size_t len) {
     const qw_hbuf *h = b ? b->handle : NULL;

@@ -244,8 +244,8 @@ struct qw_afrag_gather {
 
 // ---------------------------------------------------------------- chunks: the unit of prefetch
 // A chunk is NB consecutive blocks of one weight row, held in registers by the lane that decodes them. Kernels keep
-// two chunks per wave: while one is decoded and multiplied, the loads of the next are in flight. With 8 waves per
-// compute unit and 14 KB per wave in flight (IQ3_S, 16 rows of K = 2048) this covers the HBM latency.
+// DEPTH chunks per wave (two or three): while one is decoded and multiplied, the loads of the next one or two are in
+// flight. With 10 waves per compute unit and 7 to 14 KB per wave in flight this covers the HBM latency.
 template <int F, int NB> struct qw_chunk;
 
 template <int NB> struct qw_chunk<21, NB> {

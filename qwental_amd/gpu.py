@@ -1,5 +1,6 @@
-"""ctypes binding of libqwgpu_hip.so: the GPU interface (include/gpu.h), its HIP additions (include/qw_hip_ext.h)
-and the host side of the path (include/qw_path.h). Thin by design: one Python method per C function."""
+"""ctypes binding of libqwgpu_hip.so: the GPU interface (include/gpu.h), its HIP additions (include/qw_hip_ext.h),
+the host side of the path (include/qw_path.h) and the GGUF reader (include/qw_gguf.h). Thin by design: one Python
+method per C function."""
 import ctypes as C
 import os
 
@@ -26,9 +27,16 @@ class QwMoeLayer(C.Structure):
     _fields_ = [(n, QwTensor) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")]
 
 
-# every symbol include/gpu.h, include/qw_hip_ext.h and include/qw_path.h declare: (name, restype, argtypes)
+class QwGgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("model", C.c_char_p), ("part", C.c_uint), ("kind", C.c_int), ("type", C.c_uint32), ("nd", C.c_uint32),
+                ("dims", C.c_uint64 * 4), ("rows", C.c_uint64), ("rowbytes", C.c_uint64), ("nbytes", C.c_uint64), ("shard", C.c_int),
+                ("offset", C.c_uint64), ("res_type", C.c_int)]
+
+
+# every symbol include/gpu.h, include/qw_hip_ext.h, include/qw_path.h and include/qw_gguf.h declare: (name, restype, argtypes)
 _vp, _sz, _u, _i, _b, _d = C.c_void_p, C.c_size_t, C.c_uint, C.c_int, C.c_bool, C.c_double
-_pb, _pt, _pm = C.POINTER(QwBuf), C.POINTER(QwTensor), C.POINTER(QwMoeLayer)
+_pb, _pt, _pm, _pg = C.POINTER(QwBuf), C.POINTER(QwTensor), C.POINTER(QwMoeLayer), C.POINTER(QwGgufTensor)
+_pi = C.POINTER(C.c_int)
 SYMBOLS = [
     ("qw_gpu_open", _vp, []), ("qw_gpu_close", None, [_vp]), ("qw_gpu_name", C.c_char_p, [_vp]), ("qw_gpu_max_working_set", _sz, [_vp]),
     ("qw_gpu_compile", _b, [_vp, C.c_char_p, _sz, C.c_char_p, _sz]), ("qw_kernel_get", _vp, [_vp, C.c_char_p]),
@@ -47,6 +55,7 @@ SYMBOLS = [
     ("qw_hip_buf_new_device", _b, [_vp, _sz, _pb]), ("qw_hip_buf_mark_dirty", None, [_pb]),
     ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
+    ("qw_hip_buf_write_fd", _b, [_pb, _sz, _i, C.c_uint64, _sz]),
     ("qw_hip_set_repack", None, [_vp, _b]),
     ("qw_hip_packed_bytes", _sz, [_vp]),
     ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
@@ -65,6 +74,14 @@ SYMBOLS = [
     ("qw_path_scratch", _pb, [_vp, _i]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_pf_scratch", _pb, [_vp, _i]), ("qw_path_pf_max_tiles", C.c_uint, [_vp]),
+    # qw_gguf.h
+    ("qw_gguf_parse_parts", _u, [C.c_char_p]), ("qw_ggml_block", _b, [_i, _pi, _pi]), ("qw_ggml_name", C.c_char_p, [_i]),
+    ("qw_gguf_open", _vp, [C.c_char_p, C.c_char_p, _sz]), ("qw_gguf_close", None, [_vp]), ("qw_gguf_shards", _i, [_vp]),
+    ("qw_gguf_shard_path", C.c_char_p, [_vp, _i]), ("qw_gguf_shard_alignment", C.c_uint32, [_vp, _i]),
+    ("qw_gguf_shard_data_start", C.c_uint64, [_vp, _i]), ("qw_gguf_count", _i, [_vp]), ("qw_gguf_get", _pg, [_vp, _i]),
+    ("qw_gguf_find", _pg, [_vp, C.c_char_p]), ("qw_gguf_host", _vp, [_vp, _pg]),
+    ("qw_gguf_load", _b, [_vp, _vp, _u, C.c_char_p, _sz]), ("qw_gguf_resident_bytes", _sz, [_vp]), ("qw_gguf_load_seconds", _d, [_vp]),
+    ("qw_gguf_tensor_at", _b, [_vp, _pg, _pt]), ("qw_gguf_moe_layer", _b, [_vp, _i, _pm, _pi, _pi, _pi, C.c_char_p, _sz]),
 ]
 
 
@@ -332,3 +349,77 @@ class Path:
         if not self.L.qw_hip_buf_read(pb, 0, out.ctypes.data, out.nbytes):
             raise RuntimeError("qw_hip_buf_read failed")
         return out
+
+
+class Gguf:
+    """include/qw_gguf.h: the *.gguf files of a directory, parsed and mapped; load() makes the chosen parts resident."""
+
+    def __init__(self, directory):
+        self.L = load_lib()
+        err = C.create_string_buffer(1024)
+        self.f = self.L.qw_gguf_open(os.fsencode(directory), err, len(err))
+        if not self.f:
+            raise ValueError(err.value.decode())
+
+    def close(self):
+        if self.f:
+            self.L.qw_gguf_close(self.f)
+            self.f = None
+
+    def shards(self):
+        n = self.L.qw_gguf_shards(self.f)
+        return [dict(path=os.fsdecode(self.L.qw_gguf_shard_path(self.f, i)), alignment=self.L.qw_gguf_shard_alignment(self.f, i),
+                     data_start=self.L.qw_gguf_shard_data_start(self.f, i)) for i in range(n)]
+
+    def __len__(self):
+        return self.L.qw_gguf_count(self.f)
+
+    def get(self, i):
+        p = self.L.qw_gguf_get(self.f, i)
+        return p.contents if p else None
+
+    def find(self, name):
+        p = self.L.qw_gguf_find(self.f, name.encode())
+        return p.contents if p else None
+
+    def host(self, t):
+        """The tensor's bytes in the mapping of its file (a copy)."""
+        a = self.L.qw_gguf_host(self.f, C.byref(t))
+        if not a:
+            return None
+        return np.frombuffer((C.c_uint8 * t.nbytes).from_address(a), np.uint8).copy()
+
+    def load(self, gpu, parts="all"):
+        err = C.create_string_buffer(1024)
+        bits = parts if isinstance(parts, int) else self.L.qw_gguf_parse_parts(parts.encode())
+        if not self.L.qw_gguf_load(self.f, gpu.g, bits, err, len(err)):
+            raise RuntimeError(err.value.decode())
+
+    def resident_bytes(self):
+        return self.L.qw_gguf_resident_bytes(self.f)
+
+    def load_seconds(self):
+        return self.L.qw_gguf_load_seconds(self.f)
+
+    def tensor_at(self, t):
+        """QwTensor (buffer, offset, type) of a resident tensor, or None."""
+        out = QwTensor()
+        return out if self.L.qw_gguf_tensor_at(self.f, C.byref(t), C.byref(out)) else None
+
+    def read_resident(self, t, nbytes):
+        """nbytes of the tensor's resident copy, read back from HBM."""
+        at = self.tensor_at(t)
+        if at is None:
+            return None
+        out = np.empty(nbytes, np.uint8)
+        if not self.L.qw_hip_buf_read(at.buf, at.offset, out.ctypes.data, nbytes):
+            raise RuntimeError("qw_hip_buf_read failed")
+        return out
+
+    def moe_layer(self, layer):
+        """(QwMoeLayer, D, I, E) of blk.<layer>; the struct points into this object's arena."""
+        M, D, I, E = QwMoeLayer(), C.c_int(), C.c_int(), C.c_int()
+        err = C.create_string_buffer(1024)
+        if not self.L.qw_gguf_moe_layer(self.f, layer, C.byref(M), C.byref(D), C.byref(I), C.byref(E), err, len(err)):
+            raise ValueError(err.value.decode())
+        return M, D.value, I.value, E.value

@@ -1,0 +1,205 @@
+"""GGUF files through the reader and the residency of include/qw_gguf.h on the GPU: the bytes in HBM are the bytes of
+the file (bit-exact), small float tensors are converted as the reference converts them (src/gguf.c:444-503), a layer
+taken from the files computes what the same bytes compute when handed over directly (bit-identical) and what the
+float64 oracle computes (max|err| / max|ref| <= 2e-3, top-k indices identical), and a resident tensor dequantizes
+bit-exactly (the flow of the reference's tools/dqtest.c on a tensor of a file)."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import qwental_amd as q
+from oracle import gguf_file as gf
+from qwental_amd import gguf_writer as gw
+from qwental_amd import synth
+from helpers import DeviceLayer, dq_define_block, maxrel, run_moe
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+D, I, E, K = 2048, 512, 64, 10
+LAYER = 5
+
+
+def bf16_exact(a):
+    """float32 values with the low 16 bits cleared (exact in BF16), and their BF16 bit patterns."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32) & np.uint32(0xffff0000)
+    return u.view(np.float32), (u >> 16).astype(np.uint16)
+
+
+def write_model(tmp, rng, router_type=30):
+    """A two-shard model: layer LAYER's MoE tensors (router BF16, gate vector F32), an lm_head (Q6_K), an embedding that
+    stays in the file, and small tensors of every conversion kind."""
+    m = synth.moe_layer(rng, D, I, E)
+    m["topk"] = K
+    wr32, wr_bits = bf16_exact(rng.normal(0.0, 0.02, (E, D)))
+    wg32, wg_bits = bf16_exact(rng.normal(0.0, 0.02, D))
+    m["Wr"], m["wsg"] = wr_bits, wg_bits
+    p = "blk.%d." % LAYER
+    router_bytes = wr_bits if router_type == 30 else wr32.astype(np.float16)
+    lm = synth.matrix(rng, 14, 1000, D)
+    emb = synth.matrix(rng, 8, 64, D)
+    dt_bias = rng.normal(0, 1, 48).astype(np.float32)                 # not exact in BF16: stays F32
+    ssm_norm = rng.normal(0, 1, 128).astype(np.float16)               # F16 in the file, not exact in BF16: F32
+    conv, _ = bf16_exact(rng.normal(0, 1, (4, 96)))                   # exact: BF16
+    q_norm, _ = bf16_exact(rng.normal(0, 1, 128))                     # a norm weight is kept F32 even when exact
+    shard1 = [(p + "ffn_gate_exps.weight", 21, [D, I, E], m["Wg"]), (p + "ffn_up_exps.weight", 21, [D, I, E], m["Wu"]),
+              (p + "ffn_gate_inp.weight", router_type, [D, E], router_bytes), (p + "ffn_gate_inp_shexp.weight", 0, [D], wg32),
+              (p + "ssm_dt.bias", 0, [48], dt_bias), (p + "ssm_norm.weight", 1, [128], ssm_norm), ("token_embd.weight", 8, [D, 64], emb)]
+    shard2 = [(p + "ffn_down_exps.weight", 21, [I, D, E], m["Wd"]), (p + "ffn_gate_shexp.weight", 21, [D, I], m["Wsg"]),
+              (p + "ffn_up_shexp.weight", 21, [D, I], m["Wsu"]), (p + "ffn_down_shexp.weight", 21, [I, D], m["Wsd"]),
+              ("output.weight", 14, [D, 1000], lm), (p + "ssm_conv1d.weight", 0, [96, 4], conv), (p + "attn_q_norm.weight", 0, [128], q_norm)]
+    gw.write_gguf(os.path.join(tmp, "model-00001-of-00002.gguf"), shard1, [("general.architecture", 8, "synthetic")])
+    gw.write_gguf(os.path.join(tmp, "model-00002-of-00002.gguf"), shard2, [("general.architecture", 8, "synthetic")], alignment=128)
+    small = dict(dt_bias=dt_bias, ssm_norm=ssm_norm, conv=conv, q_norm=q_norm, wg32=wg32)
+    return m, lm, small
+
+
+class _Layer:  # what run_moe expects: .layer.c is the QwMoeLayer
+    def __init__(self, c):
+        self.layer = self
+        self.c = c
+
+
+class _Ref:  # what Batch.buf expects of a buffer, for a qw_buf that the reader owns
+    def __init__(self, pbuf):
+        self.p = pbuf
+
+    def ref(self):
+        return self.p
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    tmp = str(tmp_path_factory.mktemp("gguf"))
+    rng = np.random.default_rng(77)
+    m, lm, small = write_model(tmp, rng)
+    return tmp, m, lm, small
+
+
+@pytest.mark.parametrize("threads", ["1", "3", None])
+def test_resident_bytes_are_the_files_bytes(gpu, model, threads):
+    tmp, m, lm, small = model
+    old = os.environ.get("QW_HIP_LOAD_THREADS")
+    if threads is None:
+        os.environ.pop("QW_HIP_LOAD_THREADS", None)
+    else:
+        os.environ["QW_HIP_LOAD_THREADS"] = threads  # one thread: a 28 MB tensor passes four times through two staging buffers
+    try:
+        g = q.Gguf(tmp)
+        g.load(gpu, "moe,shared,router,lm,lin,attn")
+    finally:
+        if old is None:
+            os.environ.pop("QW_HIP_LOAD_THREADS", None)
+        else:
+            os.environ["QW_HIP_LOAD_THREADS"] = old
+    total = 0
+    for i in range(len(g)):
+        t = g.get(i)
+        name = t.name.decode()
+        if name == "token_embd.weight":  # its part was not asked for
+            assert t.res_type == -1 and g.tensor_at(t) is None
+            continue
+        at = g.tensor_at(t)
+        assert at is not None and at.offset % 256 == 0
+        if t.kind in (0, 1):  # matrices: the bytes of the file
+            assert t.res_type == t.type == at.type
+            assert np.array_equal(g.read_resident(t, t.nbytes), g.host(t)), name
+            total += t.nbytes
+    def resident(suffix, dtype, n):
+        t = g.find("blk.%d.%s" % (LAYER, suffix))
+        width = 2 if dtype == np.uint16 else 4
+        return t, g.read_resident(t, n * width).view(dtype)
+    t, v = resident("ffn_gate_inp_shexp.weight", np.uint16, D)      # F32 in the file, exact: BF16
+    assert t.res_type == 30 and np.array_equal(v, m["wsg"])
+    t, v = resident("ssm_conv1d.weight", np.uint16, 4 * 96)
+    assert t.res_type == 30 and np.array_equal(v, (small["conv"].view(np.uint32) >> 16).astype(np.uint16).ravel())
+    t, v = resident("ssm_dt.bias", np.float32, 48)                  # not exact: F32, unchanged
+    assert t.res_type == 0 and np.array_equal(v, small["dt_bias"])
+    t, v = resident("ssm_norm.weight", np.float32, 128)             # F16 widened
+    assert t.res_type == 0 and np.array_equal(v, small["ssm_norm"].astype(np.float32))
+    t, v = resident("attn_q_norm.weight", np.float32, 128)          # kept F32 although exact
+    assert t.res_type == 0 and np.array_equal(v, small["q_norm"])
+    assert g.resident_bytes() == total + 2 * D + 2 * 4 * 96 + 4 * 48 + 4 * 128 + 4 * 128
+    assert g.load_seconds() > 0
+    with pytest.raises(RuntimeError):
+        g.load(gpu, "moe")  # once per object
+    g.close()
+
+
+def test_layer_from_files_parity(gpu, oracle, model):
+    tmp, m, _, _ = model
+    g = q.Gguf(tmp)
+    g.load(gpu, "moe,shared,router")
+    M, d, i, e = g.moe_layer(LAYER)
+    assert (d, i, e) == (D, I, E)
+    assert (M.router.type, M.sh_gate_w.type, M.gate.type, M.up.type, M.down.type) == (30, 30, 21, 21, 21)
+    with pytest.raises(ValueError):
+        g.moe_layer(LAYER + 1)
+    path = q.Path(gpu, D, I, E, K, 16)
+    rng = np.random.default_rng(78)
+    dl = DeviceLayer(gpu, m, router_type=30, device_only=True)  # the same bytes, handed over directly
+    for nb in (16, 3):
+        x = synth.activations(rng, nb, D)
+        out, lg, selraw, _ = run_moe(gpu, path, _Layer(M), x, nb)
+        ref_lg = oracle.router(m["Wr"], m["wsg"], x, wfmt=30)
+        assert maxrel(lg, ref_lg) <= 1e-5
+        assert np.array_equal(oracle.topk_ids(lg, K), oracle.topk_ids(ref_lg, K))
+        assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+        out2, lg2, sel2, _ = run_moe(gpu, path, dl, x, nb)
+        assert np.array_equal(out.view(np.uint16), out2.view(np.uint16)) and np.array_equal(lg.view(np.uint32), lg2.view(np.uint32))
+        assert np.array_equal(selraw, sel2)
+    dl.free()
+    path.close()
+    g.close()
+
+
+def test_resident_tensor_dequantizes_bit_exactly(gpu, oracle, model):
+    """tools/dqtest.c:26-48 on a tensor of the file: here the Q6_K lm_head and an IQ3_S shared-expert matrix."""
+    tmp, m, lm, _ = model
+    g = q.Gguf(tmp)
+    g.load(gpu, "lm,shared")
+    for name, rows in (("output.weight", 40), ("blk.%d.ffn_gate_shexp.weight" % LAYER, 24)):
+        t = g.find(name)
+        at = g.tensor_at(t)
+        ok, err = gpu.compile(dq_define_block(t.type))
+        assert ok, err
+        k = gpu.kernel("dq_test")
+        kd, rb = int(t.dims[0]), int(t.rowbytes)
+        y = gpu.buf(rows * kd * 4)
+        b = gpu.batch()
+        b.kernel(k)
+        b.buf(0, _Ref(at.buf), at.offset + 7 * rb)  # rows 7 .. 7 + rows of the tensor
+        b.buf(1, y)
+        b.bytes(2, np.array([kd, rb], np.uint32))
+        b.dispatch(rows, 1, 1, 32, 1, 1)
+        b.end()
+        got = y.view(np.float32).reshape(rows, kd).copy()
+        raw = g.host(t).reshape(-1, rb)[7:7 + rows]
+        want = oracle.dq_rows(t.type, raw, kd)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), name
+        y.free()
+    g.close()
+
+
+def test_float_matrix_other_than_bf16_is_refused(gpu, tmp_path):
+    """src/gguf.c:417-419: an F16 or F32 matrix is an error of the load, not of the parse."""
+    rng = np.random.default_rng(79)
+    w = rng.normal(0, 1, (8, 64)).astype(np.float16)
+    gw.write_gguf(str(tmp_path / "m.gguf"), [("blk.0.ffn_gate_inp.weight", 1, [64, 8], w), ("blk.0.ffn_gate_shexp.weight", 21, [256, 4], synth.matrix(rng, 21, 4, 256))])
+    g = q.Gguf(str(tmp_path))
+    with pytest.raises(RuntimeError) as e:
+        g.load(gpu, "router")
+    assert "F16" in str(e.value)
+    g.close()
+    g = q.Gguf(str(tmp_path))
+    with pytest.raises(RuntimeError):
+        g.load(gpu, "embed")  # nothing of that part
+    g.close()
+    # a quantized tensor where a float one belongs (src/gguf.c:444)
+    gw.write_gguf(str(tmp_path / "m.gguf"), [("blk.0.ffn_gate_inp_shexp.weight", 8, [64], synth.matrix(rng, 8, 1, 64))])
+    g = q.Gguf(str(tmp_path))
+    with pytest.raises(RuntimeError) as e:
+        g.load(gpu, "router")
+    assert "floating point" in str(e.value)
+    g.close()
