@@ -49,6 +49,11 @@ def write_model(tmp, rng, router_type=30):
     shard2 = [(p + "ffn_down_exps.weight", 21, [I, D, E], m["Wd"]), (p + "ffn_gate_shexp.weight", 21, [D, I], m["Wsg"]),
               (p + "ffn_up_shexp.weight", 21, [D, I], m["Wsu"]), (p + "ffn_down_shexp.weight", 21, [I, D], m["Wsd"]),
               ("output.weight", 14, [D, 1000], lm), (p + "ssm_conv1d.weight", 0, [96, 4], conv), (p + "attn_q_norm.weight", 0, [128], q_norm)]
+    # one matrix of every other format the kernels decode, under names of the attention / linear-attention parts
+    for suffix, ft, rows in (("attn_q.weight", 12, 24), ("attn_k.weight", 13, 16), ("attn_v.weight", 14, 16), ("attn_output.weight", 20, 24),
+                             ("attn_qkv.weight", 23, 16), ("attn_gate.weight", 8, 40), ("ssm_alpha.weight", 30, 16)):
+        w = synth.matrix(rng, ft, rows, D)
+        (shard1 if ft in (12, 14, 23) else shard2).append((p + suffix, ft, [D, rows], w))
     gw.write_gguf(os.path.join(tmp, "model-00001-of-00002.gguf"), shard1, [("general.architecture", 8, "synthetic")])
     gw.write_gguf(os.path.join(tmp, "model-00002-of-00002.gguf"), shard2, [("general.architecture", 8, "synthetic")], alignment=128)
     small = dict(dt_bias=dt_bias, ssm_norm=ssm_norm, conv=conv, q_norm=q_norm, wg32=wg32)
@@ -155,30 +160,79 @@ def test_layer_from_files_parity(gpu, oracle, model):
 
 
 def test_resident_tensor_dequantizes_bit_exactly(gpu, oracle, model):
-    """tools/dqtest.c:26-48 on a tensor of the file: here the Q6_K lm_head and an IQ3_S shared-expert matrix."""
+    """The reference's tools/dqtest.py + tools/dqtest.c:26-48 on the files: for every format the first tensor of that
+    format, a few rows of it through the dq_test kernel, here out of the resident copy and against the oracle."""
     tmp, m, lm, _ = model
     g = q.Gguf(tmp)
-    g.load(gpu, "lm,shared")
-    for name, rows in (("output.weight", 40), ("blk.%d.ffn_gate_shexp.weight" % LAYER, 24)):
-        t = g.find(name)
+    g.load(gpu, "attn,lin,lm,shared")
+    pick = {}
+    for i in range(len(g)):
+        t = g.get(i)
+        if t.kind == 0 and t.res_type >= 0 and t.type not in pick:
+            pick[t.type] = t
+    assert sorted(pick) == [8, 12, 13, 14, 20, 21, 23, 30]
+    for ft, t in sorted(pick.items()):
         at = g.tensor_at(t)
         ok, err = gpu.compile(dq_define_block(t.type))
         assert ok, err
         k = gpu.kernel("dq_test")
-        kd, rb = int(t.dims[0]), int(t.rowbytes)
+        kd, rb, rows, first = int(t.dims[0]), int(t.rowbytes), 8, 7
         y = gpu.buf(rows * kd * 4)
         b = gpu.batch()
         b.kernel(k)
-        b.buf(0, _Ref(at.buf), at.offset + 7 * rb)  # rows 7 .. 7 + rows of the tensor
+        b.buf(0, _Ref(at.buf), at.offset + first * rb)  # rows 7 .. 14 of the tensor
         b.buf(1, y)
         b.bytes(2, np.array([kd, rb], np.uint32))
         b.dispatch(rows, 1, 1, 32, 1, 1)
         b.end()
         got = y.view(np.float32).reshape(rows, kd).copy()
-        raw = g.host(t).reshape(-1, rb)[7:7 + rows]
+        raw = g.host(t).reshape(-1, rb)[first:first + rows]
         want = oracle.dq_rows(t.type, raw, kd)
-        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), name
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), t.name
         y.free()
+    g.close()
+
+
+class _T:  # a resident tensor in the form Path.qmv_gg / qmv_ggm take (Tensor.c())
+    def __init__(self, at):
+        self.at = at
+
+    def c(self):
+        return self.at
+
+
+def test_matvec_on_resident_tensors(gpu, oracle, model):
+    """The projections of a layer in one multi-matrix launch and the lm_head by the dense matvec, weights straight
+    from the arena of the reader."""
+    tmp = model[0]
+    g = q.Gguf(tmp)
+    g.load(gpu, "attn,lin,lm")
+    path = q.Path(gpu, D, I, E, K, 16)
+    rng = np.random.default_rng(80)
+    nb = 5
+    x = synth.activations(rng, nb, D)
+    xb = gpu.buf_from(x)
+    names = ["blk.%d.%s" % (LAYER, n) for n in ("attn_q.weight", "attn_k.weight", "attn_v.weight", "ssm_alpha.weight")]
+    ts = [g.find(n) for n in names]
+    Ns = [int(t.rows) for t in ts]
+    ybs = [gpu.buf(nb * n * 4) for n in Ns]
+    b = gpu.batch()
+    path.qmv_ggm(b, [_T(g.tensor_at(t)) for t in ts], Ns, D, xb, ybs, nb)
+    b.end()
+    for t, n, yb in zip(ts, Ns, ybs):
+        ref = oracle.qmv(t.type, g.host(t), n, D, x, f64=True)
+        assert maxrel(yb.view(np.float32).reshape(nb, n), ref) <= TOL, t.name
+        yb.free()
+    t = g.find("language_model.lm_head.weight")  # by its model-side name
+    n = int(t.rows)
+    yb = gpu.buf(nb * n * 4)
+    b = gpu.batch()
+    path.qmv_gg(b, _T(g.tensor_at(t)), n, D, xb, yb, nb)
+    b.end()
+    assert maxrel(yb.view(np.float32).reshape(nb, n), oracle.qmv(14, g.host(t), n, D, x, f64=True)) <= TOL
+    yb.free()
+    xb.free()
+    path.close()
     g.close()
 
 
