@@ -133,6 +133,28 @@ def ragged_steps(gpu, stack, reps=5):
                     "decode_groups_GBps": (U_groups * stack.exp_bytes) / t_dec / 1e9, "packing_path_GBps": (U * stack.exp_bytes) / t_pk / 1e9})
         for bb in [xb, ib, wb, ob] + [y for t4 in bufs for y in t4]:
             bb.free()
+    # the step planner (include/qw_par.h) on these measurements: one group of b rows timed for a few sizes, the packing
+    # path from the table above; what it would run for each row count, with its two estimates
+    import qwental_amd as q
+    par = q.Par()
+    rng = np.random.default_rng(999)
+    for b_ in (1, 2, 4, 8, 12, 16):
+        ids = synth.zipf_ids(rng, b_, E, K)
+        bufs = (gpu.buf_from(synth.activations(rng, b_, D)), gpu.buf_from(synth.logits_for_ids(rng, ids, E)), gpu.buf(path.sel_bytes(b_)), gpu.buf(b_ * D * 2))
+        for _ in range(reps + 1):  # the planner drops the first sample of a size
+            b = gpu.batch()
+            path.gg_moe_lg(b, layer, b_, *bufs)
+            par.observe(b_, b.end() * 1e6)
+        for bb in bufs:
+            bb.free()
+    for row in out:
+        for _ in range(2):
+            par.observe_packed(row["rows"], row["packing_path_us"])
+    for row in out:
+        packed, groups = par.choose(row["rows"])
+        row["planner"] = {"form": "packing path" if packed else "groups", "groups": groups, "estimate_groups_us": par.cost(min(row["rows"], 64)) if row["rows"] <= 64 else None,
+                          "estimate_packing_us": par.packed_cost(row["rows"])}
+    par.free()
     return out
 
 

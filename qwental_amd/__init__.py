@@ -6,4 +6,4 @@ of the benchmark configurations. Nothing here computes on the CPU in place of th
 without a gfx950 device every entry point raises.
 """
 from . import synth  # noqa: F401
-from .gpu import Gpu, Buf, Path, Tensor, MoeLayer, Gguf, lib_path, load_lib  # noqa: F401
+from .gpu import Gpu, Buf, Path, Tensor, MoeLayer, Gguf, Par, lib_path, load_lib  # noqa: F401

@@ -4,7 +4,7 @@
 
 Two steps, both cross-compile without a GPU:
   1. hipcc --genco: csrc/kernels/qw_kernels.hip -> csrc/qw_kernels_gfx950.hsaco
-  2. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c + csrc/qw_gguf.c -> qwental_amd/libqwgpu_hip.so
+  2. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c + csrc/qw_gguf.c + csrc/qw_par.c -> qwental_amd/libqwgpu_hip.so
 """
 import os
 import subprocess
@@ -37,7 +37,7 @@ def build(verbose=False):
     if verbose and out.strip():
         print(out)
     out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-                "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), "-pthread", "-o", LIB,
+                "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), os.path.join(CSRC, "qw_par.c"), "-pthread", "-o", LIB,
                 "-L", os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
     if verbose and out.strip():
         print(out)

@@ -1,0 +1,100 @@
+// The cut of a step into launches from measured times (include/qw_par.h). Plain host arithmetic, no GPU call.
+#include "qw_par.h"
+#include <stdlib.h>
+
+#define NBUCKET (QW_PAR_PACK_MAX / 16)
+
+struct qw_par {
+    double cost[QW_PAR_VBMAX + 1];
+    int seen[QW_PAR_VBMAX + 1];
+    double pcost[NBUCKET + 1]; // bucket k: rows 16 (k - 1) + 1 .. 16 k
+    int pseen[NBUCKET + 1];
+};
+
+qw_par *qw_par_new(void) { return calloc(1, sizeof(qw_par)); }
+void qw_par_free(qw_par *p) { free(p); }
+
+// src/engine.c:9037: the first sample of a size is dropped, the second starts the average, later ones move it by a tenth
+static void observe(double *cost, int *seen, double ms) {
+    if ((*seen)++) *cost = *cost > 0 ? 0.9 * *cost + 0.1 * ms : ms;
+}
+void qw_par_observe(qw_par *p, int b, double ms) {
+    if (b >= 1 && b <= QW_PAR_VBMAX && ms > 0) observe(&p->cost[b], &p->seen[b], ms);
+}
+double qw_par_group_cost(const qw_par *p, int b) { return b >= 1 && b <= QW_PAR_VBMAX ? p->cost[b] : 0; }
+
+// Sizes never measured, filled in on the line through the smallest and the largest measured size (one size: flat).
+static bool fill_line(const double *c, int n, double *out) {
+    int lo = 0, hi = 0;
+    for (int b = 1; b <= n; b++)
+        if (c[b] > 0) {
+            if (!lo) lo = b;
+            hi = b;
+        }
+    if (!lo) return false;
+    double a = c[lo], k = 0;
+    if (hi > lo) {
+        k = (c[hi] - c[lo]) / (hi - lo);
+        a = c[lo] - k * lo;
+    }
+    for (int b = 1; b <= n; b++) out[b] = c[b] > 0 ? c[b] : a + k * b;
+    return true;
+}
+
+double qw_par_cost(const qw_par *p, int B) { // src/engine.c:8764-8781
+    if (B < 1) return 0;
+    double c[QW_PAR_VBMAX + 1], best[QW_PAR_MAX + 1];
+    if (!fill_line(p->cost, QW_PAR_VBMAX, c)) return 0;
+    if (B > QW_PAR_MAX) B = QW_PAR_MAX;
+    best[0] = 0;
+    for (int n = 1; n <= B; n++) {
+        best[n] = 1e30;
+        for (int b = 1; b <= QW_PAR_VBMAX && b <= n; b++)
+            if (best[n - b] + c[b] < best[n]) best[n] = best[n - b] + c[b];
+    }
+    return best[B];
+}
+
+int qw_par_split(const qw_par *p, int B, int *g) { // src/engine.c:8783-8797
+    if (B < 1 || B > QW_PAR_MAX) return 0;
+    double best[QW_PAR_MAX + 1];
+    int arg[QW_PAR_MAX + 1], ng = 0;
+    best[0] = 0;
+    for (int n = 1; n <= B; n++) {
+        best[n] = 1e30;
+        arg[n] = 1;
+        for (int b = 1; b <= QW_PAR_VBMAX && b <= n; b++) // "<=": at equal cost the larger group wins; a size never measured costs 0
+            if (best[n - b] + p->cost[b] <= best[n]) {
+                best[n] = best[n - b] + p->cost[b];
+                arg[n] = b;
+            }
+    }
+    for (int n = B; n > 0; n -= arg[n]) g[ng++] = arg[n];
+    return ng;
+}
+
+static int bucket(int rows) { return (rows + 15) / 16; }
+void qw_par_observe_packed(qw_par *p, int rows, double ms) {
+    if (rows >= 1 && rows <= QW_PAR_PACK_MAX && ms > 0) observe(&p->pcost[bucket(rows)], &p->pseen[bucket(rows)], ms);
+}
+double qw_par_packed_cost(const qw_par *p, int rows) {
+    if (rows < 1) return 0;
+    double c[NBUCKET + 1];
+    if (!fill_line(p->pcost, NBUCKET, c)) return 0;
+    const int k = bucket(rows > QW_PAR_PACK_MAX ? QW_PAR_PACK_MAX : rows);
+    return c[k];
+}
+
+bool qw_par_choose(const qw_par *p, int rows, int *groups, int *ngroups) {
+    *ngroups = rows <= QW_PAR_MAX ? qw_par_split(p, rows, groups) : 0;
+    if (rows < 1) return false;
+    // the grouped form beyond QW_PAR_MAX rows: full steps of QW_PAR_MAX rows plus the rest
+    double grouped = 0;
+    for (int left = rows; left > 0; left -= QW_PAR_MAX) {
+        const double c = qw_par_cost(p, left > QW_PAR_MAX ? QW_PAR_MAX : left);
+        if (c <= 0) return false;
+        grouped += c;
+    }
+    const double packed = qw_par_packed_cost(p, rows);
+    return packed > 0 && packed < grouped;
+}

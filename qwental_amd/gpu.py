@@ -1,5 +1,6 @@
 """ctypes binding of libqwgpu_hip.so: the GPU interface (include/gpu.h), its HIP additions (include/qw_hip_ext.h),
-the host side of the path (include/qw_path.h) and the GGUF reader (include/qw_gguf.h). Thin by design: one Python
+the host side of the path (include/qw_path.h), the GGUF reader (include/qw_gguf.h) and the step planner
+(include/qw_par.h). Thin by design: one Python
 method per C function."""
 import ctypes as C
 import os
@@ -82,6 +83,10 @@ SYMBOLS = [
     ("qw_gguf_find", _pg, [_vp, C.c_char_p]), ("qw_gguf_host", _vp, [_vp, _pg]),
     ("qw_gguf_load", _b, [_vp, _vp, _u, C.c_char_p, _sz]), ("qw_gguf_resident_bytes", _sz, [_vp]), ("qw_gguf_load_seconds", _d, [_vp]),
     ("qw_gguf_tensor_at", _b, [_vp, _pg, _pt]), ("qw_gguf_moe_layer", _b, [_vp, _i, _pm, _pi, _pi, _pi, C.c_char_p, _sz]),
+    # qw_par.h
+    ("qw_par_new", _vp, []), ("qw_par_free", None, [_vp]), ("qw_par_observe", None, [_vp, _i, _d]), ("qw_par_group_cost", _d, [_vp, _i]),
+    ("qw_par_cost", _d, [_vp, _i]), ("qw_par_split", _i, [_vp, _i, _pi]), ("qw_par_observe_packed", None, [_vp, _i, _d]),
+    ("qw_par_packed_cost", _d, [_vp, _i]), ("qw_par_choose", _b, [_vp, _i, _pi, _pi]),
 ]
 
 
@@ -423,3 +428,41 @@ class Gguf:
         if not self.L.qw_gguf_moe_layer(self.f, layer, C.byref(M), C.byref(D), C.byref(I), C.byref(E), err, len(err)):
             raise ValueError(err.value.decode())
         return M, D.value, I.value, E.value
+
+
+class Par:
+    """include/qw_par.h: the cut of a step into groups (or the packing path) from measured times."""
+
+    def __init__(self):
+        self.L = load_lib()
+        self.p = self.L.qw_par_new()
+
+    def free(self):
+        if self.p:
+            self.L.qw_par_free(self.p)
+            self.p = None
+
+    def observe(self, b, ms):
+        self.L.qw_par_observe(self.p, b, ms)
+
+    def group_cost(self, b):
+        return self.L.qw_par_group_cost(self.p, b)
+
+    def cost(self, B):
+        return self.L.qw_par_cost(self.p, B)
+
+    def split(self, B):
+        g = (C.c_int * 64)()
+        return list(g[:self.L.qw_par_split(self.p, B, g)])
+
+    def observe_packed(self, rows, ms):
+        self.L.qw_par_observe_packed(self.p, rows, ms)
+
+    def packed_cost(self, rows):
+        return self.L.qw_par_packed_cost(self.p, rows)
+
+    def choose(self, rows):
+        """(use the packing path, group sizes otherwise)."""
+        g, n = (C.c_int * 64)(), C.c_int()
+        packed = self.L.qw_par_choose(self.p, rows, g, C.byref(n))
+        return bool(packed), list(g[:n.value])

@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_functions():
     names = set()
-    for h in ("gpu.h", "qw_hip_ext.h", "qw_path.h", "qw_gguf.h"):
+    for h in ("gpu.h", "qw_hip_ext.h", "qw_path.h", "qw_gguf.h", "qw_par.h"):
         text = open(os.path.join(ROOT, "include", h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names |= set(re.findall(r"\b(qw_[a-z0-9_]+)\s*\(", text))
