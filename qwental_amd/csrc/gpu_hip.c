@@ -109,6 +109,9 @@ struct qw_batch {
     // a grouped product over IQ3_S rows that waits for its twin (gate, then up over the same packed rows: one launch
     // over the tile-major copy that holds both); launched alone at the next other dispatch or at submit
     struct { bool valid; qwk_pf_args a; qw_hbuf *hw, *hx, *hy; int E; } pend_pf;
+    // a down projection over a few tokens that waits for the combine of the same layer: both in one launch
+    // (qwk_dnc_*); launched as it is at any other dispatch or at submit
+    struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid; } pend_dn;
 };
 
 #define QW_LD_MAX 16
@@ -1101,6 +1104,22 @@ static bool tr_gu(qw_batch *b) {
     return add_launch(b, intern(fn), persistent_grid(b->g, tasks, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 
+// Token count up to which the down projection and the combine run as one launch (QW_HIP_DNC_NB in the environment
+// overrides it, 0 turns the fusion off).
+static unsigned dnc_maxnb(void) {
+    const char *e = getenv("QW_HIP_DNC_NB");
+    const unsigned n = e ? (unsigned)atoi(e) : 2;
+    return n > QW_DNC_MAXNB ? QW_DNC_MAXNB : n;
+}
+static bool flush_dn(qw_batch *b) {
+    if (!b->pend_dn.valid) return true;
+    b->pend_dn.valid = false;
+    const int first = b->nl;
+    if (!add_launch(b, b->pend_dn.fname, b->pend_dn.grid, 64 * QW_WAVES_DNR, &b->pend_dn.a, sizeof b->pend_dn.a)) return false;
+    if (b->nl > first) b->l[b->nl - 1].kname = b->pend_dn.kname, b->l[b->nl - 1].last_of_dispatch = true;
+    return true;
+}
+
 // src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
 // The shared down tiles (remembered from moe_gu_gg) run in the same launch.
 static bool tr_dn(qw_batch *b) {
@@ -1141,7 +1160,19 @@ static bool tr_dn(qw_batch *b) {
         const int ch = fd == 8 ? 4 : p->I / 256;
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
-        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
+        const unsigned grid = persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR);
+        // a few tokens: wait for the combine, the two run as one launch (tile-major IQ3_S or Q8_0 routed rows; a shared
+        // expert in either of these)
+        if (nbr <= dnc_maxnb() && (fd == QW_F_PACKED || fd == 8) && (fs == 0 || fs == 8 || (fs == QW_F_PACKED && fd == QW_F_PACKED))) {
+            char fu[48];
+            if (fs) fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
+            else fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d", fd, ch);
+            b->pend_dn.valid = true;
+            b->pend_dn.a = a;
+            b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid;
+            return true;
+        }
+        return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
     }
     // wider rows: one tile at a time, operand A from global memory
     fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any%s", p->fd, sfx);
@@ -1156,6 +1187,19 @@ static bool tr_cmb(qw_batch *b) {
     qwk_cmb_args a = {.D = (uint32_t)p->D, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb};
     if (!bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, false, "Pg", (void **)&a.Pg) || !bind_ptr(b, 1, (size_t)nbr * p->D * 4, false, "Psh", (void **)&a.Psh) ||
         !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel) || !bind_ptr(b, 4, (size_t)nbr * p->D * 2, true, "out", (void **)&a.out)) return false;
+    if (b->pend_dn.valid) {
+        qwk_dn_args *d = &b->pend_dn.a;
+        // the down dispatch counts tokens by its compiled NB, the combine by the bound count: the masks carry the rest
+        const bool same = d->P == a.Pg && d->sel == a.sel && d->nbr >= nbr && d->D == a.D && d->topk == a.topk && d->gnb == a.gnb && (!d->Wsd || (d->Psh == a.Psh && d->snbr >= nbr));
+        if (same) {
+            b->pend_dn.valid = false;
+            d->nbr = nbr;
+            d->out = a.out;
+            d->Psh = (float *)a.Psh;
+            return add_launch(b, b->pend_dn.fused, a.D / 16, 64 * QW_WAVES_DNR, d, sizeof *d);
+        }
+        if (!flush_dn(b)) return false;
+    }
     return add_launch(b, "qwk_cmb", cdiv(nbr * (unsigned)p->D, 256), 256, &a, sizeof a);
 }
 
@@ -1309,6 +1353,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     bool ok;
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
     if (b->k->fam != FAM_PF && !flush_pf(b)) return;
+    if (b->k->fam != FAM_CMB && !flush_dn(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
     case FAM_QMV_GGM: ok = tr_qmvm(b); break;
@@ -1338,7 +1383,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
-    if (b->failed || !flush_select(b) || !flush_pf(b)) return false;
+    if (b->failed || !flush_select(b) || !flush_pf(b) || !flush_dn(b)) return false;
     if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
     // host -> device for what this segment binds
     const unsigned mark = ++g->mark;

@@ -95,7 +95,11 @@ typedef struct {
     const uint8_t *Wsd;
     float *Psh;
     uint32_t sd_rowbytes, snbr; /* snbr: token count of the shared part */
+    /* down + combine in one launch (qwk_dnc_*, at most QW_DNC_MAXNB tokens): the layer's output [nbr][D] binary16;
+     * Psh is then also read when the launch carries no shared expert */
+    uint16_t *out;
 } qwk_dn_args;
+#define QW_DNC_MAXNB 4
 
 /* front part of a layer: router rows on the first nrouter workgroups; when g.Wsg != NULL the shared expert's gate/up
  * on the workgroups after them (g: its arguments, shared = 1), one chunk of a tile per wave, summed through LDS. */

@@ -1117,6 +1117,93 @@ QW_DN_RANGE(121, 2, 0, 1, qwk_dnr_f121_c2) QW_DN_RANGE(121, 2, 121, 2, qwk_dnr_f
 QW_DN_RANGE(121, 1, 0, 1, qwk_dnr_f121_c1) QW_DN_RANGE(121, 1, 121, 1, qwk_dnr_f121_c1_s121_c1) QW_DN_RANGE(121, 1, 8, 4, qwk_dnr_f121_c1_s8_c4)
 QW_DN_RANGE(8, 4, 0, 1, qwk_dnr_f8_c4) QW_DN_RANGE(8, 4, 8, 4, qwk_dnr_f8_c4_s8_c4) QW_DN_RANGE(8, 4, 21, 2, qwk_dnr_f8_c4_s21_c2) QW_DN_RANGE(8, 4, 21, 1, qwk_dnr_f8_c4_s21_c1)
 
+// Down + combine in one launch for a few tokens (at most QW_DNC_MAXNB; kernels/moe_gg.metal:639-663 in one pass).
+// With one or two tokens the layer is bound by its launches, and the combine is a launch that only adds up what the
+// down launch wrote. Here a workgroup owns one tile of 16 output rows: its waves take the shared expert and the unique
+// routed experts of the record, one (expert, tile) product each (operand A straight from the H planes, only the lanes
+// of tokens that picked the expert read), leave the partial results in LDS by (token, slot), and after one barrier
+// sixteen lanes per token add them up in rank order, the shared expert last, exactly as the combine kernel does.
+// Pg and Psh are still written, so that the buffers hold what the two separate launches would have left.
+template <int F, int CH, class S>
+__device__ __forceinline__ f4 dnc_tile(const qwk_dn_args &a, const u2 *lut, const uint8_t *W, uint32_t rowbytes, uint32_t tile, const qw_afrag_gather &af, S ready) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), kg = lane >> 4, cpr = a.I / (C::BLK_K * CH);
+    f4 acc = {0, 0, 0, 0};
+    qw_task_pipeline<C>(1, 0, 1, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
+        [&](uint32_t) {
+            if constexpr (F == QW_F_PACKED) return W + (size_t)tile * rowbytes; // rowbytes = bytes of a tile
+            else return W + (size_t)(16 * tile + (lane >> 2)) * rowbytes;
+        },
+        [&](uint32_t, uint32_t ci, const C &c) { c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc); }, ready);
+    return acc;
+}
+template <int F, int CH, int FSD, int CHSD>
+__device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *part /* [QW_DNC_MAXNB][topk + 1][16] */, float *wl /* [QW_DNC_MAXNB][topk + 1] */, qw_sel_cache *sc) {
+    const uint32_t K = a.topk, gnb = a.gnb, tpe = a.D / 16, tile = blockIdx.x, lane = qw_lane(), n = lane & 15, kg = lane >> 4, nwv = blockDim.x >> 6;
+    qw_sel_load(*sc, a.sel, K, gnb);
+    const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K));
+    for (uint32_t i = threadIdx.x; i < a.nbr * (K + 1); i += blockDim.x) wl[i] = wg[i];
+    if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // awaited in ready()
+    __syncthreads();
+    uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
+    if (U > gnb * K) U = gnb * K;
+    const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0, V = nsh + U;
+    bool staged = false;
+    auto ready = [&] { // once per wave, behind its first weight loads: the table has landed, for every wave
+        if (staged) return;
+        staged = true;
+        qw_lds_arrive();
+        __syncthreads();
+    };
+    for (uint32_t v = qw_wave(); v < V; v += nwv) {
+        const bool sh = v < nsh;
+        const uint32_t u = sh ? 0 : v - nsh;
+        const uint32_t mask = sh ? qw_all_tokens(a.snbr) : (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->mask[u]) & qw_all_tokens(a.nbr);
+        const bool on = (mask >> n) & 1; // token n of the batch takes part in this product
+        const uint32_t sl = sh || !on ? K : sc->slot[u * gnb + n];
+        const uint16_t *rowhi = a.H + ((size_t)(on ? n : 0) * (K + 1) + sl) * a.I;
+        h8 xhi[4] = {}, xlo[4] = {}; // the columns of tokens that are off stay zero
+        const qw_afrag_gather af = {rowhi, rowhi + a.hplane, on, xhi, xlo};
+        f4 acc;
+        if (sh) {
+            if constexpr (FSD != 0) acc = dnc_tile<FSD, CHSD>(a, lut, a.Wsd, a.sd_rowbytes, tile, af, ready);
+            else acc = f4{0, 0, 0, 0};
+        } else {
+            const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->ue[u]);
+            acc = dnc_tile<F, CH>(a, lut, a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, a.rowbytes, tile, af, ready);
+        }
+        const uint32_t r = 16 * tile + n;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) {
+            const uint32_t tok = 4 * kg + j;
+            if (tok < QW_DNC_MAXNB && ((mask >> tok) & 1)) {
+                const uint32_t s = sh ? K : sc->slot[u * gnb + tok];
+                part[(tok * (K + 1) + s) * 16 + n] = acc[j];
+                if (sh) a.Psh[(size_t)tok * a.D + r] = acc[j];
+                else a.P[((size_t)tok * K + s) * a.D + r] = acc[j];
+            }
+        }
+    }
+    ready(); // waves without a product still meet the others at the barrier
+    __syncthreads();
+    if (threadIdx.x < a.nbr * 16) { // rank order, then the shared expert (qwk_cmb's arithmetic)
+        const uint32_t t = threadIdx.x >> 4, i = threadIdx.x & 15, r = 16 * tile + i;
+        const float *w = wl + t * (K + 1), *p = part + t * (K + 1) * 16 + i;
+        float o = 0;
+        for (uint32_t s = 0; s < K; s++) o = __builtin_fmaf(w[s], p[s * 16], o);
+        o = __builtin_fmaf(w[K], nsh ? p[K * 16] : a.Psh[(size_t)t * a.D + r], o);
+        a.out[(size_t)t * a.D + r] = qw_f2h(o);
+    }
+}
+#define QW_DNC(F, CH, FSD, CHSD, NAME)                                                              \
+    extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                    \
+        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; float part[QW_DNC_MAXNB * 17 * 16], wl[QW_DNC_MAXNB * 17]; qw_sel_cache sc; } L; \
+        dnc_body<F, CH, FSD, CHSD>(a, L.lut, L.part, L.wl, &L.sc);                                  \
+    }
+QW_DNC(121, 2, 0, 1, qwk_dnc_f121_c2) QW_DNC(121, 2, 121, 2, qwk_dnc_f121_c2_s121_c2) QW_DNC(121, 2, 8, 4, qwk_dnc_f121_c2_s8_c4)
+QW_DNC(121, 1, 0, 1, qwk_dnc_f121_c1) QW_DNC(121, 1, 121, 1, qwk_dnc_f121_c1_s121_c1) QW_DNC(121, 1, 8, 4, qwk_dnc_f121_c1_s8_c4)
+QW_DNC(8, 4, 0, 1, qwk_dnc_f8_c4) QW_DNC(8, 4, 8, 4, qwk_dnc_f8_c4_s8_c4)
+
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
     typedef qw_chunk<F, 1> C;

@@ -329,6 +329,47 @@ def test_moe_batched_equals_single(gpu):
     path.close()
 
 
+@pytest.mark.parametrize("nb,limit", [(1, 2), (2, 2), (3, 4), (4, 4)])
+@pytest.mark.parametrize("fd,fshd,dev", [(21, 21, True), (21, 8, True), (8, 8, False), (8, 8, True)])
+def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev):
+    """With a few tokens the down projection and the combine run as one launch (kernels/moe_gg.metal:639-663 in one
+    pass). Its output, Pg and Psh must equal bit for bit what the two separate launches leave, and the output must meet
+    the float64 layer."""
+    if dev and fd == 21 and os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
+    D, I, E, K = 2048, 512, 32, 10
+    rng = np.random.default_rng(900 + nb + fd + fshd)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=fd, fsh=21 if fshd == 21 else 8, fshd=fshd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    if nb > 1:
+        x[nb - 1] = x[0]  # two tokens on the same experts: one product serves both
+    dl = DeviceLayer(gpu, m, device_only=dev)
+    old = os.environ.get("QW_HIP_DNC_NB")
+    res = {}
+    try:
+        for lim in (0, limit):
+            os.environ["QW_HIP_DNC_NB"] = str(lim)
+            path = q.Path(gpu, D, I, E, K, 16)
+            gpu.profile(True)
+            out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            res[lim] = (out, lg, path.scratch(2).view(np.float32)[:nb * D].copy(), path.scratch(3).view(np.float32)[:nb * K * D].copy(), names)
+            path.close()
+    finally:
+        if old is None:
+            os.environ.pop("QW_HIP_DNC_NB", None)
+        else:
+            os.environ["QW_HIP_DNC_NB"] = old
+    a, b = res[0], res[limit]
+    assert any(n.startswith("qwk_dnc_") for n in b[4]) and not any(n.startswith("qwk_dnc_") for n in a[4]), (a[4], b[4])
+    assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
+    assert np.array_equal(a[2].view(np.uint32), b[2].view(np.uint32)) and np.array_equal(a[3].view(np.uint32), b[3].view(np.uint32))
+    assert maxrel(b[0], oracle.moe_layer_f64(m, b[1], x)) <= TOL
+    dl.free()
+
+
 @pytest.mark.parametrize("nb,valu", [(1, False), (3, False), (16, False), (1, True), (2, True), (4, True)])
 def test_qmv_packed_and_valu_forms(gpu, oracle, nb, valu):
     """Weights in a device-only buffer take the tile-major copy; with QW_VALU in the block the VALU GEMV runs instead of
