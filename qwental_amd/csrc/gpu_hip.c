@@ -392,7 +392,8 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             FAIL("moe_gg: E, TOPK, D, I and NB must be integer macros");
         if (p.NB < 1 || p.NB > 16) FAIL("moe_gg: NB %d outside 1..16", p.NB);
         if (p.E < 1 || p.E > 1024 || p.topk < 1 || p.topk > 16 || p.topk > p.E) FAIL("moe_gg: E %d / TOPK %d outside this build (E <= 1024, TOPK <= 16)", p.E, p.topk);
-        if (p.D % 256 || p.I % 256 || p.D > 2560 || p.D < 256 || p.I < 256) FAIL("moe_gg: D %d / I %d outside this build (multiples of 256, D <= 2560)", p.D, p.I);
+        // the reference asks D % 512 == 0 and I % 128 == 0 (kernels/moe_gg.metal:419); its model has D = 2560, I = 640
+        if (p.D % 256 || p.I % 128 || p.D > 2560 || p.D < 256 || p.I < 256) FAIL("moe_gg: D %d / I %d outside this build (D a multiple of 256 up to 2560, I a multiple of 128 from 256)", p.D, p.I);
         p.gnb = p.NB <= 8 ? 8 : 16; // 8 = the reference's gg_sel layout; 16 = the wide layout
         p.rwf = 30;
         if (def_int(d, n, "RWF", &v)) { if (v != 1 && v != 30) FAIL("moe_gg: RWF %d (router weight type) must be 1 or 30", v); p.rwf = v; }
@@ -406,11 +407,13 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             if (!reg_kernel(g, d, n, "moe_pre_gg", FAM_PRE, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 2) {
             if (!def_int(d, n, "FGU", &p.fgu) || !def_int(d, n, "FSD", &p.fsd)) FAIL("moe_gu_gg: FGU, FSD missing");
-            if (!fmt_ok(p.fgu) || !fmt_ok(p.fsd)) FAIL("moe_gu_gg: types %d/%d have no gfx950 build (have 8, 21)", p.fgu, p.fsd);
+            if (!fmt_ok(p.fgu) || !(fmt_ok(p.fsd) || p.fsd == 20)) FAIL("moe_gu_gg: types %d/%d have no gfx950 build (have 8, 21; shared down also 20)", p.fgu, p.fsd);
+            if (p.fsd == 21 && p.I % 256) FAIL("moe_gu_gg: I %d does not fit IQ3_S shared down rows", p.I);
             if (!reg_kernel(g, d, n, "moe_gu_gg", FAM_GU, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 3) {
             if (!def_int(d, n, "FD", &p.fd)) FAIL("moe_dn_gg: FD missing");
-            if (!fmt_ok(p.fd)) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 21)", p.fd);
+            if (!fmt_ok(p.fd) && p.fd != 20) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 20, 21)", p.fd);
+            if (p.fd == 21 && p.I % 256) FAIL("moe_dn_gg: I %d does not fit IQ3_S rows", p.I);
             if (!reg_kernel(g, d, n, "moe_dn_gg", FAM_DN, &p, err, errlen) || !reg_kernel(g, d, n, "moe_cmb_gg", FAM_CMB, &p, err, errlen)) { ok = false; goto out; }
         } else if (part != 5) FAIL("moe_gg: GG_PART %d has no gfx950 build (have 0..3, 5 and GG_ROUTER)", part);
     }
@@ -1156,7 +1159,9 @@ static bool tr_dn(qw_batch *b) {
     }
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
-    if (p->I <= 512) { // contiguous task ranges per workgroup, operand A staged in LDS
+    if (fd == 20 || fs == 20) { // IQ4_NL rows run in the any-shape kernel; the shared expert's may be IQ4_NL or Q8_0 beside them
+        if (fd != 20 || (fs != 0 && fs != 20 && fs != 8)) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
+    } else if (p->I <= 512 && p->I % 256 == 0) { // contiguous task ranges per workgroup, operand A staged in LDS
         const int ch = fd == 8 ? 4 : p->I / 256;
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);

@@ -21,6 +21,7 @@
 #include "iq3s_codes.h"
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
@@ -211,6 +212,8 @@ template <bool LO> struct qw_afrag_glb {
     static constexpr bool has_lo = LO;
     __device__ __forceinline__ h8 hi(uint32_t koff) const { return rowhi ? *(const h8 *)(rowhi + koff) : h8{}; }
     __device__ __forceinline__ h8 lo(uint32_t koff) const { return rowlo ? *(const h8 *)(rowlo + koff) : h8{}; }
+    __device__ __forceinline__ h4 hi4(uint32_t koff) const { return rowhi ? *(const h4 *)(rowhi + koff) : h4{}; } // four values
+    __device__ __forceinline__ h4 lo4(uint32_t koff) const { return rowlo ? *(const h4 *)(rowlo + koff) : h4{}; }
 };
 
 // One token's row of both planes staged in LDS as [hi I halves][lo I halves].

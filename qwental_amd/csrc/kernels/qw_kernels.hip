@@ -1209,6 +1209,7 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
     typedef qw_chunk<F, 1> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
     if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook (IQ3_S never meets it here)
     qw_sel_load(*sc, a.sel, K, gnb);
     __syncthreads();
     const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
@@ -1236,11 +1237,13 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
 }
 #define QW_DN_ANY(F, FSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
-        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : 1]; qw_sel_cache sc; } L; \
+        __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : (F == 20 || FSD == 20) ? QW_KQ_TAB / 2 : 1]; qw_sel_cache sc; } L; \
         dn_any_body<F, FSD>(a, L.lut, &L.sc);                                         \
     }
 QW_DN_ANY(21, 0, qwk_dn_f21_any) QW_DN_ANY(21, 21, qwk_dn_f21_any_s21) QW_DN_ANY(21, 8, qwk_dn_f21_any_s8)
 QW_DN_ANY(8, 0, qwk_dn_f8_any) QW_DN_ANY(8, 21, qwk_dn_f8_any_s21) QW_DN_ANY(8, 8, qwk_dn_f8_any_s8)
+// IQ4_NL down rows (the routed and shared down projections of a layer with I = 640, bench/moe_bw.c:22-24 of the reference)
+QW_DN_ANY(20, 0, qwk_dn_f20_any) QW_DN_ANY(20, 20, qwk_dn_f20_any_s20) QW_DN_ANY(20, 8, qwk_dn_f20_any_s8)
 
 // ================================================================ ragged packing (kernels/moe_prefill.metal:15-119)
 // P (token, expert) pairs -> per-expert counts -> exclusive prefix sums (first packed row of every expert, tile table)

@@ -14,7 +14,6 @@
 #pragma once
 #include "qw_common.hip.h"
 
-typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
 typedef uint32_t __attribute__((aligned(2))) u1a2;
 
@@ -317,6 +316,59 @@ template <int F, int S = 0> __device__ __forceinline__ void qw_kq_values(const q
         qw_kq_values<F, S + 1>(b, tab, kg, y);
     }
 }
+
+// IQ4_NL rows for the MoE kernels (the interface of qw_chunk<8, NB>): NB blocks of 18 bytes, loaded in quad order
+// (lane & 3 takes bytes 4 kl .. 4 kl + 3 of qs), pulled to matrix-core lane order. "lut" is the 256-entry byte table
+// of qw_kq_tab_build. Operand A of a block: x[4 kg .. + 4] and x[16 + 4 kg .. + 4], the values the lane's four bytes hold.
+template <int NB> struct qw_chunk<20, NB> {
+    static constexpr uint32_t BLK_K = 32, BLK_B = 18;
+    static constexpr int DEPTH = 2;
+    uint32_t q[NB];
+    uint16_t d[NB];
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t kl) {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            q[b] = *(const u1a2 *)(p + 18 * b + 2 + 4 * kl);
+            d[b] = *(const uint16_t *)(p + 18 * b);
+        }
+    }
+    __device__ __forceinline__ void transpose() {
+        const uint32_t src4 = qw_pull_addr();
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            q[b] = qw_pull(q[b], src4);
+            d[b] = (uint16_t)qw_pull(d[b], src4);
+        }
+    }
+    static __device__ __forceinline__ h8 join(h4 a, h4 b) { return h8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]}; }
+    template <class AF> __device__ __forceinline__ void mac(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const h8 w = qw_iq4_bytes((const uint32_t *)lut, q[b]);
+            const uint32_t kb = k0 + 32 * b + 4 * kg;
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(join(af.hi4(kb), af.hi4(kb + 16)), w, sub);
+            if (AF::has_lo) sub = qw_mfma(join(af.lo4(kb), af.lo4(kb + 16)), w, sub);
+            acc += qw_h2f(d[b]) * sub;
+        }
+    }
+    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const uint32_t kb = k0 + 32 * b + 4 * kg;
+            h8 xh = {}, xl = {};
+            if (af.on) {
+                xh = join(*(const h4 *)(af.rowhi + kb), *(const h4 *)(af.rowhi + kb + 16));
+                xl = join(*(const h4 *)(af.rowlo + kb), *(const h4 *)(af.rowlo + kb + 16));
+            }
+            const h8 w = qw_iq4_bytes((const uint32_t *)lut, q[b]);
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(xh, w, sub);
+            sub = qw_mfma(xl, w, sub);
+            acc += qw_h2f(d[b]) * sub;
+        }
+    }
+};
 
 // NB blocks of one row for the task pipeline: loaded in quad order, pulled to matrix-core lane order.
 template <int F, int NB> struct qw_chunk_kq {

@@ -125,6 +125,11 @@ def test_bad_calls_fail_without_launching(gpu):
     ok, err = gpu.compile("#define IQ_DQ_ONLY 1\n#define qmv_gg q_bad\n#define GF 21\n#define KD 2048\n#define RB 881\n#define NB 1\n")
     assert not ok
     assert not gpu.kernel("no_such_kernel")
+    head = "#define IQ_DQ_ONLY\n#define E 512\n#define TOPK 10\n#define D 2560\n#define I 640\n#define NB 8\n#define GG_PART 3\n#define DSGN 4\n"
+    ok, err = gpu.compile(head + "#define FD 21\n#define moe_dn_gg dn_bad\n#define moe_cmb_gg cmb_bad\n")  # IQ3_S rows cannot be 640 long
+    assert not ok and "640" in err
+    ok, err = gpu.compile(head + "#define FD 20\n#define moe_dn_gg dn_640_nl\n#define moe_cmb_gg cmb_640_nl\n")
+    assert ok, err
     path = q.Path(gpu, 2048, 512, 512, 10, 16)
     W = gpu.buf(100)  # far too small for 4096 rows
     x, y = gpu.buf(4096), gpu.buf(4096 * 4)
@@ -288,6 +293,11 @@ def test_moe_layer_parity(gpu, oracle, nb, fmt):
     (1536, 512, 256, 16, 16, 21, 8, 8, 21, True),    # sixteen picks per token; mixed formats per projection
     (256, 256, 1024, 10, 3, 21, 21, 21, 21, False),  # the smallest rows, the most experts
     (2048, 512, 48, 10, 9, 21, 21, 21, 21, True),    # an expert count without a register build of the selection
+    (2560, 640, 64, 10, 16, 21, 20, 21, 20, True),   # the reference model's shape and routed formats (src/model.h:10-18, bench/moe_bw.c:16-24): IQ4_NL down rows of 640
+    (2560, 640, 64, 10, 1, 21, 20, 21, 20, True),    # the same, one token
+    (2560, 640, 64, 10, 7, 21, 20, 8, 8, False),     # IQ4_NL routed down beside a Q8_0 shared expert
+    (2560, 640, 64, 10, 12, 21, 8, 21, 8, True),     # I = 640 with Q8_0 down rows
+    (1024, 384, 32, 4, 5, 8, 20, 8, 20, False),      # I a multiple of 128 only
 ])
 def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
     """Shapes and format mixes off the benchmark's: every kernel variant the host can pick is reached by one of them."""
