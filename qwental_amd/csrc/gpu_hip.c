@@ -139,6 +139,7 @@ struct qw_gpu {
     int npacks, cappacks;
     struct qw_ldlane { void *pin[2]; hipStream_t st; hipEvent_t ev[2]; } ld[QW_LD_MAX]; // staging of qw_hip_buf_write_fd, made at first use
     int nld;
+    float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes;
 };
@@ -196,6 +197,7 @@ qw_gpu *qw_gpu_open(void) {
         qwk_tab_args ta;
         void *params[] = {&ta};
         if (hipMalloc(&g->tabs, QW_TAB_BYTES) != hipSuccess || hipMemset(g->tabs, 0, QW_TAB_BYTES) != hipSuccess ||
+            hipMalloc((void **)&g->shgu, (size_t)2 * 2 * 16 * 4096 * 4) != hipSuccess ||
             hipModuleGetFunction(&f, g->mod, "qwk_tab_init") != hipSuccess) { free(g->kernels); free(g); return NULL; }
         ta = (qwk_tab_args){.tab = g->tabs, .slot_order = 1};
         if (hipDeviceSynchronize() != hipSuccess || hipModuleLaunchKernel(f, 32, 1, 1, 256, 1, 1, 0, g->stream[0], params, NULL) != hipSuccess ||
@@ -227,6 +229,7 @@ void qw_gpu_close(qw_gpu *g) {
     }
     free(g->packs);
     (void)hipFree(g->tabs);
+    (void)hipFree(g->shgu);
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
     free(g);
@@ -403,7 +406,9 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             if (!reg_kernel(g, d, n, "gg_tab_init", FAM_TAB_INIT, &p, err, errlen) || !reg_kernel(g, d, n, "moe_sel_gg", FAM_SEL, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 1) {
             if (!def_int(d, n, "FSG", &p.fsg) || !def_int(d, n, "FSU", &p.fsu) || !def_int(d, n, "RBF", &p.rbf)) FAIL("moe_pre_gg: FSG, FSU, RBF missing");
-            if (!fmt_ok(p.fsg) || p.fsu != p.fsg) FAIL("moe_pre_gg: shared gate/up types %d/%d: this build needs equal types from {8, 21}", p.fsg, p.fsu);
+            if (!(fmt_ok(p.fsg) && p.fsu == p.fsg) && !(kq_ok(p.fsg) && kq_ok(p.fsu)))
+                FAIL("moe_pre_gg: shared gate/up types %d/%d: this build needs equal types from {8, 21} or two of {1, 12, 13, 14, 20, 23, 30}", p.fsg, p.fsu);
+            if (kq_ok(p.fsg) && (p.D > (int)QW_KQ_MAXK)) FAIL("moe_pre_gg: D %d too wide for shared gate/up types %d/%d", p.D, p.fsg, p.fsu);
             if (!reg_kernel(g, d, n, "moe_pre_gg", FAM_PRE, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 2) {
             if (!def_int(d, n, "FGU", &p.fgu) || !def_int(d, n, "FSD", &p.fsd)) FAIL("moe_gu_gg: FGU, FSD missing");
@@ -1004,6 +1009,22 @@ static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nb
     return bind_bytes(b, 2, &nbr, 4, "nbr") && nbr_ok(b, nbr) && launch_select(b, 0, 1, nbr);
 }
 
+// A shared expert whose gate and up rows are in the other format family (Q4_K gate and IQ4_XS up in the reference's
+// model, bench/moe_bw.c:19-20): the multi-format matvec over the two matrices, then SwiGLU into H.
+#define QW_SHGU_MAXI 4096
+static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t *h) {
+    const qw_kparams *p = &b->k->p;
+    if (p->I > QW_SHGU_MAXI) return fail(b, "moe_pre_gg: I %d too wide for shared gate/up types %d/%d", p->I, p->fsg, p->fsu);
+    if (b->buf[2].off % 16 || b->buf[6].off % 16 || b->buf[7].off % 16) return fail(b, "moe_pre_gg: x and shared gate/up offsets must be 16-byte aligned for types %d/%d", p->fsg, p->fsu);
+    float *gy = b->g->shgu + (size_t)b->stream * 2 * 16 * QW_SHGU_MAXI, *uy = gy + (size_t)16 * p->I;
+    qwk_qmvm_args m = {.K = (uint32_t)p->D, .xstride = (uint32_t)p->D, .nb = nbr, .yfloat = 1, .nmat = 2, .x = x,
+                       .W = {b->pend_sg.Wsg, b->pend_sg.Wsu}, .y = {gy, uy}, .N = {(uint32_t)p->I, (uint32_t)p->I}, .fmt = {(uint32_t)p->fsg, (uint32_t)p->fsu},
+                       .rowbytes = {(uint32_t)fmt_rb(p->fsg, p->D), (uint32_t)fmt_rb(p->fsu, p->D)}, .ystride = {(uint32_t)p->I, (uint32_t)p->I}};
+    qwk_shact_args sa = {.g = gy, .u = uy, .H = h, .I = (uint32_t)p->I, .nb = nbr, .topk = (uint32_t)p->topk, .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
+    b->pend_sg.valid = false; // done here
+    return launch_qmvm(b, &m) && add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa);
+}
+
 // src/engine.c:588-607: 0 Wr, 1 shared gate vector, 2 x, 3 logits, 4 counter, 5 sel, 6/7 shared gate/up, 8 H, 13 tables, 14 nbr.
 // Two launches: router rows, then the selection. The shared expert's gate/up is checked and remembered here and
 // runs inside the gate/up launch that follows.
@@ -1014,7 +1035,7 @@ static bool tr_pre(qw_batch *b) {
     const size_t rb = fmt_rb(p->fsg, p->D);
     uint16_t *h;
     b->pend_sg.valid = false;
-    if (!bind_ptr(b, 6, (size_t)p->I * rb, false, "shared gate weights", (void **)&b->pend_sg.Wsg) || !bind_ptr(b, 7, (size_t)p->I * rb, false, "shared up weights", (void **)&b->pend_sg.Wsu) ||
+    if (!bind_ptr(b, 6, (size_t)p->I * rb, false, "shared gate weights", (void **)&b->pend_sg.Wsg) || !bind_ptr(b, 7, (size_t)p->I * fmt_rb(p->fsu, p->D), false, "shared up weights", (void **)&b->pend_sg.Wsu) ||
         !bind_ptr(b, 8, (size_t)p->NB * (p->topk + 1) * p->I * 4, true, "H", (void **)&h)) return false;
     b->pend_sg.valid = true;
     b->pend_sg.hg = b->buf[6].h;
@@ -1022,7 +1043,10 @@ static bool tr_pre(qw_batch *b) {
     b->pend_sg.fmt = p->fsg;
     b->pend_sg.rowbytes = (uint32_t)rb;
     b->pend_sg.nbr = nbr;
-    if (!p->rbf) return true; // router and selection come as dispatches of their own
+    if (!p->rbf) { // router and selection come as dispatches of their own
+        const uint16_t *x;
+        return !kq_ok(p->fsg) || (bind_ptr(b, 2, (size_t)nbr * p->D * 2, false, "x", (void **)&x) && shared_gu_kq(b, nbr, x, h));
+    }
     // router rows per workgroup: 16 on the matrix cores (binary16 router), 8 on the vector units (bf16 router)
     qwk_pre_args a = {.nrouter = cdiv((unsigned)p->E + 1, p->rwf == 1 ? 16 : 8)};
     if (!fill_router(b, &a.r, 0, 1, 2, 3, nbr)) return false;
@@ -1048,7 +1072,9 @@ static bool tr_pre(qw_batch *b) {
         }
     }
     // the counter buffer of the reference's hand-over (index 4) is not used
-    if (!add_launch(b, intern(fn), grid, 512, &a, sizeof a) || !fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
+    if (!add_launch(b, intern(fn), grid, 512, &a, sizeof a)) return false;
+    if (kq_ok(p->fsg) && !shared_gu_kq(b, nbr, a.r.x, h)) return false;
+    if (!fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
     b->pend_sel.valid = true; // made by the gate/up launch if one follows for the same record, else by its own launch
     return true;
 }

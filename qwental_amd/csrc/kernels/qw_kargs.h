@@ -47,6 +47,14 @@ typedef struct {
     uint32_t split, pad;                         /* waves a tile's K range is cut over (1, 2, 4; > 1 needs K % (256 * split) == 0) */
 } qwk_qmvm_args;
 
+/* SwiGLU of the shared expert when its gate/up rows went through the multi-format matvec: g, u float [nb][I] ->
+ * H[t][topk][j] as binary16 hi + lo planes */
+typedef struct {
+    const float *g, *u;
+    uint16_t *H;
+    uint32_t I, nb, topk, hplane;
+} qwk_shact_args;
+
 typedef struct { /* router: logits[t][r], r in [0, E] (row E = shared gate vector), row stride E + 1 */
     const uint16_t *Wr, *Wsg, *x;
     float *logits;

@@ -939,6 +939,19 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
 QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
 QW_PRE(1, 121, 2, qwk_pre_w1_s121_c2) QW_PRE(30, 121, 2, qwk_pre_w30_s121_c2) QW_PRE(1, 8, 16, qwk_pre_w1_s8_c16) QW_PRE(30, 8, 16, qwk_pre_w30_s8_c16)
 
+// SwiGLU of the shared expert (kernels/moe_gg.metal:563-573) after a matvec of its gate and up rows in another format
+// family: the arithmetic and the two-plane store of pre_shared. One thread per (token, column).
+extern "C" __global__ __launch_bounds__(256) void qwk_sh_act(qwk_shact_args a) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.nb * a.I) return;
+    const uint32_t t = i / a.I, j = i % a.I;
+    const float g = a.g[i], up = a.u[i], h = g / (1.0f + __expf(-g)) * up;
+    const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
+    const size_t o = ((size_t)t * (a.topk + 1) + a.topk) * a.I + j;
+    a.H[o] = __builtin_bit_cast(uint16_t, hi);
+    a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
+}
+
 // ================================================================ down (kernels/moe_gg.metal:456-483, 606-617, 639-652)
 // The shared expert's down projection rides in the same launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
 // planes) of every token straight from global memory. Wave w takes tiles w, w + nw, ...

@@ -64,15 +64,16 @@ def router(rng, E, D):
     return rng.normal(0.0, 0.02, (E, D)).astype(np.float16), rng.normal(0.0, 0.02, D).astype(np.float16)
 
 
-def moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21, fshd=None, experts=None, d_scale=MOE_D_SCALE):
+def moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21, fshd=None, experts=None, d_scale=MOE_D_SCALE, fshu=None):
     """One MoE layer as a dict of numpy arrays (the field names of qwo_moe_weights / MoeLayer).
     experts: generate only this many routed experts' bytes (the others are never read when ids are < experts)."""
     ne = E if experts is None else experts
     fshd = fsh if fshd is None else fshd
+    fshu = fsh if fshu is None else fshu  # the shared expert's up rows may have a format of their own
     Wr, wsg = router(rng, E, D)
-    return dict(D=D, I=I, E=E, fgu=fgu, fd=fd, fsg=fsh, fsu=fsh, fsd=fshd, Wr=Wr, wsg=wsg,
+    return dict(D=D, I=I, E=E, fgu=fgu, fd=fd, fsg=fsh, fsu=fshu, fsd=fshd, Wr=Wr, wsg=wsg,
                 Wg=matrix(rng, fgu, ne * I, D, d_scale), Wu=matrix(rng, fgu, ne * I, D, d_scale), Wd=matrix(rng, fd, ne * D, I, d_scale),
-                Wsg=matrix(rng, fsh, I, D, d_scale), Wsu=matrix(rng, fsh, I, D, d_scale), Wsd=matrix(rng, fshd, D, I, d_scale))
+                Wsg=matrix(rng, fsh, I, D, d_scale), Wsu=matrix(rng, fshu, I, D, d_scale), Wsd=matrix(rng, fshd, D, I, d_scale))
 
 
 def expert_bytes(D, I, fgu=21, fd=21):

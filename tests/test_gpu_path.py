@@ -339,6 +339,42 @@ def test_moe_batched_equals_single(gpu):
     path.close()
 
 
+@pytest.mark.parametrize("nb", [1, 2, 5, 16])
+@pytest.mark.parametrize("D,I,fsg,fsu,fsd,fd", [
+    (2560, 640, 12, 23, 20, 20),   # the formats of the reference model's layer (bench/moe_bw.c:19-24): Q4_K gate, IQ4_XS up, IQ4_NL down
+    (2048, 512, 14, 13, 8, 21),    # Q6_K gate, Q5_K up beside IQ3_S routed rows and a Q8_0 shared down
+    (1024, 256, 20, 30, 21, 21),   # IQ4_NL gate, bfloat16 up
+])
+def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd):
+    """The shared expert's gate and up rows in the K-quant / IQ4 / plain formats (different ones for gate and up):
+    the multi-format matvec and a SwiGLU launch stand in for the front launch's shared tiles. Output against the
+    float64 layer; H of the shared expert against the float oracle's."""
+    E, K = 32, 10
+    rng = np.random.default_rng(1700 + nb + D + fsg + fsu)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=fd, fsh=fsg, fshu=fsu, fshd=fsd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    path = q.Path(gpu, D, I, E, K, 16)
+    dl = DeviceLayer(gpu, m, device_only=True)
+    gpu.profile(True)
+    out, lg, selraw, _ = run_moe(gpu, path, dl, x, nb)
+    names = [n for n, _ in gpu.profile_entries()]
+    gpu.profile(False)
+    assert "qwk_qmvm" in names and "qwk_sh_act" in names, names
+    gnb = 8 if nb <= 8 else 16
+    ref = oracle.moe_layer_f64(m, lg, x)
+    assert np.isfinite(out.astype(np.float64)).all()
+    assert maxrel(out, ref) <= TOL, maxrel(out, ref)
+    _, H32, _ = oracle.moe_layer_f32(m, lg, x, gnb)
+    nbv = 1 if nb <= 1 else 2 if nb <= 2 else 4 if nb <= 4 else 8 if nb <= 8 else 16
+    Hraw = path.scratch(1).view(np.float16)
+    plane = nbv * (K + 1) * I
+    H = (Hraw[:nb * (K + 1) * I].astype(np.float32) + Hraw[plane:plane + nb * (K + 1) * I].astype(np.float32)).reshape(nb, K + 1, I)
+    assert maxrel(H[:, K], H32[:, K]) <= 1e-5
+    dl.free()
+    path.close()
+
+
 @pytest.mark.parametrize("nb,limit", [(1, 2), (2, 2), (3, 4), (4, 4)])
 @pytest.mark.parametrize("fd,fshd,dev", [(21, 21, True), (21, 8, True), (8, 8, False), (8, 8, True)])
 def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev):
