@@ -39,6 +39,42 @@ def timed_steps(stack, x, nb, steps, warmup):
     return time.perf_counter() - t0, gpu_s
 
 
+def model_shape_leg(gpu, layers, steps, warmup):
+    """The same decode step on the reference model's own layer (src/model.h:10-18 and bench/moe_bw.c:16-24 of the
+    reference): D = 2560, I = 640, 512 experts, top-10; routed gate/up IQ3_S, routed down IQ4_NL, shared expert Q4_K
+    gate, IQ4_XS up, IQ4_NL down. Tokens/s, GPU time and algorithmic GB/s per batch size, mean launch times at B = 16,
+    and the layer-0 output at B = 16 against the CPU oracle."""
+    from qwental_amd import synth
+    from qwental_amd.stack import MoeStack
+    from oracle import oracle as o
+    stack = MoeStack(gpu, layers=layers, D=2560, I=640, nbmax=16, model_formats=(20, 12, 23, 20))
+    xh = synth.activations(np.random.default_rng(2025), 16, stack.D)
+    x = gpu.buf_from(xh, device_only=True)
+    res = {"workload": "%d-layer MoE FFN stack decode, D=2560 I=640 E=512 top-10; IQ3_S gate/up, IQ4_NL down; shared Q4_K / IQ4_XS / IQ4_NL" % layers,
+           "resident_weight_bytes": int(stack.weight_bytes), "by_batch": {}}
+    for nb in (1, 8, 16):
+        wall, gpu_s = timed_steps(stack, x, nb, steps, warmup)
+        U = stack.unique_experts(nb)
+        byts = stack.algorithmic_bytes(nb, U)
+        res["by_batch"][str(nb)] = {"tokens_per_s": nb * steps / wall, "gpu_ms_per_step": gpu_s / steps * 1e3, "stack_GBps": sum(byts) / (gpu_s / steps) / 1e9, "mean_U": float(np.mean(U))}
+    gpu.profile(True)
+    stack.step(x, 16)
+    gpu.profile(False)
+    per = {}
+    for name, us in gpu.profile_entries():
+        per.setdefault(name, []).append(us)
+    res["kernel_us_mean"] = {k: float(np.mean(v)) for k, v in per.items()}
+    # one 16-token step of the first layer alone: `out` is the last layer's otherwise
+    stack.step(x, 16, nlayers=1)
+    lg = stack.lg[0].read(dtype=np.float32)[:16 * (stack.E + 1)].reshape(16, stack.E + 1).copy()
+    got = stack.out.view(np.float16)[:16 * stack.D].reshape(16, stack.D).astype(np.float64)
+    ref = o.moe_layer_f64(stack.layer_weights_host(0), lg, xh)
+    res["layer0_max_rel_err"] = float(np.abs(got - ref).max() / np.abs(ref).max())
+    x.free()
+    stack.free()
+    return res
+
+
 def committed_traffic():
     """HBM bytes per launch of the dominant kernel as the committed counter summary states them (two rocprofv3
     --pmc runs of this file with --copy-calib, FETCH_SIZE and WRITE_SIZE, scaled by the copy kernel); None without it."""
@@ -356,6 +392,7 @@ def main():
     ap.add_argument("--traffic", type=float, default=None, help="HBM bytes per launch of the dominant kernel from the counter runs, to report")
     ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
     ap.add_argument("--gguf-only", action="store_true", help="only the GGUF load measurement")
+    ap.add_argument("--model-shape-only", action="store_true", help="only the stack of the reference model's layer shape and formats")
     ap.add_argument("--ragged-only", action="store_true", help="only the continuous-batching step table (config 4) on a one-layer stack: for profiling runs")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -371,6 +408,9 @@ def main():
         return 0
     if a.gguf_only:
         print(json.dumps({"gguf_load": gguf_load(gpu)}))
+        return 0
+    if a.model_shape_only:
+        print(json.dumps({"model_shape": model_shape_leg(gpu, a.layers, a.steps, a.warmup)}))
         return 0
     if a.ragged_only:
         stack = MoeStack(gpu, layers=1, nbmax=16)

@@ -1185,9 +1185,14 @@ static bool tr_dn(qw_batch *b) {
     }
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
-    if (fd == 20 || fs == 20) { // IQ4_NL rows run in the any-shape kernel; the shared expert's may be IQ4_NL or Q8_0 beside them
-        if (fd != 20 || (fs != 0 && fs != 20 && fs != 8)) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
-    } else if (p->I <= 512 && p->I % 256 == 0) { // contiguous task ranges per workgroup, operand A staged in LDS
+    // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
+    if ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8))) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
+    if (fd == 20 && p->I <= 640 && !getenv("QW_HIP_DN_ANY")) { // the range kernel with rows of up to 640 staged
+        if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c4_s%d_c4", fs);
+        else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c4");
+        return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
+    }
+    if (fd != 20 && p->I <= 512 && p->I % 256 == 0) { // contiguous task ranges per workgroup, operand A staged in LDS
         const int ch = fd == 8 ? 4 : p->I / 256;
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
@@ -1368,7 +1373,7 @@ static bool tr_mem(qw_batch *b, unsigned gx) {
 static bool tr_fill_blocks(qw_batch *b) {
     struct { uint64_t nblocks, seed; uint32_t type; float sigma; } in;
     if (!bind_bytes(b, 2, &in, sizeof in, "{nblocks, seed, type, sigma}")) return false;
-    if (!fmt_ok((int)in.type)) return fail(b, "qw_fill_blocks: type %u", in.type);
+    if (!fmt_ok((int)in.type) && in.type != 20) return fail(b, "qw_fill_blocks: type %u", in.type);
     qwk_fill_args a = {.nblocks = in.nblocks, .seed = in.seed, .type = in.type, .sigma = in.sigma};
     if (!bind_ptr(b, 1, (size_t)in.nblocks * (size_t)fmt_bb((int)in.type), true, "dst", (void **)&a.dst)) return false;
     if (b->buf[1].off % 2) return fail(b, "qw_fill_blocks: odd offset");

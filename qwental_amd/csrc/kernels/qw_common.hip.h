@@ -185,6 +185,9 @@ struct qw_afrag_lds2 {
     static constexpr bool has_lo = true;
     __device__ __forceinline__ h8 hi(uint32_t koff) const { return __builtin_bit_cast(h8, hi_[(koff >> 3) * 16 + m]); }
     __device__ __forceinline__ h8 lo(uint32_t koff) const { return __builtin_bit_cast(h8, lo_[(koff >> 3) * 16 + m]); }
+    // four values (koff a multiple of 4): one half of a 16-byte unit
+    __device__ __forceinline__ h4 hi4(uint32_t koff) const { return __builtin_bit_cast(h4, ((const u2 *)hi_)[((koff >> 3) * 16 + m) * 2 + ((koff >> 2) & 1)]); }
+    __device__ __forceinline__ h4 lo4(uint32_t koff) const { return __builtin_bit_cast(h4, ((const u2 *)lo_)[((koff >> 3) * 16 + m) * 2 + ((koff >> 2) & 1)]); }
 };
 
 // Every workgroup of a launch copies the same bytes: each starts at a different place (a rotation by its index), so

@@ -1035,6 +1035,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     auto div_tpe = [&](uint32_t x) { return tp2 ? x >> tsh : x / tpe; };
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
     if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // lands in LDS meanwhile; awaited in ready()
+    if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook instead
     __syncthreads();
     const uint32_t *ue = sc->ue, *mask = sc->mask;
     const uint8_t *slot = sc->slot;
@@ -1085,8 +1086,9 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
             const uint32_t lane = qw_lane(), t = lane & 15, rows = g0.mask | (both ? g1.mask << 16 : 0), nrows = (uint32_t)__builtin_popcount(rows);
             if (nrows * 2 * upr <= blockDim.x) {
                 // few rows (a token or two per expert): one 16-byte unit per thread through a register, the waves
-                // of a row finding its bit in the mask by a scalar walk
-                const uint32_t i = threadIdx.x, k = (uint32_t)__builtin_amdgcn_readfirstlane((int)(i / (2 * upr))), r = i % (2 * upr), pl = r / upr, c = r % upr;
+                // of a row finding its bit in the mask by a (mostly scalar) walk
+                // (a row of both planes is 2 upr threads: whole waves when I is a multiple of 256, else a wave may span two rows)
+                const uint32_t i = threadIdx.x, kl = i / (2 * upr), k = (2 * upr) % 64 == 0 ? (uint32_t)__builtin_amdgcn_readfirstlane((int)kl) : kl, r = i % (2 * upr), pl = r / upr, c = r % upr;
                 if (k < nrows) {
                     uint32_t m = rows;
                     for (uint32_t j = 0; j < k; j++) m &= m - 1;
@@ -1123,6 +1125,14 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; uint16_t arows[2 * 16 * 2 * 512]; qw_sel_cache sc; } L; \
         dn_range_body<F, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
     }
+// IQ4_NL rows (the reference model's down projections: I = 640, five chunks of 4 blocks a row): no IQ3_S table in LDS,
+// so the staged H rows may be 640 wide
+#define QW_DN_RANGE_NL(FSD, CHSD, NAME)                                                           \
+    extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
+        __shared__ struct { u2 lut[QW_KQ_TAB / 2]; uint16_t arows[2 * 16 * 2 * 640]; qw_sel_cache sc; } L; \
+        dn_range_body<20, 4, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
+    }
+QW_DN_RANGE_NL(0, 1, qwk_dnr_f20_c4) QW_DN_RANGE_NL(20, 4, qwk_dnr_f20_c4_s20_c4) QW_DN_RANGE_NL(8, 4, qwk_dnr_f20_c4_s8_c4)
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
 QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
 QW_DN_RANGE(21, 1, 0, 1, qwk_dnr_f21_c1) QW_DN_RANGE(21, 1, 21, 1, qwk_dnr_f21_c1_s21_c1) QW_DN_RANGE(21, 1, 8, 4, qwk_dnr_f21_c1_s8_c4)
@@ -1529,10 +1539,10 @@ extern "C" __global__ __launch_bounds__(256) void qwk_fill_random(qwk_mem_args a
 }
 
 // Synthetic GGUF blocks, one thread per block: d = binary16(|N(0, sigma)|) by Box-Muller over two hashed uniforms,
-// every other byte uniform (IQ3_S), or int8 uniform in [-127, 127] (Q8_0). Blocks are 2-byte aligned: 16-bit stores.
+// every other byte uniform (IQ3_S, IQ4_NL), or int8 uniform in [-127, 127] (Q8_0). Blocks are 2-byte aligned: 16-bit stores.
 extern "C" __global__ __launch_bounds__(256) void qwk_fill_blocks(qwk_fill_args a) {
     const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
-    const uint32_t bb = a.type == 21 ? 110 : 34;
+    const uint32_t bb = a.type == 21 ? 110 : a.type == 20 ? 18 : 34; // IQ4_NL: d and sixteen uniform bytes
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.nblocks; i += step) {
         uint16_t *p = (uint16_t *)(a.dst + i * bb);
         const uint64_t c = a.seed + i * 64;

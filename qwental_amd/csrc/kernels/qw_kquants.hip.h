@@ -352,6 +352,7 @@ template <int NB> struct qw_chunk<20, NB> {
             acc += qw_h2f(d[b]) * sub;
         }
     }
+    template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {

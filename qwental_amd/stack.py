@@ -28,32 +28,44 @@ def fill_blocks(gpu, batch, buf, offset, nblocks, ftype, seed, sigma):
 
 
 class MoeStack:
-    def __init__(self, gpu, layers=48, D=2048, I=512, E=512, topk=10, nbmax=16, q8_every=4, seed=1234, d_scale=synth.MOE_D_SCALE):
+    """model_formats: None for the benchmark's layer (IQ3_S throughout, Q8_0 shared expert every q8_every-th layer), or
+    (routed down, shared gate, shared up, shared down) ggml types for a layer of other formats — (20, 12, 23, 20) with
+    D = 2560, I = 640 is the reference model's layer (src/model.h:10-18, bench/moe_bw.c:16-24). The routed rows are
+    generated on the device, a shared expert of other formats on the host."""
+
+    def __init__(self, gpu, layers=48, D=2048, I=512, E=512, topk=10, nbmax=16, q8_every=4, seed=1234, d_scale=synth.MOE_D_SCALE, model_formats=None):
         self.gpu, self.L, self.D, self.I, self.E, self.topk, self.nbmax = gpu, layers, D, I, E, topk, nbmax
         self.path = Path(gpu, D, I, E, topk, nbmax, device_scratch=True)
         rng = np.random.default_rng(seed)
-        rb_gu, rb_d = synth.row_bytes(21, D), synth.row_bytes(21, I)
-        self.exp_bytes = 2 * I * rb_gu + D * rb_d           # one IQ3_S expert
+        self.fd = fd = model_formats[0] if model_formats else 21
+        rb_gu, rb_d = synth.row_bytes(21, D), synth.row_bytes(fd, I)
+        self.exp_bytes = 2 * I * rb_gu + D * rb_d           # one routed expert
         self.gu_bytes = 2 * I * rb_gu
         self.layers, self.bufs, self.shared_fmt = [], [], []
         self.router_bytes = (E + 1) * D * 2
+        sigma = lambda f: (synth.D_SIGMA[f] if f in synth.D_SIGMA else synth.SCALE_FIELDS[f][1]) * d_scale
         b = gpu.batch()
         for l in range(layers):
             fsh = 8 if q8_every and l % q8_every == q8_every - 1 else 21
-            sz_e = E * I * rb_gu                              # gate, up and down each: E * I * rb(D) == E * D * rb(I)
-            assert sz_e == E * D * rb_d
-            sh_gu, sh_d = I * synth.row_bytes(fsh, D), D * synth.row_bytes(fsh, I)
-            w = gpu.buf(3 * sz_e, device_only=True)
-            sh = gpu.buf(2 * sh_gu + sh_d, device_only=True)
-            fill_blocks(gpu, b, w, 0, 3 * sz_e // 110, 21, seed * 1000003 + l * 7919, synth.D_SIGMA[21] * d_scale)
-            fill_blocks(gpu, b, sh, 0, (2 * sh_gu + sh_d) // synth.BLOCK[fsh][1], fsh, seed * 1000003 + l * 7919 + 1, synth.D_SIGMA[fsh] * d_scale)
+            fs3 = tuple(model_formats[1:]) if model_formats else (fsh, fsh, fsh)
+            sz_gu, sz_d = E * I * rb_gu, E * D * rb_d         # gate and up each; down
+            sh_g, sh_u, sh_d = I * synth.row_bytes(fs3[0], D), I * synth.row_bytes(fs3[1], D), D * synth.row_bytes(fs3[2], I)
+            w = gpu.buf(2 * sz_gu + sz_d, device_only=True)
+            fill_blocks(gpu, b, w, 0, 2 * sz_gu // 110, 21, seed * 1000003 + l * 7919, sigma(21))
+            fill_blocks(gpu, b, w, 2 * sz_gu, sz_d // synth.BLOCK[fd][1], fd, seed * 1000003 + l * 7919 + 2, sigma(fd))
+            if model_formats:
+                hr = np.random.default_rng(seed * 31 + l)
+                sh = gpu.buf_from(np.concatenate([synth.matrix(hr, fs3[0], I, D, d_scale), synth.matrix(hr, fs3[1], I, D, d_scale), synth.matrix(hr, fs3[2], D, I, d_scale)]), device_only=True)
+            else:
+                sh = gpu.buf(sh_g + sh_u + sh_d, device_only=True)
+                fill_blocks(gpu, b, sh, 0, (sh_g + sh_u + sh_d) // synth.BLOCK[fsh][1], fsh, seed * 1000003 + l * 7919 + 1, sigma(fsh))
             Wr, wsg = synth.router(rng, E, D)
             r = gpu.buf_from(np.concatenate([Wr.ravel(), wsg]).view(np.uint16), device_only=True)
             T = Tensor
-            self.layers.append(MoeLayer(router=T(r, 1), sh_gate_w=T(r, 1, E * D * 2), gate=T(w, 21), up=T(w, 21, sz_e), down=T(w, 21, 2 * sz_e),
-                                        sh_gate=T(sh, fsh), sh_up=T(sh, fsh, sh_gu), sh_down=T(sh, fsh, 2 * sh_gu)))
+            self.layers.append(MoeLayer(router=T(r, 1), sh_gate_w=T(r, 1, E * D * 2), gate=T(w, 21), up=T(w, 21, sz_gu), down=T(w, fd, 2 * sz_gu),
+                                        sh_gate=T(sh, fs3[0]), sh_up=T(sh, fs3[1], sh_g), sh_down=T(sh, fs3[2], sh_g + sh_u)))
             self.bufs += [w, sh, r]
-            self.shared_fmt.append(fsh)
+            self.shared_fmt.append(fs3)
         b.end()
         self.layers_c = (QwMoeLayer * layers)(*[m.c for m in self.layers])
         self.lg = [gpu.buf(self.path.logits_bytes(nbmax), device_only=True) for _ in range(layers)]
@@ -66,7 +78,7 @@ class MoeStack:
 
     def shared_bytes(self, l):
         f = self.shared_fmt[l]
-        return 2 * self.I * synth.row_bytes(f, self.D) + self.D * synth.row_bytes(f, self.I)
+        return self.I * (synth.row_bytes(f[0], self.D) + synth.row_bytes(f[1], self.D)) + self.D * synth.row_bytes(f[2], self.I)
 
     def step(self, x, nb, nlayers=None):
         """One decode step over the stack; returns GPU seconds (events around the kernels)."""
@@ -89,10 +101,10 @@ class MoeStack:
         E, I, D = self.E, self.I, self.D
         sz_e = E * I * synth.row_bytes(21, D)
         f = self.shared_fmt[l]
-        sh_gu = I * synth.row_bytes(f, D)
+        sh_g, sh_u = I * synth.row_bytes(f[0], D), I * synth.row_bytes(f[1], D)
         wb, sb, rb = w.read(), sh.read(), r.read(dtype=np.uint16)
-        return dict(D=D, I=I, E=E, topk=self.topk, fgu=21, fd=21, fsg=f, fsu=f, fsd=f, Wg=wb[:sz_e], Wu=wb[sz_e:2 * sz_e], Wd=wb[2 * sz_e:],
-                    Wsg=sb[:sh_gu], Wsu=sb[sh_gu:2 * sh_gu], Wsd=sb[2 * sh_gu:], Wr=rb[:E * D].view(np.float16).reshape(E, D), wsg=rb[E * D:].view(np.float16))
+        return dict(D=D, I=I, E=E, topk=self.topk, fgu=21, fd=self.fd, fsg=f[0], fsu=f[1], fsd=f[2], Wg=wb[:sz_e], Wu=wb[sz_e:2 * sz_e], Wd=wb[2 * sz_e:],
+                    Wsg=sb[:sh_g], Wsu=sb[sh_g:sh_g + sh_u], Wsd=sb[sh_g + sh_u:], Wr=rb[:E * D].view(np.float16).reshape(E, D), wsg=rb[E * D:].view(np.float16))
 
     def free(self):
         for b in self.bufs:

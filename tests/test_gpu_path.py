@@ -319,6 +319,36 @@ def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
     path.close()
 
 
+def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
+    """IQ4_NL down rows normally take the range kernel (rows of up to 640 staged in LDS); wider rows, or
+    QW_HIP_DN_ANY in the environment, take the any-shape kernel. Both against the float64 layer."""
+    D, I, E, K, nb = 1024, 640, 32, 10, 6
+    rng = np.random.default_rng(2020)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=20, fsh=8, fshd=20)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    dl = DeviceLayer(gpu, m)
+    old = os.environ.get("QW_HIP_DN_ANY")
+    try:
+        for env, want in ((None, "qwk_dnr_f20_c4_s20_c4"), ("1", "qwk_dn_f20_any_s20")):
+            os.environ.pop("QW_HIP_DN_ANY", None)
+            if env:
+                os.environ["QW_HIP_DN_ANY"] = env
+            path = q.Path(gpu, D, I, E, K, 16)
+            gpu.profile(True)
+            out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            assert want in names, names
+            assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+            path.close()
+    finally:
+        os.environ.pop("QW_HIP_DN_ANY", None)
+        if old is not None:
+            os.environ["QW_HIP_DN_ANY"] = old
+    dl.free()
+
+
 def test_moe_batched_equals_single(gpu):
     """Each row of a batched layer call equals the single-token call bit for bit (src/engine.c:7977-7987)."""
     D, I, E, K, nb = 2048, 512, 64, 10, 8
