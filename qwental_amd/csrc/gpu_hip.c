@@ -1188,8 +1188,9 @@ static bool tr_dn(qw_batch *b) {
     // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
     if ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8))) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
     if (fd == 20 && p->I <= 640 && !getenv("QW_HIP_DN_ANY")) { // the range kernel with rows of up to 640 staged
-        if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c4_s%d_c4", fs);
-        else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c4");
+        const int ch = p->I % 320 == 0 && !getenv("QW_HIP_NL_C4") ? 10 : 4; // blocks per chunk
+        if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d_s%d_c%d", ch, fs, fs == 20 ? ch : 4);
+        else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d", ch);
         return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
     }
     if (fd != 20 && p->I <= 512 && p->I % 256 == 0) { // contiguous task ranges per workgroup, operand A staged in LDS

@@ -1127,12 +1127,14 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     }
 // IQ4_NL rows (the reference model's down projections: I = 640, five chunks of 4 blocks a row): no IQ3_S table in LDS,
 // so the staged H rows may be 640 wide
-#define QW_DN_RANGE_NL(FSD, CHSD, NAME)                                                           \
+#define QW_DN_RANGE_NL(CH, FSD, CHSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
         __shared__ struct { u2 lut[QW_KQ_TAB / 2]; uint16_t arows[2 * 16 * 2 * 640]; qw_sel_cache sc; } L; \
-        dn_range_body<20, 4, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                                \
+        dn_range_body<20, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                               \
     }
-QW_DN_RANGE_NL(0, 1, qwk_dnr_f20_c4) QW_DN_RANGE_NL(20, 4, qwk_dnr_f20_c4_s20_c4) QW_DN_RANGE_NL(8, 4, qwk_dnr_f20_c4_s8_c4)
+QW_DN_RANGE_NL(4, 0, 1, qwk_dnr_f20_c4) QW_DN_RANGE_NL(4, 20, 4, qwk_dnr_f20_c4_s20_c4) QW_DN_RANGE_NL(4, 8, 4, qwk_dnr_f20_c4_s8_c4)
+// rows of 320 or 640: chunks of ten blocks (a row of 640 in two), 5760 bytes a tile in flight per wave
+QW_DN_RANGE_NL(10, 0, 1, qwk_dnr_f20_c10) QW_DN_RANGE_NL(10, 20, 10, qwk_dnr_f20_c10_s20_c10) QW_DN_RANGE_NL(10, 8, 4, qwk_dnr_f20_c10_s8_c4)
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
 QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
 QW_DN_RANGE(21, 1, 0, 1, qwk_dnr_f21_c1) QW_DN_RANGE(21, 1, 21, 1, qwk_dnr_f21_c1_s21_c1) QW_DN_RANGE(21, 1, 8, 4, qwk_dnr_f21_c1_s8_c4)

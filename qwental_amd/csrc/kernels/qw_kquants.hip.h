@@ -322,7 +322,7 @@ template <int F, int S = 0> __device__ __forceinline__ void qw_kq_values(const q
 // of qw_kq_tab_build. Operand A of a block: x[4 kg .. + 4] and x[16 + 4 kg .. + 4], the values the lane's four bytes hold.
 template <int NB> struct qw_chunk<20, NB> {
     static constexpr uint32_t BLK_K = 32, BLK_B = 18;
-    static constexpr int DEPTH = 2;
+    static constexpr int DEPTH = 3; // blocks are small: two chunks ahead keep enough bytes in flight
     uint32_t q[NB];
     uint16_t d[NB];
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t kl) {

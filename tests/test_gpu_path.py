@@ -330,7 +330,7 @@ def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
     dl = DeviceLayer(gpu, m)
     old = os.environ.get("QW_HIP_DN_ANY")
     try:
-        for env, want in ((None, "qwk_dnr_f20_c4_s20_c4"), ("1", "qwk_dn_f20_any_s20")):
+        for env, want in ((None, "qwk_dnr_f20_c10_s20_c10"), ("1", "qwk_dn_f20_any_s20")):
             os.environ.pop("QW_HIP_DN_ANY", None)
             if env:
                 os.environ["QW_HIP_DN_ANY"] = env
