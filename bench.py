@@ -52,6 +52,8 @@ def model_shape_leg(gpu, layers, steps, warmup):
     x = gpu.buf_from(xh, device_only=True)
     res = {"workload": "%d-layer MoE FFN stack decode, D=2560 I=640 E=512 top-10; IQ3_S gate/up, IQ4_NL down; shared Q4_K / IQ4_XS / IQ4_NL" % layers,
            "resident_weight_bytes": int(stack.weight_bytes), "by_batch": {}}
+    for _ in range(30):  # the legs before this one may have left the device idle for seconds: bring the clocks back up
+        stack.step(x, 16)
     for nb in (1, 8, 16):
         wall, gpu_s = timed_steps(stack, x, nb, steps, warmup)
         U = stack.unique_experts(nb)
@@ -469,8 +471,11 @@ def main():
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)
-    print(json.dumps(line))
+    x.free()
     stack.free()
+    if not a.quick:
+        line["model_shape"] = model_shape_leg(gpu, a.layers, min(a.steps, 10), a.warmup)
+    print(json.dumps(line))
     gpu.close()
     return 0
 

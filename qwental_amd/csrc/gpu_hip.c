@@ -80,6 +80,8 @@ typedef struct {
     size_t argsz;
     const char *kname; // caller-visible kernel name (for profiling)
     bool last_of_dispatch;
+    bool side; // independent of the launches before it in the batch: runs on the side stream, beside them
+    bool join; // needs the side stream's results: the main stream waits for them first
 } qw_launch;
 
 typedef struct { qw_hbuf *b; bool out; } qw_use;
@@ -139,6 +141,9 @@ struct qw_gpu {
     int npacks, cappacks;
     struct qw_ldlane { void *pin[2]; hipStream_t st; hipEvent_t ev[2]; } ld[QW_LD_MAX]; // staging of qw_hip_buf_write_fd, made at first use
     int nld;
+    hipStream_t side[2]; // one beside each stream: launches of a batch that do not depend on the ones before them (made at first use)
+    hipEvent_t sev[256];  // fork / join events between a stream and its side stream, used round robin (made at first use)
+    unsigned nsev;
     float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes;
@@ -215,6 +220,10 @@ void qw_gpu_close(qw_gpu *g) {
     if (!g) return;
     (void)hipDeviceSynchronize();
     for (int i = 0; i < 2; i++) (void)hipStreamDestroy(g->stream[i]);
+    for (int i = 0; i < 2; i++)
+        if (g->side[i]) (void)hipStreamDestroy(g->side[i]);
+    for (int i = 0; i < 256; i++)
+        if (g->sev[i]) (void)hipEventDestroy(g->sev[i]);
     for (int i = 0; i < g->nld; i++) {
         for (int k = 0; k < 2; k++) {
             if (g->ld[i].ev[k]) (void)hipEventDestroy(g->ld[i].ev[k]);
@@ -761,6 +770,7 @@ static bool add_launch(qw_batch *b, const char *fname, unsigned gx, unsigned bx,
     memcpy(l->args, args, argsz);
     l->argsz = argsz;
     l->kname = b->k->name;
+    l->join = !strncmp(fname, "qwk_dn", 6); // the down launches read H of the shared expert, which a side launch may write
     return true;
 }
 
@@ -1022,7 +1032,16 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
                        .rowbytes = {(uint32_t)fmt_rb(p->fsg, p->D), (uint32_t)fmt_rb(p->fsu, p->D)}, .ystride = {(uint32_t)p->I, (uint32_t)p->I}};
     qwk_shact_args sa = {.g = gy, .u = uy, .H = h, .I = (uint32_t)p->I, .nb = nbr, .topk = (uint32_t)p->topk, .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
     b->pend_sg.valid = false; // done here
-    return launch_qmvm(b, &m) && add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa);
+    // These two depend on x alone. With one or two tokens, where the layer is a chain of short launches, they run
+    // beside the router and the routed gate/up on the side stream (48 layers of the reference model's shape: 2.89 ->
+    // 2.70 ms a token); with more tokens the fork and join cost more than the overlap gives (6.81 -> 6.93 ms at 16).
+    // QW_HIP_SIDE in the environment: 0 never, 1 always.
+    const int first = b->nl;
+    if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
+    const char *e = getenv("QW_HIP_SIDE");
+    if (e ? e[0] == '1' : nbr <= 2)
+        for (int i = first; i < b->nl; i++) b->l[i].side = true;
+    return true;
 }
 
 // src/engine.c:588-607: 0 Wr, 1 shared gate vector, 2 x, 3 logits, 4 counter, 5 sel, 6/7 shared gate/up, 8 H, 13 tables, 14 nbr.
@@ -1072,8 +1091,8 @@ static bool tr_pre(qw_batch *b) {
         }
     }
     // the counter buffer of the reference's hand-over (index 4) is not used
+    if (kq_ok(p->fsg) && !shared_gu_kq(b, nbr, a.r.x, h)) return false; // first: side launches fork where they stand in the batch
     if (!add_launch(b, intern(fn), grid, 512, &a, sizeof a)) return false;
-    if (kq_ok(p->fsg) && !shared_gu_kq(b, nbr, a.r.x, h)) return false;
     if (!fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
     b->pend_sel.valid = true; // made by the gate/up launch if one follows for the same record, else by its own launch
     return true;
@@ -1417,6 +1436,19 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
 }
 
 // ---------------------------------------------------------------- batches: submission
+// The side stream of a stream (default priority, made at first use), and an ordering edge "to goes on after what from
+// holds now" through an event of the pool.
+static hipStream_t side_of(qw_gpu *g, int stream) {
+    if (!g->side[stream] && hipStreamCreateWithFlags(&g->side[stream], hipStreamNonBlocking) != hipSuccess) g->side[stream] = NULL;
+    return g->side[stream];
+}
+static bool side_link(qw_gpu *g, hipStream_t from, hipStream_t to) {
+    if (!from || !to) { set_err(g, "no side stream"); return false; }
+    hipEvent_t *e = &g->sev[g->nsev++ % 256];
+    if (!*e && !HIPOK(g, hipEventCreateWithFlags(e, hipEventDisableTiming))) return false;
+    return HIPOK(g, hipEventRecord(*e, from)) && HIPOK(g, hipStreamWaitEvent(to, *e, 0));
+}
+
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
@@ -1438,8 +1470,19 @@ static bool submit_segment(qw_batch *b) {
     if (!HIPOK(g, hipEventCreate(&ev[0])) || !HIPOK(g, hipEventCreate(&ev[1]))) { b->failed = true; return false; }
     b->nseg++;
     if (!HIPOK(g, hipEventRecord(ev[0], st))) { b->failed = true; return false; }
+    bool side_open = false;
     for (int i = b->done_l; i < b->nl; i++) {
         qw_launch *l = &b->l[i];
+        if (l->side && !b->prof) { // fork: the side stream starts from where the main stream stands now
+            if (!side_open && !(side_open = side_link(g, st, side_of(g, b->stream)))) { b->failed = true; return false; }
+            void *sparams[] = {l->args};
+            if (!HIPOK(g, hipModuleLaunchKernel(l->f, l->gx, l->gy, l->gz, l->bx, 1, 1, 0, g->side[b->stream], sparams, NULL))) { b->failed = true; return false; }
+            continue;
+        }
+        if (l->join && side_open) { // join: the main stream goes on once the side stream has finished
+            side_open = false;
+            if (!side_link(g, g->side[b->stream], st)) { b->failed = true; return false; }
+        }
         if (b->prof) { // an event pair brackets every launch
             b->pev = realloc(b->pev, sizeof *b->pev * (size_t)(b->npev + 2));
             if (!HIPOK(g, hipEventCreate(&b->pev[b->npev])) || !HIPOK(g, hipEventCreate(&b->pev[b->npev + 1])) || !HIPOK(g, hipEventRecord(b->pev[b->npev], st))) { b->failed = true; return false; }
@@ -1451,6 +1494,7 @@ static bool submit_segment(qw_batch *b) {
             b->npev += 2;
         }
     }
+    if (side_open && !side_link(g, g->side[b->stream], st)) { b->failed = true; return false; }
     if (!HIPOK(g, hipEventRecord(ev[1], st))) { b->failed = true; return false; }
     b->done_l = b->nl;
     b->done_use = b->nuse;

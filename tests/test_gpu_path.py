@@ -401,6 +401,30 @@ def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd
     plane = nbv * (K + 1) * I
     H = (Hraw[:nb * (K + 1) * I].astype(np.float32) + Hraw[plane:plane + nb * (K + 1) * I].astype(np.float32)).reshape(nb, K + 1, I)
     assert maxrel(H[:, K], H32[:, K]) <= 1e-5
+    # unprofiled, the two shared launches run on a side stream beside the router and the routed gate/up: three layers
+    # in one batch (three forks and joins), twice, against the same launches kept in line
+    def three(side):
+        old = os.environ.pop("QW_HIP_SIDE", None)
+        os.environ["QW_HIP_SIDE"] = "1" if side else "0"  # by default the side stream is taken with one or two tokens only
+        try:
+            xb = gpu.buf_from(x)
+            lgs, sels, outs = [gpu.buf(path.logits_bytes(nb)) for _ in range(3)], [gpu.buf(path.sel_bytes(nb)) for _ in range(3)], [gpu.buf(nb * D * 2) for _ in range(3)]
+            b = gpu.batch()
+            for i in range(3):
+                path.gg_moe(b, dl.layer, nb, xb, lgs[i], sels[i], outs[i])
+            assert b.end() >= 0, gpu.last_error()
+            res = [o_.view(np.uint16)[:nb * D].copy() for o_ in outs]
+            for bb in [xb] + lgs + sels + outs:
+                bb.free()
+            return res
+        finally:
+            os.environ.pop("QW_HIP_SIDE", None)
+            if old is not None:
+                os.environ["QW_HIP_SIDE"] = old
+    inline = three(False)
+    assert all(np.array_equal(r, out.view(np.uint16).ravel()) for r in inline)
+    for _ in range(2):
+        assert all(np.array_equal(r, inline[0]) for r in three(True))
     dl.free()
     path.close()
 
