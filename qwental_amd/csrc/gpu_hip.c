@@ -822,6 +822,13 @@ static int chunk_of(int F, int K) { return K % 512 == 0 ? (F == 21 ? 2 : 16) : 1
 
 static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf *hb, const void *B, uint64_t ntiles, uint32_t nblk, uint32_t rowbytes, uint32_t split);
 // One launch of the multi-format matvec over nmat matrices; W / y already bound into a.
+// Few tiles: the parts a tile's K range is cut into, one wave each — the largest divisor of the chunk count up to 6
+// that the wave slots of the device hold (a workgroup's waves beyond a whole number of tiles stay idle).
+static unsigned pick_split(unsigned chunks, unsigned tiles, unsigned slots) {
+    for (unsigned s = 6; s > 1; s--)
+        if (chunks % s == 0 && tiles * s <= slots) return s;
+    return 1;
+}
 static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a) {
     unsigned tiles = 0;
     a->sums = 0;
@@ -833,9 +840,7 @@ static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a) {
     if (!tiles) return true;
     // few tiles: cut every tile's K range over several waves, as far as the wave slots of the device and K allow
     const unsigned waves = QW_WAVES_GU, slots = (unsigned)b->g->ncu * waves;
-    a->split = 1;
-    if (a->K % 256 == 0)
-        while (a->split < 4 && tiles * a->split * 2 <= slots && (a->K / 256) % (a->split * 2) == 0) a->split *= 2;
+    a->split = a->K % 256 == 0 ? pick_split(a->K / 256, tiles, slots) : 1;
     if (a->split > 1) {
         unsigned groups = 0;
         for (uint32_t j = 0; j < a->nmat; j++) groups += cdiv(a->ntiles[j], waves / a->split);
@@ -904,10 +909,9 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
         const int base = 21 == F || F == QW_F_PACKED ? 21 : F, ch = p->K > 2560 ? 1 : chunk_of(base, p->K);
         if (p->K > 2560) fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c1g", F);
         else fname_fmt(fn, sizeof fn, "qwk_qmv_f%d_c%d", F, ch);
-        // few tiles: cut every tile's chunks over 2 or 4 waves, as far as the wave slots of the device allow
+        // few tiles: cut every tile's chunks over several waves, as far as the wave slots of the device allow
         const unsigned cpr = (unsigned)p->K / ((unsigned)fmt_qb(base) * (unsigned)ch), slots = (unsigned)b->g->ncu * QW_WAVES_GU;
-        a.split = 1;
-        while (a.split < 4 && a.ntiles * a.split * 2 <= slots && cpr % (a.split * 2) == 0) a.split *= 2;
+        a.split = pick_split(cpr, a.ntiles, slots);
         if (a.split > 1) return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, cdiv(a.ntiles, QW_WAVES_GU / a.split)), 64 * QW_WAVES_GU, &a, sizeof a);
     }
     a.split = 1;

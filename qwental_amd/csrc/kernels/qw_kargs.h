@@ -32,7 +32,7 @@ typedef struct { /* dense matvec, y[b][row] = W[row] . x[b] */
     void *y;           /* binary16 or float [nb][ystride] */
     uint32_t N, K, rowbytes, xstride, ystride, nb, yfloat, ntiles;
     const void *glut; /* the backend's pre-signed IQ3_S table in global memory (64 KB) */
-    uint32_t split, pad; /* waves a tile's chunks are cut over (1, 2, 4; the chunk count of a row is a multiple of it) */
+    uint32_t split, pad; /* waves a tile's chunks are cut over (1 .. 6; the chunk count of a row is a multiple of it) */
 } qwk_qmv_args;
 
 /* Dense matvec over up to four matrices that share the activations (kernels/qmv_ggm.metal:232-262; one matrix:
@@ -44,7 +44,7 @@ typedef struct {
     const uint16_t *x; /* binary16 [nb][xstride] */
     uint32_t N[4], fmt[4], rowbytes[4], ystride[4], ntiles[4];
     uint32_t K, xstride, nb, yfloat, nmat, sums; /* sums: some matrix is Q4_K / Q5_K (needs the 32-value sums of x) */
-    uint32_t split, pad;                         /* waves a tile's K range is cut over (1, 2, 4; > 1 needs K % (256 * split) == 0) */
+    uint32_t split, pad;                         /* waves a tile's K range is cut over (1 .. 6; > 1 needs K % (256 * split) == 0) */
 } qwk_qmvm_args;
 
 /* SwiGLU of the shared expert when its gate/up rows went through the multi-format matvec: g, u float [nb][I] ->

@@ -145,7 +145,7 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
         const uint32_t wave = qw_wave(), sp = a.split, tpg = (QW_WG_GU / 64) / sp, part = wave % sp, cpp = cpr / sp;
         const uint32_t ngroups = (a.ntiles + tpg - 1) / tpg;
         for (uint32_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
-            const uint32_t t = g * tpg + wave / sp;
+            const uint32_t t = wave / sp < tpg ? g * tpg + wave / sp : a.ntiles; // waves past a whole number of tiles: none
             acc = f4{0, 0, 0, 0};
             if (t < a.ntiles)
                 qw_task_pipeline<C>(1, 0, 1, cpp, CH * C::BLK_B, F == QW_F_PACKED ? lane : kl, [&](uint32_t) { return rowp(t) + (size_t)part * cpp * CH * C::BLK_B; },
@@ -229,7 +229,7 @@ template <int F, int NB> __device__ __forceinline__ void qmvm_matrix_split(const
     const uint32_t cpp = a.K / (C::BLK_K * NB) / sp, part = wave % sp; // chunks per part
     const uint32_t ngroups = (a.ntiles[j] + tpg - 1) / tpg;
     for (uint32_t g = g0; g < ngroups; g += ng) {
-        const uint32_t t = g * tpg + wave / sp;
+        const uint32_t t = wave / sp < tpg ? g * tpg + wave / sp : a.ntiles[j]; // waves past a whole number of tiles: none
         f4 acc = {0, 0, 0, 0};
         if (t < a.ntiles[j])
             qw_task_pipeline<C>(1, 0, 1, cpp, NB * C::BLK_B, lane & 3, [&](uint32_t) { return T.rowp(t) + (size_t)part * cpp * NB * C::BLK_B; },

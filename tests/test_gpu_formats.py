@@ -77,7 +77,8 @@ def test_dq_extreme_fields(gpu, oracle):
 @pytest.mark.parametrize("nb", [1, 5, 16])
 def test_qmv_parity(gpu, oracle, ftype, nb):
     path = q.Path(gpu, 2048, 512, 512, 10, 16)
-    for N, K, fout in ((1000 + 7, 2048, True), (64, 4096, True), (48, 256, False)):
+    # K = 2560 (the reference model's hidden size) and 1536: the K range of a tile is cut into 5 and 6 parts
+    for N, K, fout in ((1000 + 7, 2048, True), (64, 4096, True), (48, 256, False), (640, 2560, True), (100, 1536, True)):
         rng = np.random.default_rng(1000 + ftype + N)
         W = synth.matrix(rng, ftype, N, K)
         x = synth.activations(rng, nb, K)

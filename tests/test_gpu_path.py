@@ -118,6 +118,31 @@ def test_qmv_ragged_rows_and_half_output(gpu, oracle):
     path.close()
 
 
+@pytest.mark.parametrize("ftype", [21, 8])
+@pytest.mark.parametrize("N,K,dev", [(640, 2560, True), (640, 2560, False), (200, 1536, True), (48, 1280, False)])
+def test_qmv_k_cut_into_odd_parts(gpu, oracle, ftype, N, K, dev):
+    """Few tiles and a chunk count of 5 or 3 (K = 2560 is the reference model's hidden size): a tile's K range is cut
+    over 5, 3 or 6 waves. Against the float64 matvec; every row of the 16-token call equals the 1-token call."""
+    nb = 16
+    rng = np.random.default_rng(K + N + ftype)
+    W = synth.matrix(rng, ftype, N, K)
+    x = synth.activations(rng, nb, K)
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    wb, xb, yb, y1 = gpu.buf_from(W, device_only=dev), gpu.buf_from(x), gpu.buf(nb * N * 4), gpu.buf(N * 4)
+    b = gpu.batch()
+    path.qmv_gg(b, q.Tensor(wb, ftype), N, K, xb, yb, nb, fout=True)
+    assert b.end() >= 0, gpu.last_error()
+    y = yb.view(np.float32)[:nb * N].reshape(nb, N).copy()
+    assert maxrel(y, oracle.qmv(ftype, W, N, K, x, f64=True)) <= 1e-5
+    b = gpu.batch()
+    path.qmv_gg(b, q.Tensor(wb, ftype), N, K, xb, y1, 1, xoff=5 * K * 2)
+    assert b.end() >= 0, gpu.last_error()
+    assert np.array_equal(y1.view(np.uint32)[:N], y[5].view(np.uint32))
+    for bb in (wb, xb, yb, y1):
+        bb.free()
+    path.close()
+
+
 def test_bad_calls_fail_without_launching(gpu):
     """Undersized buffers, unknown formats and unknown kernels are refused on the host."""
     ok, err = gpu.compile("#define IQ_DQ_ONLY 1\n#define DQ_TEST 10\n")  # Q2_K
