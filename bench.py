@@ -468,13 +468,12 @@ def main():
         line["qmv"] = qmv_table(gpu)
         line["qmv_formats"] = formats_table(gpu)
         line["gguf_load"] = gguf_load(gpu)
+        line["model_shape"] = model_shape_leg(gpu, a.layers, min(a.steps, 10), a.warmup)  # 92 GB beside the 67 GB of the main stack
     if not a.no_cpu:
         lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
         line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)
     x.free()
     stack.free()
-    if not a.quick:
-        line["model_shape"] = model_shape_leg(gpu, a.layers, min(a.steps, 10), a.warmup)
     print(json.dumps(line))
     gpu.close()
     return 0
