@@ -947,7 +947,8 @@ static bool nbr_ok(qw_batch *b, uint32_t nbr) {
 }
 
 // gate/up arguments. shared: one expert at (iWg, iWu), all tokens, slot topk.
-// The packed copy of IQ3_S rows: tiles of `split` rows of A and 16 - split rows of B (B = NULL, split 16: one matrix).
+// The packed copy of IQ3_S rows: tiles of `split` rows of A and 16 - split rows of B (B = NULL, split 16: one matrix);
+// split = QW_F_PACKED_NL: the packed copy of one matrix of IQ4_NL rows, nblk chunks of ten blocks a row.
 // Made at the first request, on the batch's stream, and complete when this returns; NULL when packing is off, the
 // source may change without notice (a small buffer with a host shadow is copied at every submit) or memory is short:
 // the caller then reads the GGUF rows directly.
@@ -968,9 +969,10 @@ static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf 
             h->dirty = false;
         }
     }
-    hipFunction_t f = get_func(g, "qwk_pack_iq3");
+    const bool nl = split == QW_F_PACKED_NL; // IQ4_NL rows: nblk counts chunks of ten blocks
+    hipFunction_t f = get_func(g, nl ? "qwk_pack_nl" : "qwk_pack_iq3");
     if (!f) return NULL;
-    const size_t bytes = (size_t)ntiles * nblk * QW_SLAB_BYTES;
+    const size_t bytes = (size_t)ntiles * nblk * (nl ? QW_NL_CHUNK_BYTES : QW_SLAB_BYTES);
     void *dst;
     if (hipMalloc(&dst, bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -1211,6 +1213,18 @@ static bool tr_dn(qw_batch *b) {
     // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
     if ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8))) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
     if (fd == 20 && p->I <= 640 && !getenv("QW_HIP_DN_ANY")) { // the range kernel with rows of up to 640 staged
+        if (p->I % 320 == 0) { // tile-major copies, as for IQ3_S rows (the shared expert's only together with the routed ones)
+            const uint32_t nch = (uint32_t)p->I / 320, tileb = nch * QW_NL_CHUNK_BYTES;
+            const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wd, NULL, NULL, (uint64_t)p->E * (uint64_t)(p->D / 16), nch, a.rowbytes, QW_F_PACKED_NL);
+            const uint8_t *ps = pk && fs == 20 ? get_pack(b, hsd, a.Wsd, NULL, NULL, (uint64_t)(p->D / 16), nch, a.sd_rowbytes, QW_F_PACKED_NL) : NULL;
+            if (pk && (fs != 20 || ps)) {
+                a.Wd = pk, a.rowbytes = tileb;
+                if (fs == 20) a.Wsd = ps, a.sd_rowbytes = tileb;
+                if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10_s%d_c%d", fs == 20 ? QW_F_PACKED_NL : fs, fs == 20 ? 10 : 4);
+                else fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10");
+                return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
+            }
+        }
         const int ch = p->I % 320 == 0 && !getenv("QW_HIP_NL_C4") ? 10 : 4; // blocks per chunk
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d_s%d_c%d", ch, fs, fs == 20 ? ch : 4);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d", ch);

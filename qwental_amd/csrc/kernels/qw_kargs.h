@@ -142,6 +142,15 @@ typedef struct { /* pure-read ceiling and fill helpers */
  * (row tile * (16 - split) + n - split): split 16 = one matrix, split 8 = gate rows and up rows side by side. */
 #define QW_SLAB_BYTES 1792u
 #define QW_F_PACKED 121
+/* Tile-major copy of IQ4_NL rows (format code QW_F_PACKED_NL; qwk_pack_args with split = QW_F_PACKED_NL, nblk = chunks
+ * of ten blocks per row, so the row length is a multiple of 320): every (tile of 16 rows, chunk) becomes
+ * QW_NL_CHUNK_BYTES = 16 x 180 contiguous bytes in the lane order of the matrix instruction (lane = row & 15 | k-group
+ * << 4; a lane owns bytes 4 kg .. 4 kg + 3 of qs of every block of its row):
+ *   [0, 1024)    blocks 0..3: 16 bytes per lane      [1024, 2048)  blocks 4..7: 16 bytes per lane
+ *   [2048, 2560) blocks 8..9:  8 bytes per lane      [2560, 2880)  d of the ten blocks, 20 bytes per row
+ * A wave reads a chunk with three fully coalesced loads plus 20 bytes of scales per lane. */
+#define QW_F_PACKED_NL 120
+#define QW_NL_CHUNK_BYTES 2880u
 typedef struct {
     const uint8_t *A, *B;
     uint8_t *dst;

@@ -104,6 +104,26 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) 
     }
 }
 
+// The tile-major copy of IQ4_NL rows (layout: QW_F_PACKED_NL in qw_kargs.h); a wave per (tile, chunk of ten blocks).
+extern "C" __global__ __launch_bounds__(256) void qwk_pack_nl(qwk_pack_args a) {
+    const uint64_t nchunk = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
+    for (uint64_t ch = (uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); ch < nchunk; ch += step) {
+        const uint64_t tile = ch / a.nblk;
+        const uint8_t *src = a.A + (tile * 16 + n) * a.rowbytes + 180 * (ch % a.nblk);
+        uint8_t *dst = a.dst + ch * QW_NL_CHUNK_BYTES;
+        uint32_t q[10];
+#pragma unroll
+        for (int b = 0; b < 10; b++) q[b] = *(const u1a2 *)(src + 18 * b + 2 + 4 * kg);
+        *(u4 *)(dst + 16 * lane) = u4{q[0], q[1], q[2], q[3]};
+        *(u4 *)(dst + 1024 + 16 * lane) = u4{q[4], q[5], q[6], q[7]};
+        *(u2 *)(dst + 2048 + 8 * lane) = u2{q[8], q[9]};
+        if (kg == 0)
+#pragma unroll
+            for (int b = 0; b < 10; b++) *(uint16_t *)(dst + 2560 + 20 * n + 2 * b) = *(const uint16_t *)(src + 18 * b);
+    }
+}
+
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
 // y[b][row] = sum_k W[row][k] x[b][k] for up to 16 activations; the weights are streamed once for all of them.
 // Tiles of 16 rows are dealt round-robin to the waves of a persistent grid; a row is CPR chunks of CH blocks.
@@ -981,6 +1001,7 @@ template <int F, int CH> __device__ __forceinline__ void shared_down_tiles(const
 // range of at most D / 16 tasks, which touches at most two experts: their H rows (both planes, only the tokens
 // that picked them) are copied into LDS once, in fragment order, and the waves then stream the range's tiles with operand A read
 // from LDS. The first weight loads are issued before the table copy, the row copy and the barrier.
+constexpr bool qw_tiled(int F) { return F == QW_F_PACKED || F == QW_F_PACKED_NL; } // weights come from a tile-major copy
 struct qw_dn_seg { // one expert's part of a workgroup's range (all fields wave-uniform)
     const uint8_t *W;  // the expert's matrix
     float *P;          // Pg or Psh
@@ -1002,13 +1023,13 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
         off1[j] = !both || !((g1.mask >> tok) & 1) ? ~0u : (g1.sh ? tok : tok * K + slots1[tok]) * a.D;
     }
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
+    qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
         [&](uint32_t i) {
             // (field by field: a reference chosen between the two records would put them in scratch memory)
             const bool second = i >= g0.ntile;
             const uint8_t *W = second ? g1.W : g0.W;
             const uint32_t tile = second ? g1.tile0 + i - g0.ntile : g0.tile0 + i, rbs = second ? g1.rowbytes : g0.rowbytes;
-            if constexpr (F == QW_F_PACKED) return W + (size_t)tile * rbs; // rowbytes = bytes of a tile
+            if constexpr (qw_tiled(F)) return W + (size_t)tile * rbs; // rowbytes = bytes of a tile
             else return W + (size_t)(16 * tile + nl) * rbs;
         },
         [&](uint32_t i, uint32_t ci, const C &c) {
@@ -1035,14 +1056,14 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
     auto div_tpe = [&](uint32_t x) { return tp2 ? x >> tsh : x / tpe; };
     qw_sel_load(*sc, a.sel, K, gnb); // one memory round trip for everything the ranges depend on
     if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // lands in LDS meanwhile; awaited in ready()
-    if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook instead
+    if (F == 20 || FSD == 20 || F == QW_F_PACKED_NL || FSD == QW_F_PACKED_NL) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook instead
     __syncthreads();
     const uint32_t *ue = sc->ue, *mask = sc->mask;
     const uint8_t *slot = sc->slot;
     uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
     if (U > GU) U = GU;
     // a shared-expert tile of a wider format counts as several tasks, so that ranges hold about the same bytes
-    const uint32_t tb = F == QW_F_PACKED ? a.rowbytes : 16 * a.rowbytes, stb = FSD == QW_F_PACKED ? a.sd_rowbytes : 16 * a.sd_rowbytes; // bytes of a tile
+    const uint32_t tb = qw_tiled(F) ? a.rowbytes : 16 * a.rowbytes, stb = qw_tiled(FSD) ? a.sd_rowbytes : 16 * a.sd_rowbytes; // bytes of a tile
     const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0, shw = nsh ? (stb + tb - 1) / tb : 1, vsh = nsh * shw * tpe;
     const uint32_t V = vsh + U * tpe;
     uint32_t per = (V + gridDim.x - 1) / gridDim.x;
@@ -1066,7 +1087,7 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
                 g.tile0 = lo - first;
                 g.ntile = hi - lo;
                 const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ue[g.u]);
-                g.W = a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, g.P = a.P, g.rowbytes = a.rowbytes;
+                g.W = a.Wd + (size_t)e * (qw_tiled(F) ? tpe : a.D) * a.rowbytes, g.P = a.P, g.rowbytes = a.rowbytes;
                 g.mask = (uint32_t)__builtin_amdgcn_readfirstlane((int)mask[g.u]) & qw_all_tokens(a.nbr);
             }
             return g;
@@ -1133,6 +1154,13 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         dn_range_body<20, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                               \
     }
 QW_DN_RANGE_NL(4, 0, 1, qwk_dnr_f20_c4) QW_DN_RANGE_NL(4, 20, 4, qwk_dnr_f20_c4_s20_c4) QW_DN_RANGE_NL(4, 8, 4, qwk_dnr_f20_c4_s8_c4)
+#define QW_DN_RANGE_NLP(FSD, CHSD, NAME)                                                          \
+    extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
+        __shared__ struct { u2 lut[QW_KQ_TAB / 2]; uint16_t arows[2 * 16 * 2 * 640]; qw_sel_cache sc; } L; \
+        dn_range_body<QW_F_PACKED_NL, 10, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                   \
+    }
+// the tile-major copy: rows of 320 or 640
+QW_DN_RANGE_NLP(0, 10, qwk_dnr_f120_c10) QW_DN_RANGE_NLP(QW_F_PACKED_NL, 10, qwk_dnr_f120_c10_s120_c10) QW_DN_RANGE_NLP(8, 4, qwk_dnr_f120_c10_s8_c4)
 // rows of 320 or 640: chunks of ten blocks (a row of 640 in two), 5760 bytes a tile in flight per wave
 QW_DN_RANGE_NL(10, 0, 1, qwk_dnr_f20_c10) QW_DN_RANGE_NL(10, 20, 10, qwk_dnr_f20_c10_s20_c10) QW_DN_RANGE_NL(10, 8, 4, qwk_dnr_f20_c10_s8_c4)
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks

@@ -371,6 +371,38 @@ template <int NB> struct qw_chunk<20, NB> {
     }
 };
 
+// The same rows from their tile-major copy (layout: QW_F_PACKED_NL in qw_kargs.h): one chunk = ten blocks of the 16
+// rows of a tile, already in matrix-core lane order. BLK_B is the bytes of a block of all 16 rows, so that
+// NB * BLK_B is the chunk's size as for the other chunk types.
+typedef u4 __attribute__((aligned(4))) u4a4;
+template <> struct qw_chunk<QW_F_PACKED_NL, 10> {
+    static constexpr uint32_t BLK_K = 32, BLK_B = 288;
+    static constexpr int DEPTH = 3;
+    uint32_t q[10], dd[5];
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t lane) {
+        const u4 a = *(const u4 *)(p + 16 * lane), b = *(const u4 *)(p + 1024 + 16 * lane);
+        const u2 c = *(const u2 *)(p + 2048 + 8 * lane);
+        const uint8_t *ds = p + 2560 + 20 * (lane & 15);
+        const u4 d0 = *(const u4a4 *)ds;
+        q[0] = a.x, q[1] = a.y, q[2] = a.z, q[3] = a.w, q[4] = b.x, q[5] = b.y, q[6] = b.z, q[7] = b.w, q[8] = c.x, q[9] = c.y;
+        dd[0] = d0.x, dd[1] = d0.y, dd[2] = d0.z, dd[3] = d0.w, dd[4] = *(const uint32_t *)(ds + 16);
+    }
+    __device__ __forceinline__ void transpose() {}
+    __device__ __forceinline__ float scale(int b) const { return qw_h2f((uint16_t)(dd[b >> 1] >> (16 * (b & 1)))); }
+    template <class AF> __device__ __forceinline__ void mac(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < 10; b++) {
+            const h8 w = qw_iq4_bytes((const uint32_t *)lut, q[b]);
+            const uint32_t kb = k0 + 32 * b + 4 * kg;
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(qw_chunk<20, 1>::join(af.hi4(kb), af.hi4(kb + 16)), w, sub);
+            if (AF::has_lo) sub = qw_mfma(qw_chunk<20, 1>::join(af.lo4(kb), af.lo4(kb + 16)), w, sub);
+            acc += scale(b) * sub;
+        }
+    }
+    template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+};
+
 // NB blocks of one row for the task pipeline: loaded in quad order, pulled to matrix-core lane order.
 template <int F, int NB> struct qw_chunk_kq {
     static constexpr uint32_t BLK_K = qw_kq<F>::BLK_K, BLK_B = qw_kq<F>::BLK_B;

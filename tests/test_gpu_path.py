@@ -352,7 +352,7 @@ def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
     m = synth.moe_layer(rng, D, I, E, fgu=21, fd=20, fsh=8, fshd=20)
     m["topk"] = K
     x = synth.activations(rng, nb, D)
-    dl = DeviceLayer(gpu, m)
+    dl = DeviceLayer(gpu, m)  # host-shadowed buffers: no tile-major copies
     old = os.environ.get("QW_HIP_DN_ANY")
     try:
         for env, want in ((None, "qwk_dnr_f20_c10_s20_c10"), ("1", "qwk_dn_f20_any_s20")):
@@ -372,6 +372,41 @@ def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
         if old is not None:
             os.environ["QW_HIP_DN_ANY"] = old
     dl.free()
+
+
+@pytest.mark.parametrize("D,I,nb,fshd", [(2560, 640, 16, 20), (2560, 640, 2, 20), (1024, 640, 9, 8), (1024, 640, 5, 20)])
+def test_iq4_nl_down_from_the_tile_major_copy(gpu, oracle, D, I, nb, fshd):
+    """Device-only IQ4_NL down matrices with rows of 640 get a tile-major copy (the IQ3_S scheme); the layer from
+    the copy equals the layer from the GGUF rows bit for bit (same products in the same order) and meets the float64 layer."""
+    if os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
+    E, K = 32, 10
+    rng = np.random.default_rng(3000 + D + I + nb)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=20, fsh=8, fshd=fshd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    outs = []
+    try:
+        for copies in (True, False):
+            gpu.L.qw_hip_set_repack(gpu.g, copies)
+            path = q.Path(gpu, D, I, E, K, 16)
+            dl = DeviceLayer(gpu, m, device_only=True)
+            before = gpu.L.qw_hip_packed_bytes(gpu.g)
+            gpu.profile(True)
+            out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            want = "qwk_dnr_f120_c10" if copies else "qwk_dnr_f20_c10"
+            assert any(n.startswith(want) for n in names), names
+            if copies:  # the routed matrix, and the shared one when it is IQ4_NL too (the IQ3_S gate/up copies come on top)
+                assert gpu.L.qw_hip_packed_bytes(gpu.g) - before >= (E + (fshd == 20)) * D * I // 32 * 18
+            assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+            outs.append(out)
+            dl.free()
+            path.close()
+    finally:
+        gpu.L.qw_hip_set_repack(gpu.g, True)
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
 
 
 def test_moe_batched_equals_single(gpu):
