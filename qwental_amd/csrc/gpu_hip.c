@@ -434,8 +434,8 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
     if (part == 5) { // the grouped product over packed rows, src/engine.c:3244-3248
         p = (qw_kparams){0};
         if (!def_int(d, n, "PFF", &p.F) || !def_int(d, n, "KD", &p.K) || !def_int(d, n, "TM", &p.tm) || !def_int(d, n, "E", &p.E)) FAIL("moe_pf_gg: PFF, KD, TM and E must be integer macros");
-        if (!fmt_ok(p.F)) FAIL("moe_pf_gg: ggml type %d has no gfx950 build (have 8, 21)", p.F);
-        if (p.K <= 0 || p.K % fmt_qb(p.F) || (p.F == 8 && p.K % 128)) FAIL("moe_pf_gg: KD %d does not fit type %d", p.K, p.F);
+        if (!fmt_ok(p.F) && p.F != 20) FAIL("moe_pf_gg: ggml type %d has no gfx950 build (have 8, 20, 21)", p.F);
+        if (p.K <= 0 || p.K % fmt_qb(p.F) || ((p.F == 8 || p.F == 20) && p.K % 128)) FAIL("moe_pf_gg: KD %d does not fit type %d", p.K, p.F);
         if (p.tm < 1 || p.tm > 64) FAIL("moe_pf_gg: TM %d outside this build (1..64 rows per tile entry)", p.tm);
         if (p.E < 1 || p.E > 1024) FAIL("moe_pf_gg: E %d outside this build (E <= 1024)", p.E);
         if (!reg_kernel(g, d, n, "moe_pf_gg", FAM_PF, &p, err, errlen)) { ok = false; goto out; }
@@ -1348,7 +1348,7 @@ static bool launch_pf(qw_batch *b, qwk_pf_args *a, int F, int E, qw_hbuf *hw, qw
         if (wb) return false; // the caller launches the two matrices one by one
     }
     if (F == 21) fname_fmt(fn, sizeof fn, "qwk_pf_f21_c%d", a->K % 512 == 0 ? 2 : 1);
-    else fname_fmt(fn, sizeof fn, "qwk_pf_f8_c4");
+    else fname_fmt(fn, sizeof fn, "qwk_pf_f%d_c4", F == 20 ? 20 : 8);
     // every entry can hold a tile: the grid covers the whole table, the kernel counts the entries in use
     return add_launch(b, intern(fn), persistent_grid(b->g, a->max_tiles * a->ntn, 8), 512, a, sizeof *a);
 }

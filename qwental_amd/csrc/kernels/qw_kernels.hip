@@ -1389,6 +1389,7 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
     if (threadIdx.x == 0) *cnt = 0;
     if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (F == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook
     __syncthreads();
     uint32_t mine = 0;
     for (uint32_t t = threadIdx.x; t < a.max_tiles; t += blockDim.x) {
@@ -1449,10 +1450,11 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
 }
 #define QW_PF(F, CH, NAME)                                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pf_args a) {                    \
-        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 tl[2048]; uint32_t cnt; } L; \
+        __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : F == 20 ? QW_KQ_TAB / 2 : 1]; u4 tl[2048]; uint32_t cnt; } L; \
         pf_body<F, CH>(a, L.lut, L.tl, &L.cnt);                                                  \
     }
 QW_PF(21, 2, qwk_pf_f21_c2) QW_PF(21, 1, qwk_pf_f21_c1) QW_PF(8, 4, qwk_pf_f8_c4)
+QW_PF(20, 4, qwk_pf_f20_c4) // IQ4_NL rows (the down projection of the reference model's layer: K = 640)
 QW_PF(121, 2, qwk_pf_f121_c2) QW_PF(121, 1, qwk_pf_f121_c1) // tile-major IQ3_S: one matrix, or gate and up rows side by side
 
 // The same product for entries of at most 16 packed rows over tile-major weights, the way the decode kernels work:

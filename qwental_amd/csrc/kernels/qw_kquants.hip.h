@@ -353,6 +353,20 @@ template <int NB> struct qw_chunk<20, NB> {
         }
     }
     template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    // NG groups of 16 activation rows (binary16, one plane, global memory) against the same decoded weights
+    template <int NG> __device__ __forceinline__ void mac_groups(const u2 *lut, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const h8 w = qw_iq4_bytes((const uint32_t *)lut, q[b]);
+            const uint32_t kb = k0 + 32 * b + 4 * kg;
+#pragma unroll
+            for (int g = 0; g < NG; g++) {
+                f4 sub = {0, 0, 0, 0};
+                sub = qw_mfma(join(*(const h4 *)(rows[g] + kb), *(const h4 *)(rows[g] + kb + 16)), w, sub);
+                acc[g] += qw_h2f(d[b]) * sub;
+            }
+        }
+    }
     __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {

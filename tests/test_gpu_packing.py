@@ -26,9 +26,9 @@ def expert_ref(o, m, e, x):
     return h, Wd
 
 
-def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed, device_only=False):
+def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed, device_only=False, fd=None):
     rng = np.random.default_rng(seed)
-    m = synth.moe_layer(rng, D, I, E, fgu=fmt, fd=fmt, fsh=fmt)
+    m = synth.moe_layer(rng, D, I, E, fgu=fmt, fd=fmt if fd is None else fd, fsh=fmt)
     x = synth.activations(rng, T, D)
     w = rng.uniform(0.05, 1.0, (T, K)).astype(np.float32)
     w /= w.sum(axis=1, keepdims=True)
@@ -40,7 +40,7 @@ def run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, seed, device_only=False):
     b = gpu.batch()
     path.pf_moe(b, dl.layer, T, xb, ib, wb, ob)
     assert b.end() >= 0, gpu.last_error()
-    if device_only and fmt == 21:  # weights that live in HBM only get the tile-major copies: gate + up as one, down
+    if device_only and fmt == 21 and fd is None:  # weights that live in HBM only get the tile-major copies: gate + up as one, down
         assert gpu.L.qw_hip_packed_bytes(gpu.g) - packed0 == (2 * E * I * (D // 256) + E * D * (I // 256)) // 16 * 1792
     P = T * K
     # integer stages against the oracle (kernels/moe_prefill.metal:15-93)
@@ -76,6 +76,15 @@ def test_packing_uniform_routing(gpu, oracle, fmt, tm):
     rng = np.random.default_rng(7 + tm)
     ids = np.stack([rng.choice(E, K, replace=False) for _ in range(T)])
     run_case(gpu, oracle, T, ids, E, K, D, I, fmt, tm, 70 + tm)
+
+
+@pytest.mark.parametrize("dev", [False, True])
+def test_packing_iq4_nl_down_rows(gpu, oracle, dev):
+    """The reference model's formats on the packing path: IQ3_S gate/up, IQ4_NL down rows of 640 values."""
+    T, E, K, D, I = 40, 32, 4, 512, 640
+    rng = np.random.default_rng(19)
+    ids = synth.zipf_ids(rng, T, E, K)
+    run_case(gpu, oracle, T, ids, E, K, D, I, 21, 16, 190, device_only=dev, fd=20)
 
 
 @pytest.mark.parametrize("tm", [16, 64])
