@@ -529,7 +529,10 @@ bool qw_gguf_moe_layer(const qw_gguf *G, int layer, qw_moe_layer *M, int *D, int
     ok = ok && sg->dims[0] == d && sg->dims[1] == in && su->dims[0] == d && su->dims[1] == in && sd->dims[0] == in && sd->dims[1] == d;
     if (!ok) return fail(err, errlen, "GGUF: layer %d: the shapes of the MoE tensors do not agree", layer);
     if (ga->type != up->type) return fail(err, errlen, "GGUF: layer %d: gate is %s but up is %s", layer, qw_ggml_name((int)ga->type), qw_ggml_name((int)up->type));
-    if (sg->type != su->type) return fail(err, errlen, "GGUF: layer %d: shared gate is %s but shared up is %s", layer, qw_ggml_name((int)sg->type), qw_ggml_name((int)su->type));
+    // The shared expert's gate and up may differ inside the K-quant / IQ4 / plain family (Q4_K gate and IQ4_XS up in the
+    // reference's model, bench/moe_bw.c:19-20); Q8_0 and IQ3_S rows run in kernels that take one type for both.
+    if (sg->type != su->type && (sg->type == 8 || sg->type == 21 || su->type == 8 || su->type == 21))
+        return fail(err, errlen, "GGUF: layer %d: shared gate is %s but shared up is %s", layer, qw_ggml_name((int)sg->type), qw_ggml_name((int)su->type));
     if (M->sh_gate_w.type != M->router.type)
         return fail(err, errlen, "GGUF: layer %d: the shared-expert gate vector is %s but the router is %s", layer, qw_ggml_name(M->sh_gate_w.type), qw_ggml_name(M->router.type));
     *D = (int)d;

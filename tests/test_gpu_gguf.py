@@ -159,6 +159,37 @@ def test_layer_from_files_parity(gpu, oracle, model):
     g.close()
 
 
+def test_layer_in_the_reference_models_formats_from_files(gpu, oracle, tmp_path):
+    """A layer as a GGUF of the reference's model holds it (bench/moe_bw.c:16-24 of the reference): IQ3_S gate/up,
+    IQ4_NL down rows of 640, shared expert Q4_K gate, IQ4_XS up, IQ4_NL down; read from a file, made resident, run."""
+    d, i, e, k, layer = 512, 640, 16, 4, 2
+    rng = np.random.default_rng(91)
+    m = synth.moe_layer(rng, d, i, e, fgu=21, fd=20, fsh=12, fshu=23, fshd=20)
+    m["topk"] = k
+    wr32, wr_bits = bf16_exact(rng.normal(0.0, 0.02, (e, d)))
+    wg32, wg_bits = bf16_exact(rng.normal(0.0, 0.02, d))
+    m["Wr"], m["wsg"] = wr_bits, wg_bits
+    p = "blk.%d." % layer
+    gw.write_gguf(os.path.join(str(tmp_path), "model.gguf"),
+                  [(p + "ffn_gate_exps.weight", 21, [d, i, e], m["Wg"]), (p + "ffn_up_exps.weight", 21, [d, i, e], m["Wu"]), (p + "ffn_down_exps.weight", 20, [i, d, e], m["Wd"]),
+                   (p + "ffn_gate_inp.weight", 30, [d, e], wr_bits), (p + "ffn_gate_inp_shexp.weight", 0, [d], wg32),
+                   (p + "ffn_gate_shexp.weight", 12, [d, i], m["Wsg"]), (p + "ffn_up_shexp.weight", 23, [d, i], m["Wsu"]), (p + "ffn_down_shexp.weight", 20, [i, d], m["Wsd"])],
+                  [("general.architecture", 8, "synthetic")])
+    g = q.Gguf(str(tmp_path))
+    g.load(gpu, "moe,shared,router")
+    M, d2, i2, e2 = g.moe_layer(layer)
+    assert (d2, i2, e2) == (d, i, e)
+    assert (M.gate.type, M.down.type, M.sh_gate.type, M.sh_up.type, M.sh_down.type) == (21, 20, 12, 23, 20)
+    path = q.Path(gpu, d, i, e, k, 16)
+    for nb in (1, 11):
+        x = synth.activations(rng, nb, d)
+        out, lg, _, _ = run_moe(gpu, path, _Layer(M), x, nb)
+        assert maxrel(lg, oracle.router(m["Wr"], m["wsg"], x, wfmt=30)) <= 1e-5
+        assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+    path.close()
+    g.close()
+
+
 def test_resident_tensor_dequantizes_bit_exactly(gpu, oracle, model):
     """The reference's tools/dqtest.py + tools/dqtest.c:26-48 on the files: for every format the first tensor of that
     format, a few rows of it through the dq_test kernel, here out of the resident copy and against the oracle."""
