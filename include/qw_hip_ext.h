@@ -40,7 +40,7 @@ void *qw_hip_buf_devptr(const qw_buf *b);
 
 /* IQ3_S weight matrices of the MoE kernels are copied once, at their first use, into a tile-major layout that a wave
  * reads with fully coalesced loads (the copy costs 1792 / 1760 of the matrix's bytes of HBM; the GGUF bytes stay where
- * they are). The copy is dropped when the source buffer is freed, marked dirty, uploaded, written, or bound as a
+ * they are); IQ4_NL down matrices with rows of 640 values likewise (a copy of exactly their size). The copy is dropped when the source buffer is freed, marked dirty, uploaded, written, or bound as a
  * kernel's output. Buffers of at most QW_HIP_SMALL_BYTES with a host shadow are never copied. QW_HIP_REPACK=0 in the
  * environment, or qw_hip_set_repack(g, false), turns the copies off (kernels then read the GGUF rows directly). */
 void qw_hip_set_repack(qw_gpu *g, bool on);
