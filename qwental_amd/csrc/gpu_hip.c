@@ -1220,9 +1220,19 @@ static bool tr_dn(qw_batch *b) {
             if (pk && (fs != 20 || ps)) {
                 a.Wd = pk, a.rowbytes = tileb;
                 if (fs == 20) a.Wsd = ps, a.sd_rowbytes = tileb;
-                if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10_s%d_c%d", fs == 20 ? QW_F_PACKED_NL : fs, fs == 20 ? 10 : 4);
-                else fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10");
-                return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
+                char tail[24] = "";
+                if (fs) fname_fmt(tail, sizeof tail, "_s%d_c%d", fs == 20 ? QW_F_PACKED_NL : fs, fs == 20 ? 10 : 4);
+                fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10%s", tail);
+                const unsigned grid = persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR);
+                if (nbr <= dnc_maxnb()) { // a few tokens: wait for the combine, the two run as one launch
+                    char fu[48];
+                    fname_fmt(fu, sizeof fu, "qwk_dnc_f120_c10%s", tail);
+                    b->pend_dn.valid = true;
+                    b->pend_dn.a = a;
+                    b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid;
+                    return true;
+                }
+                return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
             }
         }
         const int ch = p->I % 320 == 0 && !getenv("QW_HIP_NL_C4") ? 10 : 4; // blocks per chunk

@@ -1182,9 +1182,9 @@ __device__ __forceinline__ f4 dnc_tile(const qwk_dn_args &a, const u2 *lut, cons
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), kg = lane >> 4, cpr = a.I / (C::BLK_K * CH);
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(1, 0, 1, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
+    qw_task_pipeline<C>(1, 0, 1, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
         [&](uint32_t) {
-            if constexpr (F == QW_F_PACKED) return W + (size_t)tile * rowbytes; // rowbytes = bytes of a tile
+            if constexpr (qw_tiled(F)) return W + (size_t)tile * rowbytes; // rowbytes = bytes of a tile
             else return W + (size_t)(16 * tile + (lane >> 2)) * rowbytes;
         },
         [&](uint32_t, uint32_t ci, const C &c) { c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc); }, ready);
@@ -1197,6 +1197,7 @@ __device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *p
     const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K));
     for (uint32_t i = threadIdx.x; i < a.nbr * (K + 1); i += blockDim.x) wl[i] = wg[i];
     if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // awaited in ready()
+    if (F == QW_F_PACKED_NL || FSD == QW_F_PACKED_NL) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook instead
     __syncthreads();
     uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
     if (U > gnb * K) U = gnb * K;
@@ -1223,7 +1224,7 @@ __device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *p
             else acc = f4{0, 0, 0, 0};
         } else {
             const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->ue[u]);
-            acc = dnc_tile<F, CH>(a, lut, a.Wd + (size_t)e * (F == QW_F_PACKED ? tpe : a.D) * a.rowbytes, a.rowbytes, tile, af, ready);
+            acc = dnc_tile<F, CH>(a, lut, a.Wd + (size_t)e * (qw_tiled(F) ? tpe : a.D) * a.rowbytes, a.rowbytes, tile, af, ready);
         }
         const uint32_t r = 16 * tile + n;
 #pragma unroll
@@ -1250,12 +1251,13 @@ __device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *p
 }
 #define QW_DNC(F, CH, FSD, CHSD, NAME)                                                              \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                    \
-        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : 1]; float part[QW_DNC_MAXNB * 17 * 16], wl[QW_DNC_MAXNB * 17]; qw_sel_cache sc; } L; \
+        __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : (F == QW_F_PACKED_NL || FSD == QW_F_PACKED_NL) ? QW_KQ_TAB / 2 : 1]; float part[QW_DNC_MAXNB * 17 * 16], wl[QW_DNC_MAXNB * 17]; qw_sel_cache sc; } L; \
         dnc_body<F, CH, FSD, CHSD>(a, L.lut, L.part, L.wl, &L.sc);                                  \
     }
 QW_DNC(121, 2, 0, 1, qwk_dnc_f121_c2) QW_DNC(121, 2, 121, 2, qwk_dnc_f121_c2_s121_c2) QW_DNC(121, 2, 8, 4, qwk_dnc_f121_c2_s8_c4)
 QW_DNC(121, 1, 0, 1, qwk_dnc_f121_c1) QW_DNC(121, 1, 121, 1, qwk_dnc_f121_c1_s121_c1) QW_DNC(121, 1, 8, 4, qwk_dnc_f121_c1_s8_c4)
 QW_DNC(8, 4, 0, 1, qwk_dnc_f8_c4) QW_DNC(8, 4, 8, 4, qwk_dnc_f8_c4_s8_c4)
+QW_DNC(120, 10, 0, 10, qwk_dnc_f120_c10) QW_DNC(120, 10, 120, 10, qwk_dnc_f120_c10_s120_c10) QW_DNC(120, 10, 8, 4, qwk_dnc_f120_c10_s8_c4) // tile-major IQ4_NL rows of 640
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {

@@ -415,6 +415,23 @@ template <> struct qw_chunk<QW_F_PACKED_NL, 10> {
         }
     }
     template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    // operand A gathered from the two H planes in global memory by the lanes whose token is in use
+    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < 10; b++) {
+            const uint32_t kb = k0 + 32 * b + 4 * kg;
+            h8 xh = {}, xl = {};
+            if (af.on) {
+                xh = qw_chunk<20, 1>::join(*(const h4 *)(af.rowhi + kb), *(const h4 *)(af.rowhi + kb + 16));
+                xl = qw_chunk<20, 1>::join(*(const h4 *)(af.rowlo + kb), *(const h4 *)(af.rowlo + kb + 16));
+            }
+            const h8 w = qw_iq4_bytes((const uint32_t *)lut, q[b]);
+            f4 sub = {0, 0, 0, 0};
+            sub = qw_mfma(xh, w, sub);
+            sub = qw_mfma(xl, w, sub);
+            acc += scale(b) * sub;
+        }
+    }
 };
 
 // NB blocks of one row for the task pipeline: loaded in quad order, pulled to matrix-core lane order.
