@@ -1043,7 +1043,18 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
     // 2.70 ms a token); with more tokens the fork and join cost more than the overlap gives (6.81 -> 6.93 ms at 16).
     // QW_HIP_SIDE in the environment: 0 never, 1 always.
     const int first = b->nl;
-    if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
+    // one launch when the K range splits so that a workgroup holds whole (gate tile, up tile) pairs; else matvec, then SwiGLU
+    unsigned sw = 0;
+    for (unsigned s = 6; s > 1 && !sw; s--)
+        if (s != 4 && (unsigned)(p->D / 256) % s == 0 && !getenv("QW_HIP_NO_SWIGLU_MATVEC")) sw = s;
+    if (sw) {
+        m.split = sw, m.sums = 0, m.H = h, m.topk = (uint32_t)p->topk, m.hplane = sa.hplane;
+        for (int j = 0; j < 2; j++) {
+            m.ntiles[j] = cdiv((unsigned)p->I, 16);
+            if (m.fmt[j] == 12 || m.fmt[j] == 13) m.sums = 1;
+        }
+        if (!add_launch(b, "qwk_qmvm_swiglu", umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2)), 64 * QW_WAVES_GU, &m, sizeof m)) return false;
+    } else if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
     const char *e = getenv("QW_HIP_SIDE");
     if (e ? e[0] == '1' : nbr <= 2)
         for (int i = first; i < b->nl; i++) b->l[i].side = true;

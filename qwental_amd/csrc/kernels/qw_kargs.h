@@ -45,6 +45,10 @@ typedef struct {
     uint32_t N[4], fmt[4], rowbytes[4], ystride[4], ntiles[4];
     uint32_t K, xstride, nb, yfloat, nmat, sums; /* sums: some matrix is Q4_K / Q5_K (needs the 32-value sums of x) */
     uint32_t split, pad;                         /* waves a tile's K range is cut over (1 .. 6; > 1 needs K % (256 * split) == 0) */
+    /* qwk_qmvm_swiglu (matrix 0 = gate rows, matrix 1 = up rows of a shared expert, N[0] = N[1] = I, split in
+     * {2, 3, 5, 6}): nothing goes to y; H[t][topk][r] = silu(gate) * up as binary16 hi + lo planes, hplane halves apart */
+    uint16_t *H;
+    uint32_t topk, hplane;
 } qwk_qmvm_args;
 
 /* SwiGLU of the shared expert when its gate/up rows went through the multi-format matvec: g, u float [nb][I] ->

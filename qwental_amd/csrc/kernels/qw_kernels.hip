@@ -264,6 +264,80 @@ template <int F, int NB> __device__ __forceinline__ void qmvm_matrix_split(const
         __syncthreads();
     }
 }
+// One part of one tile: the product over chunks [part * cpp, (part + 1) * cpp) of the rows of tile t of matrix j.
+template <int F, int NB> __device__ __forceinline__ f4 qmvm_part(const qwk_qmvm_args &a, uint32_t j, const uint32_t *tab, const qw_afrag_kq &af, uint32_t t, uint32_t part) {
+    typedef qw_chunk_kq<F, NB> C;
+    const qmvm_tile<F, NB> T = {a, j};
+    const uint32_t lane = qw_lane(), kg = lane >> 4, cpp = a.K / (C::BLK_K * NB) / a.split;
+    f4 acc = {0, 0, 0, 0};
+    qw_task_pipeline<C>(1, 0, 1, cpp, NB * C::BLK_B, lane & 3, [&](uint32_t) { return T.rowp(t) + (size_t)part * cpp * NB * C::BLK_B; },
+                        [&](uint32_t, uint32_t ci, const C &c) { c.mac(tab, af, (part * cpp + ci) * NB * C::BLK_K, kg, acc); });
+    return acc;
+}
+// The shared expert's gate/up in the other format family with SwiGLU in the same launch (kernels/moe_gg.metal:563-573):
+// matrix 0 holds the gate rows, matrix 1 the up rows, each of its own format. A workgroup takes 12 / split / 2 pairs of
+// tiles (gate tile t and up tile t side by side), split waves a tile as in qwk_qmvm; the partial sums meet in LDS, and
+// the first wave of a gate tile adds up both tiles in part order, applies SwiGLU and stores H's two planes.
+extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmvm_args a) {
+    __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; } L;
+    qw_kq_tab_build(L.tab);
+    qw_stage_x(L.xf, a.x, a.xstride, a.K, a.nb);
+    __syncthreads();
+    if (a.sums) { // sums of 32 activations per token, in index order
+        for (uint32_t i = threadIdx.x; i < (a.K >> 5) * 16; i += blockDim.x) {
+            const uint32_t c = i >> 4, m = i & 15;
+            float sum = 0;
+#pragma unroll
+            for (uint32_t f = 0; f < 4; f++) {
+                const h8 v = __builtin_bit_cast(h8, L.xf[(4 * c + f) * 16 + m]);
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += (float)v[e];
+            }
+            L.xs[i] = sum;
+        }
+        __syncthreads();
+    }
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, wave = qw_wave(), sp = a.split;
+    const qw_afrag_kq af = {L.xf, L.xs, n, kg};
+    const uint32_t pairs = (QW_WG_QMVM / 64) / sp / 2, slot = wave / sp, part = wave % sp, which = slot & 1, ntiles = a.ntiles[0];
+    const uint32_t ngroups = (ntiles + pairs - 1) / pairs;
+    for (uint32_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
+        const uint32_t t = slot < 2 * pairs ? g * pairs + slot / 2 : ntiles; // waves past a whole number of pairs: none
+        f4 acc = {0, 0, 0, 0};
+        if (t < ntiles) {
+            switch (a.fmt[which]) { // uniform in a wave
+            case 12: acc = qmvm_part<12, 1>(a, which, L.tab, af, t, part); break;
+            case 13: acc = qmvm_part<13, 1>(a, which, L.tab, af, t, part); break;
+            case 14: acc = qmvm_part<14, 1>(a, which, L.tab, af, t, part); break;
+            case 23: acc = qmvm_part<23, 1>(a, which, L.tab, af, t, part); break;
+            case 20: acc = qmvm_part<20, 8>(a, which, L.tab, af, t, part); break;
+            case 1: acc = qmvm_part<1, 8>(a, which, L.tab, af, t, part); break;
+            case 30: acc = qmvm_part<30, 8>(a, which, L.tab, af, t, part); break;
+            }
+        }
+        L.red[wave * 64 + lane] = acc;
+        __syncthreads();
+        if (part == 0 && which == 0 && t < ntiles) {
+            f4 gate = L.red[wave * 64 + lane], up = L.red[(wave + sp) * 64 + lane];
+            for (uint32_t q = 1; q < sp; q++) gate += L.red[(wave + q) * 64 + lane], up += L.red[(wave + sp + q) * 64 + lane];
+            const uint32_t r = 16 * t + n;
+            if (r < a.N[0])
+#pragma unroll
+                for (uint32_t j = 0; j < 4; j++) {
+                    const uint32_t tok = 4 * kg + j;
+                    if (tok < a.nb) {
+                        const float gv = gate[j], h = gv / (1.0f + __expf(-gv)) * up[j];
+                        const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
+                        const size_t o = ((size_t)tok * (a.topk + 1) + a.topk) * a.N[0] + r;
+                        a.H[o] = __builtin_bit_cast(uint16_t, hi);
+                        a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+}
+
 extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args a) {
     __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; } L;
     qw_kq_tab_build(L.tab);
