@@ -323,6 +323,9 @@ def test_moe_layer_parity(gpu, oracle, nb, fmt):
     (2560, 640, 64, 10, 7, 21, 20, 8, 8, False),     # IQ4_NL routed down beside a Q8_0 shared expert
     (2560, 640, 64, 10, 12, 21, 8, 21, 8, True),     # I = 640 with Q8_0 down rows
     (1024, 384, 32, 4, 5, 8, 20, 8, 20, False),      # I a multiple of 128 only
+    (256, 640, 16, 1, 4, 8, 20, 8, 20, True),        # the narrowest layer, one pick per token, tile-major IQ4_NL rows
+    (512, 1280, 16, 16, 3, 21, 20, 21, 20, True),    # IQ4_NL rows wider than the staged 640: the any-shape kernel; every expert picked
+    (2560, 640, 512, 10, 16, 21, 20, 8, 8, True),    # 512 experts at the reference model's shape, Q8_0 shared expert
 ])
 def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
     """Shapes and format mixes off the benchmark's: every kernel variant the host can pick is reached by one of them."""
