@@ -114,6 +114,8 @@ struct qw_batch {
     // a down projection over a few tokens that waits for the combine of the same layer: both in one launch
     // (qwk_dnc_*); launched as it is at any other dispatch or at submit
     struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid; } pend_dn;
+    // measurement switches, read from the environment once when the batch begins
+    struct { unsigned dnc_nb; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select; } sw;
 };
 
 #define QW_LD_MAX 16
@@ -692,6 +694,14 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     b->stream = g->cur_stream;
     b->prof = g->prof;
     g->err[0] = 0;
+    const char *e = getenv("QW_HIP_DNC_NB"); // token count up to which down + combine run as one launch (0: never)
+    b->sw.dnc_nb = e ? (unsigned)atoi(e) : 2;
+    if (b->sw.dnc_nb > QW_DNC_MAXNB) b->sw.dnc_nb = QW_DNC_MAXNB;
+    e = getenv("QW_HIP_SIDE"); // the side stream: 0 never, 1 always, unset: with one or two tokens
+    b->sw.side = e ? (e[0] == '1' ? 1 : 0) : -1;
+    b->sw.dn_any = getenv("QW_HIP_DN_ANY") != NULL, b->sw.nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
+    b->sw.no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, b->sw.shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
+    b->sw.split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
     return b;
 }
 
@@ -1046,7 +1056,7 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
     // one launch when the K range splits so that a workgroup holds whole (gate tile, up tile) pairs; else matvec, then SwiGLU
     unsigned sw = 0;
     for (unsigned s = 6; s > 1 && !sw; s--)
-        if (s != 4 && (unsigned)(p->D / 256) % s == 0 && !getenv("QW_HIP_NO_SWIGLU_MATVEC")) sw = s;
+        if (s != 4 && (unsigned)(p->D / 256) % s == 0 && !b->sw.no_swiglu_matvec) sw = s;
     if (sw) {
         m.split = sw, m.sums = 0, m.H = h, m.topk = (uint32_t)p->topk, m.hplane = sa.hplane;
         for (int j = 0; j < 2; j++) {
@@ -1055,8 +1065,7 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
         }
         if (!add_launch(b, "qwk_qmvm_swiglu", umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2)), 64 * QW_WAVES_GU, &m, sizeof m)) return false;
     } else if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
-    const char *e = getenv("QW_HIP_SIDE");
-    if (e ? e[0] == '1' : nbr <= 2)
+    if (b->sw.side < 0 ? nbr <= 2 : b->sw.side == 1)
         for (int i = first; i < b->nl; i++) b->l[i].side = true;
     return true;
 }
@@ -1095,7 +1104,7 @@ static bool tr_pre(qw_batch *b) {
     fname_fmt(fn, sizeof fn, "qwk_pre_w%d", p->rwf == 30 ? 30 : 1);
     unsigned grid = a.nrouter;
     const unsigned cpr = (unsigned)p->D / 512;
-    if (p->D % 512 == 0 && cpr <= 8 && !getenv("QW_HIP_SHARED_IN_GU")) {
+    if (p->D % 512 == 0 && cpr <= 8 && !b->sw.shared_in_gu) {
         const uint32_t nblk = (uint32_t)p->D / 256;
         const uint8_t *ps = p->fsg == 21 ? get_pack(b, b->pend_sg.hg, b->pend_sg.Wsg, b->pend_sg.hu, b->pend_sg.Wsu, (uint64_t)(p->I / 8), nblk, (uint32_t)rb, 8) : NULL;
         if (p->fsg == 8 || ps) {
@@ -1146,7 +1155,7 @@ static bool tr_gu(qw_batch *b) {
         if (cg == 1 || cs == 1) cg = cs = 1; // any-shape builds come in pairs
     }
     if (b->pend_sel.valid && b->pend_sel.a.sel == a.sel && b->pend_sel.a.nbr == nbr && b->pend_sel.a.E == (uint32_t)p->E && b->pend_sel.a.topk == (uint32_t)p->topk &&
-        b->pend_sel.a.gnb == (uint32_t)p->gnb && !getenv("QW_HIP_SPLIT_SELECT")) {
+        b->pend_sel.a.gnb == (uint32_t)p->gnb && !b->sw.split_select) {
         a.logits = b->pend_sel.a.logits;
         a.E = (uint32_t)p->E;
         b->pend_sel.valid = false;
@@ -1169,13 +1178,6 @@ static bool tr_gu(qw_batch *b) {
     return add_launch(b, intern(fn), persistent_grid(b->g, tasks, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 
-// Token count up to which the down projection and the combine run as one launch (QW_HIP_DNC_NB in the environment
-// overrides it, 0 turns the fusion off).
-static unsigned dnc_maxnb(void) {
-    const char *e = getenv("QW_HIP_DNC_NB");
-    const unsigned n = e ? (unsigned)atoi(e) : 2;
-    return n > QW_DNC_MAXNB ? QW_DNC_MAXNB : n;
-}
 static bool flush_dn(qw_batch *b) {
     if (!b->pend_dn.valid) return true;
     b->pend_dn.valid = false;
@@ -1223,7 +1225,7 @@ static bool tr_dn(qw_batch *b) {
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
     // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
     if ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8))) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
-    if (fd == 20 && p->I <= 640 && !getenv("QW_HIP_DN_ANY")) { // the range kernel with rows of up to 640 staged
+    if (fd == 20 && p->I <= 640 && !b->sw.dn_any) { // the range kernel with rows of up to 640 staged
         if (p->I % 320 == 0) { // tile-major copies, as for IQ3_S rows (the shared expert's only together with the routed ones)
             const uint32_t nch = (uint32_t)p->I / 320, tileb = nch * QW_NL_CHUNK_BYTES;
             const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wd, NULL, NULL, (uint64_t)p->E * (uint64_t)(p->D / 16), nch, a.rowbytes, QW_F_PACKED_NL);
@@ -1235,7 +1237,7 @@ static bool tr_dn(qw_batch *b) {
                 if (fs) fname_fmt(tail, sizeof tail, "_s%d_c%d", fs == 20 ? QW_F_PACKED_NL : fs, fs == 20 ? 10 : 4);
                 fname_fmt(fn, sizeof fn, "qwk_dnr_f120_c10%s", tail);
                 const unsigned grid = persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR);
-                if (nbr <= dnc_maxnb()) { // a few tokens: wait for the combine, the two run as one launch
+                if (nbr <= b->sw.dnc_nb) { // a few tokens: wait for the combine, the two run as one launch
                     char fu[48];
                     fname_fmt(fu, sizeof fu, "qwk_dnc_f120_c10%s", tail);
                     b->pend_dn.valid = true;
@@ -1246,7 +1248,7 @@ static bool tr_dn(qw_batch *b) {
                 return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
             }
         }
-        const int ch = p->I % 320 == 0 && !getenv("QW_HIP_NL_C4") ? 10 : 4; // blocks per chunk
+        const int ch = p->I % 320 == 0 && !b->sw.nl_c4 ? 10 : 4; // blocks per chunk
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d_s%d_c%d", ch, fs, fs == 20 ? ch : 4);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d", ch);
         return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR), 64 * QW_WAVES_DNR, &a, sizeof a);
@@ -1258,7 +1260,7 @@ static bool tr_dn(qw_batch *b) {
         const unsigned grid = persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR);
         // a few tokens: wait for the combine, the two run as one launch (tile-major IQ3_S or Q8_0 routed rows; a shared
         // expert in either of these)
-        if (nbr <= dnc_maxnb() && (fd == QW_F_PACKED || fd == 8) && (fs == 0 || fs == 8 || (fs == QW_F_PACKED && fd == QW_F_PACKED))) {
+        if (nbr <= b->sw.dnc_nb && (fd == QW_F_PACKED || fd == 8) && (fs == 0 || fs == 8 || (fs == QW_F_PACKED && fd == QW_F_PACKED))) {
             char fu[48];
             if (fs) fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
             else fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d", fd, ch);
