@@ -146,6 +146,14 @@ struct qw_gpu {
     hipStream_t side[2]; // one beside each stream: launches of a batch that do not depend on the ones before them (made at first use)
     hipEvent_t sev[256];  // fork / join events between a stream and its side stream, used round robin (made at first use)
     unsigned nsev;
+    // Launch sequences that come again unchanged (a decode step over resident weights) replayed as HIP graphs: hash of
+    // the sequence, a copy of it for the exact comparison, the instantiated graph; seen = hashes of the last sequences
+    // that were launched eagerly (a graph is built only when a sequence repeats). Off unless QW_HIP_GRAPH=1 / qw_hip_set_graphs.
+    struct qw_graph { uint64_t hash; int nl; size_t bytes; unsigned char *key; hipGraphExec_t exec; } graphs[8];
+    unsigned ngraph_next, ngraph_launches;
+    uint64_t seen_hash[8];
+    unsigned nseen;
+    bool use_graphs;
     float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes;
@@ -198,6 +206,8 @@ qw_gpu *qw_gpu_open(void) {
     {
         const char *e = getenv("QW_HIP_REPACK");
         g->repack = !(e && e[0] == '0');
+        e = getenv("QW_HIP_GRAPH"); // off unless asked for: measured as no gain on this path (the steps are bound by the GPU)
+        g->use_graphs = e && e[0] == '1';
     }
     { // build the pre-signed table once; every weight kernel copies it into LDS
         hipFunction_t f;
@@ -240,6 +250,10 @@ void qw_gpu_close(qw_gpu *g) {
     }
     free(g->packs);
     (void)hipFree(g->tabs);
+    for (int i = 0; i < 8; i++) {
+        if (g->graphs[i].exec) (void)hipGraphExecDestroy(g->graphs[i].exec);
+        free(g->graphs[i].key);
+    }
     (void)hipFree(g->shgu);
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
@@ -582,6 +596,8 @@ void qw_hip_buf_mark_dirty(qw_buf *b) {
     packs_drop(b->handle);
 }
 void qw_hip_set_repack(qw_gpu *g, bool on) { g->repack = on; }
+unsigned qw_hip_graph_launches(const qw_gpu *g) { return g->ngraph_launches; }
+void qw_hip_set_graphs(qw_gpu *g, bool on) { g->use_graphs = on; }
 size_t qw_hip_packed_bytes(const qw_gpu *g) { return g->pack_bytes; }
 void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle ? ((qw_hbuf *)b->handle)->dptr : NULL; }
 static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return off <= h->size && len <= h->size - off; }
@@ -1490,6 +1506,70 @@ static bool side_link(qw_gpu *g, hipStream_t from, hipStream_t to) {
     return HIPOK(g, hipEventRecord(*e, from)) && HIPOK(g, hipStreamWaitEvent(to, *e, 0));
 }
 
+// A batch's launches as a HIP graph. The key of a sequence is every launch's function, grid and argument record;
+// it is replayed only after an exact comparison. Returns 1 when the sequence ran as a graph, 0 when the caller should
+// launch it eagerly, -1 on an error. Graphs hold kernel nodes only (no copies, no memsets).
+static size_t graph_key(const qw_batch *b, unsigned char *out) {
+    size_t n = 0;
+    for (int i = 0; i < b->nl; i++) {
+        const qw_launch *l = &b->l[i];
+        const unsigned hdr[4] = {l->gx, l->bx, (unsigned)l->argsz, 0};
+        if (out) { memcpy(out + n, &l->f, sizeof l->f); memcpy(out + n + sizeof l->f, hdr, sizeof hdr); memcpy(out + n + sizeof l->f + sizeof hdr, l->args, l->argsz); }
+        n += sizeof l->f + sizeof hdr + l->argsz;
+    }
+    return n;
+}
+static int graph_run(qw_batch *b, hipStream_t st) {
+    qw_gpu *g = b->g;
+    if (!g->use_graphs || b->prof || b->done_l != 0 || b->nl < 8) return 0;
+    for (int i = 0; i < b->nl; i++)
+        if (b->l[i].side) return 0;
+    const size_t bytes = graph_key(b, NULL);
+    unsigned char *key = malloc(bytes);
+    if (!key) return 0;
+    graph_key(b, key);
+    uint64_t h = 1469598103934665603ull; // FNV-1a
+    for (size_t i = 0; i < bytes; i++) h = (h ^ key[i]) * 1099511628211ull;
+    for (int i = 0; i < 8; i++) {
+        struct qw_graph *c = &g->graphs[i];
+        if (c->exec && c->hash == h && c->nl == b->nl && c->bytes == bytes && !memcmp(c->key, key, bytes)) {
+            free(key);
+            g->ngraph_launches++;
+            return HIPOK(g, hipGraphLaunch(c->exec, st)) ? 1 : -1;
+        }
+    }
+    bool seen = false;
+    for (int i = 0; i < 8; i++) seen = seen || g->seen_hash[i] == h;
+    if (!seen) { // first time: eagerly, and remembered
+        g->seen_hash[g->nseen++ % 8] = h;
+        free(key);
+        return 0;
+    }
+    hipGraph_t graph = NULL;
+    hipGraphExec_t exec = NULL;
+    if (hipStreamBeginCapture(st, hipStreamCaptureModeRelaxed) != hipSuccess) { (void)hipGetLastError(); free(key); return 0; }
+    bool ok = true;
+    for (int i = 0; i < b->nl && ok; i++) {
+        qw_launch *l = &b->l[i];
+        void *params[] = {l->args};
+        ok = hipModuleLaunchKernel(l->f, l->gx, l->gy, l->gz, l->bx, 1, 1, 0, st, params, NULL) == hipSuccess;
+    }
+    if (hipStreamEndCapture(st, &graph) != hipSuccess || !ok || !graph || hipGraphInstantiate(&exec, graph, NULL, NULL, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        free(key);
+        g->use_graphs = false; // this runtime does not capture these launches: stay eager
+        return 0;
+    }
+    (void)hipGraphDestroy(graph);
+    struct qw_graph *c = &g->graphs[g->ngraph_next++ % 8];
+    if (c->exec) (void)hipGraphExecDestroy(c->exec);
+    free(c->key);
+    *c = (struct qw_graph){.hash = h, .nl = b->nl, .bytes = bytes, .key = key, .exec = exec};
+    g->ngraph_launches++;
+    return HIPOK(g, hipGraphLaunch(exec, st)) ? 1 : -1;
+}
+
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
@@ -1511,8 +1591,10 @@ static bool submit_segment(qw_batch *b) {
     if (!HIPOK(g, hipEventCreate(&ev[0])) || !HIPOK(g, hipEventCreate(&ev[1]))) { b->failed = true; return false; }
     b->nseg++;
     if (!HIPOK(g, hipEventRecord(ev[0], st))) { b->failed = true; return false; }
+    const int as_graph = graph_run(b, st);
+    if (as_graph < 0) { b->failed = true; return false; }
     bool side_open = false;
-    for (int i = b->done_l; i < b->nl; i++) {
+    for (int i = as_graph ? b->nl : b->done_l; i < b->nl; i++) {
         qw_launch *l = &b->l[i];
         if (l->side && !b->prof) { // fork: the side stream starts from where the main stream stands now
             if (!side_open && !(side_open = side_link(g, st, side_of(g, b->stream)))) { b->failed = true; return false; }

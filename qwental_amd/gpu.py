@@ -57,7 +57,7 @@ SYMBOLS = [
     ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
     ("qw_hip_buf_write_fd", _b, [_pb, _sz, _i, C.c_uint64, _sz]),
-    ("qw_hip_set_repack", None, [_vp, _b]),
+    ("qw_hip_set_repack", None, [_vp, _b]), ("qw_hip_graph_launches", C.c_uint, [_vp]), ("qw_hip_set_graphs", None, [_vp, _b]),
     ("qw_hip_packed_bytes", _sz, [_vp]),
     ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
     ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),

@@ -412,6 +412,40 @@ def test_iq4_nl_down_from_the_tile_major_copy(gpu, oracle, D, I, nb, fshd):
     assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
 
 
+@pytest.mark.parametrize("nb", [1, 16])
+def test_repeated_step_replayed_as_a_graph(gpu, oracle, nb):
+    """With graphs switched on, a step recorded again over the same buffers runs as a HIP graph from its second
+    repetition on. Six steps with
+    fresh activations each, eager work and synchronisations of the program between them (the reference run below):
+    every one must equal the eager run bit for bit."""
+    gpu.L.qw_hip_set_graphs(gpu.g, True)  # off by default
+    D, I, E, K = 1024, 512, 32, 4
+    rng = np.random.default_rng(4100 + nb)
+    m = synth.moe_layer(rng, D, I, E)
+    m["topk"] = K
+    path = q.Path(gpu, D, I, E, K, 16)
+    dl = DeviceLayer(gpu, m, device_only=True)
+    xb, outs = gpu.buf(nb * D * 2), [gpu.buf(nb * D * 2) for _ in range(3)]
+    lgs, sels = [gpu.buf(path.logits_bytes(nb)) for _ in range(3)], [gpu.buf(path.sel_bytes(nb)) for _ in range(3)]
+    before = gpu.L.qw_hip_graph_launches(gpu.g)
+    for step in range(6):
+        x = synth.activations(rng, nb, D)
+        xb.fill(x)
+        b = gpu.batch()
+        for i in range(3):  # three layers' worth of launches: long enough to be worth a graph
+            path.gg_moe(b, dl.layer, nb, xb, lgs[i], sels[i], outs[i])
+        assert b.end() >= 0, gpu.last_error()
+        got = [o_.view(np.uint16)[:nb * D].copy() for o_ in outs]
+        ref, _, _, _ = run_moe(gpu, path, dl, x, nb)  # fresh buffers: another sequence, launched eagerly
+        assert all(np.array_equal(g_, ref.view(np.uint16).ravel()) for g_ in got), step
+    gpu.L.qw_hip_set_graphs(gpu.g, os.environ.get("QW_HIP_GRAPH") == "1")
+    assert gpu.L.qw_hip_graph_launches(gpu.g) - before >= 4  # steps 1 .. 5 of the fixed buffers at least
+    for bb in [xb] + outs + lgs + sels:
+        bb.free()
+    dl.free()
+    path.close()
+
+
 def test_moe_batched_equals_single(gpu):
     """Each row of a batched layer call equals the single-token call bit for bit (src/engine.c:7977-7987)."""
     D, I, E, K, nb = 2048, 512, 64, 10, 8
