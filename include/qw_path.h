@@ -70,6 +70,13 @@ bool qw_path_gg_moe_lg(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
  * each in turn, out. Equivalent to nlayers calls of qw_path_gg_moe. */
 bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,
                           const qw_buf *sel, const qw_buf *out);
+/* After which layers of a stack the recorded part is submitted (qw_batch_flush) so that the GPU runs while the host
+ * records the rest: bit l = after layer l, the reference's vb_flush (src/engine.c:142, :5997, where the default is 0).
+ * Default here: 0x101 (after layers 0 and 8) — this backend launches at submit, so without it the GPU waits for the
+ * whole step to be recorded; measured on the 48-layer step at one token: 1.73 ms a step unsplit, 1.72 with bit 0, 1.65
+ * with bits 0 and 8, 1.72–1.97 with six flushes (each costs the host two events and a pass over the bound buffers).
+ * A batch takes at most 8 flushes; a profiled batch is never split. */
+void qw_path_set_flush(qw_path *p, uint64_t mask);
 /* Ragged batch through the packing path (the routed part of the reference's pf_moe(), src/engine.c:4203-4254, with
  * the kernels of kernels/moe_prefill.metal and moe_pf_gg): T rows of x, P = T * topk (token, expert) pairs given by
  * ids [P] (uint32) and weights w [P] (float); count -> plan -> scatter -> gate / up products -> SiLU -> down product

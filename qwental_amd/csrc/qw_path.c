@@ -17,6 +17,7 @@ struct qw_path {
     int pf_tmax, pf_tm;
     int rbf; // 1: moe_pre_gg computes the router (src/engine.c:577); 0: the logits are given
     unsigned pf_max_tiles;
+    uint64_t flush_mask; // bit l: submit what is recorded after layer l of a stack (src/engine.c:142, :5997 vb_flush)
 };
 
 static int blk_values(int type) { // src/gguf.c:15-25
@@ -52,7 +53,7 @@ qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool 
     if (!g || nbmax < 1 || nbmax > 16) return NULL;
     qw_path *p = calloc(1, sizeof *p);
     if (!p) return NULL;
-    *p = (qw_path){.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = nbmax};
+    *p = (qw_path){.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = nbmax, .flush_mask = 0x101};
     const size_t nb = (size_t)qw_path_nbv(nbmax);
     bool (*mk)(qw_gpu *, size_t, qw_buf *) = device_scratch ? qw_hip_buf_new_device : qw_buf_new;
     // sizes as the engine allocates them: H [nb][topk + 1][I] float, Psh [nb][D] float, Pg [nb][topk][D] float (src/engine.c:157)
@@ -292,10 +293,14 @@ static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const
 
 bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nlayers, int nb, const qw_buf *x, const qw_buf *lg,
                           const qw_buf *sel, const qw_buf *out) {
-    for (int l = 0; l < nlayers; l++)
+    for (int l = 0; l < nlayers; l++) {
         if (!qw_path_gg_moe(p, b, &M[l], nb, x, &lg[l], &sel[l], out)) return false;
+        // the recorded part goes to the GPU while the host records the rest (at most 8 times a batch, src/gpu.h:54-56)
+        if (l < 64 && (p->flush_mask >> l & 1) && l + 1 < nlayers) qw_batch_flush(b);
+    }
     return true;
 }
+void qw_path_set_flush(qw_path *p, uint64_t mask) { p->flush_mask = mask; }
 
 // ---------------------------------------------------------------- ragged batch through the packing path (src/engine.c:4133-4254)
 bool qw_path_pf_reserve(qw_path *p, int tmax, int tm) {

@@ -71,7 +71,7 @@ SYMBOLS = [
     ("qw_path_gg_router", _b, [_vp, _vp, _pm, _i, _pb, _pb]),
     ("qw_path_gg_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
-    ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]),
+    ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]), ("qw_path_set_flush", None, [_vp, C.c_uint64]),
     ("qw_path_scratch", _pb, [_vp, _i]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_pf_scratch", _pb, [_vp, _i]), ("qw_path_pf_max_tiles", C.c_uint, [_vp]),
@@ -321,6 +321,9 @@ class Path:
         """The layer with the caller's logits (forced routing)."""
         if not self.L.qw_path_gg_moe_lg(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
             raise RuntimeError("qw_path_gg_moe_lg failed")
+
+    def set_flush(self, mask):
+        self.L.qw_path_set_flush(self.p, mask)
 
     def gg_moe_stack(self, batch, layers_c, nlayers, nb, x, lg_c, sel_c, out):
         """layers_c: ctypes array of QwMoeLayer; lg_c / sel_c: ctypes arrays of QwBuf, one per layer."""

@@ -446,6 +446,41 @@ def test_repeated_step_replayed_as_a_graph(gpu, oracle, nb):
     path.close()
 
 
+def test_stack_flush_points_do_not_change_results(gpu, oracle):
+    """A stack of layers in one batch with the recorded part submitted after chosen layers (the reference's vb_flush,
+    src/engine.c:5997): the same results whatever the mask, and the GPU time still covers every segment."""
+    from qwental_amd.gpu import QwBuf, QwMoeLayer
+    D, I, E, K, nb, L = 1024, 512, 32, 4, 7, 5
+    rng = np.random.default_rng(5150)
+    ms = [synth.moe_layer(rng, D, I, E) for _ in range(L)]
+    for m in ms:
+        m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    path = q.Path(gpu, D, I, E, K, 16)
+    dls = [DeviceLayer(gpu, m, device_only=True) for m in ms]
+    layers_c = (QwMoeLayer * L)(*[d.layer.c for d in dls])
+    xb, out = gpu.buf_from(x), gpu.buf(nb * D * 2)
+    lgs, sels = [gpu.buf(path.logits_bytes(nb)) for _ in range(L)], [gpu.buf(path.sel_bytes(nb)) for _ in range(L)]
+    lg_c, sel_c = (QwBuf * L)(*[b_.c for b_ in lgs]), (QwBuf * L)(*[b_.c for b_ in sels])
+    res = {}
+    for mask in (0, 1, 0b1011, (1 << 64) - 1):
+        path.set_flush(mask)
+        b = gpu.batch()
+        path.gg_moe_stack(b, layers_c, L, nb, xb, lg_c, sel_c, out)
+        t = b.end()
+        assert t > 0, gpu.last_error()
+        res[mask] = (out.view(np.uint16)[:nb * D].copy(), [l_.view(np.uint32)[:nb * (E + 1)].copy() for l_ in lgs], t)
+    ref = oracle.moe_layer_f64(ms[L - 1], res[0][1][L - 1].view(np.float32).reshape(nb, E + 1), x)  # out holds the last layer's
+    assert maxrel(res[0][0].view(np.float16).reshape(nb, D), ref) <= TOL
+    for mask in res:
+        assert np.array_equal(res[mask][0], res[0][0]) and all(np.array_equal(a, b_) for a, b_ in zip(res[mask][1], res[0][1]))
+    for bb in [xb, out] + lgs + sels:
+        bb.free()
+    for d in dls:
+        d.free()
+    path.close()
+
+
 def test_moe_batched_equals_single(gpu):
     """Each row of a batched layer call equals the single-token call bit for bit (src/engine.c:7977-7987)."""
     D, I, E, K, nb = 2048, 512, 64, 10, 8
