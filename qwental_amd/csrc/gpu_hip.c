@@ -713,8 +713,8 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     const char *e = getenv("QW_HIP_DNC_NB"); // token count up to which down + combine run as one launch (0: never)
     b->sw.dnc_nb = e ? (unsigned)atoi(e) : 2;
     if (b->sw.dnc_nb > QW_DNC_MAXNB) b->sw.dnc_nb = QW_DNC_MAXNB;
-    e = getenv("QW_HIP_SIDE"); // the side stream: 0 never, 1 always, unset: with one or two tokens
-    b->sw.side = e ? (e[0] == '1' ? 1 : 0) : -1;
+    e = getenv("QW_HIP_SIDE"); // the side stream for launches that depend on the step's input alone: 1 on
+    b->sw.side = e && e[0] == '1';
     b->sw.dn_any = getenv("QW_HIP_DN_ANY") != NULL, b->sw.nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
     b->sw.no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, b->sw.shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
     b->sw.split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
@@ -1064,10 +1064,10 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
                        .rowbytes = {(uint32_t)fmt_rb(p->fsg, p->D), (uint32_t)fmt_rb(p->fsu, p->D)}, .ystride = {(uint32_t)p->I, (uint32_t)p->I}};
     qwk_shact_args sa = {.g = gy, .u = uy, .H = h, .I = (uint32_t)p->I, .nb = nbr, .topk = (uint32_t)p->topk, .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I};
     b->pend_sg.valid = false; // done here
-    // These two depend on x alone. With one or two tokens, where the layer is a chain of short launches, they run
-    // beside the router and the routed gate/up on the side stream (48 layers of the reference model's shape: 2.89 ->
-    // 2.70 ms a token); with more tokens the fork and join cost more than the overlap gives (6.81 -> 6.93 ms at 16).
-    // QW_HIP_SIDE in the environment: 0 never, 1 always.
+    // This work depends on x alone, so it may run beside the router and the routed gate/up on the side stream
+    // (QW_HIP_SIDE=1). Off by default: with the matvec and SwiGLU as two launches it paid with one or two tokens (48
+    // layers of the reference model's shape: 2.89 -> 2.70 ms a token) and cost with more (6.81 -> 6.93 ms at 16); as
+    // the one launch it is now, the fork and join cost as much as the overlap gives at every token count.
     const int first = b->nl;
     // one launch when the K range splits so that a workgroup holds whole (gate tile, up tile) pairs; else matvec, then SwiGLU
     unsigned sw = 0;
@@ -1081,7 +1081,7 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
         }
         if (!add_launch(b, "qwk_qmvm_swiglu", umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2)), 64 * QW_WAVES_GU, &m, sizeof m)) return false;
     } else if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
-    if (b->sw.side < 0 ? nbr <= 2 : b->sw.side == 1)
+    if (b->sw.side == 1)
         for (int i = first; i < b->nl; i++) b->l[i].side = true;
     return true;
 }
