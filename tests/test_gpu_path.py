@@ -535,11 +535,11 @@ def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd
     plane = nbv * (K + 1) * I
     H = (Hraw[:nb * (K + 1) * I].astype(np.float32) + Hraw[plane:plane + nb * (K + 1) * I].astype(np.float32)).reshape(nb, K + 1, I)
     assert maxrel(H[:, K], H32[:, K]) <= 1e-5
-    # unprofiled, the two shared launches run on a side stream beside the router and the routed gate/up: three layers
+    # with QW_HIP_SIDE=1 (and no profiling) the shared expert's launches run on a side stream beside the router and the routed gate/up: three layers
     # in one batch (three forks and joins), twice, against the same launches kept in line
     def three(side):
         old = os.environ.pop("QW_HIP_SIDE", None)
-        os.environ["QW_HIP_SIDE"] = "1" if side else "0"  # by default the side stream is taken with one or two tokens only
+        os.environ["QW_HIP_SIDE"] = "1" if side else "0"  # off by default
         try:
             xb = gpu.buf_from(x)
             lgs, sels, outs = [gpu.buf(path.logits_bytes(nb)) for _ in range(3)], [gpu.buf(path.sel_bytes(nb)) for _ in range(3)], [gpu.buf(nb * D * 2) for _ in range(3)]
