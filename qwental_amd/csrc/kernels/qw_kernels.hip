@@ -130,7 +130,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_nl(qwk_pack_args a) {
 template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(const qwk_qmv_args &a, u2 *lut, u4 *xf, f4 *red) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4;
-    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
     const uint32_t cpr = a.K / (C::BLK_K * CH);
     const uint32_t nl = lane >> 2, kl = lane & 3; // (row, k-group) this lane loads
     auto rowp = [&](uint32_t t) {
@@ -357,7 +357,7 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args 
         }
         __syncthreads();
     }
-    const uint32_t lane = qw_lane(), nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t lane = qw_lane(), nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
     const qw_afrag_kq af = {L.xf, L.xs, lane & 15, lane >> 4};
     const bool k256 = a.K % 256 == 0;
     uint32_t toff = 0; // tiles (split == 1) or tile groups (split > 1) of the matrices before j
@@ -905,7 +905,9 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
         qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
         __syncthreads();
     };
-    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    // Waves are numbered wave-major (wave w of workgroup b is number w * gridDim.x + b), so that when the tiles do not
+    // divide evenly the waves with one tile more are spread over all compute units instead of filling the first ones.
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x;
     if (FSG != 0) {
         if (a.Wsg) { // the shared expert's tiles go to the first waves
             qwk_gu_args sa = a;
@@ -1341,7 +1343,7 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
     if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook (IQ3_S never meets it here)
     qw_sel_load(*sc, a.sel, K, gnb);
     __syncthreads();
-    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
     if (FSD != 0) {
         if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, 1>(a, lut, w0, nw);
     }
@@ -1476,7 +1478,7 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
     if (mine) atomicAdd(cnt, mine);
     __syncthreads();
     const uint32_t used = *cnt, ntn = a.ntn, ntasks = used * ntn, cpr = a.K / (C::BLK_K * CH);
-    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = blockIdx.x * (blockDim.x >> 6) + qw_wave();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
     f4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
     qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3,
         [&](uint32_t task) {
