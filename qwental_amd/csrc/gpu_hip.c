@@ -1191,7 +1191,10 @@ static bool tr_gu(qw_batch *b) {
     if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", fgu, cg, fs, cs);
     else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", fgu, cg);
     const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (fs ? (unsigned)p->I / 8 : 0);
-    return add_launch(b, intern(fn), persistent_grid(b->g, tasks, QW_WAVES_GU), 64 * QW_WAVES_GU, &a, sizeof a);
+    // With few tiles (one or two tokens: 640 to 1280 of them) every compute unit still gets a workgroup: the waves are
+    // numbered wave-major, so the tiles spread over all compute units instead of filling the waves of the first
+    // workgroups (48-layer step at one token: gate/up launch 18.3 -> 13.4 us, 615 -> 715 tokens/s).
+    return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, tasks), 64 * QW_WAVES_GU, &a, sizeof a);
 }
 
 static bool flush_dn(qw_batch *b) {
