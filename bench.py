@@ -106,23 +106,66 @@ def copy_calibration(gpu, nbytes=1 << 30):
     dst.free()
 
 
-def cpu_baseline(stack, x, nb, lg_dev, budget_s=20.0):
+def cpu_baseline(stack, x_dev, xh, nb, budget_s=20.0):
     """The CPU oracle (float dot products over dequantized rows, OpenMP over all cores) on the first layers of the
-    same stack with the same logits; stops after about budget_s seconds. Also the full-size parity check."""
+    same stack, timed; stops after about budget_s seconds of oracle time. Every sampled layer is also the full-size
+    parity check of the benchmarked configuration: the stack call with l + 1 layers leaves layer l's output, which is
+    compared with the oracle's (binary16 both), and the layer's picks with the oracle's own router and top-k."""
     from oracle import oracle as o
     cores = o.max_threads()
-    t_used, n, worst = 0.0, 0, 0.0
-    while t_used < budget_s and n < stack.L and n < len(lg_dev):
+    t_used, n, worst, topk_ok = 0.0, 0, 0.0, True
+    while t_used < budget_s and n < stack.L:
+        stack.step(x_dev, nb, nlayers=n + 1)
+        got = stack.out.view(np.float16)[:nb * stack.D].reshape(nb, stack.D).astype(np.float64)
+        lg = stack.lg[n].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy()
         m = stack.layer_weights_host(n)
-        lg = lg_dev[n]
         t0 = time.perf_counter()
-        out32, _, _ = o.moe_layer_f32(m, lg, x[:nb], 8 if nb <= 8 else 16)
+        out32, _, _ = o.moe_layer_f32(m, lg, xh[:nb], 8 if nb <= 8 else 16)
         t_used += time.perf_counter() - t0
+        ref = out32.astype(np.float64)
+        worst = max(worst, float(np.abs(got - ref).max() / np.abs(ref).max()))
+        topk_ok = topk_ok and bool(np.array_equal(o.topk_ids(lg, stack.topk), o.topk_ids(o.router(m["Wr"], m["wsg"], xh[:nb]), stack.topk)))
         n += 1
         del m
     per_layer = t_used / n
     return {"value": nb / (per_layer * stack.L), "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": "oracle moe_layer_f32 on layers 0..%d of the stack (B = %d), %.1f s; scaled to %d layers" % (n - 1, nb, t_used, stack.L)}
+            "sample": "oracle moe_layer_f32 on layers 0..%d of the stack (B = %d), %.1f s; scaled to %d layers" % (n - 1, nb, t_used, stack.L),
+            "max_rel_err": worst, "topk_identical": topk_ok, "layers_compared": n, "tolerance": 2e-3}
+
+
+def read_ceiling(gpu, stack, nb, reps=5):
+    """What this device gives a kernel that only reads (the method of bench/moe_bw.c:50-89 and kernels/ceiling_mem.metal of
+    the reference): (a) the pure-read kernel over the resident gate/up rows of the experts the last step picked, one
+    launch per layer over the same bytes the gate/up launch streams (one contiguous range per layer of the same
+    size: the experts' rows themselves are contiguous pieces of 901,120 bytes); (b) the same kernel over 1 GiB; (c) the
+    copy kernel over 1 GiB (read + write)."""
+    ok, err = gpu.compile("#define QW_HIP_MEM 1\n")
+    assert ok, err
+    sink = gpu.buf(64, device_only=True)
+    U = stack.unique_experts(nb)
+
+    def timed(kernel, launches):
+        best = 1e9
+        for _ in range(reps):
+            b = gpu.batch()
+            b.kernel(gpu.kernel(kernel))
+            for src, off, n, dst in launches:
+                b.buf(0, src, off)
+                b.buf(1, dst)
+                b.bytes(2, np.array([n // 16, 0], np.uint64))
+                b.dispatch(256 * 8)
+            best = min(best, b.end())
+        return best
+    # (a) per layer: U_l experts' gate/up bytes out of the layer's weight buffer (each layer another 692 MB allocation)
+    launches = [(stack.bufs[3 * l], 0, U[l] * stack.gu_bytes, sink) for l in range(stack.L)]
+    t = timed("qw_bw_read", launches)
+    out = {"gate_up_bytes_per_layer_GBps": sum(n for _, _, n, _ in launches) / t / 1e9, "us_per_launch": t / stack.L * 1e6}
+    big, big2 = gpu.buf(1 << 30, device_only=True), gpu.buf(1 << 30, device_only=True)
+    out["read_1GiB_GBps"] = (1 << 30) / timed("qw_bw_read", [(big, 0, 1 << 30, sink)]) / 1e9
+    out["copy_1GiB_GBps_read_plus_write"] = 2 * (1 << 30) / timed("qw_copy", [(big, 0, 1 << 30, big2)]) / 1e9
+    for bb in (sink, big, big2):
+        bb.free()
+    return out
 
 
 def ragged_steps(gpu, stack, reps=5):
@@ -132,7 +175,7 @@ def ragged_steps(gpu, stack, reps=5):
     path (count -> prefix sums -> scatter -> grouped product -> combine) in one pass. Routed experts' bytes are read
     once per group on the first way and once on the second; the table gives the crossover in rows per step."""
     from qwental_amd import synth
-    from oracle import oracle as o
+    from qwental_amd.gpu import SelRecord
     layer, path, E, K, D = stack.layers[0], stack.path, stack.E, stack.topk, stack.D
     out = []
     for target in (16, 32, 64, 128):
@@ -153,7 +196,7 @@ def ragged_steps(gpu, stack, reps=5):
             for (g0, nb), (xb, lb, sb, ob) in zip(groups, bufs):
                 path.gg_moe_lg(b, layer, nb, xb, lb, sb, ob)
             t_dec = min(t_dec, b.end())
-        w = np.concatenate([o.Sel(sb.view(np.uint8).copy(), 8 if nb <= 8 else 16, K).w[:nb, :K] for (g0, nb), (xb, lb, sb, ob) in zip(groups, bufs)])
+        w = np.concatenate([SelRecord(sb.view(np.uint8).copy(), 8 if nb <= 8 else 16, K).w[:nb, :K] for (g0, nb), (xb, lb, sb, ob) in zip(groups, bufs)])
         path.pf_reserve(T, 16)
         xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.astype(np.float32).ravel()), gpu.buf(T * D * 2)
         t_pk = 1e9
@@ -458,6 +501,7 @@ def main():
             "config": {"workload": "configs[4]: %d-layer MoE FFN stack decode, B=%d, D=2048 I=512 E=512 top-10, IQ3_S experts, shared expert Q8_0 every 4th layer" % (stack.L, nb),
                        "resident_weight_bytes": int(stack.weight_bytes), "packed_copy_bytes": int(gpu.L.qw_hip_packed_bytes(gpu.g)), "device": gpu.name()},
             "roofline": roof,
+            "read_ceiling": read_ceiling(gpu, stack, nb),
             "stack": {"GBps_algorithmic": res[nb]["stack_GBps"], "frac_of_peak": res[nb]["stack_GBps"] / HBM_PEAK_GBS, "gpu_ms_per_step": res[nb]["gpu_ms_per_step"],
                       "mean_unique_experts": res[nb]["mean_U"], "bytes_per_step": res[nb]["bytes_per_step"]},
             "by_batch": {str(k): v for k, v in res.items()},
@@ -470,8 +514,7 @@ def main():
         line["gguf_load"] = gguf_load(gpu)
         line["model_shape"] = model_shape_leg(gpu, a.layers, min(a.steps, 10), a.warmup)  # 92 GB beside the 67 GB of the main stack
     if not a.no_cpu:
-        lg = [stack.lg[l].read(dtype=np.float32)[:nb * (stack.E + 1)].reshape(nb, stack.E + 1).copy() for l in range(stack.L)]
-        line["cpu_baseline"] = cpu_baseline(stack, xh, nb, lg)
+        line["cpu_baseline"] = cpu_baseline(stack, x, xh, nb)
     x.free()
     stack.free()
     print(json.dumps(line))

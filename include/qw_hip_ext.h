@@ -5,7 +5,10 @@
  *   - host -> device, when a batch is submitted, for every buffer a dispatch of the batch binds:
  *       a buffer of at most QW_HIP_SMALL_BYTES is copied every time;
  *       a larger one is copied the first time it is bound and again only after qw_hip_buf_mark_dirty();
- *       qw_buf_wrap() buffers are copied once; device-only buffers never.
+ *       qw_buf_wrap() buffers are copied once; device-only buffers never;
+ *       none of this for a buffer that a submitted batch (or an earlier, flushed part of this one) binds in an
+ *       output role and that has not been waited for yet: HBM then holds the newer contents (a layer's output that the
+ *       next layer reads), and they stay until the wait copies them back.
  *   - device -> host, when the batch completes, for every buffer bound in an output role:
  *       always, unless the buffer is device-only or larger than QW_HIP_BIG_OUT_BYTES (then: qw_hip_buf_download()).
  */
@@ -55,6 +58,19 @@ size_t qw_hip_packed_bytes(const qw_gpu *g);
  * environment at qw_gpu_open, or qw_hip_set_graphs(g, true), turns it on. Number of batches run as graphs so far: */
 void qw_hip_set_graphs(qw_gpu *g, bool on);
 unsigned qw_hip_graph_launches(const qw_gpu *g);
+
+/* Measurement switches, read from the environment by every qw_batch_begin(). Each routes a layer through kernels that
+ * other shapes or formats reach by themselves, so that both forms can be timed on one shape; results do not change
+ * (tests/test_gpu_path.py runs a layer with each of them set).
+ *   QW_HIP_DNC_NB=n           token count up to which moe_dn_gg + moe_cmb_gg run as one launch (default 2, at most 4; 0: never)
+ *   QW_HIP_SIDE=1             a shared expert's gate/up in the K-quant / IQ4 / plain formats runs on a side stream beside the router
+ *   QW_HIP_DN_ANY             IQ4_NL down rows take the any-shape kernel instead of the range kernel
+ *   QW_HIP_NL_C4              IQ4_NL down rows from GGUF order in chunks of four blocks instead of ten
+ *   QW_HIP_NO_SWIGLU_MATVEC   such a shared expert's gate/up as two launches (matvec, then SwiGLU) instead of one
+ *   QW_HIP_SHARED_IN_GU       an IQ3_S / Q8_0 shared expert's gate/up inside the gate/up launch instead of the front launch
+ *   QW_HIP_SPLIT_SELECT       the selection as a launch of its own instead of inside the gate/up launch
+ * QW_HIP_REPACK=0 and QW_HIP_GRAPH=1 are read once, by qw_gpu_open() (see above); QW_HIP_LOAD_THREADS by qw_hip_buf_write_fd();
+ * QW_HIP_VERBOSE prints every error text to stderr as it is set, QW_HIP_QUIET keeps qw_batch_wait from printing one. */
 
 /* The define-block front end of qw_gpu_compile() without a device: parses src as qw_gpu_compile would, and on
  * success writes the names of the kernels it would register to names (comma separated). For host-side tests. */

@@ -31,11 +31,13 @@ def _run(cmd):
     return out
 
 
-def build(verbose=False):
-    out = _run([HIPCC] + HIPFLAGS + ["--genco", "-I", os.path.join(CSRC, "kernels"), "-o", HSACO,
-                                    os.path.join(CSRC, "kernels", "qw_kernels.hip")])
-    if verbose and out.strip():
-        print(out)
+def build(verbose=False, kernels=True):
+    """kernels=False keeps the code object of the last build (host-side iterations: `python -m qwental_amd.build --host-only`)."""
+    if kernels or not os.path.exists(HSACO):
+        out = _run([HIPCC] + HIPFLAGS + ["--genco", "-I", os.path.join(CSRC, "kernels"), "-o", HSACO,
+                                        os.path.join(CSRC, "kernels", "qw_kernels.hip")])
+        if verbose and out.strip():
+            print(out)
     out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
                 "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), os.path.join(CSRC, "qw_par.c"), "-pthread", "-o", LIB,
                 "-L", os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
@@ -43,9 +45,9 @@ def build(verbose=False):
         print(out)
     # command-line tool with the reference's dqtest contract
     _run([CLANG, "-std=c23", "-O2", "-Wall", "-I", os.path.join(ROOT, "include"), os.path.join(CSRC, "tools", "dqhip.c"), "-o",
-          os.path.join(HERE, "dqhip"), "-L", HERE, "-lqwgpu_hip", "-Wl,-rpath," + HERE, "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+          os.path.join(HERE, "dqhip"), "-L", HERE, "-lqwgpu_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
     return LIB
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, kernels="--host-only" not in sys.argv))

@@ -31,7 +31,7 @@ enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES 
 typedef enum {
     FAM_DQ_TEST, FAM_QMV_GG, FAM_QMV_GGM, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
     FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
-    FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PF, // ragged packing and the grouped product
+    FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PK_ZERO, FAM_PF, // ragged packing and the grouped product
 } qw_family;
 
 typedef struct { // parameters taken from the define block
@@ -58,6 +58,8 @@ typedef struct qw_hbuf {
     bool wrapped, device_only;
     bool dirty;      // host copy is newer than HBM (or HBM never received it)
     unsigned mark;   // scratch for de-duplication while a batch is submitted
+    int pending_out; // submitted batches that bind it in an output role and have not been waited for: HBM is newer than the shadow
+    uint64_t out_seq; // the last batch that counted itself in pending_out
     struct qw_gpu *g;
     int npack;       // packed copies made from this buffer (dropped when its contents change)
 } qw_hbuf;
@@ -98,6 +100,9 @@ struct qw_batch {
     int nl, capl, done_l; // done_l: launches already submitted by a flush
     qw_use *use;
     int nuse, capuse, done_use;
+    uint64_t seq;      // this batch's number (qw_hbuf.out_seq)
+    qw_hbuf **outs;    // buffers whose pending_out this batch raised
+    int nouts, capouts;
     hipEvent_t ev[2 * 9]; // start/stop per submitted segment (end + at most 8 flushes)
     int nseg;
     hipEvent_t *pev;      // profiling: 2 events per launch
@@ -139,6 +144,7 @@ struct qw_gpu {
     const char *prof_fname[QW_PROF_MAX];
     double prof_us[QW_PROF_MAX];
     unsigned mark;
+    uint64_t batch_seq;
     qw_pack *packs;
     int npacks, cappacks;
     struct qw_ldlane { void *pin[2]; hipStream_t st; hipEvent_t ev[2]; } ld[QW_LD_MAX]; // staging of qw_hip_buf_write_fd, made at first use
@@ -464,7 +470,8 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
         if (p.K < 8 || p.K % 8 || p.I < 1 || p.tm < 1) FAIL("moe_prefill: KD %d / I %d / TM %d outside this build (KD a multiple of 8)", p.K, p.I, p.tm);
         if (!reg_kernel(g, d, n, "moe_count", FAM_PK_COUNT, &p, err, errlen) || !reg_kernel(g, d, n, "moe_plan", FAM_PK_PLAN, &p, err, errlen) ||
             !reg_kernel(g, d, n, "moe_plan_t", FAM_PK_PLAN_T, &p, err, errlen) || !reg_kernel(g, d, n, "moe_scatter", FAM_PK_SCATTER, &p, err, errlen) ||
-            !reg_kernel(g, d, n, "moe_act", FAM_PK_ACT, &p, err, errlen) || !reg_kernel(g, d, n, "p_act2", FAM_PK_ACT2, &p, err, errlen) || !reg_kernel(g, d, n, "moe_combine", FAM_PK_COMBINE, &p, err, errlen)) { ok = false; goto out; }
+            !reg_kernel(g, d, n, "moe_act", FAM_PK_ACT, &p, err, errlen) || !reg_kernel(g, d, n, "p_act2", FAM_PK_ACT2, &p, err, errlen) || !reg_kernel(g, d, n, "moe_combine", FAM_PK_COMBINE, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "p_zero", FAM_PK_ZERO, &p, err, errlen)) { ok = false; goto out; }
     }
     if (def_get(d, n, "QW_HIP_MEM")) { // this backend's own measurement helpers
         p = (qw_kparams){0};
@@ -522,7 +529,7 @@ bool qw_buf_new(qw_gpu *g, size_t size, qw_buf *out) {
         if (!h->host) { (void)hipFree(h->dptr); free(h); return false; }
     }
     h->own_host = true;
-    h->dirty = false; // both sides are zero
+    h->dirty = true; // the caller may fill it through ptr at any time before its first use: the first bind copies it
     out->handle = h;
     out->ptr = h->host;
     out->size = size;
@@ -707,6 +714,7 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     qw_batch *b = calloc(1, sizeof *b);
     if (!b) return NULL;
     b->g = g;
+    b->seq = ++g->batch_seq;
     b->stream = g->cur_stream;
     b->prof = g->prof;
     g->err[0] = 0;
@@ -990,6 +998,10 @@ static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf 
         qw_hbuf *h = hs[i];
         if (!h) continue;
         if (!h->device_only && !h->wrapped && h->size <= QW_HIP_SMALL_BYTES) return NULL;
+        // A dispatch recorded earlier in this batch writes the source and has not been launched yet (launches wait for
+        // the submit): a copy made now would hold the old bytes.
+        for (int u = b->done_use; u < b->nuse; u++)
+            if (b->use[u].b == h && b->use[u].out) return NULL;
         if (h->dirty && h->host) { // what the next submit would do for this buffer
             if (hipMemcpyAsync(h->dptr, h->host, h->size, hipMemcpyHostToDevice, g->stream[b->stream]) != hipSuccess) return NULL;
             h->dirty = false;
@@ -1325,6 +1337,11 @@ static bool tr_pk_count(qw_batch *b) { // 0 ids, 1 counts, 2 P
     if (!bind_bytes(b, 2, &a.P, 4, "P") || !bind_ptr(b, 0, (size_t)a.P * 4, false, "ids", (void **)&a.ids) || !bind_ptr(b, 1, (size_t)a.E * 4, true, "counts", (void **)&a.counts)) return false;
     return add_launch(b, "qwk_moe_count", cdiv(a.P, 256), 256, &a, sizeof a);
 }
+static bool tr_pk_zero(qw_batch *b) { // kernels/prefill.metal:601-603: 0 x, 1 n (dwords to clear)
+    qwk_zero_args a = {0};
+    if (!bind_bytes(b, 1, &a.n, 4, "n") || !bind_ptr(b, 0, (size_t)a.n * 4, true, "x", (void **)&a.x)) return false;
+    return add_launch(b, "qwk_zero", cdiv(a.n, 256), 256, &a, sizeof a);
+}
 static bool tr_pk_plan(qw_batch *b, bool tm_bound) { // 0 counts, 1 offs, 2 cursor, 3 tiles, 4 max_tiles (, 5 tm)
     const qw_kparams *p = &b->k->p;
     qwk_plan_args a = {.E = (uint32_t)p->E, .tm = (uint32_t)p->tm};
@@ -1482,6 +1499,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     case FAM_DN: ok = tr_dn(b); break;
     case FAM_CMB: ok = tr_cmb(b); break;
     case FAM_FILL_BLOCKS: ok = tr_fill_blocks(b); break;
+    case FAM_PK_ZERO: ok = tr_pk_zero(b); break;
     case FAM_PK_COUNT: ok = tr_pk_count(b); break;
     case FAM_PK_PLAN: ok = tr_pk_plan(b, false); break;
     case FAM_PK_PLAN_T: ok = tr_pk_plan(b, true); break;
@@ -1585,10 +1603,24 @@ static bool submit_segment(qw_batch *b) {
         if (h->mark == mark) continue;
         h->mark = mark;
         if (h->device_only || !h->host) continue;
+        // A kernel of a batch that was submitted (or of an earlier segment of this one) and not yet waited for wrote
+        // this buffer: HBM holds the newer contents, and the shadow must not overwrite them.
+        if (h->pending_out > 0 && !h->dirty) continue;
         if (h->dirty || (!h->wrapped && h->size <= QW_HIP_SMALL_BYTES)) {
             if (!HIPOK(g, hipMemcpyAsync(h->dptr, h->host, h->size, hipMemcpyHostToDevice, st))) { b->failed = true; return false; }
             h->dirty = false;
         }
+    }
+    for (int i = b->done_use; i < b->nuse; i++) { // outputs of this segment: the device side is the newer one until the batch is waited for
+        qw_hbuf *h = b->use[i].b;
+        if (!b->use[i].out || h->device_only || !h->host || h->wrapped || h->out_seq == b->seq) continue;
+        if (b->nouts == b->capouts) {
+            b->capouts = b->capouts ? 2 * b->capouts : 16;
+            b->outs = realloc(b->outs, sizeof *b->outs * (size_t)b->capouts);
+        }
+        h->out_seq = b->seq;
+        h->pending_out++;
+        b->outs[b->nouts++] = h;
     }
     hipEvent_t *ev = &b->ev[2 * b->nseg];
     if (!HIPOK(g, hipEventCreate(&ev[0])) || !HIPOK(g, hipEventCreate(&ev[1]))) { b->failed = true; return false; }
@@ -1645,6 +1677,8 @@ bool qw_batch_poll(qw_batch *b) {
 }
 
 static void batch_free(qw_batch *b) {
+    for (int i = 0; i < b->nouts; i++) b->outs[i]->pending_out--;
+    free(b->outs);
     for (int i = 0; i < 2 * b->nseg; i++) (void)hipEventDestroy(b->ev[i]);
     for (int i = 0; i < b->npev; i++) (void)hipEventDestroy(b->pev[i]);
     free(b->pev);

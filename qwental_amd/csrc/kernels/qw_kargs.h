@@ -164,6 +164,10 @@ typedef struct {
 
 /* Ragged packing of (token, expert) pairs and the grouped product over the packed rows (kernels/moe_prefill.metal,
  * kernels/moe_gg.metal:761-838). P pairs, flat index p = token * topk + rank. */
+typedef struct { /* clear n dwords (kernels/prefill.metal:601-603) */
+    uint32_t *x;
+    uint32_t n, pad;
+} qwk_zero_args;
 typedef struct {
     const uint32_t *ids; /* [P] expert of pair p */
     uint32_t *counts;    /* [E] */

@@ -1379,6 +1379,12 @@ QW_DN_ANY(20, 0, qwk_dn_f20_any) QW_DN_ANY(20, 20, qwk_dn_f20_any_s20) QW_DN_ANY
 // ================================================================ ragged packing (kernels/moe_prefill.metal:15-119)
 // P (token, expert) pairs -> per-expert counts -> exclusive prefix sums (first packed row of every expert, tile table)
 // -> rows copied to packed order -> grouped product -> gathered, weighted sum. Integer work; bit-exact.
+// The counters are cleared on the device, inside the recorded sequence (kernels/prefill.metal:601-603): a batch may hold
+// the packing sequence several times, and all of it is recorded before any of it runs.
+extern "C" __global__ __launch_bounds__(256) void qwk_zero(qwk_zero_args a) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < a.n) a.x[i] = 0;
+}
 extern "C" __global__ __launch_bounds__(256) void qwk_moe_count(qwk_count_args a) {
     const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p < a.P && a.ids[p] < a.E) atomicAdd(&a.counts[a.ids[p]], 1u);

@@ -16,6 +16,7 @@ struct qw_path {
     qw_buf pcnt, poffs, pcur, ptiles, ppos, pXs, pGg, pGu, pH, pDm;
     int pf_tmax, pf_tm;
     int rbf; // 1: moe_pre_gg computes the router (src/engine.c:577); 0: the logits are given
+    bool device_scratch; // scratch without host shadows (qw_path_open)
     unsigned pf_max_tiles;
     uint64_t flush_mask; // bit l: submit what is recorded after layer l of a stack (src/engine.c:142, :5997 vb_flush)
 };
@@ -53,7 +54,7 @@ qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool 
     if (!g || nbmax < 1 || nbmax > 16) return NULL;
     qw_path *p = calloc(1, sizeof *p);
     if (!p) return NULL;
-    *p = (qw_path){.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = nbmax, .flush_mask = 0x101};
+    *p = (qw_path){.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = nbmax, .flush_mask = 0x101, .device_scratch = device_scratch};
     const size_t nb = (size_t)qw_path_nbv(nbmax);
     bool (*mk)(qw_gpu *, size_t, qw_buf *) = device_scratch ? qw_hip_buf_new_device : qw_buf_new;
     // sizes as the engine allocates them: H [nb][topk + 1][I] float, Psh [nb][D] float, Pg [nb][topk][D] float (src/engine.c:157)
@@ -311,10 +312,12 @@ bool qw_path_pf_reserve(qw_path *p, int tmax, int tm) {
     const size_t P = (size_t)tmax * (size_t)p->topk, E = (size_t)p->E;
     p->pf_max_tiles = (unsigned)((P + (size_t)tm - 1) / (size_t)tm + E); // src/engine.c:4135
     p->pf_tmax = 0;
-    if (!qw_buf_new(p->g, E * 4, &p->pcnt) || !qw_buf_new(p->g, E * 4, &p->poffs) || !qw_buf_new(p->g, E * 4, &p->pcur) ||
-        !qw_buf_new(p->g, (size_t)p->pf_max_tiles * 16, &p->ptiles) || !qw_buf_new(p->g, P * 4, &p->ppos) || !qw_buf_new(p->g, P * (size_t)p->D * 2, &p->pXs) ||
-        !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pGg) || !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pGu) || !qw_buf_new(p->g, P * (size_t)p->I * 2, &p->pH) ||
-        !qw_buf_new(p->g, P * (size_t)p->D * 2, &p->pDm)) return false;
+    // with host shadows every one of these (several MB at full size) would be copied back at every wait
+    bool (*mk)(qw_gpu *, size_t, qw_buf *) = p->device_scratch ? qw_hip_buf_new_device : qw_buf_new;
+    if (!mk(p->g, E * 4, &p->pcnt) || !mk(p->g, E * 4, &p->poffs) || !mk(p->g, E * 4, &p->pcur) ||
+        !mk(p->g, (size_t)p->pf_max_tiles * 16, &p->ptiles) || !mk(p->g, P * 4, &p->ppos) || !mk(p->g, P * (size_t)p->D * 2, &p->pXs) ||
+        !mk(p->g, P * (size_t)p->I * 2, &p->pGg) || !mk(p->g, P * (size_t)p->I * 2, &p->pGu) || !mk(p->g, P * (size_t)p->I * 2, &p->pH) ||
+        !mk(p->g, P * (size_t)p->D * 2, &p->pDm)) return false;
     p->pf_tmax = tmax;
     p->pf_tm = tm;
     return true;
@@ -363,7 +366,12 @@ bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const
     }
     const uint32_t P = (uint32_t)T * (uint32_t)p->topk, tm = (uint32_t)p->pf_tm, n = P * (uint32_t)p->I;
     qw_kernel *k;
-    memset(p->pcnt.ptr, 0, p->pcnt.size); // the engine clears the counters on the GPU (p_zero); here the host shadow is copied at submit
+    const uint32_t ne = (uint32_t)p->E; // the counters are cleared on the GPU, inside the batch (src/engine.c:4201-4206)
+    if (!(k = pk_kernel(p, "p_zero"))) return false;
+    qw_batch_kernel(b, k);
+    qw_batch_buf(b, 0, &p->pcnt, 0);
+    qw_batch_bytes(b, 1, &ne, 4);
+    qw_batch_dispatch(b, (ne + 255) / 256, 1, 1, 256, 1, 1);
     if (!(k = pk_kernel(p, "moe_count"))) return false;
     qw_batch_kernel(b, k);
     qw_batch_buf(b, 0, ids, 0);

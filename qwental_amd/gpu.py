@@ -165,6 +165,23 @@ class Buf:
         return C.byref(self.c)
 
 
+class SelRecord:
+    """The selection record a layer leaves (kernels/moe_gg.metal:110-116 of the reference; QW_SEL_* in csrc/kernels/qw_kargs.h):
+    U | ue[GU] | mask[GU] | slot[GU][gnb] | w[gnb][topk + 1] with GU = gnb * topk; gnb = 8 for up to 8 tokens, else 16."""
+
+    def __init__(self, raw, gnb, topk):
+        gu = gnb * topk
+        raw = np.ascontiguousarray(raw, np.uint8)
+        self.gnb, self.topk = gnb, topk
+        self.U = int(raw[:4].view(np.uint32)[0])
+        self.ue = raw[4:4 + 4 * gu].view(np.uint32)
+        self.mask = raw[4 + 4 * gu:4 + 8 * gu].view(np.uint32)
+        o = 4 + 8 * gu
+        self.slot = raw[o:o + gu * gnb].reshape(gu, gnb)
+        o += gu * gnb
+        self.w = raw[o:o + 4 * gnb * (topk + 1)].view(np.float32).reshape(gnb, topk + 1)
+
+
 class Tensor:
     def __init__(self, buf, ftype, offset=0):
         self.buf, self.ftype, self.offset = buf, ftype, offset

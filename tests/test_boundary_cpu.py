@@ -113,7 +113,7 @@ def test_packing_blocks_register_the_reference_names():
     blk = "#define moe_scatter moe_scatter_x\n#define E 512\n#define TOPK 10\n#define KD 2048\n#define I 512\n#define TM 64\n"  # bench/moe_prefill.c:86-87
     ok, err, names = compile_check(blk)
     assert ok, err
-    assert names == ["moe_count", "moe_plan", "moe_plan_t", "moe_scatter_x", "moe_act", "p_act2", "moe_combine"]
+    assert names == ["moe_count", "moe_plan", "moe_plan_t", "moe_scatter_x", "moe_act", "p_act2", "moe_combine", "p_zero"]
     pf = ("#define IQ_DQ_ONLY\n#define E 512\n#define TOPK 10\n#define D 2048\n#define I 512\n#define NB 1\n#define GG_PART 5\n#define PFF 21\n#define KD 2048\n"
           "#define TM 64\n#define TN 64\n#define SG 4\n#define KC 64\n#define PFS 1\n#define PFT 1\n#define PFDBG 0\n#define moe_pf_gg moe_pf_gg_21_k2048_tm64\n")  # src/engine.c:3244-3248
     ok, err, names = compile_check(pf)
@@ -145,3 +145,18 @@ def test_valu_gemv_is_asked_for_by_a_macro():
     blk = "#define qmv_gg q1\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 2\n#define YT float\n#define QW_VALU 1\n"
     ok, err, names = compile_check(blk)
     assert ok and names == ["q1"]
+
+
+def test_reference_clients_link_against_the_library():
+    """The reference's tools/dqtest.c and tools/ggmtest.c, compiled unchanged by oracle/Makefile (`make ref`, where the
+    reference tree is mounted), ask the library for nothing it does not export."""
+    import subprocess
+    L = q.load_lib()
+    exes = [os.path.join(ROOT, "oracle", "_ref", n) for n in ("dqtest_ref", "ggmtest_ref")]
+    if not os.path.isdir("/root/reference"):
+        pytest.skip("no reference tree here")
+    for exe in exes:
+        assert os.path.exists(exe), "oracle/_ref is stale: run `make -C oracle ref` after building the library"
+        und = subprocess.run(["nm", "-D", "--undefined-only", exe], stdout=subprocess.PIPE, text=True, check=True).stdout
+        asked = set(re.findall(r"\b(qw_[a-z0-9_]+)", und))
+        assert asked and all(hasattr(L, n) for n in asked), asked

@@ -662,3 +662,94 @@ def test_packed_copy_follows_the_source(gpu, oracle):
         assert maxrel(yb.view(np.float32)[:nb * N].reshape(nb, N), oracle.qmv(21, W, N, K, x, f64=True)) <= 1e-5
     for bb in (wb, xb, yb):
         bb.free()
+
+
+@pytest.mark.parametrize("switch,shape,want", [
+    ("QW_HIP_SPLIT_SELECT", (2048, 512, 64, 10, 16, 21, 21, 21, 21, None), "qwk_select"),                 # the selection as a launch of its own
+    ("QW_HIP_SHARED_IN_GU", (2048, 512, 64, 10, 16, 21, 21, 21, 21, None), "qwk_gu_f121_c2_s121_c2"),    # shared gate/up inside the gate/up launch
+    ("QW_HIP_NL_C4", (1024, 640, 32, 10, 6, 21, 20, 8, 20, None), "qwk_dnr_f20_c4_s20_c4"),              # IQ4_NL down in chunks of four blocks
+    ("QW_HIP_NO_SWIGLU_MATVEC", (2560, 640, 32, 10, 4, 21, 20, 12, 20, 23), "qwk_sh_act"),               # shared gate/up: matvec, then SwiGLU
+])
+def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, oracle, switch, shape, want):
+    """The environment switches that qw_batch_begin reads (include/qw_hip_ext.h) route a layer through kernels that other
+    shapes reach by themselves; with a switch set the named kernel runs and the layer still meets the float64 oracle."""
+    D, I, E, K, nb, fgu, fd, fsh, fshd, fshu = shape
+    rng = np.random.default_rng(len(switch) + D)
+    m = synth.moe_layer(rng, D, I, E, fgu=fgu, fd=fd, fsh=fsh, fshd=fshd, fshu=fshu)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    dl = DeviceLayer(gpu, m, device_only=switch != "QW_HIP_NL_C4")  # host-shadowed rows: no tile-major copy of the IQ4_NL matrix
+    old = os.environ.get(switch)
+    outs = {}
+    try:
+        for on in (False, True):
+            os.environ.pop(switch, None)
+            if on:
+                os.environ[switch] = "1"
+            path = q.Path(gpu, D, I, E, K, 16)
+            gpu.profile(True)
+            out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            assert (want in names) == on, (on, names)
+            assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+            outs[on] = out
+            path.close()
+    finally:
+        os.environ.pop(switch, None)
+        if old is not None:
+            os.environ[switch] = old
+    if switch in ("QW_HIP_SPLIT_SELECT", "QW_HIP_NO_SWIGLU_MATVEC"):  # the same products in the same order (the shared gate/up inside
+        # the gate/up launch adds a row's blocks one after the other, the front launch per chunk first)
+        assert np.array_equal(outs[False].view(np.uint16), outs[True].view(np.uint16))
+    dl.free()
+
+
+def test_chained_layers_across_a_flush_keep_the_device_results(gpu, oracle):
+    """Two layers in one batch, the first one's output the second one's input, with the recorded part submitted in
+    between (qw_batch_flush) and every buffer host-visible: the second segment must read what the first one's kernels
+    left in HBM, not the buffer's host side (still zero until the batch is waited for)."""
+    D, I, E, K, nb = 1024, 512, 32, 4, 8
+    rng = np.random.default_rng(77)
+    # the first layer's output is a few hundred times larger than N(0, 1): the second layer's block scales are drawn that much
+    # smaller, so that its binary16 output stays finite
+    ma, mb = synth.moe_layer(rng, D, I, E), synth.moe_layer(rng, D, I, E, d_scale=synth.MOE_D_SCALE / 50)
+    ma["topk"] = mb["topk"] = K
+    x = synth.activations(rng, nb, D)
+    path = q.Path(gpu, D, I, E, K, 16)
+    da, db = DeviceLayer(gpu, ma), DeviceLayer(gpu, mb)
+    xb, mid, out = gpu.buf_from(x), gpu.buf(nb * D * 2), gpu.buf(nb * D * 2)
+    lgs, sels = [gpu.buf(path.logits_bytes(nb)) for _ in range(2)], [gpu.buf(path.sel_bytes(nb)) for _ in range(2)]
+    for flush in (False, True):
+        mid.view(np.uint16)[:] = 0
+        b = gpu.batch()
+        path.gg_moe(b, da.layer, nb, xb, lgs[0], sels[0], mid)
+        if flush:
+            b.flush()
+        path.gg_moe(b, db.layer, nb, mid, lgs[1], sels[1], out)
+        b.end()
+        h = mid.view(np.float16)[:nb * D].reshape(nb, D).copy()
+        assert maxrel(h, oracle.moe_layer_f64(ma, lgs[0].view(np.float32)[:nb * (E + 1)].reshape(nb, E + 1), x)) <= TOL
+        lg1 = lgs[1].view(np.float32)[:nb * (E + 1)].reshape(nb, E + 1).copy()
+        assert maxrel(lg1, oracle.router(mb["Wr"], mb["wsg"], h)) <= 1e-5, flush  # the second layer saw the first one's output
+        got = out.view(np.float16)[:nb * D].reshape(nb, D)
+        assert np.isfinite(got.astype(np.float64)).all() and np.abs(got.astype(np.float64)).max() > 0
+        assert maxrel(got, oracle.moe_layer_f64(mb, lg1, h)) <= TOL, flush
+    # the same across two batches, the first one submitted and not waited for when the second is submitted
+    mid.view(np.uint16)[:] = 0
+    b1 = gpu.batch()
+    path.gg_moe(b1, da.layer, nb, xb, lgs[0], sels[0], mid)
+    gpu.L.qw_batch_submit(b1.b)
+    b2 = gpu.batch()
+    path.gg_moe(b2, db.layer, nb, mid, lgs[1], sels[1], out)
+    gpu.L.qw_batch_submit(b2.b)
+    assert gpu.L.qw_batch_wait(b1.b) >= 0 and gpu.L.qw_batch_wait(b2.b) >= 0
+    h = mid.view(np.float16)[:nb * D].reshape(nb, D).copy()
+    lg1 = lgs[1].view(np.float32)[:nb * (E + 1)].reshape(nb, E + 1).copy()
+    assert maxrel(lg1, oracle.router(mb["Wr"], mb["wsg"], h)) <= 1e-5
+    assert maxrel(out.view(np.float16)[:nb * D].reshape(nb, D), oracle.moe_layer_f64(mb, lg1, h)) <= TOL
+    for bb in [xb, mid, out] + lgs + sels:
+        bb.free()
+    da.free()
+    db.free()
+    path.close()
