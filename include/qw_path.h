@@ -88,6 +88,30 @@ bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const
 const qw_buf *qw_path_pf_scratch(const qw_path *p, int which);
 unsigned qw_path_pf_max_tiles(const qw_path *p);
 
+/* The layer for callers that cannot allocate. No counterpart in the reference: it exists for callers that must not call
+ * hipMalloc or any allocating routine while they run the layer — a stream under HIP graph capture, a tight serving loop,
+ * a harness that forbids allocation. It is qw_path_gg_moe() (same dispatches, same kernels, same results bit for bit)
+ * with plain device pointers: the weights, x [nb][D] and out [nb][D] (binary16) are the caller's device memory; the
+ * layer's intermediates (logits, selection record, H, Psh, Pg: what qw_path_open() allocates for qw_path_gg_moe()) live
+ * in a per-device array of 4 MiB inside the library that the device holds until the process ends. Limits (larger shapes
+ * are refused with a message): QW_NOALLOC_MAX_NB tokens, D <= QW_NOALLOC_MAX_D, I <= QW_NOALLOC_MAX_I, E <=
+ * QW_NOALLOC_MAX_E, topk <= QW_NOALLOC_MAX_TOPK, and the formats qw_path_gg_moe() takes. The call records and launches on
+ * `stream` (a hipStream_t; NULL = the stream qw_gpu_set_stream selected) and returns without waiting: no device or pinned
+ * memory is allocated or freed, no event or stream is made, nothing is copied, and a tile-major copy of the weights is
+ * used when an earlier allocating call made one, never made here (the GGUF rows are read directly otherwise; same
+ * results). Every call on a device uses the same array, which keeps the last call's contents (nothing in it has to
+ * start from zero): calls that overlap on one device, on any streams, race. */
+#define QW_NOALLOC_MAX_NB 16
+#define QW_NOALLOC_MAX_D 2560
+#define QW_NOALLOC_MAX_I 640
+#define QW_NOALLOC_MAX_E 1024
+#define QW_NOALLOC_MAX_TOPK 16
+typedef struct { /* device addresses and ggml types of one layer's weights (qw_moe_layer without the buffers) */
+    const void *router, *sh_gate_w, *gate, *up, *down, *sh_gate, *sh_up, *sh_down;
+    int router_type, gate_type, down_type, sh_gate_type, sh_up_type, sh_down_type;
+} qw_moe_weights_dev;
+bool qw_path_gg_moe_noalloc(qw_gpu *g, int D, int I, int E, int topk, const qw_moe_weights_dev *W, int nb, const void *x, void *out, void *stream);
+
 /* The scratch buffers, for tests: 0 = lookup tables, 1 = H, 2 = Psh, 3 = Pg. */
 const qw_buf *qw_path_scratch(const qw_path *p, int which);
 

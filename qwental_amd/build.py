@@ -2,9 +2,10 @@
 
     python -m qwental_amd.build
 
-Two steps, both cross-compile without a GPU:
+Three steps, all cross-compile without a GPU:
   1. hipcc --genco: csrc/kernels/qw_kernels.hip -> csrc/qw_kernels_gfx950.hsaco
-  2. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c + csrc/qw_gguf.c + csrc/qw_par.c -> qwental_amd/libqwgpu_hip.so
+  2. hipcc -c: csrc/qw_noalloc.hip (host + device: the per-device scratch array of the entry point that allocates nothing) -> csrc/qw_noalloc.o
+  3. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c + csrc/qw_gguf.c + csrc/qw_par.c + qw_noalloc.o -> qwental_amd/libqwgpu_hip.so
 """
 import os
 import subprocess
@@ -38,8 +39,10 @@ def build(verbose=False, kernels=True):
                                         os.path.join(CSRC, "kernels", "qw_kernels.hip")])
         if verbose and out.strip():
             print(out)
+    noalloc_o = os.path.join(CSRC, "qw_noalloc.o")
+    _run([HIPCC] + HIPFLAGS + ["-fPIC", "-I", CSRC, "-I", os.path.join(ROOT, "include"), "-c", os.path.join(CSRC, "qw_noalloc.hip"), "-o", noalloc_o])
     out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-                "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), os.path.join(CSRC, "qw_par.c"), "-pthread", "-o", LIB,
+                "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), os.path.join(CSRC, "qw_par.c"), noalloc_o, "-pthread", "-o", LIB,
                 "-L", os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
     if verbose and out.strip():
         print(out)

@@ -11,6 +11,7 @@
 #define __HIP_PLATFORM_AMD__ 1
 #include "gpu.h"
 #include "qw_hip_ext.h"
+#include "qw_internal.h"
 #include "kernels/qw_kargs.h"
 #include <hip/hip_runtime_api.h>
 #include <pthread.h>
@@ -100,6 +101,8 @@ struct qw_batch {
     int nl, capl, done_l; // done_l: launches already submitted by a flush
     qw_use *use;
     int nuse, capuse, done_use;
+    bool noalloc;      // the device's static recorder (qw_hip_batch_begin_static): fixed storage, no tile-major copies made
+    hipStream_t xstream; // noalloc: the caller's stream (NULL: the device's)
     uint64_t seq;      // this batch's number (qw_hbuf.out_seq)
     qw_hbuf **outs;    // buffers whose pending_out this batch raised
     int nouts, capouts;
@@ -160,6 +163,11 @@ struct qw_gpu {
     uint64_t seen_hash[8];
     unsigned nseen;
     bool use_graphs;
+    void *na_scratch;    // the scratch array of the no-allocation entry point on this device (csrc/qw_noalloc.hip); NULL: set-up failed
+    size_t na_bytes;
+    const char *na_err;
+    struct qw_batch *na_batch; // its recorder, with fixed storage (made by qw_gpu_open)
+    bool na_busy;
     float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes;
@@ -231,6 +239,13 @@ qw_gpu *qw_gpu_open(void) {
             return NULL;
         }
     }
+    // the entry point that allocates nothing: its scratch array's address on this device and its recorder, made now
+    if (!qw_noalloc_scratch(g->dev, &g->na_scratch, &g->na_bytes, &g->na_err)) g->na_scratch = NULL;
+    g->na_batch = calloc(1, sizeof *g->na_batch);
+    if (g->na_batch) {
+        g->na_batch->capl = 64, g->na_batch->l = calloc(64, sizeof(qw_launch));
+        g->na_batch->capuse = 1024, g->na_batch->use = calloc(1024, sizeof(qw_use));
+    }
     return g;
 }
 
@@ -261,6 +276,7 @@ void qw_gpu_close(qw_gpu *g) {
         free(g->graphs[i].key);
     }
     (void)hipFree(g->shgu);
+    if (g->na_batch) { free(g->na_batch->l); free(g->na_batch->use); free(g->na_batch); }
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
     free(g);
@@ -772,6 +788,7 @@ static bool bind_ptr(qw_batch *b, unsigned index, size_t need, bool out, const c
     if (out) packs_drop(h); // a kernel is about to write it
     *p = (char *)h->dptr + off;
     if (b->nuse == b->capuse) {
+        if (b->noalloc) return fail(b, "%s: more than %d bindings in the fixed recorder", b->k->name, b->capuse);
         b->capuse = b->capuse ? 2 * b->capuse : 64;
         b->use = realloc(b->use, sizeof *b->use * (size_t)b->capuse);
     }
@@ -793,6 +810,7 @@ static bool add_launch(qw_batch *b, const char *fname, unsigned gx, unsigned bx,
     if (!f) return fail(b, "%s: entry point %s missing from the code object", b->k->name, fname);
     if (gx == 0) return true; // nothing to do
     if (b->nl == b->capl) {
+        if (b->noalloc) return fail(b, "%s: more than %d launches in the fixed recorder", b->k->name, b->capl);
         b->capl = b->capl ? 2 * b->capl : 64;
         b->l = realloc(b->l, sizeof *b->l * (size_t)b->capl);
     }
@@ -993,6 +1011,7 @@ static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf 
         const qw_pack *p = &g->packs[i];
         if (p->A == A && p->B == B && p->ntiles == ntiles && p->nblk == nblk && p->split == split) return p->dst;
     }
+    if (b->noalloc) return NULL; // a copy that exists was found above; none is made here
     qw_hbuf *hs[2] = {ha, hb};
     for (int i = 0; i < 2; i++) {
         qw_hbuf *h = hs[i];
@@ -1742,6 +1761,48 @@ double qw_batch_end(qw_batch *b) {
 }
 
 void qw_gpu_set_stream(qw_gpu *g, int s) { g->cur_stream = s == 1 ? 1 : 0; }
+
+// ---------------------------------------------------------------- the recorder with fixed storage (qw_internal.h)
+_Static_assert(sizeof(qw_hbuf) <= sizeof(qw_hip_view), "qw_hip_view is too small for a buffer handle");
+void qw_hip_view_init(qw_gpu *g, qw_hip_view *v, void *devptr, size_t size, qw_buf *out) {
+    qw_hbuf *h = (qw_hbuf *)v;
+    memset(h, 0, sizeof *h);
+    h->dptr = devptr;
+    h->size = size;
+    h->device_only = true;
+    h->g = g;
+    *out = (qw_buf){.handle = h, .ptr = NULL, .size = size};
+}
+bool qw_hip_noalloc_scratch(qw_gpu *g, void **ptr, size_t *bytes) {
+    if (!g->na_scratch) { set_err(g, "no scratch array on this device: %s", g->na_err ? g->na_err : "not set up"); return false; }
+    *ptr = g->na_scratch;
+    *bytes = g->na_bytes;
+    return true;
+}
+qw_batch *qw_hip_batch_begin_static(qw_gpu *g, void *stream) {
+    qw_batch *b = g->na_batch;
+    if (!b || !b->l || !b->use || g->na_busy) return NULL;
+    qw_launch *l = b->l;
+    qw_use *use = b->use;
+    memset(b, 0, sizeof *b);
+    *b = (qw_batch){.g = g, .seq = ++g->batch_seq, .stream = g->cur_stream, .noalloc = true, .xstream = (hipStream_t)stream, .l = l, .capl = 64, .use = use, .capuse = 1024};
+    b->sw.dnc_nb = 2; // the defaults of qw_batch_begin; the measurement switches of the environment do not apply here
+    g->na_busy = true;
+    g->err[0] = 0;
+    return b;
+}
+bool qw_hip_batch_launch_static(qw_batch *b) {
+    qw_gpu *g = b->g;
+    hipStream_t st = b->xstream ? b->xstream : g->stream[b->stream];
+    bool ok = !b->failed && flush_select(b) && flush_pf(b) && flush_dn(b) && !b->failed;
+    for (int i = 0; ok && i < b->nl; i++) {
+        qw_launch *l = &b->l[i];
+        void *params[] = {l->args};
+        ok = HIPOK(g, hipModuleLaunchKernel(l->f, l->gx, l->gy, l->gz, l->bx, 1, 1, 0, st, params, NULL));
+    }
+    g->na_busy = false;
+    return ok;
+}
 
 // ---------------------------------------------------------------- profiling and bench utilities
 void qw_profile_enable(qw_gpu *g, bool on) { g->prof = on; }

@@ -2,6 +2,7 @@
 // (src/engine.c:439-724), written against the interface only. See include/qw_path.h.
 #include "qw_path.h"
 #include "qw_hip_ext.h"
+#include "qw_internal.h"
 #include "kernels/qw_kargs.h"
 #include <stdio.h>
 #include <stdlib.h>
@@ -412,4 +413,64 @@ bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const
     qw_batch_buf(b, 3, out, 0);
     qw_batch_dispatch(b, (unsigned)p->D / 4 / 64, (unsigned)T, 1, 64, 1, 1);
     return true;
+}
+
+// ---------------------------------------------------------------- the layer without any allocation (include/qw_path.h)
+// qw_path_gg_moe over memory the caller owns and the device's scratch array: the same dispatches, translators and
+// kernels, recorded into the device's fixed recorder and launched on the caller's stream.
+bool qw_path_gg_moe_noalloc(qw_gpu *g, int D, int I, int E, int topk, const qw_moe_weights_dev *W, int nb, const void *x, void *out, void *stream) {
+    if (!g || !W || !x || !out) return false;
+    if (nb < 1 || nb > QW_NOALLOC_MAX_NB || D < 256 || D > QW_NOALLOC_MAX_D || I < 256 || I > QW_NOALLOC_MAX_I || E < 1 || E > QW_NOALLOC_MAX_E || topk < 1 ||
+        topk > QW_NOALLOC_MAX_TOPK) {
+        fprintf(stderr, "qw_path_gg_moe_noalloc: nb %d / D %d / I %d / E %d / top-%d beyond what the scratch array holds (%d tokens, D %d, I %d, E %d, top-%d)\n", nb, D, I, E,
+                topk, QW_NOALLOC_MAX_NB, QW_NOALLOC_MAX_D, QW_NOALLOC_MAX_I, QW_NOALLOC_MAX_E, QW_NOALLOC_MAX_TOPK);
+        return false;
+    }
+    void *base;
+    size_t have;
+    if (!qw_hip_noalloc_scratch(g, &base, &have)) {
+        fprintf(stderr, "qw_path_gg_moe_noalloc: %s\n", qw_hip_last_error(g));
+        return false;
+    }
+    // the array, cut at its largest shape (so that every shape finds its pieces at the same places), 256-byte aligned
+    const size_t nbv = 16, gnb = 16, sz[7] = {QW_TAB_BYTES, nbv * (QW_NOALLOC_MAX_E + 1) * 4, QW_SEL_BYTES(gnb, (size_t)QW_NOALLOC_MAX_TOPK),
+                                              nbv * (QW_NOALLOC_MAX_TOPK + 1) * (size_t)QW_NOALLOC_MAX_I * 4, nbv * (size_t)QW_NOALLOC_MAX_D * 4,
+                                              nbv * QW_NOALLOC_MAX_TOPK * (size_t)QW_NOALLOC_MAX_D * 4, 16};
+    size_t off[7], end = 0;
+    for (int i = 0; i < 7; i++) off[i] = end, end = (end + sz[i] + 255) & ~(size_t)255;
+    if (end > have) {
+        fprintf(stderr, "qw_path_gg_moe_noalloc: the scratch array holds %zu bytes, the layer's intermediates need %zu\n", have, end);
+        return false;
+    }
+    qw_hip_view v[7 + 10];
+    qw_buf s[7], w[8], xb, ob;
+    for (int i = 0; i < 7; i++) qw_hip_view_init(g, &v[i], (char *)base + off[i], sz[i], &s[i]);
+    const int rt = W->router_type;
+    if ((rt != 1 && rt != 30) || !blk_values(W->gate_type) || !blk_values(W->down_type) || !blk_values(W->sh_gate_type) || !blk_values(W->sh_up_type) || !blk_values(W->sh_down_type)) {
+        fprintf(stderr, "qw_path_gg_moe_noalloc: unknown weight type\n");
+        return false;
+    }
+    const size_t e = (size_t)E, ws[8] = {e * (size_t)D * 2, (size_t)D * 2, e * (size_t)I * (size_t)row_bytes(W->gate_type, D), e * (size_t)I * (size_t)row_bytes(W->gate_type, D),
+                                         e * (size_t)D * (size_t)row_bytes(W->down_type, I), (size_t)I * (size_t)row_bytes(W->sh_gate_type, D), (size_t)I * (size_t)row_bytes(W->sh_up_type, D),
+                                         (size_t)D * (size_t)row_bytes(W->sh_down_type, I)};
+    const void *wp[8] = {W->router, W->sh_gate_w, W->gate, W->up, W->down, W->sh_gate, W->sh_up, W->sh_down};
+    for (int i = 0; i < 8; i++) {
+        if (!wp[i]) return false;
+        qw_hip_view_init(g, &v[7 + i], (void *)(uintptr_t)wp[i], ws[i], &w[i]);
+    }
+    qw_hip_view_init(g, &v[15], (void *)(uintptr_t)x, (size_t)nb * (size_t)D * 2, &xb);
+    qw_hip_view_init(g, &v[16], out, (size_t)nb * (size_t)D * 2, &ob);
+    const qw_moe_layer M = {.router = {&w[0], 0, rt}, .sh_gate_w = {&w[1], 0, rt}, .gate = {&w[2], 0, W->gate_type}, .up = {&w[3], 0, W->gate_type}, .down = {&w[4], 0, W->down_type},
+                            .sh_gate = {&w[5], 0, W->sh_gate_type}, .sh_up = {&w[6], 0, W->sh_up_type}, .sh_down = {&w[7], 0, W->sh_down_type}};
+    // the kernels of this backend read its own table, never the caller's: no gg_tab_init dispatch here
+    qw_path p = {.g = g, .D = D, .I = I, .E = E, .topk = topk, .nbmax = QW_NOALLOC_MAX_NB, .tab = s[0], .H = s[3], .psh = s[4], .pd = s[5], .cnt = s[6], .tab_ready = true};
+    qw_batch *b = qw_hip_batch_begin_static(g, stream);
+    if (!b) {
+        fprintf(stderr, "qw_path_gg_moe_noalloc: the device's fixed recorder is missing or in use\n");
+        return false;
+    }
+    const bool rec = gg_moe(&p, b, &M, nb, &xb, &s[1], &s[2], &ob, false);
+    const bool ok = qw_hip_batch_launch_static(b) && rec; // also releases the recorder when the recording failed (nothing is launched then)
+    if (!ok) fprintf(stderr, "qw_path_gg_moe_noalloc: %s\n", qw_hip_last_error(g));
+    return ok;
 }

@@ -28,6 +28,11 @@ class QwMoeLayer(C.Structure):
     _fields_ = [(n, QwTensor) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")]
 
 
+class QwMoeWeightsDev(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")] + \
+               [(n, C.c_int) for n in ("router_type", "gate_type", "down_type", "sh_gate_type", "sh_up_type", "sh_down_type")]
+
+
 class QwGgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("model", C.c_char_p), ("part", C.c_uint), ("kind", C.c_int), ("type", C.c_uint32), ("nd", C.c_uint32),
                 ("dims", C.c_uint64 * 4), ("rows", C.c_uint64), ("rowbytes", C.c_uint64), ("nbytes", C.c_uint64), ("shard", C.c_int),
@@ -73,6 +78,7 @@ SYMBOLS = [
     ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]), ("qw_path_set_flush", None, [_vp, C.c_uint64]),
     ("qw_path_scratch", _pb, [_vp, _i]),
+    ("qw_path_gg_moe_noalloc", _b, [_vp, _i, _i, _i, _i, C.POINTER(QwMoeWeightsDev), _i, _vp, _vp, _vp]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_pf_scratch", _pb, [_vp, _i]), ("qw_path_pf_max_tiles", C.c_uint, [_vp]),
     # qw_gguf.h
