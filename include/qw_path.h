@@ -77,6 +77,22 @@ bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nl
  * with bits 0 and 8, 1.72–1.97 with six flushes (each costs the host two events and a pass over the bound buffers).
  * A batch takes at most 8 flushes; a profiled batch is never split. */
 void qw_path_set_flush(qw_path *p, uint64_t mask);
+/* A ragged step of one layer, the way the reference's scheduler hands it over (qw_engine_par_vstep, src/engine.c:9138-9161,
+ * and qw_engine_par_step, :8798-8814): slot i contributes n[i] >= 1 consecutive rows of x [R][D] (binary16), its first row
+ * being r0[i] = n[0] + ... + n[i - 1]; R = sum n[i] <= QW_PAR_MAX. The rows are cut into groups of at most 16 by par's
+ * measured table (qw_par_split), each group runs the layer in a batch of its own (the weights of the experts it picks are
+ * read once per group) into the same rows of out [R][D], and the wall time of every group is fed back to par
+ * (qw_par_observe; the first sample of a size is dropped, as src/engine.c:9037 does). A row's result does not depend on
+ * the group it falls into (bit for bit). The path must have been opened for 16 tokens. info (may be NULL) receives the cut.
+ * The packing path (qw_path_pf_moe) is the other form of such a step when the routing is known to the caller;
+ * qw_par_choose() weighs the two. */
+typedef struct {
+    int rows, ngroups, groups[64], r0[64];
+    double gpu_ms, wall_ms; /* summed over the groups */
+} qw_vstep_info;
+struct qw_par;
+bool qw_path_par_vstep(qw_path *p, struct qw_par *par, const qw_moe_layer *M, const int *n, int B, const qw_buf *x, const qw_buf *out, qw_vstep_info *info);
+
 /* Ragged batch through the packing path (the routed part of the reference's pf_moe(), src/engine.c:4203-4254, with
  * the kernels of kernels/moe_prefill.metal and moe_pf_gg): T rows of x, P = T * topk (token, expert) pairs given by
  * ids [P] (uint32) and weights w [P] (float); count -> plan -> scatter -> gate / up products -> SiLU -> down product

@@ -2,6 +2,7 @@
 // (src/engine.c:439-724), written against the interface only. See include/qw_path.h.
 #include "qw_path.h"
 #include "qw_hip_ext.h"
+#include "qw_par.h"
 #include "qw_internal.h"
 #include "kernels/qw_kargs.h"
 #include <stdio.h>
@@ -20,6 +21,7 @@ struct qw_path {
     bool device_scratch; // scratch without host shadows (qw_path_open)
     unsigned pf_max_tiles;
     uint64_t flush_mask; // bit l: submit what is recorded after layer l of a stack (src/engine.c:142, :5997 vb_flush)
+    qw_buf vlg, vsel;    // logits and selection record of one group of a ragged step (qw_path_par_vstep), made at first use
 };
 
 static int blk_values(int type) { // src/gguf.c:15-25
@@ -70,6 +72,7 @@ qw_path *qw_path_open(qw_gpu *g, int D, int I, int E, int topk, int nbmax, bool 
 void qw_path_close(qw_path *p) {
     if (!p) return;
     qw_buf_free(&p->tab); qw_buf_free(&p->H); qw_buf_free(&p->psh); qw_buf_free(&p->pd); qw_buf_free(&p->cnt);
+    qw_buf_free(&p->vlg); qw_buf_free(&p->vsel);
     qw_buf *pf[] = {&p->pcnt, &p->poffs, &p->pcur, &p->ptiles, &p->ppos, &p->pXs, &p->pGg, &p->pGu, &p->pH, &p->pDm};
     for (size_t i = 0; i < sizeof pf / sizeof *pf; i++) qw_buf_free(pf[i]);
     free(p);
@@ -203,7 +206,11 @@ bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
 }
 
 // src/engine.c:568-647: front part (router + shared gate/up + selection) -> routed gate/up + shared down -> routed down -> combine
-static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, bool given);
+static bool gg_moe_at(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, size_t xoff, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, size_t outoff,
+                      bool given);
+static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, bool given) {
+    return gg_moe_at(p, b, M, nb, x, 0, lg, sel, out, 0, given);
+}
 bool qw_path_gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel,
                     const qw_buf *out) {
     return gg_moe(p, b, M, nb, x, lg, sel, out, false);
@@ -212,7 +219,9 @@ bool qw_path_gg_moe_lg(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, c
                        const qw_buf *out) {
     return gg_moe(p, b, M, nb, x, lg, sel, out, true);
 }
-static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, bool given) {
+// x and out may be rows of larger buffers (byte offsets): the rows of one group of a step
+static bool gg_moe_at(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, size_t xoff, const qw_buf *lg, const qw_buf *sel, const qw_buf *out, size_t outoff,
+                      bool given) {
     p->rbf = given ? 0 : 1;
     if (nb < 1 || nb > p->nbmax) {
         fprintf(stderr, "gg_moe: %d tokens, scratch was sized for %d\n", nb, p->nbmax);
@@ -240,7 +249,7 @@ static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const
     qw_batch_kernel(b, k);
     bind_t(b, 0, &M->router);
     bind_t(b, 1, &M->sh_gate_w);
-    qw_batch_buf(b, 2, x, 0);
+    qw_batch_buf(b, 2, x, xoff);
     qw_batch_buf(b, 3, lg, 0);
     qw_batch_buf(b, 4, &p->cnt, 0);
     qw_batch_buf(b, 5, sel, 0);
@@ -261,7 +270,7 @@ static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const
     bind_t(b, 1, &M->up);
     bind_t(b, 2, &M->sh_down);
     qw_batch_buf(b, 3, &p->psh, 0);
-    qw_batch_buf(b, 4, x, 0);
+    qw_batch_buf(b, 4, x, xoff);
     qw_batch_buf(b, 5, sel, 0);
     qw_batch_buf(b, 6, &p->H, 0);
     bind_t(b, 7, &M->sh_down);
@@ -286,7 +295,7 @@ static bool gg_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const
     qw_batch_kernel(b, k);
     qw_batch_buf(b, 1, &p->psh, 0);
     qw_batch_buf(b, 3, sel, 0);
-    qw_batch_buf(b, 4, out, 0);
+    qw_batch_buf(b, 4, out, outoff);
     qw_batch_bytes(b, 8, &nbr, 4);
     qw_batch_buf(b, 9, &p->pd, 0);
     qw_batch_dispatch(b, D / 256, 1, 1, 256, 1, 1);
@@ -303,6 +312,49 @@ bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nl
     return true;
 }
 void qw_path_set_flush(qw_path *p, uint64_t mask) { p->flush_mask = mask; }
+
+// ---------------------------------------------------------------- a ragged step (src/engine.c:8783-8814, :9138-9161, :9037)
+// Slot i brings n[i] rows; its first row is r0[i] = n[0] + ... + n[i - 1] (src/engine.c:9150-9161). The R rows are cut
+// into groups by the measured table (qw_par_split: the reference's par_split with groups of up to 16 rows), every
+// group is one batch through the layer (the reference's par_step runs its groups one after the other, each reading
+// the weights once, src/engine.c:8805-8812), and each group's wall time goes back into the table (src/engine.c:9037).
+bool qw_path_par_vstep(qw_path *p, qw_par *par, const qw_moe_layer *M, const int *n, int B, const qw_buf *x, const qw_buf *out, qw_vstep_info *info) {
+    if (!p || !par || !M || !n || !x || !out || B < 1 || B > QW_PAR_MAX) return false;
+    int R = 0, r0[QW_PAR_MAX];
+    for (int i = 0; i < B; i++) {
+        if (n[i] < 1) return false; // src/engine.c:9141
+        r0[i] = R;
+        R += n[i];
+    }
+    if (R > QW_PAR_MAX || p->nbmax < QW_PAR_VBMAX) {
+        fprintf(stderr, "qw_path_par_vstep: %d rows (at most %d), path opened for %d tokens (needs %d)\n", R, QW_PAR_MAX, p->nbmax, QW_PAR_VBMAX);
+        return false;
+    }
+    if ((size_t)R * (size_t)p->D * 2 > x->size || (size_t)R * (size_t)p->D * 2 > out->size) return false;
+    if (!p->vlg.handle && (!qw_hip_buf_new_device(p->g, qw_path_logits_bytes(p, QW_PAR_VBMAX), &p->vlg) || !qw_hip_buf_new_device(p->g, qw_path_sel_bytes(p, QW_PAR_VBMAX), &p->vsel)))
+        return false;
+    int grp[QW_PAR_MAX];
+    const int ng = qw_par_split(par, R, grp);
+    if (info) {
+        *info = (qw_vstep_info){.rows = R, .ngroups = ng};
+        memcpy(info->r0, r0, sizeof(int) * (size_t)B);
+        memcpy(info->groups, grp, sizeof(int) * (size_t)ng);
+    }
+    double gpu = 0, wall = 0;
+    for (int gi = 0, c = 0; gi < ng; c += grp[gi++]) {
+        const double t0 = qw_now();
+        qw_batch *b = qw_batch_begin(p->g, false);
+        if (!b) return false;
+        const bool rec = gg_moe_at(p, b, M, grp[gi], x, (size_t)c * (size_t)p->D * 2, &p->vlg, &p->vsel, out, (size_t)c * (size_t)p->D * 2, false);
+        const double t = qw_batch_end(b);
+        if (!rec || t < 0) return false;
+        const double ms = (qw_now() - t0) * 1e3;
+        qw_par_observe(par, grp[gi], ms);
+        gpu += t * 1e3, wall += ms;
+    }
+    if (info) info->gpu_ms = gpu, info->wall_ms = wall;
+    return true;
+}
 
 // ---------------------------------------------------------------- ragged batch through the packing path (src/engine.c:4133-4254)
 bool qw_path_pf_reserve(qw_path *p, int tmax, int tm) {

@@ -33,6 +33,10 @@ class QwMoeWeightsDev(C.Structure):
                [(n, C.c_int) for n in ("router_type", "gate_type", "down_type", "sh_gate_type", "sh_up_type", "sh_down_type")]
 
 
+class QwVstepInfo(C.Structure):
+    _fields_ = [("rows", C.c_int), ("ngroups", C.c_int), ("groups", C.c_int * 64), ("r0", C.c_int * 64), ("gpu_ms", C.c_double), ("wall_ms", C.c_double)]
+
+
 class QwGgufTensor(C.Structure):
     _fields_ = [("name", C.c_char_p), ("model", C.c_char_p), ("part", C.c_uint), ("kind", C.c_int), ("type", C.c_uint32), ("nd", C.c_uint32),
                 ("dims", C.c_uint64 * 4), ("rows", C.c_uint64), ("rowbytes", C.c_uint64), ("nbytes", C.c_uint64), ("shard", C.c_int),
@@ -78,6 +82,7 @@ SYMBOLS = [
     ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]), ("qw_path_set_flush", None, [_vp, C.c_uint64]),
     ("qw_path_scratch", _pb, [_vp, _i]),
+    ("qw_path_par_vstep", _b, [_vp, _vp, _pm, _pi, _i, _pb, _pb, C.POINTER(QwVstepInfo)]),
     ("qw_path_gg_moe_noalloc", _b, [_vp, _i, _i, _i, _i, C.POINTER(QwMoeWeightsDev), _i, _vp, _vp, _vp]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_pf_scratch", _pb, [_vp, _i]), ("qw_path_pf_max_tiles", C.c_uint, [_vp]),
@@ -352,6 +357,14 @@ class Path:
         """layers_c: ctypes array of QwMoeLayer; lg_c / sel_c: ctypes arrays of QwBuf, one per layer."""
         if not self.L.qw_path_gg_moe_stack(self.p, batch.b, layers_c, nlayers, nb, x.ref(), lg_c, sel_c, out.ref()):
             raise RuntimeError("qw_path_gg_moe_stack failed")
+
+    def par_vstep(self, par, layer, n, x, out):
+        """A ragged step (slot i: n[i] rows) cut by the planner `par`; returns the QwVstepInfo of the cut."""
+        na = (C.c_int * len(n))(*[int(v) for v in n])
+        info = QwVstepInfo()
+        if not self.L.qw_path_par_vstep(self.p, par.p, C.byref(layer.c), na, len(n), x.ref(), out.ref(), C.byref(info)):
+            raise RuntimeError("qw_path_par_vstep failed: " + self.gpu.last_error())
+        return info
 
     def pf_reserve(self, tmax, tm):
         if not self.L.qw_path_pf_reserve(self.p, tmax, tm):
