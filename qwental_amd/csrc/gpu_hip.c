@@ -32,6 +32,7 @@ enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES 
 typedef enum {
     FAM_DQ_TEST, FAM_QMV_GG, FAM_QMV_GGM, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
     FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
+    FAM_BW_CHUNKS, FAM_BW_ROWS, // read pattern of a decode layer (bench/moe_bw.c)
     FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PK_ZERO, FAM_PF, // ragged packing and the grouped product
 } qw_family;
 
@@ -42,6 +43,7 @@ typedef struct { // parameters taken from the define block
     int tm;                              // packing: rows per tile entry
     int valu;                            // qmv_gg: QW_VALU in the block asks for the VALU GEMV (measurement)
     int nmat, gf[4];                     // qmv_ggm: number of matrices and their formats
+    int sl, ld, ub;                      // bw_chunks / bw_rows (with RB)
 } qw_kparams;
 
 struct qw_kernel {
@@ -488,6 +490,13 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             !reg_kernel(g, d, n, "moe_plan_t", FAM_PK_PLAN_T, &p, err, errlen) || !reg_kernel(g, d, n, "moe_scatter", FAM_PK_SCATTER, &p, err, errlen) ||
             !reg_kernel(g, d, n, "moe_act", FAM_PK_ACT, &p, err, errlen) || !reg_kernel(g, d, n, "p_act2", FAM_PK_ACT2, &p, err, errlen) || !reg_kernel(g, d, n, "moe_combine", FAM_PK_COMBINE, &p, err, errlen) ||
             !reg_kernel(g, d, n, "p_zero", FAM_PK_ZERO, &p, err, errlen)) { ok = false; goto out; }
+    }
+    if (def_get(d, n, "SL") && def_get(d, n, "LD") && def_get(d, n, "UB")) { // bench/moe_bw.c:29-41: one source, one of its two kernels renamed
+        memset(&p, 0, sizeof p);
+        if (!def_int(d, n, "SL", &p.sl) || !def_int(d, n, "LD", &p.ld) || !def_int(d, n, "RB", &p.RB) || !def_int(d, n, "UB", &p.ub)) FAIL("bw_chunks / bw_rows: SL, LD, RB and UB must be integers");
+        // Both kernels are in the source; the one the block renames is the one the caller asks for. Its parameters are
+        // checked when it is dispatched (the other one's are placeholders).
+        if (!reg_kernel(g, d, n, "bw_chunks", FAM_BW_CHUNKS, &p, err, errlen) || !reg_kernel(g, d, n, "bw_rows", FAM_BW_ROWS, &p, err, errlen)) { ok = false; goto out; }
     }
     if (def_get(d, n, "QW_HIP_MEM")) { // this backend's own measurement helpers
         p = (qw_kparams){0};
@@ -1485,6 +1494,28 @@ static bool tr_mem(qw_batch *b, unsigned gx) {
     return add_launch(b, f == FAM_BW_READ ? "qwk_bw_read" : f == FAM_COPY ? "qwk_copy" : "qwk_fill_random", gx, 256, &a, sizeof a);
 }
 
+// bench/moe_bw.c:82-91, 106-112: 0 arena, 1 chunk records at the dispatch's first chunk, 2 sink; grid (slices or row groups, chunks)
+static bool tr_bwpat(qw_batch *b, unsigned gx, unsigned gy, unsigned tx) {
+    const qw_kparams *p = &b->k->p;
+    const bool rows = b->k->fam == FAM_BW_ROWS;
+    qwk_bwpat_args a = {.sl = (uint32_t)p->sl, .ld = (uint32_t)p->ld, .rb = (uint32_t)p->RB, .ub = (uint32_t)p->ub};
+    if (rows) {
+        if (p->RB <= 0 || p->ub < 2 || p->ub % 2 || tx != 256) return fail(b, "bw_rows: RB %d, UB %d (even, at least 2), %u threads (256)", p->RB, p->ub, tx);
+    } else if (p->sl <= 0 || (p->ld != 1 && p->ld != 2 && p->ld != 4 && p->ld != 8) || tx == 0 || tx > 1024 || tx % 64)
+        return fail(b, "bw_chunks: SL %d, LD %d (1, 2, 4 or 8), %u threads (a multiple of 64 up to 1024)", p->sl, p->ld, tx);
+    if (gy == 0 || gy > 65535) return fail(b, "%s: %u chunks in one dispatch", b->k->name, gy);
+    if (!b->buf[0].h) return fail(b, "%s: no arena bound at 0", b->k->name);
+    if (b->buf[0].off > b->buf[0].h->size) return fail(b, "%s: arena offset past its end", b->k->name);
+    const size_t avail = b->buf[0].h->size - b->buf[0].off;
+    if (b->buf[0].off % 16 || !bind_ptr(b, 0, avail, false, "arena", (void **)&a.src)) return fail(b, "%s: arena binding", b->k->name);
+    a.src_n = avail / 16;
+    if (b->buf[1].off % 8 || !bind_ptr(b, 1, (size_t)gy * 8, false, "chunk records", (void **)&a.chunks)) return false;
+    if (!bind_ptr(b, 2, 1024 * 4, true, "sink", (void **)&a.out)) return false;
+    if (!add_launch(b, rows ? "qwk_bw_rows" : "qwk_bw_chunks", gx, tx, &a, sizeof a)) return false;
+    if (gx) b->l[b->nl - 1].gy = gy;
+    return true;
+}
+
 // synthetic weights: 1 dst (+ offset), 2 {nblocks (uint64), seed (uint64), type (uint32), sigma (float)}
 static bool tr_fill_blocks(qw_batch *b) {
     struct { uint64_t nblocks, seed; uint32_t type; float sigma; } in;
@@ -1518,6 +1549,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     case FAM_DN: ok = tr_dn(b); break;
     case FAM_CMB: ok = tr_cmb(b); break;
     case FAM_FILL_BLOCKS: ok = tr_fill_blocks(b); break;
+    case FAM_BW_CHUNKS: case FAM_BW_ROWS: ok = tr_bwpat(b, gx, gy, tx); break;
     case FAM_PK_ZERO: ok = tr_pk_zero(b); break;
     case FAM_PK_COUNT: ok = tr_pk_count(b); break;
     case FAM_PK_PLAN: ok = tr_pk_plan(b, false); break;

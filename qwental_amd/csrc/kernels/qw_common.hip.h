@@ -167,6 +167,17 @@ __device__ __forceinline__ h8 qw_q8_cvt(u2 q) {
     return __builtin_bit_cast(h8, raw);
 }
 
+// ---------------------------------------------------------------- result stores of the streaming kernels
+// Loads and stores share one counter of outstanding operations on this hardware, and stores may complete out of order
+// with respect to loads; once the compiler has seen a store it therefore no longer waits for "all but the youngest N
+// loads" but for everything in flight, which empties the prefetch queue. The few result stores at the end of a tile are
+// issued as assembly that this bookkeeping does not see. That is safe in the direction that matters: an outstanding
+// store only makes the hardware counter larger than the number of outstanding loads, so "at most N outstanding" still
+// implies that all but the N youngest loads have returned. A store reads its data registers when it is issued, and it
+// has completed when the kernel ends, which is when its readers start.
+__device__ __forceinline__ void qw_store_u16(uint16_t *p, uint16_t v) { asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"((uint32_t)v) : "memory"); }
+__device__ __forceinline__ void qw_store_f32(float *p, float v) { asm volatile("global_store_dword %0, %1, off" : : "v"(p), "v"(v) : "memory"); }
+
 // ---------------------------------------------------------------- activation fragment providers (operand A)
 // Fragment order in LDS: chunk c (8 consecutive k-values) of token m lives at xf[c * 16 + m], 16 bytes, so that the
 // 16 lanes of a k-group read 256 contiguous bytes. Tokens >= nb are stored as zeros.
@@ -649,6 +660,55 @@ __device__ __forceinline__ void qw_task_pipeline(uint32_t ntasks, uint32_t w0, u
             done = consume(buf[i]);
         }
     }
+}
+
+
+// The streaming form of qw_task_pipeline, for the kernels whose waves each run through several tasks (the routed
+// gate/up and down products): same arguments and the same calls of rowp, use and ready, plus spare, which is null or the
+// address of 64 KB of readable memory that stays in cache (the lookup table).
+template <class C, int DEPTH = C::DEPTH, class R, class U, class S>
+__device__ __forceinline__ void qw_task_stream(uint32_t ntasks, uint32_t w0, uint32_t nw, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use, S ready, const uint8_t *spare = nullptr) {
+    if (w0 >= ntasks) {
+        ready();
+        return;
+    }
+    // DEPTH chunk buffers: the loads run DEPTH - 1 chunks ahead of the arithmetic
+    C buf[DEPTH];
+    uint32_t left = ((ntasks - w0 + nw - 1) / nw) * cpr;
+    uint32_t lt = w0, lc = 0, ut = w0, uc = 0;
+    const uint8_t *lrow = rowp(lt);
+    // Every step issues one chunk's loads, whatever happens: once the wave's rows are used up the loads read a row's worth
+    // of valid, cached memory that is never consumed (the caller's spare region of at least 64 KB if a row fits in it,
+    // else the wave's own first row again). The loop below then has no memory operation under a condition and a fixed
+    // trip structure, so the number of loads in flight at each wait is the same on every path and the compiler waits for
+    // "all but the youngest DEPTH - 1 chunks" instead of emptying the queue.
+    const uint8_t *const past = spare && cpr * cstride <= 65536u ? spare : lrow;
+    auto load = [&](C &x) {
+        x.load(lrow + (size_t)lc * cstride, kl);
+        if (++lc == cpr) {
+            lc = 0;
+            lt += nw;
+            lrow = lt < ntasks ? rowp(lt) : past;
+        }
+    };
+    auto consume = [&](C &x) {
+        x.transpose();
+        use(ut, uc, x);
+        if (++uc == cpr) uc = 0, ut += nw;
+    };
+#pragma unroll
+    for (int i = 0; i + 1 < DEPTH; i++) load(buf[i]);
+    ready();
+    for (; left >= DEPTH; left -= DEPTH) {
+#pragma unroll
+        for (int i = 0; i < DEPTH; i++) {
+            load(buf[(i + DEPTH - 1) % DEPTH]);
+            consume(buf[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i + 1 < DEPTH; i++)
+        if (left > (uint32_t)i) consume(buf[i]);
 }
 
 

@@ -135,6 +135,14 @@ typedef struct { /* pure-read ceiling and fill helpers */
     uint64_t seed;
 } qwk_mem_args;
 
+typedef struct { /* read-pattern ceiling of a decode layer (the reference's kernels/moe_bw.metal:7-41) */
+    const void *src;          /* the arena the chunks lie in */
+    const uint32_t *chunks;   /* {start, length} per chunk, in 16-byte units; workgroup row y reads chunks[y] */
+    uint32_t *out;            /* sink that is practically never written; holds at least one dword per thread */
+    uint64_t src_n;           /* 16-byte units readable at src: chunk records that reach past it are clamped */
+    uint32_t sl, ld, rb, ub;  /* SL: units per workgroup; LD: independent loads per thread and round; RB, UB: bytes per row and per unit */
+} qwk_bwpat_args;
+
 /* Tile-major copy of IQ3_S rows ("packed", format code QW_F_PACKED below): rows are taken 16 at a time (a tile) and
  * every (tile, block) slab of 16 x 110 bytes becomes QW_SLAB_BYTES contiguous bytes in the lane order of the matrix
  * instructions (lane l: row l & 15 of the tile, 64-value slice l >> 4 of the block):

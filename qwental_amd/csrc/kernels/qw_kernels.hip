@@ -152,8 +152,9 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
                 }
             }
     };
-    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
-    if (XLDS) qw_stage_x(xf, a.x, a.xstride, a.K, a.nb);
+    if (qw_has_lut(F)) qw_lut_copy_issue(lut, (const u2 *)a.glut);
+    if (XLDS) qw_stage_x_issue(xf, a.x, a.xstride, a.K, a.nb);
+    qw_lds_arrive(); // both awaited once
     __syncthreads();
     const qw_afrag_lds afl = {xf, n};
     const qw_afrag_glb<false> afg = {n < a.nb ? a.x + (size_t)n * a.xstride : nullptr, nullptr};
@@ -842,7 +843,7 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
         else return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + 8 * (task % tpe) + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
+    qw_task_stream<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
         c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
@@ -856,12 +857,12 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
                 const float h = g / (1.0f + __expf(-g)) * up;
                 const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
                 const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
-                a.H[o] = __builtin_bit_cast(uint16_t, hi);
-                a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
+                qw_store_u16(a.H + o, __builtin_bit_cast(uint16_t, hi));
+                qw_store_u16(a.H + o + a.hplane, __builtin_bit_cast(uint16_t, lo));
             }
         }
         acc = f4{0, 0, 0, 0};
-    }, ready);
+    }, ready, qw_has_lut(F) ? (const uint8_t *)a.glut : nullptr);
 }
 
 // FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
@@ -901,8 +902,9 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
     auto ready = [&] {
         if (staged) return;
         staged = true;
-        if (!tabled && (qw_has_lut(FGU) || qw_has_lut(FSG))) qw_lut_copy(lut, (const u2 *)a.glut);
-        qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+        if (!tabled && (qw_has_lut(FGU) || qw_has_lut(FSG))) qw_lut_copy_issue(lut, (const u2 *)a.glut);
+        qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
+        qw_lds_arrive();
         __syncthreads();
     };
     // Waves are numbered wave-major (wave w of workgroup b is number w * gridDim.x + b), so that when the tiles do not
@@ -996,8 +998,10 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
         if constexpr (F == QW_F_PACKED) c.load(a.Wg + (size_t)tile * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane);
         else c.load(((lane >> 2) < 8 ? a.Wg : a.Wu) + ((size_t)8 * tile + ((lane >> 2) & 7)) * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane & 3);
     }
-    if (qw_has_lut(F)) qw_lut_copy(lut, (const u2 *)a.glut);
-    qw_stage_x(xf, a.x, a.D, a.D, a.nbr);
+    // the table and the activations behind the weights, all awaited once: one memory round trip before the barrier
+    if (qw_has_lut(F)) qw_lut_copy_issue(lut, (const u2 *)a.glut);
+    qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
+    qw_lds_arrive();
     __syncthreads();
     f4 acc = {0, 0, 0, 0};
     if (on) {
@@ -1099,7 +1103,7 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
         off1[j] = !both || !((g1.mask >> tok) & 1) ? ~0u : (g1.sh ? tok : tok * K + slots1[tok]) * a.D;
     }
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
+    qw_task_stream<C>(ntask, qw_wave(), nwv, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
         [&](uint32_t i) {
             // (field by field: a reference chosen between the two records would put them in scratch memory)
             const bool second = i >= g0.ntile;
@@ -1119,11 +1123,11 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++) {
                 const uint32_t o = second ? off1[j] : off0[j];
-                if (o != ~0u) P[o + r] = acc[j];
+                if (o != ~0u) qw_store_f32(P + o + r, acc[j]);
             }
             acc = f4{0, 0, 0, 0};
         },
-        ready);
+        ready, qw_has_lut(F) ? (const uint8_t *)a.glut : nullptr);
 }
 template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_range_body(const qwk_dn_args &a, u2 *lut, uint16_t *arows /* [2][16][2][I] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, GU = gnb * K, tpe = a.D / 16;
@@ -1632,6 +1636,53 @@ extern "C" __global__ __launch_bounds__(256) void qwk_bw_read(qwk_mem_args a) {
     }
     for (; i < a.n; i += step) s ^= p[i];
     if ((s.x ^ s.y ^ s.z ^ s.w) == 0x9e3779b9u && a.seed == 0x1234) ((u4 *)a.dst)[0] = s; // practically never taken
+}
+// Read pattern of a decode layer without the decoding (kernels/moe_bw.metal:7-26): workgroup (x, c) reads slice x
+// (SL 16-byte units) of chunk c, every thread LD independent loads a round, folded into an XOR sink.
+template <int LD> __device__ __forceinline__ void bw_chunks_body(const qwk_bwpat_args &a) {
+    const uint32_t nt = blockDim.x, tid = threadIdx.x;
+    const uint64_t start = a.chunks[2 * blockIdx.y];
+    uint64_t len = a.chunks[2 * blockIdx.y + 1];
+    if (start >= a.src_n) return;
+    if (start + len > a.src_n) len = a.src_n - start; // a record that reaches past the arena reads what there is
+    const uint64_t b = (uint64_t)blockIdx.x * a.sl;
+    if (b >= len) return;
+    const uint64_t e = b + a.sl < len ? b + a.sl : len;
+    const u4 *p = (const u4 *)a.src + start;
+    u4 acc[LD];
+#pragma unroll
+    for (int k = 0; k < LD; k++) acc[k] = u4{0, 0, 0, 0};
+    uint64_t i = b + tid;
+    for (; i + (uint64_t)(LD - 1) * nt < e; i += (uint64_t)LD * nt)
+#pragma unroll
+        for (int k = 0; k < LD; k++) acc[k] ^= p[i + (uint64_t)k * nt];
+    for (; i < e; i += nt) acc[0] ^= p[i];
+    u4 s = acc[0];
+#pragma unroll
+    for (int k = 1; k < LD; k++) s ^= acc[k];
+    const uint32_t r = s.x ^ s.y ^ s.z ^ s.w;
+    if (r == 0x9e3779b9u) a.out[tid] = r; // practically never taken
+}
+extern "C" __global__ __launch_bounds__(1024) void qwk_bw_chunks(qwk_bwpat_args a) {
+    switch (a.ld) {
+    case 1: bw_chunks_body<1>(a); break;
+    case 2: bw_chunks_body<2>(a); break;
+    case 4: bw_chunks_body<4>(a); break;
+    default: bw_chunks_body<8>(a); break; // the host admits 1, 2, 4, 8
+    }
+}
+// The row pattern (kernels/moe_bw.metal:30-41): a group of 32 lanes takes one row of RB bytes and reads it two bytes
+// at a time, a unit of UB bytes per lane and step; workgroup (x, c) takes rows 8 x .. 8 x + 7 of chunk c. The
+// reference's group is the 32-lane SIMD group of its hardware: here it is half of a wave, the same rows and loads.
+extern "C" __global__ __launch_bounds__(256) void qwk_bw_rows(qwk_bwpat_args a) {
+    const uint32_t sg = threadIdx.x >> 5, lane = threadIdx.x & 31;
+    const uint64_t off = (uint64_t)a.chunks[2 * blockIdx.y] * 16 + ((uint64_t)blockIdx.x * 8 + sg) * a.rb;
+    if (off + a.rb > a.src_n * 16) return; // a row past the arena is not read
+    const uint8_t *row = (const uint8_t *)a.src + off;
+    uint32_t acc = 0;
+    for (uint32_t u = lane; u < a.rb / a.ub; u += 32)
+        for (uint32_t j = 0; j < a.ub; j += 2) acc ^= *(const uint16_t *)(row + (size_t)u * a.ub + j);
+    if (acc == 0x9e3779b9u) a.out[lane] = acc; // practically never taken
 }
 // Plain copy of n 16-byte units (the known-size kernel the hardware traffic counters are scaled against).
 extern "C" __global__ __launch_bounds__(256) void qwk_copy(qwk_mem_args a) {

@@ -73,21 +73,24 @@ const char *qw_ggml_name(int type) {
     return "?";
 }
 
+// One word of a QW_GGUF_PARTS list (src/gguf.c:38-52 gives the words and what they select).
+static unsigned part_of_word(const char *w, size_t n) {
+    static const char *const words[] = {"moe", "shared", "router", "attn", "lin", "hyper", "lm", "embed", "ple"};
+    static const unsigned bits[] = {QW_GG_MOE, QW_GG_SHARED, QW_GG_ROUTER, QW_GG_ATTN, QW_GG_LIN, QW_GG_HYPER, QW_GG_LM, QW_GG_EMBED, QW_GG_PLE};
+    for (size_t i = 0; i < sizeof bits / sizeof *bits; i++)
+        if (strlen(words[i]) == n && !memcmp(w, words[i], n)) return bits[i];
+    return 0; // a word that names nothing selects nothing
+}
 unsigned qw_gguf_parse_parts(const char *s) {
     if (!s || !*s || !strcmp(s, "all")) return QW_GG_ALL;
-    static const struct { const char *n; unsigned b; } tab[] = {
-        {"moe", QW_GG_MOE},     {"shared", QW_GG_SHARED}, {"router", QW_GG_ROUTER}, {"attn", QW_GG_ATTN}, {"lin", QW_GG_LIN},
-        {"hyper", QW_GG_HYPER}, {"lm", QW_GG_LM},         {"embed", QW_GG_EMBED},   {"ple", QW_GG_PLE},
-    };
-    unsigned r = 0;
-    for (const char *p = s; *p;) { // comma-separated words; unknown words are ignored
-        const char *e = strchr(p, ',');
-        const size_t n = e ? (size_t)(e - p) : strlen(p);
-        for (size_t i = 0; i < sizeof tab / sizeof *tab; i++)
-            if (strlen(tab[i].n) == n && !strncmp(p, tab[i].n, n)) r |= tab[i].b;
-        p += n + (e ? 1 : 0);
+    unsigned parts = 0;
+    while (*s) { // comma-separated, read in place
+        const size_t n = strcspn(s, ",");
+        parts |= part_of_word(s, n);
+        s += n;
+        if (*s == ',') s++;
     }
-    return r;
+    return parts;
 }
 
 // ---------------------------------------------------------------- names (src/gguf.c:181-273)

@@ -116,3 +116,80 @@ def test_reference_ggmtest_runs_unchanged(oracle, tmp_path, ftype, nb):
     got = np.fromfile(fy, np.float32).reshape(nb, rows).astype(np.float64)
     ref = oracle.qmv(ftype, raw, rows, K, x, f64=True)
     assert np.abs(got - ref).max() / np.abs(ref).max() <= 2e-3
+
+
+def bw_block(base, name, sl, ld, rb, ub):
+    """The define block bench/moe_bw.c:34 puts before the reference's kernels/moe_bw.metal."""
+    return "#define SL %d\n#define LD %d\n#define RB %d\n#define UB %d\n#define %s %s\n" % (sl, ld, rb, ub, base, name)
+
+
+def test_bw_chunks_reads_the_slices_the_reference_kernel_reads(gpu):
+    """kernels/moe_bw.metal:7-26 folds what it reads into a sink that is only stored when it equals one constant. An
+    arena of zeros with that constant in one place shows which workgroup and thread read that place: unit
+    start + SL + nt + 44 belongs to slice 1, second load of thread 44."""
+    sl, ld, nt = 1024, 4, 256
+    ok, err = gpu.compile(bw_block("bw_chunks", "bw_chunks_t", sl, ld, 0, 0))
+    assert ok, err
+    n16 = 8192
+    arena = np.zeros((n16, 4), np.uint32)
+    start, length = 100, 3000
+    arena[start + sl + nt + 44, 2] = 0x9e3779b9
+    a, out = gpu.buf_from(arena), gpu.buf_from(np.zeros(1024, np.uint32))
+    ch = gpu.buf_from(np.array([[7, 9], [start, length], [start + 5000, 10**9]], np.uint32))  # the last record reaches past the arena: clamped
+    b = gpu.batch()
+    b.kernel(gpu.kernel("bw_chunks_t"))
+    b.buf(0, a)
+    b.buf(1, ch, 8)  # from the second record on, as the driver binds a layer's records at an offset
+    b.buf(2, out)
+    b.dispatch((length + sl - 1) // sl, 2, 1, nt, 1, 1)
+    b.end()
+    got = out.view(np.uint32)
+    want = np.zeros(1024, np.uint32)
+    want[44] = 0x9e3779b9
+    assert np.array_equal(got, want)
+    for x in (a, out, ch):
+        x.free()
+
+
+def test_bw_rows_and_refusals(gpu):
+    ok, err = gpu.compile(bw_block("bw_rows", "bw_rows_t", 1, 1, 1100, 8))
+    assert ok, err
+    a, out = gpu.buf_from(np.ones(1 << 20, np.uint8)), gpu.buf_from(np.zeros(1024, np.uint32))
+    ch = gpu.buf_from(np.array([[64, 4096], [60000, 5536]], np.uint32))  # rows of the second chunk run past the arena: not read
+    b = gpu.batch()
+    b.kernel(gpu.kernel("bw_rows_t"))
+    b.buf(0, a)
+    b.buf(1, ch)
+    b.buf(2, out)
+    b.dispatch(8, 2, 1, 256, 1, 1)
+    b.end()
+    assert not out.view(np.uint32).any()
+    # an odd unit, a thread count the row kernel is not written for, more records than the buffer holds
+    ok, err = gpu.compile(bw_block("bw_rows", "bw_rows_odd", 1, 1, 1100, 7))
+    assert ok, err
+    for name, gy, tx in (("bw_rows_odd", 2, 256), ("bw_rows_t", 2, 128), ("bw_rows_t", 3, 256)):
+        b = gpu.batch()
+        b.kernel(gpu.kernel(name))
+        b.buf(0, a)
+        b.buf(1, ch)
+        b.buf(2, out)
+        b.dispatch(8, gy, 1, tx, 1, 1)
+        assert b.end(check=False) < 0 and gpu.last_error()
+    for x in (a, out, ch):
+        x.free()
+
+
+def test_reference_moe_bw_runs_unchanged():
+    """The reference's bench/moe_bw.c (read-pattern ceiling of a decode layer) over this backend: it allocates a 2 GiB
+    arena, compiles its kernels/moe_bw.metal with four parameters and prints a table of microseconds per layer."""
+    exe = os.path.join(REF, "moe_bw_ref")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/moe_bw_ref is not built (the reference tree was absent at build time)")
+    r = run([exe])
+    assert r.returncode == 0, r.stdout
+    rows = [ln for ln in r.stdout.splitlines() if ln.startswith("| ") and ln.count("|") == 7 and ln.split("|")[5].strip().replace(".", "").isdigit()]
+    assert len(rows) == 5, r.stdout  # three dispatches a layer; front, gate/up, down alone; the row pattern
+    for ln in rows:
+        us, gbs = float(ln.split("|")[5]), float(ln.split("|")[6])
+        assert 1 < us < 1e4 and 50 < gbs < 8000, ln
+    print(r.stdout)
