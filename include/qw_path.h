@@ -7,6 +7,7 @@
  *     gg_router()   src/engine.c:544-552      qw_path_gg_router()
  *     gg_kernel()   src/engine.c:460-517      (internal)
  *     gg_moe()      src/engine.c:568-647      qw_path_gg_moe()
+ *     hyper_gg()    src/engine.c:1344-1412    qw_path_hyper_gg()
  * with the same binding indices, macro names and dispatch order, so that a parity test written against them
  * exercises exactly the call sequence engine.c would issue. The one extension is a token count above 8 (up to 16),
  * which the reference splits into two passes (src/engine.c:8783-8814).
@@ -103,6 +104,30 @@ bool qw_path_pf_reserve(qw_path *p, int tmax, int tm);
 bool qw_path_pf_moe(qw_path *p, qw_batch *b, const qw_moe_layer *M, int T, const qw_buf *x, const qw_buf *ids, const qw_buf *w, const qw_buf *out);
 const qw_buf *qw_path_pf_scratch(const qw_path *p, int which);
 unsigned qw_path_pf_max_tiles(const qw_path *p);
+
+/* The hyper-connection in front of a sublayer, GGUF profile (hyper_gg(), src/engine.c:1344-1412; kernels/hyper_gg.metal):
+ * nb tokens with QW_PATH_HC residual streams of D values each. h [nb][HC][D] float (written back when apply),
+ * out [nb][D] binary16 (the previous sublayer's output, read only when apply), inj [nb][HC][HC] float (inject sums of the
+ * previous hyper-connection) -> x [nb][D] binary16 (the sublayer's input), inj_out [nb][HC][HC] (when H has inject rows).
+ * Weights: hc_norm F32 [HC * D], mix_down BF16 [QW_PATH_HC_LR][HC * D], mix_up BF16 [HC * D][QW_PATH_HC_LR], inject
+ * BF16 [HC][HC * D] (inject.buf NULL: none, as the reference's final mixer). pd is scratch of
+ * qw_path_hyper_pd_bytes(nb) bytes. three: record the reference's three-kernel sequence (ghc_dsk, ghc_mid, ghc_upv;
+ * its path for more than one token) instead of the two-kernel one; same results up to the float sums' order. D is the
+ * path's; it must be a multiple of 512. All in binary32 on the device, as the reference. */
+#define QW_PATH_HC 4
+#define QW_PATH_HC_LR 320
+typedef struct { qw_tensor hc_norm, mix_down, mix_up, inject; } qw_hyper_w;
+size_t qw_path_hyper_pd_bytes(int nb);
+bool qw_path_hyper_gg(qw_path *p, qw_batch *b, const qw_hyper_w *H, int nb, bool apply, bool three, const qw_buf *h, const qw_buf *out, const qw_buf *inj,
+                      const qw_buf *inj_out, const qw_buf *pd, const qw_buf *x);
+
+/* nlayers times: hyper-connection H[l] (h, and from the second layer on — or at once when pending — the residual of out)
+ * -> x, then MoE layer M[l]: x -> out. The FFN half of the reference's layer loop (hyper_in then moe,
+ * src/engine.c:1415-1423, :2169) with a real dependency from layer to layer. inj: two buffers of nb x HC x HC floats, the
+ * first holding the inject sums to start from; they alternate as the reference swaps them. On return out holds the last
+ * layer's output, still to be applied. lg and sel: one per layer, as for qw_path_gg_moe_stack. */
+bool qw_path_hyper_moe_stack(qw_path *p, qw_batch *b, const qw_hyper_w *H, const qw_moe_layer *M, int nlayers, int nb, bool pending, const qw_buf *h,
+                             const qw_buf *inj, const qw_buf *pd, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out);
 
 /* The layer for callers that cannot allocate. No counterpart in the reference: it exists for callers that must not call
  * hipMalloc or any allocating routine while they run the layer — a stream under HIP graph capture, a tight serving loop,

@@ -53,6 +53,8 @@ def load():
     L.qwo_moe_layer_f64.argtypes = [vp, vp, vp, i, vp, i]
     L.qwo_moe_pack.restype = i
     L.qwo_moe_pack.argtypes = [vp, i, i, i, vp, vp, vp, vp, i]
+    L.qwo_hyper_gg.restype = None
+    L.qwo_hyper_gg.argtypes = [i, i, i, i, i] + [vp] * 10
     L.qwo_max_threads.restype = i
     _lib = L
     return L
@@ -193,6 +195,27 @@ def moe_layer_f64(m, logits, x, threads=0):
     L.qwo_moe_layer_f64(C.byref(s), _p(logits), _p(x), nb, _p(out), threads)
     del keep
     return out
+
+
+def hyper_gg(h, out, inj, w, Wd, Wi, Wu, apply):
+    """The GGUF profile's hyper-connection in float64. h float32 [nb, HC, D]; out float16 [nb, D]; inj float32
+    [nb, HC, HC]; w float32 [HC * D]; Wd, Wi, Wu bfloat16 bit patterns (uint16) [LR, HC * D], [HC, HC * D] or None,
+    [HC * D, LR]. Returns (h1 [nb, HC, D], x [nb, D], inject sums [nb, HC, HC] or None), all float64."""
+    L = load()
+    h = np.ascontiguousarray(h, np.float32)
+    nb, HC, D = h.shape
+    out = np.ascontiguousarray(out, np.float16)
+    inj = np.ascontiguousarray(inj, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    Wd, Wu = np.ascontiguousarray(Wd, np.uint16), np.ascontiguousarray(Wu, np.uint16)
+    LR = Wd.shape[0]
+    assert Wd.shape == (LR, HC * D) and Wu.shape == (HC * D, LR) and w.size == HC * D and out.shape == (nb, D) and inj.shape == (nb, HC, HC)
+    Wi = None if Wi is None else np.ascontiguousarray(Wi, np.uint16)
+    h1, x = np.empty((nb, HC, D), np.float64), np.empty((nb, D), np.float64)
+    io = None if Wi is None else np.empty((nb, HC, HC), np.float64)
+    L.qwo_hyper_gg(D, HC, LR, nb, 1 if apply else 0, _p(h), _p(out), _p(inj), _p(w), _p(Wd), None if Wi is None else _p(Wi), _p(Wu), _p(h1), _p(x),
+                   None if io is None else _p(io))
+    return h1, x, io
 
 
 def moe_pack(ids, E, tm, max_tiles):

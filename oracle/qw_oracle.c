@@ -544,3 +544,55 @@ int qwo_moe_pack(const uint32_t *ids, int P, int E, int tm, uint32_t *counts, ui
     free(cur);
     return nt;
 }
+
+// ---------------------------------------------------------------- hyper-connection (kernels/hyper_gg.metal:94-233, tools/hc_ref.py:60-70)
+void qwo_hyper_gg(int D, int HC, int LR, int NB, int apply, const float *h, const uint16_t *out_f16, const float *inj, const float *w,
+                  const uint16_t *Wd_bf16, const uint16_t *Wi_bf16, const uint16_t *Wu_bf16, double *h_out, double *x, double *inj_out) {
+    const size_t HCD = (size_t)HC * D;
+    double *y = malloc(sizeof(double) * HCD), *sx = malloc(sizeof(double) * (size_t)LR);
+    for (int t = 0; t < NB; t++) {
+        double *h1 = h_out + (size_t)t * HCD;
+        for (int s = 0; s < HC; s++) {
+            double js = 0;
+            if (apply) { // kernels/hyper_gg.metal:47-51: the column sum over the streams' partial sums
+                double a = 0;
+                for (int q = 0; q < HC; q++) a += inj[((size_t)t * HC + q) * HC + s];
+                js = 2.0 / (1.0 + exp(-a / HC));
+            }
+            double ss = 0;
+            for (int j = 0; j < D; j++) {
+                const double v = (double)h[(size_t)t * HCD + (size_t)s * D + j] + (apply ? (double)qwo_h2f(out_f16[(size_t)t * D + j]) * js : 0.0);
+                h1[(size_t)s * D + j] = v;
+                ss += v * v;
+            }
+            const double r = 1.0 / sqrt(ss / D + 1e-6);
+            for (int j = 0; j < D; j++) y[(size_t)s * D + j] = h1[(size_t)s * D + j] * r * (double)w[(size_t)s * D + j];
+        }
+#pragma omp parallel for
+        for (int r = 0; r < LR; r++) {
+            double d = 0;
+            for (size_t c = 0; c < HCD; c++) d += (double)qwo_bf2f(Wd_bf16[(size_t)r * HCD + c]) * y[c];
+            sx[r] = (d / HC) / (1.0 + exp(-d / HC));
+        }
+#pragma omp parallel for
+        for (int j = 0; j < D; j++) {
+            double m = 0;
+            for (int s = 0; s < HC; s++) {
+                const uint16_t *row = Wu_bf16 + ((size_t)s * D + j) * LR;
+                double u = 0;
+                for (int r = 0; r < LR; r++) u += (double)qwo_bf2f(row[r]) * sx[r];
+                m += y[(size_t)s * D + j] / (1.0 + exp(-u));
+            }
+            x[(size_t)t * D + j] = m / HC;
+        }
+        if (Wi_bf16 && inj_out)
+            for (int s = 0; s < HC; s++)
+                for (int q = 0; q < HC; q++) {
+                    double a = 0;
+                    for (int j = 0; j < D; j++) a += (double)qwo_bf2f(Wi_bf16[(size_t)q * HCD + (size_t)s * D + j]) * y[(size_t)s * D + j];
+                    inj_out[((size_t)t * HC + s) * HC + q] = a;
+                }
+    }
+    free(y);
+    free(sx);
+}

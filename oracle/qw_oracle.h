@@ -26,6 +26,12 @@
 //                             the closed-form softmax / sigmoid, and dedupe invariants.
 //   qwo_moe_layer_*           pinned by a numpy float64 recomputation on small shapes.
 //   qwo_moe_pack              pinned by counting-sort invariants (exclusive scan, permutation).
+//   qwo_hyper_gg              pinned by: the cases the mathematics fixes (a zero mix_up matrix makes every gate
+//                             sigmoid(0) = 1/2; zero inject sums make the residual coefficient exactly 1; scaling
+//                             the streams leaves the normalised vector unchanged; one-hot mix_down / mix_up rows
+//                             pick single terms), an element-by-element loop on a tiny shape, and a float64
+//                             matrix statement in numpy. The reference holds no dump of this step (its
+//                             tools/hc_ref.py reads files a model run writes).
 #pragma once
 #include <stdbool.h>
 #include <stddef.h>
@@ -106,6 +112,18 @@ void qwo_moe_layer_f64(const qwo_moe_weights *m, const float *logits, const uint
 // for row blocks of tm rows, unused tiles zeroed. Returns the number of tiles in use.
 int qwo_moe_pack(const uint32_t *ids, int P, int E, int tm, uint32_t *counts, uint32_t *offs, uint32_t *pos_of,
                  uint32_t *tiles, int max_tiles);
+
+// Hyper-connection of the GGUF profile (kernels/hyper_gg.metal:94-233; the reference's own float64 statement is
+// tools/hc_ref.py:60-70), one call for NB tokens, everything in float64:
+//   js[s]   = apply ? 2 sigmoid(sum_q inj[q][s] / HC) : 0            (kernels/hyper_gg.metal:47-51)
+//   h1[s]   = h[s] + out * js[s]
+//   r[s]    = 1 / sqrt(mean_j h1[s][j]^2 + 1e-6);  y[s][j] = h1[s][j] r[s] w[s D + j]
+//   d       = Wd y (LR rows over the HC D columns);  sx = silu(d / HC);  u = Wu sx
+//   x[j]    = mean_s sigmoid(u[s D + j]) y[s][j]
+//   injo[s][q] = sum_j Wi[q][s D + j] y[s][j]                          (only when Wi is given)
+// h1 is returned in h_out whether or not the residual was applied.
+void qwo_hyper_gg(int D, int HC, int LR, int NB, int apply, const float *h, const uint16_t *out_f16, const float *inj, const float *w,
+                  const uint16_t *Wd_bf16, const uint16_t *Wi_bf16, const uint16_t *Wu_bf16, double *h_out, double *x, double *inj_out);
 
 int qwo_max_threads(void);
 

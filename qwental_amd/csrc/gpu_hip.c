@@ -33,6 +33,7 @@ typedef enum {
     FAM_DQ_TEST, FAM_QMV_GG, FAM_QMV_GGM, FAM_ROUTER, FAM_TAB_INIT, FAM_SEL, FAM_PRE, FAM_GU, FAM_DN, FAM_CMB,
     FAM_BW_READ, FAM_COPY, FAM_FILL, FAM_FILL_BLOCKS,
     FAM_BW_CHUNKS, FAM_BW_ROWS, // read pattern of a decode layer (bench/moe_bw.c)
+    FAM_HC_DOWN, FAM_HC_MID, FAM_HC_UP, FAM_HC_UPV, // hyper-connection of the GGUF profile (kernels/hyper_gg.metal)
     FAM_PK_COUNT, FAM_PK_PLAN, FAM_PK_PLAN_T, FAM_PK_SCATTER, FAM_PK_ACT, FAM_PK_ACT2, FAM_PK_COMBINE, FAM_PK_ZERO, FAM_PF, // ragged packing and the grouped product
 } qw_family;
 
@@ -490,6 +491,18 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             !reg_kernel(g, d, n, "moe_plan_t", FAM_PK_PLAN_T, &p, err, errlen) || !reg_kernel(g, d, n, "moe_scatter", FAM_PK_SCATTER, &p, err, errlen) ||
             !reg_kernel(g, d, n, "moe_act", FAM_PK_ACT, &p, err, errlen) || !reg_kernel(g, d, n, "p_act2", FAM_PK_ACT2, &p, err, errlen) || !reg_kernel(g, d, n, "moe_combine", FAM_PK_COMBINE, &p, err, errlen) ||
             !reg_kernel(g, d, n, "p_zero", FAM_PK_ZERO, &p, err, errlen)) { ok = false; goto out; }
+    }
+    if (def_get(d, n, "HC") && (def_get(d, n, "ghc_down") || def_get(d, n, "ghc_up") || def_get(d, n, "ghc_dsk"))) { // src/engine.c:1323-1341
+        memset(&p, 0, sizeof p);
+        int hc;
+        if (!def_int(d, n, "D", &p.D) || !def_int(d, n, "HC", &hc) || !def_int(d, n, "NB", &p.NB)) FAIL("hyper_gg: D, HC and NB must be integers");
+        if (hc != (int)QW_HC) FAIL("hyper_gg: HC %d (this build has %u streams)", hc, QW_HC);
+        if (p.D <= 0 || p.D % 512 || p.D > 8192) FAIL("hyper_gg: D %d must be a multiple of 512 up to 8192", p.D);
+        if (p.NB < 1 || p.NB > 16) FAIL("hyper_gg: NB %d (1 to 16)", p.NB);
+        // GH_R, GH_G, GU_SG, GV_SG, GV_RP and GK tune the reference's own kernels; the ones here have their own shape
+        if (!reg_kernel(g, d, n, "ghc_down", FAM_HC_DOWN, &p, err, errlen) || !reg_kernel(g, d, n, "ghc_up", FAM_HC_UP, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "ghc_dsk", FAM_HC_DOWN, &p, err, errlen) || !reg_kernel(g, d, n, "ghc_mid", FAM_HC_MID, &p, err, errlen) ||
+            !reg_kernel(g, d, n, "ghc_upv", FAM_HC_UPV, &p, err, errlen)) { ok = false; goto out; }
     }
     if (def_get(d, n, "SL") && def_get(d, n, "LD") && def_get(d, n, "UB")) { // bench/moe_bw.c:29-41: one source, one of its two kernels renamed
         memset(&p, 0, sizeof p);
@@ -1494,6 +1507,52 @@ static bool tr_mem(qw_batch *b, unsigned gx) {
     return add_launch(b, f == FAM_BW_READ ? "qwk_bw_read" : f == FAM_COPY ? "qwk_copy" : "qwk_fill_random", gx, 256, &a, sizeof a);
 }
 
+// Hyper-connection (src/engine.c:1344-1412). Bindings of ghc_down / ghc_dsk: 0 h, 1 out, 2 inj, 3 norm weights, 4 mix_down,
+// 5 inject, 6 partial sums, 7 {apply, want inject}; ghc_up: 0 h, 1 out, 2 inj, 3 norm weights, 4 mix_up, 5 partial sums, 6 x,
+// 7 new inject sums, 8 flags; ghc_mid: 0 partial sums, 1 sx, 2 rs, 3 new inject sums, 4 flags; ghc_upv: as ghc_up with 5 sx, 6 rs,
+// 7 x, 8 flags. The caller's grids are the reference kernels' own; these launches have theirs.
+static bool hc_aligned(qw_batch *b, const unsigned *idx, int n) {
+    for (int i = 0; i < n; i++)
+        if (b->buf[idx[i]].off % 16) return fail(b, "%s: the offset of binding %u must be a multiple of 16", b->k->name, idx[i]);
+    return true;
+}
+static bool tr_hc(qw_batch *b) {
+    const qw_kparams *p = &b->k->p;
+    const qw_family f = b->k->fam;
+    const size_t D = (size_t)p->D, nb = (size_t)p->NB, HCD = QW_HC * D;
+    uint32_t fl[2];
+    qwk_hc_args a = {.D = (uint32_t)p->D, .nb = (uint32_t)p->NB};
+    if (!bind_bytes(b, f == FAM_HC_DOWN ? 7 : f == FAM_HC_MID ? 4 : 8, fl, sizeof fl, "{apply, want inject}")) return false;
+    a.apply = fl[0] != 0, a.want_inj = fl[1] != 0;
+    if (f == FAM_HC_MID) {
+        static const unsigned al[] = {0, 1, 2, 3};
+        if (!hc_aligned(b, al, 4)) return false;
+        if (!bind_ptr(b, 0, nb * QW_HC * QW_HC_PDS * 4, false, "partial sums", (void **)&a.pd) || !bind_ptr(b, 1, nb * QW_HC_LR * 4, true, "sx", (void **)&a.sx) ||
+            !bind_ptr(b, 2, nb * QW_HC * 4, true, "rs", (void **)&a.rs)) return false;
+        if (a.want_inj && !bind_ptr(b, 3, nb * QW_HC * QW_HC * 4, true, "new inject sums", (void **)&a.injo)) return false;
+        return add_launch(b, "qwk_hc_mid", (unsigned)nb, QW_HC_LR, &a, sizeof a);
+    }
+    static const unsigned al[] = {0, 1, 2, 3, 4, 5, 6, 7};
+    if (!hc_aligned(b, al, f == FAM_HC_DOWN ? 7 : 8)) return false;
+    // h is written back by the up kernels when the residual is applied; out is only read then (it may not exist yet otherwise)
+    if (!bind_ptr(b, 0, nb * HCD * 4, a.apply && f != FAM_HC_DOWN, "h", (void **)&a.h) || !bind_ptr(b, 3, HCD * 4, false, "norm weights", (void **)&a.w)) return false;
+    if (a.apply && (!bind_ptr(b, 1, nb * D * 2, false, "out", (void **)&a.out) || !bind_ptr(b, 2, nb * QW_HC * QW_HC * 4, false, "inject sums", (void **)&a.inj))) return false;
+    if (f == FAM_HC_DOWN) {
+        if (!bind_ptr(b, 4, QW_HC_LR * HCD * 2, false, "mix_down", (void **)&a.Wd) || !bind_ptr(b, 6, nb * QW_HC * QW_HC_PDS * 4, true, "partial sums", (void **)&a.pd)) return false;
+        if (a.want_inj && !bind_ptr(b, 5, QW_HC * HCD * 2, false, "inject", (void **)&a.Wi)) return false;
+        if (!add_launch(b, "qwk_hc_down", QW_HC_LR / QW_HC_ROWS + (a.want_inj ? 1 : 0), (unsigned)(D / 8), &a, sizeof a)) return false;
+        b->l[b->nl - 1].gy = QW_HC;
+        return true;
+    }
+    if (!bind_ptr(b, 4, HCD * QW_HC_LR * 2, false, "mix_up", (void **)&a.Wu)) return false;
+    if (f == FAM_HC_UP) {
+        if (!bind_ptr(b, 5, nb * QW_HC * QW_HC_PDS * 4, false, "partial sums", (void **)&a.pd) || !bind_ptr(b, 6, nb * D * 2, true, "x", (void **)&a.x)) return false;
+        if (a.want_inj && !bind_ptr(b, 7, nb * QW_HC * QW_HC * 4, true, "new inject sums", (void **)&a.injo)) return false;
+    } else if (!bind_ptr(b, 5, nb * QW_HC_LR * 4, false, "sx", (void **)&a.sx) || !bind_ptr(b, 6, nb * QW_HC * 4, false, "rs", (void **)&a.rs) ||
+               !bind_ptr(b, 7, nb * D * 2, true, "x", (void **)&a.x)) return false;
+    return add_launch(b, f == FAM_HC_UP ? "qwk_hc_up" : "qwk_hc_upv", (unsigned)(D / 8), 256, &a, sizeof a);
+}
+
 // bench/moe_bw.c:82-91, 106-112: 0 arena, 1 chunk records at the dispatch's first chunk, 2 sink; grid (slices or row groups, chunks)
 static bool tr_bwpat(qw_batch *b, unsigned gx, unsigned gy, unsigned tx) {
     const qw_kparams *p = &b->k->p;
@@ -1550,6 +1609,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     case FAM_CMB: ok = tr_cmb(b); break;
     case FAM_FILL_BLOCKS: ok = tr_fill_blocks(b); break;
     case FAM_BW_CHUNKS: case FAM_BW_ROWS: ok = tr_bwpat(b, gx, gy, tx); break;
+    case FAM_HC_DOWN: case FAM_HC_MID: case FAM_HC_UP: case FAM_HC_UPV: ok = tr_hc(b); break;
     case FAM_PK_ZERO: ok = tr_pk_zero(b); break;
     case FAM_PK_COUNT: ok = tr_pk_count(b); break;
     case FAM_PK_PLAN: ok = tr_pk_plan(b, false); break;

@@ -135,6 +135,26 @@ typedef struct { /* pure-read ceiling and fill helpers */
     uint64_t seed;
 } qwk_mem_args;
 
+/* Hyper-connection of the GGUF profile (the reference's kernels/hyper_gg.metal): QW_HC streams of D values a token,
+ * low rank QW_HC_LR. pd holds, per (token, stream), QW_HC_PDS floats: [0, LR) the stream's part of the mix_down sums
+ * before normalisation, [LR, LR + HC) the same for the inject rows, [LR + HC] the stream's sum of squares. */
+#define QW_HC 4u
+#define QW_HC_LR 320u
+#define QW_HC_PDS (QW_HC_LR + 2 * QW_HC)
+#define QW_HC_ROWS 4u /* weight rows per workgroup of the down kernel */
+typedef struct {
+    float *h;                      /* [nb][HC][D]; the up kernels write it back when the residual is applied */
+    const uint16_t *out;           /* binary16 [nb][D]: the sublayer output the residual adds */
+    const float *inj;              /* [nb][HC][HC]: inject sums of the previous hyper-connection */
+    const float *w;                /* [HC * D] norm weights */
+    const uint16_t *Wd, *Wi, *Wu;  /* bfloat16: mix_down [LR][HC * D], inject [HC][HC * D], mix_up [HC * D][LR] */
+    float *pd;                     /* [nb][HC][QW_HC_PDS] */
+    float *sx, *rs;                /* three-kernel form: silu(mix_down) [nb][LR] and the streams' 1 / rms [nb][HC] */
+    uint16_t *x;                   /* binary16 [nb][D] */
+    float *injo;                   /* [nb][HC][HC] */
+    uint32_t D, nb, apply, want_inj;
+} qwk_hc_args;
+
 typedef struct { /* read-pattern ceiling of a decode layer (the reference's kernels/moe_bw.metal:7-41) */
     const void *src;          /* the arena the chunks lie in */
     const uint32_t *chunks;   /* {start, length} per chunk, in 16-byte units; workgroup row y reads chunks[y] */

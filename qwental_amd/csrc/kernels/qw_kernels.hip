@@ -1637,6 +1637,172 @@ extern "C" __global__ __launch_bounds__(256) void qwk_bw_read(qwk_mem_args a) {
     for (; i < a.n; i += step) s ^= p[i];
     if ((s.x ^ s.y ^ s.z ^ s.w) == 0x9e3779b9u && a.seed == 0x1234) ((u4 *)a.dst)[0] = s; // practically never taken
 }
+// ================================================================ hyper-connection, GGUF profile (kernels/hyper_gg.metal:94-233)
+// Everything in binary32, as there. Two launches a hyper-connection whatever the token count: a launch boundary costs
+// more here than recomputing nb x 320 activations per workgroup, which is what the reference's third kernel avoids.
+__device__ __forceinline__ float qw_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+// 2 sigmoid(sum over the streams of their inject sums for stream s / HC) (kernels/hyper_gg.metal:47-51)
+__device__ __forceinline__ float hc_coef(const float *injp, uint32_t s) {
+    float t = 0;
+#pragma unroll
+    for (uint32_t q = 0; q < QW_HC; q++) t += injp[q * QW_HC + s];
+    return 2.0f / (1.0f + expf(-t / QW_HC));
+}
+// Down: residual, sums of squares and the un-normalised mix_down / inject sums (kernels/hyper_gg.metal:94-137).
+// Workgroup (rb, s): QW_HC_ROWS weight rows (block 80 = the inject rows) against stream s; thread c owns columns
+// 8 c .. 8 c + 7 (16 bytes of a bfloat16 row, kept in registers for every token). Per token: the lane's eight
+// h' w products, four dot products of eight and the squares, summed over the wave, then over the waves in order.
+extern "C" __global__ __launch_bounds__(1024) void qwk_hc_down(qwk_hc_args a) {
+    __shared__ float part[16][16][QW_HC_ROWS + 1]; // [wave][token][row | squares]
+    const uint32_t rb = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nwv = blockDim.x >> 6;
+    const bool is_inj = rb == QW_HC_LR / QW_HC_ROWS;
+    const size_t HCD = (size_t)QW_HC * a.D, c0 = (size_t)s * a.D + 8 * tid;
+    const uint16_t *W = is_inj ? a.Wi : a.Wd + (size_t)rb * QW_HC_ROWS * HCD;
+    float wf[QW_HC_ROWS][8];
+#pragma unroll
+    for (uint32_t r = 0; r < QW_HC_ROWS; r++) {
+        const u4 u = *(const u4 *)(W + (size_t)r * HCD + c0);
+#pragma unroll
+        for (int k = 0; k < 4; k++) wf[r][2 * k] = __builtin_bit_cast(float, u[k] << 16), wf[r][2 * k + 1] = __builtin_bit_cast(float, u[k] & 0xffff0000u);
+    }
+    const f4 w0 = *(const f4 *)(a.w + c0), w1 = *(const f4 *)(a.w + c0 + 4);
+    for (uint32_t t = 0; t < a.nb; t++) {
+        const f4 h0 = *(const f4 *)(a.h + t * HCD + c0), h1 = *(const f4 *)(a.h + t * HCD + c0 + 4);
+        float v[8] = {h0[0], h0[1], h0[2], h0[3], h1[0], h1[1], h1[2], h1[3]};
+        if (a.apply) { // out is not read otherwise: it may never have been written
+            const float js = hc_coef(a.inj + t * QW_HC * QW_HC, s);
+            const u4 o = *(const u4 *)(a.out + (size_t)t * a.D + 8 * tid);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                v[2 * k] = fmaf(qw_h2f((uint16_t)o[k]), js, v[2 * k]);
+                v[2 * k + 1] = fmaf(qw_h2f((uint16_t)(o[k] >> 16)), js, v[2 * k + 1]);
+            }
+        }
+        float ss = 0, x[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) ss = fmaf(v[k], v[k], ss), x[k] = v[k] * (k < 4 ? w0[k] : w1[k - 4]);
+        float d[QW_HC_ROWS];
+#pragma unroll
+        for (uint32_t r = 0; r < QW_HC_ROWS; r++) {
+            d[r] = 0;
+#pragma unroll
+            for (int k = 0; k < 8; k++) d[r] = fmaf(wf[r][k], x[k], d[r]);
+            d[r] = qw_wave_sum(d[r]);
+        }
+        ss = qw_wave_sum(ss);
+        if (lane == 0) {
+#pragma unroll
+            for (uint32_t r = 0; r < QW_HC_ROWS; r++) part[wave][t][r] = d[r];
+            part[wave][t][QW_HC_ROWS] = ss;
+        }
+    }
+    __syncthreads();
+    for (uint32_t j = tid; j < a.nb * (QW_HC_ROWS + 1); j += blockDim.x) {
+        const uint32_t t = j / (QW_HC_ROWS + 1), r = j % (QW_HC_ROWS + 1);
+        float sum = 0;
+        for (uint32_t q = 0; q < nwv; q++) sum += part[q][t][r];
+        float *pd = a.pd + ((size_t)t * QW_HC + s) * QW_HC_PDS;
+        if (r < QW_HC_ROWS) pd[(is_inj ? QW_HC_LR : rb * QW_HC_ROWS) + r] = sum;
+        else if (rb == 0) pd[QW_HC_LR + QW_HC] = sum;
+    }
+}
+// What follows the down kernel for tokens t0 .. t0 + nt - 1, by the threads of one workgroup: the streams' 1 / rms,
+// silu of the normalised mix_down sums, and (injo given) the inject sums in the caller's format
+// (kernels/hyper_gg.metal:165-181, 312-340). rs [nt][HC] and sx [nt][LR] are in LDS; ends with a barrier.
+__device__ __forceinline__ void hc_mid(const qwk_hc_args &a, uint32_t t0, uint32_t nt, float *rs, float *sx, float *injo) {
+    const float *pd = a.pd + (size_t)t0 * QW_HC * QW_HC_PDS;
+    for (uint32_t j = threadIdx.x; j < nt * QW_HC; j += blockDim.x) rs[j] = rsqrtf(pd[j * QW_HC_PDS + QW_HC_LR + QW_HC] / (float)a.D + 1e-6f);
+    __syncthreads();
+    for (uint32_t j = threadIdx.x; j < nt * QW_HC_LR; j += blockDim.x) {
+        const uint32_t t = j / QW_HC_LR, r = j % QW_HC_LR;
+        float d = 0;
+#pragma unroll
+        for (uint32_t q = 0; q < QW_HC; q++) d = fmaf(rs[t * QW_HC + q], pd[(t * QW_HC + q) * QW_HC_PDS + r], d);
+        d /= QW_HC;
+        sx[j] = d / (1.0f + __expf(-d));
+    }
+    if (injo)
+        for (uint32_t j = threadIdx.x; j < nt * QW_HC * QW_HC; j += blockDim.x) // j = (t, s, q)
+            injo[t0 * QW_HC * QW_HC + j] = rs[j / QW_HC] * pd[(j / QW_HC) * QW_HC_PDS + QW_HC_LR + j % QW_HC];
+    __syncthreads();
+}
+// The middle kernel of the three-kernel form (kernels/hyper_gg.metal:312-340): a workgroup a token.
+extern "C" __global__ __launch_bounds__(320) void qwk_hc_mid(qwk_hc_args a) {
+    __shared__ float rs[QW_HC], sx[QW_HC_LR];
+    const uint32_t t = blockIdx.x;
+    hc_mid(a, t, 1, rs, sx, a.want_inj ? a.injo : nullptr);
+    for (uint32_t r = threadIdx.x; r < QW_HC_LR; r += blockDim.x) a.sx[t * QW_HC_LR + r] = sx[r];
+    if (threadIdx.x < QW_HC) a.rs[t * QW_HC + threadIdx.x] = rs[threadIdx.x];
+}
+// Up: mix_up, the gates and the mix over the streams, the write-back of h (kernels/hyper_gg.metal:141-233, 344-).
+// A workgroup of 256 threads takes eight output columns i, one per group of 32 lanes; a lane holds ten low-rank columns
+// of the four mix_up rows s D + i (20 bytes each). GIVEN: sx and rs come from qwk_hc_mid instead of being made here.
+template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_args &a) {
+    __shared__ float sx[16][QW_HC_LR], rs[16][QW_HC], js[16][QW_HC];
+    const uint32_t tid = threadIdx.x, l32 = tid & 31, i = blockIdx.x * 8 + (tid >> 5);
+    const size_t HCD = (size_t)QW_HC * a.D;
+    // the weights first: their round trip overlaps what follows
+    uint32_t u[QW_HC][5];
+#pragma unroll
+    for (uint32_t q = 0; q < QW_HC; q++) {
+        const uint32_t *wr = (const uint32_t *)(a.Wu + ((size_t)q * a.D + i) * QW_HC_LR) + l32 * 5;
+#pragma unroll
+        for (int k = 0; k < 5; k++) u[q][k] = wr[k];
+    }
+    const float wn = l32 < QW_HC ? a.w[(size_t)l32 * a.D + i] : 0.0f;
+    if (GIVEN) {
+        for (uint32_t j = tid; j < a.nb * QW_HC_LR; j += blockDim.x) sx[j / QW_HC_LR][j % QW_HC_LR] = a.sx[j];
+        if (tid < a.nb * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[tid];
+    } else {
+        hc_mid(a, 0, a.nb, &rs[0][0], &sx[0][0], blockIdx.x == 0 && a.want_inj ? a.injo : nullptr);
+    }
+    if (tid < a.nb * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
+    __syncthreads();
+    float v[QW_HC][10];
+#pragma unroll
+    for (uint32_t q = 0; q < QW_HC; q++)
+#pragma unroll
+        for (int k = 0; k < 5; k++) v[q][2 * k] = __builtin_bit_cast(float, u[q][k] << 16), v[q][2 * k + 1] = __builtin_bit_cast(float, u[q][k] & 0xffff0000u);
+    for (uint32_t t = 0; t < a.nb; t++) {
+        // lanes 0..3 of the group are the four streams of column i: their h (and out) loads go out before the products
+        float hv = 0, ov = 0;
+        if (l32 < QW_HC) {
+            hv = a.h[t * HCD + (size_t)l32 * a.D + i];
+            if (a.apply) ov = qw_h2f(a.out[(size_t)t * a.D + i]);
+        }
+        float xv[10];
+#pragma unroll
+        for (int k = 0; k < 10; k++) xv[k] = sx[t][l32 * 10 + k];
+        float mine = 0;
+#pragma unroll
+        for (uint32_t q = 0; q < QW_HC; q++) {
+            float d = 0;
+#pragma unroll
+            for (int k = 0; k < 10; k++) d = fmaf(v[q][k], xv[k], d);
+#pragma unroll
+            for (int o = 16; o; o >>= 1) d += __shfl_xor(d, o); // over the 32 lanes of the group
+            mine = l32 == q ? d : mine;
+        }
+        float m = 0;
+        if (l32 < QW_HC) {
+            if (a.apply) {
+                hv = fmaf(ov, js[t][l32], hv);
+                a.h[t * HCD + (size_t)l32 * a.D + i] = hv;
+            }
+            m = (hv * rs[t][l32]) * wn / (1.0f + __expf(-mine));
+        }
+        m += __shfl_xor(m, 1);
+        m += __shfl_xor(m, 2);
+        if (l32 == 0) a.x[(size_t)t * a.D + i] = qw_f2h(m / QW_HC);
+    }
+}
+extern "C" __global__ __launch_bounds__(256) void qwk_hc_up(qwk_hc_args a) { hc_up_body<false>(a); }
+extern "C" __global__ __launch_bounds__(256) void qwk_hc_upv(qwk_hc_args a) { hc_up_body<true>(a); }
+
 // Read pattern of a decode layer without the decoding (kernels/moe_bw.metal:7-26): workgroup (x, c) reads slice x
 // (SL 16-byte units) of chunk c, every thread LD independent loads a round, folded into an XOR sink.
 template <int LD> __device__ __forceinline__ void bw_chunks_body(const qwk_bwpat_args &a) {

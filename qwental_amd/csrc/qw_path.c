@@ -192,6 +192,86 @@ static qw_kernel *gg_kernel(qw_path *p, const char *base, const qw_moe_layer *M,
 
 static void bind_t(qw_batch *b, unsigned index, const qw_tensor *t) { qw_batch_buf(b, index, t->buf, t->offset); }
 
+// ---------------------------------------------------------------- hyper-connection (src/engine.c:1323-1412)
+// The define block of gh_kernel (src/engine.c:1328-1333): the five kernel names carry the token count (and here the
+// width, since one qw_gpu may serve several shapes); GH_R, GH_G, GU_SG, GV_SG, GV_RP and GK are the reference's
+// defaults for its own kernels (src/engine.c:1295-1312) and mean nothing to this backend.
+static qw_kernel *gh_kernel(qw_path *p, const char *base, int nb) {
+    char name[64], defs[768];
+    snprintf(name, sizeof name, "%s_n%d_d%d", base, nb, p->D);
+    qw_kernel *k = qw_kernel_get(p->g, name);
+    if (k) return k;
+    snprintf(defs, sizeof defs,
+             "#define ghc_down ghc_down_n%d_d%d\n#define ghc_up ghc_up_n%d_d%d\n#define ghc_dsk ghc_dsk_n%d_d%d\n#define ghc_mid ghc_mid_n%d_d%d\n"
+             "#define ghc_upv ghc_upv_n%d_d%d\n#define D %d\n#define HC %d\n#define NB %d\n"
+             "#define GH_R %d\n#define GH_G %d\n#define GU_SG %d\n#define GV_SG %d\n#define GV_RP %d\n#define GK %d\n",
+             nb, p->D, nb, p->D, nb, p->D, nb, p->D, nb, p->D, p->D, QW_PATH_HC, nb, nb <= 4 ? 16 : 32, nb <= 2 ? 16 : 8, 8, 8, 10, 10);
+    return compile_get(p, name, defs);
+}
+size_t qw_path_hyper_pd_bytes(int nb) { return (size_t)nb * (QW_PATH_HC * (QW_PATH_HC_LR + 2 * QW_PATH_HC) + QW_PATH_HC_LR + QW_PATH_HC) * 4; }
+
+bool qw_path_hyper_gg(qw_path *p, qw_batch *b, const qw_hyper_w *H, int nb, bool apply, bool three, const qw_buf *h, const qw_buf *out, const qw_buf *inj,
+                      const qw_buf *inj_out, const qw_buf *pd, const qw_buf *x) {
+    if (nb < 1 || nb > 16) { fprintf(stderr, "hyper_gg: unsupported token count %d\n", nb); return false; }
+    if (H->hc_norm.type != 0 || H->mix_down.type != 30 || H->mix_up.type != 30 || (H->inject.buf && H->inject.type != 30)) {
+        fprintf(stderr, "hyper_gg: the norm weights must be F32 (0) and the matrices BF16 (30): got %d, %d, %d, %d\n", H->hc_norm.type, H->mix_down.type, H->mix_up.type, H->inject.type);
+        return false;
+    }
+    const uint32_t fl[2] = {apply ? 1u : 0u, H->inject.buf ? 1u : 0u};
+    const qw_tensor *inj_w = H->inject.buf ? &H->inject : &H->mix_down; // src/engine.c:1357-1358: something is bound at 5 either way
+    qw_kernel *kd = gh_kernel(p, three ? "ghc_dsk" : "ghc_down", nb);
+    if (!kd) return false;
+    qw_batch_kernel(b, kd);
+    qw_batch_buf(b, 0, h, 0);
+    qw_batch_buf(b, 1, out, 0);
+    qw_batch_buf(b, 2, inj, 0);
+    bind_t(b, 3, &H->hc_norm);
+    bind_t(b, 4, &H->mix_down);
+    bind_t(b, 5, inj_w);
+    qw_batch_buf(b, 6, pd, 0);
+    qw_batch_bytes(b, 7, fl, sizeof fl);
+    if (three) qw_batch_dispatch(b, 10, QW_PATH_HC, 10, 32 * 8, 1, 1);
+    else qw_batch_dispatch(b, QW_PATH_HC_LR / (nb <= 4 ? 16 : 32) + 1, QW_PATH_HC, 1, (unsigned)p->D / 8, 1, 1);
+    if (three) { // src/engine.c:1364-1386; sx and rs follow the partial sums in pd
+        const size_t o_sx = (size_t)nb * QW_PATH_HC * (QW_PATH_HC_LR + 2 * QW_PATH_HC) * 4, o_rs = o_sx + (size_t)nb * QW_PATH_HC_LR * 4;
+        qw_kernel *km = gh_kernel(p, "ghc_mid", nb), *kv = gh_kernel(p, "ghc_upv", nb);
+        if (!km || !kv) return false;
+        qw_batch_kernel(b, km);
+        qw_batch_buf(b, 0, pd, 0);
+        qw_batch_buf(b, 1, pd, o_sx);
+        qw_batch_buf(b, 2, pd, o_rs);
+        if (inj_out) qw_batch_buf(b, 3, inj_out, 0);
+        qw_batch_bytes(b, 4, fl, sizeof fl);
+        qw_batch_dispatch(b, (unsigned)nb, 1, 1, QW_PATH_HC_LR, 1, 1);
+        qw_batch_kernel(b, kv);
+        qw_batch_buf(b, 0, h, 0);
+        qw_batch_buf(b, 1, out, 0);
+        qw_batch_buf(b, 2, inj, 0);
+        bind_t(b, 3, &H->hc_norm);
+        bind_t(b, 4, &H->mix_up);
+        qw_batch_buf(b, 5, pd, o_sx);
+        qw_batch_buf(b, 6, pd, o_rs);
+        qw_batch_buf(b, 7, x, 0);
+        qw_batch_bytes(b, 8, fl, sizeof fl);
+        qw_batch_dispatch(b, (unsigned)p->D / 8, 1, 1, 32 * 8, 1, 1);
+        return true;
+    }
+    qw_kernel *ku = gh_kernel(p, "ghc_up", nb);
+    if (!ku) return false;
+    qw_batch_kernel(b, ku);
+    qw_batch_buf(b, 0, h, 0);
+    qw_batch_buf(b, 1, out, 0);
+    qw_batch_buf(b, 2, inj, 0);
+    bind_t(b, 3, &H->hc_norm);
+    bind_t(b, 4, &H->mix_up);
+    qw_batch_buf(b, 5, pd, 0);
+    qw_batch_buf(b, 6, x, 0);
+    if (inj_out) qw_batch_buf(b, 7, inj_out, 0);
+    qw_batch_bytes(b, 8, fl, sizeof fl);
+    qw_batch_dispatch(b, (unsigned)p->D / 8, 1, 1, 32 * 8, 1, 1);
+    return true;
+}
+
 // src/engine.c:544-552
 bool qw_path_gg_router(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nb, const qw_buf *x, const qw_buf *lg) {
     qw_kernel *k = gg_kernel(p, "moe_router_bf", M, nb);
@@ -312,6 +392,23 @@ bool qw_path_gg_moe_stack(qw_path *p, qw_batch *b, const qw_moe_layer *M, int nl
     return true;
 }
 void qw_path_set_flush(qw_path *p, uint64_t mask) { p->flush_mask = mask; }
+
+// The FFN half of a decode step, layer after layer (the hyper_in -> moe pair of the reference's layer loop,
+// src/engine.c:1415-1423 and :2169): hyper-connection l turns the streams h into the layer's input x, applying the
+// residual of what the layer before left in out; the MoE layer turns x into out. The inject sums alternate between
+// inj[0] and inj[1] as src/engine.c:1421 swaps them.
+bool qw_path_hyper_moe_stack(qw_path *p, qw_batch *b, const qw_hyper_w *H, const qw_moe_layer *M, int nlayers, int nb, bool pending, const qw_buf *h,
+                             const qw_buf *inj, const qw_buf *pd, const qw_buf *x, const qw_buf *lg, const qw_buf *sel, const qw_buf *out) {
+    int cur = 0;
+    for (int l = 0; l < nlayers; l++) {
+        if (!qw_path_hyper_gg(p, b, &H[l], nb, pending, false, h, out, &inj[cur], &inj[cur ^ 1], pd, x)) return false;
+        if (H[l].inject.buf) cur ^= 1;
+        if (!qw_path_gg_moe(p, b, &M[l], nb, x, &lg[l], &sel[l], out)) return false;
+        pending = true;
+        if (l < 64 && (p->flush_mask >> l & 1) && l + 1 < nlayers) qw_batch_flush(b);
+    }
+    return true;
+}
 
 // ---------------------------------------------------------------- a ragged step (src/engine.c:8783-8814, :9138-9161, :9037)
 // Slot i brings n[i] rows; its first row is r0[i] = n[0] + ... + n[i - 1] (src/engine.c:9150-9161). The R rows are cut

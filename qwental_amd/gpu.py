@@ -28,6 +28,10 @@ class QwMoeLayer(C.Structure):
     _fields_ = [(n, QwTensor) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")]
 
 
+class QwHyperW(C.Structure):
+    _fields_ = [(n, QwTensor) for n in ("hc_norm", "mix_down", "mix_up", "inject")]
+
+
 class QwMoeWeightsDev(C.Structure):
     _fields_ = [(n, C.c_void_p) for n in ("router", "sh_gate_w", "gate", "up", "down", "sh_gate", "sh_up", "sh_down")] + \
                [(n, C.c_int) for n in ("router_type", "gate_type", "down_type", "sh_gate_type", "sh_up_type", "sh_down_type")]
@@ -82,6 +86,9 @@ SYMBOLS = [
     ("qw_path_gg_moe_lg", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
     ("qw_path_gg_moe_stack", _b, [_vp, _vp, _pm, _i, _i, _pb, _pb, _pb, _pb]), ("qw_path_set_flush", None, [_vp, C.c_uint64]),
     ("qw_path_scratch", _pb, [_vp, _i]),
+    ("qw_path_hyper_pd_bytes", _sz, [_i]),
+    ("qw_path_hyper_moe_stack", _b, [_vp, _vp, C.POINTER(QwHyperW), _pm, _i, _i, _b, _pb, _pb, _pb, _pb, _pb, _pb, _pb]),
+    ("qw_path_hyper_gg", _b, [_vp, _vp, C.POINTER(QwHyperW), _i, _b, _b, _pb, _pb, _pb, _pb, _pb, _pb]),
     ("qw_path_par_vstep", _b, [_vp, _vp, _pm, _pi, _i, _pb, _pb, C.POINTER(QwVstepInfo)]),
     ("qw_path_gg_moe_noalloc", _b, [_vp, _i, _i, _i, _i, C.POINTER(QwMoeWeightsDev), _i, _vp, _vp, _vp]),
     ("qw_path_pf_reserve", _b, [_vp, _i, _i]), ("qw_path_pf_moe", _b, [_vp, _vp, _pm, _i, _pb, _pb, _pb, _pb]),
@@ -349,6 +356,21 @@ class Path:
         """The layer with the caller's logits (forced routing)."""
         if not self.L.qw_path_gg_moe_lg(self.p, batch.b, C.byref(layer.c), nb, x.ref(), lg.ref(), sel.ref(), out.ref()):
             raise RuntimeError("qw_path_gg_moe_lg failed")
+
+    def hyper_gg(self, batch, H, nb, apply, h, out, inj, inj_out, pd, x, three=False):
+        """H: dict of Tensor (hc_norm, mix_down, mix_up and, optionally, inject)."""
+        w = QwHyperW()
+        for n in ("hc_norm", "mix_down", "mix_up", "inject"):
+            if H.get(n) is not None:
+                setattr(w, n, H[n].c())
+        ok = self.L.qw_path_hyper_gg(self.p, batch.b, C.byref(w), nb, bool(apply), bool(three), h.ref(), out.ref(), inj.ref(),
+                                     inj_out.ref() if inj_out is not None else None, pd.ref(), x.ref())
+        if not ok:
+            raise RuntimeError("qw_path_hyper_gg failed: " + self.gpu.last_error())
+
+    def hyper_moe_stack(self, batch, hyper_c, layers_c, nlayers, nb, pending, h, inj_c, pd, x, lg_c, sel_c, out):
+        if not self.L.qw_path_hyper_moe_stack(self.p, batch.b, hyper_c, layers_c, nlayers, nb, bool(pending), h.ref(), inj_c, pd.ref(), x.ref(), lg_c, sel_c, out.ref()):
+            raise RuntimeError("qw_path_hyper_moe_stack failed: " + self.gpu.last_error())
 
     def set_flush(self, mask):
         self.L.qw_path_set_flush(self.p, mask)

@@ -10,7 +10,7 @@ import ctypes as C
 import numpy as np
 
 from . import synth
-from .gpu import Buf, MoeLayer, Path, QwBuf, QwMoeLayer, Tensor
+from .gpu import Buf, MoeLayer, Path, QwBuf, QwHyperW, QwMoeLayer, Tensor
 
 MEM_DEFS = "#define QW_HIP_MEM 1\n"
 
@@ -76,6 +76,40 @@ class MoeStack:
         self.bufs += self.lg + self.sel + [self.out]
         self.weight_bytes = sum(x.size for x in self.bufs[:3 * layers])
 
+    def add_hyper(self, seed=99):
+        """A hyper-connection in front of every layer (GGUF profile: F32 norm weights, BF16 mix_down / mix_up / inject): one
+        drawn set of weights, rotated by a different amount for every layer, plus the buffers of the step."""
+        gpu, D, L = self.gpu, self.D, self.L
+        w = synth.hyper_weights(np.random.default_rng(seed), D)
+        self.hyper_host, self.hyper_bufs, hw = [], [], []
+        for l in range(L):
+            wl = {k: np.roll(v.ravel(), 977 * l).reshape(v.shape) for k, v in w.items()}
+            bufs = {k: gpu.buf_from(v, device_only=True) for k, v in wl.items()}
+            c = QwHyperW()
+            for k in ("hc_norm", "mix_down", "mix_up", "inject"):
+                setattr(c, k, Tensor(bufs[k], 0 if k == "hc_norm" else 30).c())
+            hw.append(c)
+            self.hyper_host.append(wl)
+            self.hyper_bufs += list(bufs.values())
+        self.hyper_c = (QwHyperW * L)(*hw)
+        nb = self.nbmax
+        self.h = gpu.buf(nb * 4 * D * 4)
+        self.inj = [gpu.buf(nb * 16 * 4), gpu.buf(nb * 16 * 4)]
+        self.inj_c = (QwBuf * 2)(*[x.c for x in self.inj])
+        self.pd = gpu.buf(int(gpu.L.qw_path_hyper_pd_bytes(nb)), device_only=True)
+        self.x = gpu.buf(nb * D * 2)
+        self.hyper_bufs += [self.h, self.pd, self.x] + self.inj
+        self.hyper_bytes = sum(v.nbytes for v in w.values())
+        return self
+
+    def step_hyper(self, nb, nlayers=None, pending=False):
+        """One decode step of the FFN halves: hyper-connection -> MoE layer, layer after layer, on the streams in self.h and the
+        inject sums in self.inj[0]; returns GPU seconds."""
+        b = self.gpu.batch()
+        self.path.hyper_moe_stack(b, self.hyper_c, self.layers_c, self.L if nlayers is None else nlayers, nb, pending, self.h, self.inj_c, self.pd, self.x,
+                                  self.lg_c, self.sel_c, self.out)
+        return b.end()
+
     def shared_bytes(self, l):
         f = self.shared_fmt[l]
         return self.I * (synth.row_bytes(f[0], self.D) + synth.row_bytes(f[1], self.D)) + self.D * synth.row_bytes(f[2], self.I)
@@ -107,6 +141,6 @@ class MoeStack:
                     Wsg=sb[:sh_g], Wsu=sb[sh_g:sh_g + sh_u], Wsd=sb[sh_g + sh_u:], Wr=rb[:E * D].view(np.float16).reshape(E, D), wsg=rb[E * D:].view(np.float16))
 
     def free(self):
-        for b in self.bufs:
+        for b in self.bufs + getattr(self, "hyper_bufs", []):
             b.free()
         self.path.close()

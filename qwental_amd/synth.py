@@ -97,3 +97,25 @@ def logits_for_ids(rng, ids, E):
     for t in range(rows):
         lg[t, ids[t]] = 4.0 - 0.25 * np.arange(topk, dtype=np.float32)
     return lg
+
+
+def to_bf16(a):
+    """float -> bfloat16 bit patterns (uint16), round to nearest even."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def hyper_weights(rng, D, hc=4, lr=320, inject=True):
+    """Weights of one hyper-connection of the GGUF profile: norm weights float32 [hc * D] around 1, mix_down [lr, hc * D],
+    mix_up [hc * D, lr] and (inject) [hc, hc * D] as bfloat16 bit patterns, scaled so that their products are O(1)."""
+    return {"hc_norm": (1 + 0.1 * rng.standard_normal(hc * D)).astype(np.float32),
+            "mix_down": to_bf16(rng.standard_normal((lr, hc * D)) / np.sqrt(hc * D) * 2),
+            "mix_up": to_bf16(rng.standard_normal((hc * D, lr)) / np.sqrt(lr) * 2),
+            "inject": to_bf16(rng.standard_normal((hc, hc * D)) / np.sqrt(D)) if inject else None}
+
+
+def hyper_state(rng, nb, D, hc=4):
+    """Streams h float32 [nb, hc, D] (a different scale per stream), a sublayer output binary16 [nb, D] and inject sums
+    float32 [nb, hc, hc]."""
+    h = (rng.standard_normal((nb, hc, D)) * (0.5 + np.arange(hc))[None, :, None]).astype(np.float32)
+    return h, (0.5 * rng.standard_normal((nb, D))).astype(np.float16), rng.standard_normal((nb, hc, hc)).astype(np.float32)
