@@ -170,6 +170,48 @@ def read_ceiling(gpu, stack, nb, reps=5):
     return out
 
 
+def hyper_ffn_leg(gpu, stack, steps, warmup):
+    """The FFN half of the decode loop with its layer-to-layer dependency: hyper-connection (GGUF profile: F32 norm, BF16
+    mix_down / mix_up / inject) -> MoE layer, for every layer of the stack, at B = 1, 8, 16. Tokens/s and GPU time per
+    step, and the mean launch times of the two hyper-connection kernels with the bytes they read."""
+    from qwental_amd import synth
+    stack.add_hyper()
+    D = stack.D
+    h0, _, inj0 = synth.hyper_state(np.random.default_rng(77), 16, D)
+    res = {"workload": "%d x (hyper-connection HC=4 LR=320 -> MoE layer), D=%d" % (stack.L, D), "hyper_weight_bytes_per_layer": int(stack.hyper_bytes), "by_batch": {}}
+    for nb in (1, 8, 16):
+        def step():
+            # the streams grow with every residual: every step starts from the same state
+            stack.h.fill(h0)
+            stack.inj[0].fill(inj0)
+            return stack.step_hyper(nb)
+        for _ in range(warmup):
+            step()
+        gpu_s, t0, wall = 0.0, 0.0, 0.0
+        for _ in range(steps):
+            stack.h.fill(h0)
+            stack.inj[0].fill(inj0)
+            t0 = time.perf_counter()
+            gpu_s += stack.step_hyper(nb)
+            wall += time.perf_counter() - t0
+        gpu.profile(True)
+        step()
+        gpu.profile(False)
+        per = {}
+        for name, us in gpu.profile_entries():
+            if name.startswith("qwk_hc"):
+                per.setdefault(name, []).append(us)
+        k = {n: float(np.mean(v)) for n, v in per.items()}
+        kd = next((v for n, v in k.items() if n.startswith("qwk_hc_down")), None)
+        # down reads mix_down and inject once, up reads mix_up once; h, out and the norm weights are small beside them
+        lr, hc = 320, 4
+        b_down, b_up = (lr + hc) * hc * D * 2 + nb * hc * D * 4 + hc * D * 4, hc * D * lr * 2 + nb * hc * D * 4
+        res["by_batch"][str(nb)] = {"tokens_per_s": nb * steps / wall, "gpu_ms_per_step": gpu_s / steps * 1e3, "kernel_us_mean": k,
+                                    "down_GBps": b_down / (kd * 1e-6) / 1e9 if kd else None,
+                                    "up_GBps": b_up / (k["qwk_hc_up"] * 1e-6) / 1e9 if "qwk_hc_up" in k else None}
+    return res
+
+
 def ragged_steps(gpu, stack, reps=5):
     """BASELINE.json configs[3]: a continuous-batching step of one layer (layer 0 of the stack): 16 slots with seeded
     uniform row counts in 1..16 redrawn until the total is near the target, Zipf(1.1) routing forced through the
@@ -440,6 +482,7 @@ def main():
     ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
     ap.add_argument("--gguf-only", action="store_true", help="only the GGUF load measurement")
     ap.add_argument("--model-shape-only", action="store_true", help="only the stack of the reference model's layer shape and formats")
+    ap.add_argument("--hyper-only", action="store_true", help="only the hyper-connection -> MoE layer loop")
     ap.add_argument("--ragged-only", action="store_true", help="only the continuous-batching step table (config 4) on a one-layer stack: for profiling runs")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -458,6 +501,11 @@ def main():
         return 0
     if a.model_shape_only:
         print(json.dumps({"model_shape": model_shape_leg(gpu, a.layers, a.steps, a.warmup, not a.no_cpu)}))
+        return 0
+    if a.hyper_only:
+        stack = MoeStack(gpu, layers=a.layers, nbmax=16)
+        print(json.dumps({"hyper_ffn_step": hyper_ffn_leg(gpu, stack, a.steps, a.warmup)}))
+        stack.free()
         return 0
     if a.ragged_only:
         stack = MoeStack(gpu, layers=1, nbmax=16)
@@ -511,6 +559,7 @@ def main():
             "kernel_us_mean": {k: float(np.mean(v)) for k, v in per_kernel.items()},
             "setup_s": setup_s}
     if not a.quick:
+        line["hyper_ffn_step"] = hyper_ffn_leg(gpu, stack, min(a.steps, 10), a.warmup)
         line["ragged_step"] = ragged_steps(gpu, stack)
         line["qmv"] = qmv_table(gpu)
         line["qmv_formats"] = formats_table(gpu)

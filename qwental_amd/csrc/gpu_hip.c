@@ -497,7 +497,7 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
         int hc;
         if (!def_int(d, n, "D", &p.D) || !def_int(d, n, "HC", &hc) || !def_int(d, n, "NB", &p.NB)) FAIL("hyper_gg: D, HC and NB must be integers");
         if (hc != (int)QW_HC) FAIL("hyper_gg: HC %d (this build has %u streams)", hc, QW_HC);
-        if (p.D <= 0 || p.D % 512 || p.D > 8192) FAIL("hyper_gg: D %d must be a multiple of 512 up to 8192", p.D);
+        if (p.D <= 0 || p.D % 512 || p.D > 4096) FAIL("hyper_gg: D %d must be a multiple of 512 up to 4096", p.D);
         if (p.NB < 1 || p.NB > 16) FAIL("hyper_gg: NB %d (1 to 16)", p.NB);
         // GH_R, GH_G, GU_SG, GV_SG, GV_RP and GK tune the reference's own kernels; the ones here have their own shape
         if (!reg_kernel(g, d, n, "ghc_down", FAM_HC_DOWN, &p, err, errlen) || !reg_kernel(g, d, n, "ghc_up", FAM_HC_UP, &p, err, errlen) ||
@@ -1540,8 +1540,10 @@ static bool tr_hc(qw_batch *b) {
     if (f == FAM_HC_DOWN) {
         if (!bind_ptr(b, 4, QW_HC_LR * HCD * 2, false, "mix_down", (void **)&a.Wd) || !bind_ptr(b, 6, nb * QW_HC * QW_HC_PDS * 4, true, "partial sums", (void **)&a.pd)) return false;
         if (a.want_inj && !bind_ptr(b, 5, QW_HC * HCD * 2, false, "inject", (void **)&a.Wi)) return false;
-        if (!add_launch(b, "qwk_hc_down", QW_HC_LR / QW_HC_ROWS + (a.want_inj ? 1 : 0), (unsigned)(D / 8), &a, sizeof a)) return false;
+        const unsigned R = nb <= 4 ? 4 : 16; // rows per workgroup: many workgroups at a few tokens, less re-reading of h at many
+        if (!add_launch(b, R == 4 ? "qwk_hc_down_r4" : "qwk_hc_down_r16", QW_HC_LR / R + (a.want_inj ? 1 : 0), (unsigned)(D / 8), &a, sizeof a)) return false;
         b->l[b->nl - 1].gy = QW_HC;
+        b->l[b->nl - 1].gz = (unsigned)(nb + QW_HC_TG - 1) / QW_HC_TG; // tokens four at a time
         return true;
     }
     if (!bind_ptr(b, 4, HCD * QW_HC_LR * 2, false, "mix_up", (void **)&a.Wu)) return false;

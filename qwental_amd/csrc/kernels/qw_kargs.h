@@ -141,7 +141,7 @@ typedef struct { /* pure-read ceiling and fill helpers */
 #define QW_HC 4u
 #define QW_HC_LR 320u
 #define QW_HC_PDS (QW_HC_LR + 2 * QW_HC)
-#define QW_HC_ROWS 4u /* weight rows per workgroup of the down kernel */
+#define QW_HC_TG 4u   /* tokens per workgroup of the down kernel */
 typedef struct {
     float *h;                      /* [nb][HC][D]; the up kernels write it back when the residual is applied */
     const uint16_t *out;           /* binary16 [nb][D]: the sublayer output the residual adds */

@@ -1652,63 +1652,95 @@ __device__ __forceinline__ float hc_coef(const float *injp, uint32_t s) {
     for (uint32_t q = 0; q < QW_HC; q++) t += injp[q * QW_HC + s];
     return 2.0f / (1.0f + expf(-t / QW_HC));
 }
+// Four sums at once over the lanes of a wave (W = 64) or of each half (W = 32): two exchange steps leave every lane with
+// one of the four values summed over a quad of lanes, the remaining steps add the quads. Lane l ends with the whole sum
+// of value number 2 (l & 1) + ((l >> 1) & 1). Seven (six) shuffles instead of four times six (five).
+template <int W> __device__ __forceinline__ float qw_sum4(float d0, float d1, float d2, float d3, uint32_t lane) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+    const float e0 = (b0 ? d2 : d0) + __shfl_xor(b0 ? d0 : d2, 1), e1 = (b0 ? d3 : d1) + __shfl_xor(b0 ? d1 : d3, 1);
+    float f = (b1 ? e1 : e0) + __shfl_xor(b1 ? e0 : e1, 2);
+#pragma unroll
+    for (int o = 4; o < W; o <<= 1) f += __shfl_xor(f, o);
+    return f;
+}
 // Down: residual, sums of squares and the un-normalised mix_down / inject sums (kernels/hyper_gg.metal:94-137).
-// Workgroup (rb, s): QW_HC_ROWS weight rows (block 80 = the inject rows) against stream s; thread c owns columns
-// 8 c .. 8 c + 7 (16 bytes of a bfloat16 row, kept in registers for every token). Per token: the lane's eight
-// h' w products, four dot products of eight and the squares, summed over the wave, then over the waves in order.
-extern "C" __global__ __launch_bounds__(1024) void qwk_hc_down(qwk_hc_args a) {
-    __shared__ float part[16][16][QW_HC_ROWS + 1]; // [wave][token][row | squares]
-    const uint32_t rb = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nwv = blockDim.x >> 6;
-    const bool is_inj = rb == QW_HC_LR / QW_HC_ROWS;
+// Workgroup (rb, s, tg): R weight rows (the last block = the four inject rows) against stream s of tokens
+// 4 tg .. 4 tg + 3; thread c owns columns 8 c .. 8 c + 7 (16 bytes of a bfloat16 row). Everything a thread reads is
+// asked for before anything is used, so the kernel is one memory round trip whatever the token count. Per token: the
+// lane's eight h' w products, R dot products of eight and the squares, summed over the wave, then over the waves in
+// order. R = 4 fills the machine at a few tokens; R = 16 re-reads h and out four times less often at many.
+template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_args &a, float (*part)[QW_HC_TG][17]) {
+    const uint32_t rb = blockIdx.x, s = blockIdx.y, t0 = blockIdx.z * QW_HC_TG, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nwv = blockDim.x >> 6;
+    const uint32_t nt = a.nb - t0 < QW_HC_TG ? a.nb - t0 : QW_HC_TG;
+    const bool is_inj = rb == QW_HC_LR / R;
+    const uint32_t nrow = is_inj ? QW_HC : R; // rows of this block (uniform)
     const size_t HCD = (size_t)QW_HC * a.D, c0 = (size_t)s * a.D + 8 * tid;
-    const uint16_t *W = is_inj ? a.Wi : a.Wd + (size_t)rb * QW_HC_ROWS * HCD;
-    float wf[QW_HC_ROWS][8];
+    const uint16_t *W = is_inj ? a.Wi : a.Wd + (size_t)rb * R * HCD;
+    u4 wu[R], ou[QW_HC_TG];
+    f4 hv[QW_HC_TG][2];
 #pragma unroll
-    for (uint32_t r = 0; r < QW_HC_ROWS; r++) {
-        const u4 u = *(const u4 *)(W + (size_t)r * HCD + c0);
-#pragma unroll
-        for (int k = 0; k < 4; k++) wf[r][2 * k] = __builtin_bit_cast(float, u[k] << 16), wf[r][2 * k + 1] = __builtin_bit_cast(float, u[k] & 0xffff0000u);
-    }
+    for (uint32_t r = 0; r < R; r++)
+        if (r < nrow) wu[r] = *(const u4 *)(W + (size_t)r * HCD + c0);
     const f4 w0 = *(const f4 *)(a.w + c0), w1 = *(const f4 *)(a.w + c0 + 4);
-    for (uint32_t t = 0; t < a.nb; t++) {
-        const f4 h0 = *(const f4 *)(a.h + t * HCD + c0), h1 = *(const f4 *)(a.h + t * HCD + c0 + 4);
-        float v[8] = {h0[0], h0[1], h0[2], h0[3], h1[0], h1[1], h1[2], h1[3]};
-        if (a.apply) { // out is not read otherwise: it may never have been written
-            const float js = hc_coef(a.inj + t * QW_HC * QW_HC, s);
-            const u4 o = *(const u4 *)(a.out + (size_t)t * a.D + 8 * tid);
+#pragma unroll
+    for (uint32_t tt = 0; tt < QW_HC_TG; tt++) {
+        if (tt < nt) {
+            hv[tt][0] = *(const f4 *)(a.h + (t0 + tt) * HCD + c0), hv[tt][1] = *(const f4 *)(a.h + (t0 + tt) * HCD + c0 + 4);
+            if (a.apply) ou[tt] = *(const u4 *)(a.out + (size_t)(t0 + tt) * a.D + 8 * tid); // not read otherwise: it may never have been written
+        }
+    }
+#pragma unroll
+    for (uint32_t tt = 0; tt < QW_HC_TG; tt++) {
+        if (tt >= nt) break;
+        float v[8] = {hv[tt][0][0], hv[tt][0][1], hv[tt][0][2], hv[tt][0][3], hv[tt][1][0], hv[tt][1][1], hv[tt][1][2], hv[tt][1][3]};
+        if (a.apply) {
+            const float js = hc_coef(a.inj + (t0 + tt) * QW_HC * QW_HC, s);
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                v[2 * k] = fmaf(qw_h2f((uint16_t)o[k]), js, v[2 * k]);
-                v[2 * k + 1] = fmaf(qw_h2f((uint16_t)(o[k] >> 16)), js, v[2 * k + 1]);
+                v[2 * k] = fmaf(qw_h2f((uint16_t)ou[tt][k]), js, v[2 * k]);
+                v[2 * k + 1] = fmaf(qw_h2f((uint16_t)(ou[tt][k] >> 16)), js, v[2 * k + 1]);
             }
         }
         float ss = 0, x[8];
 #pragma unroll
         for (int k = 0; k < 8; k++) ss = fmaf(v[k], v[k], ss), x[k] = v[k] * (k < 4 ? w0[k] : w1[k - 4]);
-        float d[QW_HC_ROWS];
-#pragma unroll
-        for (uint32_t r = 0; r < QW_HC_ROWS; r++) {
-            d[r] = 0;
-#pragma unroll
-            for (int k = 0; k < 8; k++) d[r] = fmaf(wf[r][k], x[k], d[r]);
-            d[r] = qw_wave_sum(d[r]);
-        }
         ss = qw_wave_sum(ss);
-        if (lane == 0) {
+        if (lane == 0) part[wave][tt][16] = ss;
 #pragma unroll
-            for (uint32_t r = 0; r < QW_HC_ROWS; r++) part[wave][t][r] = d[r];
-            part[wave][t][QW_HC_ROWS] = ss;
+        for (uint32_t r0 = 0; r0 < R; r0 += 4) {
+            if (r0 >= nrow) break;
+            float d[4];
+#pragma unroll
+            for (uint32_t r = 0; r < 4; r++) {
+                d[r] = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    d[r] = fmaf(__builtin_bit_cast(float, wu[r0 + r][k] << 16), x[2 * k], d[r]);
+                    d[r] = fmaf(__builtin_bit_cast(float, wu[r0 + r][k] & 0xffff0000u), x[2 * k + 1], d[r]);
+                }
+            }
+            const float f = qw_sum4<64>(d[0], d[1], d[2], d[3], lane);
+            if (lane < 4) part[wave][tt][r0 + 2 * (lane & 1) + (lane >> 1)] = f;
         }
     }
     __syncthreads();
-    for (uint32_t j = tid; j < a.nb * (QW_HC_ROWS + 1); j += blockDim.x) {
-        const uint32_t t = j / (QW_HC_ROWS + 1), r = j % (QW_HC_ROWS + 1);
+    for (uint32_t j = tid; j < nt * 17; j += blockDim.x) {
+        const uint32_t tt = j / 17, r = j % 17;
+        if (r < 16 && r >= nrow) continue;
         float sum = 0;
-        for (uint32_t q = 0; q < nwv; q++) sum += part[q][t][r];
-        float *pd = a.pd + ((size_t)t * QW_HC + s) * QW_HC_PDS;
-        if (r < QW_HC_ROWS) pd[(is_inj ? QW_HC_LR : rb * QW_HC_ROWS) + r] = sum;
+        for (uint32_t q = 0; q < nwv; q++) sum += part[q][tt][r];
+        float *pd = a.pd + ((size_t)(t0 + tt) * QW_HC + s) * QW_HC_PDS;
+        if (r < 16) pd[(is_inj ? QW_HC_LR : rb * R) + r] = sum;
         else if (rb == 0) pd[QW_HC_LR + QW_HC] = sum;
     }
+}
+extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r4(qwk_hc_args a) {
+    __shared__ float part[8][QW_HC_TG][17]; // [wave][token][row | squares]
+    hc_down_body<4>(a, part);
+}
+extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r16(qwk_hc_args a) {
+    __shared__ float part[8][QW_HC_TG][17];
+    hc_down_body<16>(a, part);
 }
 // What follows the down kernel for tokens t0 .. t0 + nt - 1, by the threads of one workgroup: the streams' 1 / rms,
 // silu of the normalised mix_down sums, and (injo given) the inject sums in the caller's format
@@ -1717,13 +1749,24 @@ __device__ __forceinline__ void hc_mid(const qwk_hc_args &a, uint32_t t0, uint32
     const float *pd = a.pd + (size_t)t0 * QW_HC * QW_HC_PDS;
     for (uint32_t j = threadIdx.x; j < nt * QW_HC; j += blockDim.x) rs[j] = rsqrtf(pd[j * QW_HC_PDS + QW_HC_LR + QW_HC] / (float)a.D + 1e-6f);
     __syncthreads();
-    for (uint32_t j = threadIdx.x; j < nt * QW_HC_LR; j += blockDim.x) {
-        const uint32_t t = j / QW_HC_LR, r = j % QW_HC_LR;
-        float d = 0;
+    for (uint32_t j0 = threadIdx.x; j0 < nt * QW_HC_LR; j0 += 4 * blockDim.x) { // four elements a round: their sixteen loads go out together
+        float p[4][QW_HC];
 #pragma unroll
-        for (uint32_t q = 0; q < QW_HC; q++) d = fmaf(rs[t * QW_HC + q], pd[(t * QW_HC + q) * QW_HC_PDS + r], d);
-        d /= QW_HC;
-        sx[j] = d / (1.0f + __expf(-d));
+        for (uint32_t e = 0; e < 4; e++) {
+            const uint32_t j = j0 + e * blockDim.x, t = j / QW_HC_LR, r = j % QW_HC_LR;
+#pragma unroll
+            for (uint32_t q = 0; q < QW_HC; q++) p[e][q] = j < nt * QW_HC_LR ? pd[(t * QW_HC + q) * QW_HC_PDS + r] : 0.0f;
+        }
+#pragma unroll
+        for (uint32_t e = 0; e < 4; e++) {
+            const uint32_t j = j0 + e * blockDim.x, t = j / QW_HC_LR;
+            if (j >= nt * QW_HC_LR) break;
+            float d = 0;
+#pragma unroll
+            for (uint32_t q = 0; q < QW_HC; q++) d = fmaf(rs[t * QW_HC + q], p[e][q], d);
+            d /= QW_HC;
+            sx[j] = d / (1.0f + __expf(-d));
+        }
     }
     if (injo)
         for (uint32_t j = threadIdx.x; j < nt * QW_HC * QW_HC; j += blockDim.x) // j = (t, s, q)
@@ -1753,7 +1796,17 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
 #pragma unroll
         for (int k = 0; k < 5; k++) u[q][k] = wr[k];
     }
-    const float wn = l32 < QW_HC ? a.w[(size_t)l32 * a.D + i] : 0.0f;
+    // lane l of a group owns token l / 4 (and that plus 8) and the stream qw_sum4 leaves with it: its h, out and norm weight
+    // are asked for now as well
+    const uint32_t ts = l32 / QW_HC, sq = 2 * (l32 & 1) + ((l32 >> 1) & 1);
+    const float wn = a.w[(size_t)sq * a.D + i];
+    float hv[2] = {0, 0}, ov[2] = {0, 0};
+#pragma unroll
+    for (uint32_t r = 0; r < 2; r++)
+        if (ts + 8 * r < a.nb) {
+            hv[r] = a.h[(ts + 8 * r) * HCD + (size_t)sq * a.D + i];
+            if (a.apply) ov[r] = qw_h2f(a.out[(size_t)(ts + 8 * r) * a.D + i]);
+        }
     if (GIVEN) {
         for (uint32_t j = tid; j < a.nb * QW_HC_LR; j += blockDim.x) sx[j / QW_HC_LR][j % QW_HC_LR] = a.sx[j];
         if (tid < a.nb * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[tid];
@@ -1767,37 +1820,41 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
     for (uint32_t q = 0; q < QW_HC; q++)
 #pragma unroll
         for (int k = 0; k < 5; k++) v[q][2 * k] = __builtin_bit_cast(float, u[q][k] << 16), v[q][2 * k + 1] = __builtin_bit_cast(float, u[q][k] & 0xffff0000u);
+    // mix_up: for every token four dot products of ten, summed over the group's 32 lanes; the lanes of the token's quad
+    // keep the sums of their streams
+    float uv[2] = {0, 0};
     for (uint32_t t = 0; t < a.nb; t++) {
-        // lanes 0..3 of the group are the four streams of column i: their h (and out) loads go out before the products
-        float hv = 0, ov = 0;
-        if (l32 < QW_HC) {
-            hv = a.h[t * HCD + (size_t)l32 * a.D + i];
-            if (a.apply) ov = qw_h2f(a.out[(size_t)t * a.D + i]);
-        }
         float xv[10];
 #pragma unroll
         for (int k = 0; k < 10; k++) xv[k] = sx[t][l32 * 10 + k];
-        float mine = 0;
+        float d[QW_HC];
 #pragma unroll
         for (uint32_t q = 0; q < QW_HC; q++) {
-            float d = 0;
+            d[q] = 0;
 #pragma unroll
-            for (int k = 0; k < 10; k++) d = fmaf(v[q][k], xv[k], d);
-#pragma unroll
-            for (int o = 16; o; o >>= 1) d += __shfl_xor(d, o); // over the 32 lanes of the group
-            mine = l32 == q ? d : mine;
+            for (int k = 0; k < 10; k++) d[q] = fmaf(v[q][k], xv[k], d[q]);
         }
+        const float f = qw_sum4<32>(d[0], d[1], d[2], d[3], l32); // this lane's stream, summed over the group
+        const bool own = ts == (t & 7);
+        uv[0] = own && t < 8 ? f : uv[0];
+        uv[1] = own && t >= 8 ? f : uv[1];
+    }
+    // the gates and the mix over the streams: the four streams of a token are neighbouring lanes
+#pragma unroll
+    for (uint32_t r = 0; r < 2; r++) {
+        const uint32_t t = ts + 8 * r;
         float m = 0;
-        if (l32 < QW_HC) {
+        if (t < a.nb) {
+            float hq = hv[r];
             if (a.apply) {
-                hv = fmaf(ov, js[t][l32], hv);
-                a.h[t * HCD + (size_t)l32 * a.D + i] = hv;
+                hq = fmaf(ov[r], js[t][sq], hq);
+                a.h[t * HCD + (size_t)sq * a.D + i] = hq;
             }
-            m = (hv * rs[t][l32]) * wn / (1.0f + __expf(-mine));
+            m = (hq * rs[t][sq]) * wn / (1.0f + __expf(-uv[r]));
         }
         m += __shfl_xor(m, 1);
         m += __shfl_xor(m, 2);
-        if (l32 == 0) a.x[(size_t)t * a.D + i] = qw_f2h(m / QW_HC);
+        if (t < a.nb && sq == 0) a.x[(size_t)t * a.D + i] = qw_f2h(m / QW_HC);
     }
 }
 extern "C" __global__ __launch_bounds__(256) void qwk_hc_up(qwk_hc_args a) { hc_up_body<false>(a); }

@@ -119,7 +119,7 @@ def test_two_in_a_row_carry_the_streams_and_the_inject_sums(gpu, oracle, hyper):
 
 def test_refusals(gpu):
     blk = "#define ghc_down ghc_down_t\n#define ghc_up ghc_up_t\n#define D %d\n#define HC %d\n#define NB %d\n#define GH_R 16\n"
-    for D, hc, nb in ((2304, 4, 1), (2048, 3, 1), (2048, 4, 17), (16384, 4, 1)):
+    for D, hc, nb in ((2304, 4, 1), (2048, 3, 1), (2048, 4, 17), (8192, 4, 1)):
         ok, err = gpu.compile(blk % (D, hc, nb))
         assert not ok and err
     ok, err = gpu.compile(blk % (2048, 4, 2))
