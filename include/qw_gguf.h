@@ -34,7 +34,7 @@ enum {
     QW_GG_ROUTER = 1u << 2, /* router + shared-expert gate vector */
     QW_GG_ATTN = 1u << 3,   /* attention projections and norms */
     QW_GG_LIN = 1u << 4,    /* linear-attention projections and their small tensors */
-    QW_GG_HYPER = 1u << 5,  /* hyper-connection (not loaded here) */
+    QW_GG_HYPER = 1u << 5,  /* hyper-connections of the layers and the output mixer */
     QW_GG_LM = 1u << 6,     /* lm_head */
     QW_GG_EMBED = 1u << 7,  /* token embedding */
     QW_GG_PLE = 1u << 8,    /* per-layer embedding (not loaded here) */
@@ -91,6 +91,11 @@ double qw_gguf_load_seconds(const qw_gguf *f);
 bool qw_gguf_tensor_at(const qw_gguf *f, const qw_gguf_tensor *t, qw_tensor *out);
 /* The MoE weights of one layer (blk.<layer>.ffn_*), checked against each other; D, I, E receive the layer's sizes. */
 bool qw_gguf_moe_layer(const qw_gguf *f, int layer, qw_moe_layer *M, int *D, int *I, int *E, char *err, size_t errlen);
+
+/* The weights of one hyper-connection (src/gguf.c:222-229, :250-252): which = 0 blk.<layer>.hc_attn_*, 1 blk.<layer>.hc_ffn_*,
+ * 2 the output mixer (no inject rows; H->inject.buf stays NULL); D receives the width of a stream. The inject rows must be
+ * exact in BF16 (they are converted as a small tensor), as the reference's kernel reads them as BF16. */
+bool qw_gguf_hyper(const qw_gguf *f, int layer, int which, qw_hyper_w *H, int *D, char *err, size_t errlen);
 
 #ifdef __cplusplus
 }

@@ -119,10 +119,23 @@ static const struct { const char *g; unsigned part; const char *m; int kind; } L
     {"ssm_dt.bias", QW_GG_LIN, "linear_attn.dt_bias", QW_GK_SMALL},
     {"ssm_conv1d.weight", QW_GG_LIN, "linear_attn.conv1d.weight", QW_GK_SMALL},
     {"ssm_norm.weight", QW_GG_LIN, "linear_attn.norm.weight", QW_GK_SMALL},
+    // the two hyper-connections of a layer (src/gguf.c:222-229): BF16 matrices as they are, inject as a small tensor, norm F32
+    {"hc_attn_down.weight", QW_GG_HYPER, "attn_hyper_connection.input_mix_weight_down.weight", QW_GK_LIN},
+    {"hc_attn_up.weight", QW_GG_HYPER, "attn_hyper_connection.input_mix_weight_up.weight", QW_GK_LIN},
+    {"hc_attn_inject.weight", QW_GG_HYPER, "attn_hyper_connection.block_inject_weight.weight", QW_GK_SMALL},
+    {"hc_attn_norm.weight", QW_GG_HYPER, "attn_hyper_connection.hc_norm.weight", QW_GK_F32},
+    {"hc_ffn_down.weight", QW_GG_HYPER, "mlp_hyper_connection.input_mix_weight_down.weight", QW_GK_LIN},
+    {"hc_ffn_up.weight", QW_GG_HYPER, "mlp_hyper_connection.input_mix_weight_up.weight", QW_GK_LIN},
+    {"hc_ffn_inject.weight", QW_GG_HYPER, "mlp_hyper_connection.block_inject_weight.weight", QW_GK_SMALL},
+    {"hc_ffn_norm.weight", QW_GG_HYPER, "mlp_hyper_connection.hc_norm.weight", QW_GK_F32},
 };
 static const struct { const char *g; unsigned part; const char *m; int kind; } TOP_NAMES[] = {
     {"output.weight", QW_GG_LM, "language_model.lm_head.weight", QW_GK_LIN},
     {"token_embd.weight", QW_GG_EMBED, "language_model.model.embed_tokens.weight", QW_GK_LIN},
+    // the mixer after the last layer (src/gguf.c:250-252): no inject rows
+    {"output_hc_down.weight", QW_GG_HYPER, "language_model.model.hyper_connection_mixer.input_mix_weight_down.weight", QW_GK_LIN},
+    {"output_hc_up.weight", QW_GG_HYPER, "language_model.model.hyper_connection_mixer.input_mix_weight_up.weight", QW_GK_LIN},
+    {"output_hc_norm.weight", QW_GG_HYPER, "language_model.model.hyper_connection_mixer.hc_norm.weight", QW_GK_F32},
 };
 
 static char *map_name(const char *g, unsigned *part, int *kind) {
@@ -541,5 +554,35 @@ bool qw_gguf_moe_layer(const qw_gguf *G, int layer, qw_moe_layer *M, int *D, int
     *D = (int)d;
     *I = (int)in;
     *E = (int)e;
+    return true;
+}
+
+// The weights of one hyper-connection: which = 0 the one in front of a layer's attention / linear attention
+// (blk.<layer>.hc_attn_*), 1 the one in front of its MoE (hc_ffn_*), 2 the mixer after the last layer (output_hc_*, layer
+// ignored, no inject rows). Shapes (src/model.h:41-45): norm [HC D], mix_down [LR][HC D], mix_up [HC D][LR], inject [HC][HC D].
+bool qw_gguf_hyper(const qw_gguf *G, int layer, int which, qw_hyper_w *H, int *D, char *err, size_t errlen) {
+    if (err && errlen) err[0] = 0;
+    if (which < 0 || which > 2) return fail(err, errlen, "GGUF: hyper-connection %d (0 attention, 1 MoE, 2 output mixer)", which);
+    static const char *const part[4] = {"norm", "down", "up", "inject"};
+    qw_tensor *const dst[4] = {&H->hc_norm, &H->mix_down, &H->mix_up, &H->inject};
+    const qw_gguf_tensor *t[4] = {0};
+    memset(H, 0, sizeof *H);
+    for (int i = 0; i < (which == 2 ? 3 : 4); i++) {
+        char name[128];
+        if (which == 2) snprintf(name, sizeof name, "output_hc_%s.weight", part[i]);
+        else snprintf(name, sizeof name, "blk.%d.hc_%s_%s.weight", layer, which ? "ffn" : "attn", part[i]);
+        t[i] = qw_gguf_find(G, name);
+        if (!t[i]) return fail(err, errlen, "GGUF: %s is missing", name);
+        if (!qw_gguf_tensor_at(G, t[i], dst[i])) return fail(err, errlen, "GGUF: %s is not resident", name);
+    }
+    const uint64_t hcd = t[0]->dims[0] * t[0]->rows;
+    if (hcd % QW_PATH_HC) return fail(err, errlen, "GGUF: hyper-connection norm of %llu values is not %d streams", (unsigned long long)hcd, QW_PATH_HC);
+    bool ok = t[1]->nd == 2 && t[1]->dims[0] == hcd && t[1]->dims[1] == QW_PATH_HC_LR && t[2]->nd == 2 && t[2]->dims[0] == QW_PATH_HC_LR && t[2]->dims[1] == hcd;
+    if (t[3]) ok = ok && t[3]->dims[0] == hcd && t[3]->rows == QW_PATH_HC;
+    if (!ok) return fail(err, errlen, "GGUF: the shapes of the hyper-connection tensors do not agree");
+    if (H->hc_norm.type != 0 || H->mix_down.type != 30 || H->mix_up.type != 30 || (t[3] && H->inject.type != 30))
+        return fail(err, errlen, "GGUF: hyper-connection tensors must be resident as F32 norm and BF16 matrices (got %s, %s, %s, %s)", qw_ggml_name(H->hc_norm.type),
+                    qw_ggml_name(H->mix_down.type), qw_ggml_name(H->mix_up.type), t[3] ? qw_ggml_name(H->inject.type) : "-");
+    *D = (int)(hcd / QW_PATH_HC);
     return true;
 }

@@ -100,6 +100,7 @@ SYMBOLS = [
     ("qw_gguf_shard_data_start", C.c_uint64, [_vp, _i]), ("qw_gguf_count", _i, [_vp]), ("qw_gguf_get", _pg, [_vp, _i]),
     ("qw_gguf_find", _pg, [_vp, C.c_char_p]), ("qw_gguf_host", _vp, [_vp, _pg]),
     ("qw_gguf_load", _b, [_vp, _vp, _u, C.c_char_p, _sz]), ("qw_gguf_resident_bytes", _sz, [_vp]), ("qw_gguf_load_seconds", _d, [_vp]),
+    ("qw_gguf_hyper", _b, [_vp, _i, _i, C.POINTER(QwHyperW), _pi, C.c_char_p, _sz]),
     ("qw_gguf_tensor_at", _b, [_vp, _pg, _pt]), ("qw_gguf_moe_layer", _b, [_vp, _i, _pm, _pi, _pi, _pi, C.c_char_p, _sz]),
     # qw_par.h
     ("qw_par_new", _vp, []), ("qw_par_free", None, [_vp]), ("qw_par_observe", None, [_vp, _i, _d]), ("qw_par_group_cost", _d, [_vp, _i]),
@@ -489,6 +490,36 @@ class Gguf:
         if not self.L.qw_gguf_moe_layer(self.f, layer, C.byref(M), C.byref(D), C.byref(I), C.byref(E), err, len(err)):
             raise ValueError(err.value.decode())
         return M, D.value, I.value, E.value
+
+    def hyper(self, layer, which):
+        """(HyperW, D) of blk.<layer>.hc_attn_* (which 0), hc_ffn_* (1) or the output mixer (2)."""
+        H, D = QwHyperW(), C.c_int()
+        err = C.create_string_buffer(1024)
+        if not self.L.qw_gguf_hyper(self.f, layer, which, C.byref(H), C.byref(D), err, len(err)):
+            raise ValueError(err.value.decode())
+        return HyperW(H), D.value
+
+
+class HyperW:
+    """A QwHyperW filled by the GGUF reader, in the form Path.hyper_gg takes."""
+
+    def __init__(self, c):
+        self.c = c
+
+    def get(self, name):
+        t = getattr(self.c, name)
+        return _Fixed(t) if t.buf else None
+
+    def __getitem__(self, name):
+        return self.get(name)
+
+
+class _Fixed:
+    def __init__(self, t):
+        self.t = t
+
+    def c(self):
+        return self.t
 
 
 class Par:

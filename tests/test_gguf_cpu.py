@@ -89,12 +89,13 @@ def test_names_parts_and_kinds(tmp_path):
         "blk.0.attn_qkv.weight": ("lin", lay % 0 + "linear_attn.in_proj_qkv.weight", "lin"),
         "blk.0.ssm_out.weight": ("lin", lay % 0 + "linear_attn.out_proj.weight", "lin"),
         "blk.10.ffn_down_shexp.weight": ("shared", lay % 10 + "mlp.shared_expert.down_proj.weight", "lin"),
+        "blk.3.hc_ffn_norm.weight": ("hyper", lay % 3 + "mlp_hyper_connection.hc_norm.weight", "f32"),
     }
     for name, (part, model, kind) in want.items():
         t = g.find(name)
         assert (t.part, t.model.decode(), t.kind) == (PARTS[part], model, KIND[kind]), name
         assert g.find(model).name.decode() == name  # found by the model-side name too
-    for name in ("some.other.tensor", "blk.3.hc_ffn_norm.weight", "per_layer_token_embd.weight"):  # not part of this path
+    for name in ("some.other.tensor", "per_layer_token_embd.weight"):  # not part of this path
         t = g.find(name)
         assert t.part == 0 and t.model == b""
     g.close()

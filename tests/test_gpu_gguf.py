@@ -288,3 +288,54 @@ def test_float_matrix_other_than_bf16_is_refused(gpu, tmp_path):
         g.load(gpu, "router")
     assert "floating point" in str(e.value)
     g.close()
+
+
+def test_hyper_connections_from_files(gpu, oracle, tmp_path):
+    """The hyper-connection tensors of a layer and the output mixer (src/gguf.c:222-229, :250-252) made resident and run: the
+    same bits as the same weights handed over directly; inject rows given as F32 in the file become BF16 when exact."""
+    rng = np.random.default_rng(90)
+    d, layer, HC, LR = 2048, 3, 4, 320
+    w = synth.hyper_weights(rng, d)
+    mixer = synth.hyper_weights(rng, d, inject=False)
+    inj32 = (w["inject"].astype(np.uint32) << 16).view(np.float32)  # F32 in the file, exact in BF16
+    p = "blk.%d.hc_ffn_" % layer
+    tensors = [(p + "norm.weight", 0, [HC * d], w["hc_norm"]), (p + "down.weight", 30, [HC * d, LR], w["mix_down"]), (p + "up.weight", 30, [LR, HC * d], w["mix_up"]),
+               (p + "inject.weight", 0, [HC * d, HC], inj32), ("output_hc_norm.weight", 0, [HC * d], mixer["hc_norm"]),
+               ("output_hc_down.weight", 30, [HC * d, LR], mixer["mix_down"]), ("output_hc_up.weight", 30, [LR, HC * d], mixer["mix_up"])]
+    gw.write_gguf(str(tmp_path / "hc.gguf"), tensors)
+    g = q.Gguf(str(tmp_path))
+    g.load(gpu, "hyper")
+    H, dd = g.hyper(layer, 1)
+    Hm, dm = g.hyper(0, 2)
+    assert dd == d and dm == d and H["inject"] is not None and Hm["inject"] is None
+    with pytest.raises(ValueError):
+        g.hyper(layer, 0)  # this file has no hc_attn_* tensors
+    path = q.Path(gpu, d, 512, 64, 4, 16)
+    nb = 6
+    h, out, inj = synth.hyper_state(rng, nb, d)
+    pd = gpu.buf(int(gpu.L.qw_path_hyper_pd_bytes(nb)))
+
+    def run(Hw, want_inj):
+        hb, ob, ib, io, x = gpu.buf_from(h), gpu.buf_from(out), gpu.buf_from(inj), gpu.buf_from(np.zeros((nb, HC, HC), np.float32)), gpu.buf(nb * d * 2)
+        b = gpu.batch()
+        path.hyper_gg(b, Hw, nb, 1, hb, ob, ib, io, pd, x)
+        b.end()
+        res = (hb.view(np.float32).copy(), x.view(np.float16).copy(), io.view(np.float32).copy())
+        for bb in (hb, ob, ib, io, x):
+            bb.free()
+        return res
+
+    for Hw, host in ((H, w), (Hm, mixer)):
+        bufs = {k: gpu.buf_from(v) for k, v in host.items() if v is not None}
+        direct = {"hc_norm": q.Tensor(bufs["hc_norm"], 0), "mix_down": q.Tensor(bufs["mix_down"], 30), "mix_up": q.Tensor(bufs["mix_up"], 30),
+                  "inject": q.Tensor(bufs["inject"], 30) if "inject" in bufs else None}
+        a, b2 = run(Hw, host["inject"] is not None), run(direct, host["inject"] is not None)
+        for u, v in zip(a, b2):
+            assert np.array_equal(u.view(np.uint8), v.view(np.uint8))
+        rh, rx, ri = oracle.hyper_gg(h, out, inj, host["hc_norm"], host["mix_down"], host["inject"], host["mix_up"], 1)
+        assert np.abs(a[1].reshape(nb, d).astype(np.float64) - rx).max() / np.abs(rx).max() <= 1e-3
+        for bb in bufs.values():
+            bb.free()
+    pd.free()
+    path.close()
+    g.close()
