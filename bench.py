@@ -482,6 +482,7 @@ def main():
     ap.add_argument("--dense-only", action="store_true", help="only the dense matvec tables (configs 1-2 and the other formats): for profiling runs")
     ap.add_argument("--gguf-only", action="store_true", help="only the GGUF load measurement")
     ap.add_argument("--model-shape-only", action="store_true", help="only the stack of the reference model's layer shape and formats")
+    ap.add_argument("--release-source", action="store_true", help="after the first step keep only the tile-major copies of the routed experts (frees their GGUF-order bytes); implies --no-cpu --quick")
     ap.add_argument("--hyper-only", action="store_true", help="only the hyper-connection -> MoE layer loop")
     ap.add_argument("--ragged-only", action="store_true", help="only the continuous-batching step table (config 4) on a one-layer stack: for profiling runs")
     a = ap.parse_args()
@@ -521,6 +522,11 @@ def main():
 
     if a.copy_calib:
         copy_calibration(gpu)
+    released = None
+    if a.release_source:  # the oracle leg reads the weights back from HBM, so it cannot follow
+        a.no_cpu = a.quick = True
+        stack.step(x, 16)
+        released = stack.release_sources()
     res = {}
     for nb in ([a.nb] if a.quick else sorted({1, 8, a.nb})):
         wall, gpu_s = timed_steps(stack, x, nb, a.steps, a.warmup)
@@ -550,9 +556,9 @@ def main():
             "vs_baseline": None, "dtype": "u8 blocks -> f16 matrix-core operands, f32 accumulate", "data": "synthetic (seeded, generated on device)",
             "config": {"workload": "configs[4]: %d-layer MoE FFN stack decode, B=%d, D=2048 I=512 E=512 top-10, IQ3_S experts, shared expert Q8_0 every 4th layer; "
                                    "every layer reads the same x and overwrites one out, launched in order on one stream (a bandwidth bench: no overlap between layers is used)" % (stack.L, nb),
-                       "resident_weight_bytes": int(stack.weight_bytes), "packed_copy_bytes": int(gpu.L.qw_hip_packed_bytes(gpu.g)), "device": gpu.name()},
+                       "resident_weight_bytes": int(stack.weight_bytes), "packed_copy_bytes": int(gpu.L.qw_hip_packed_bytes(gpu.g)), "released_source_bytes": released, "device": gpu.name()},
             "roofline": roof,
-            "read_ceiling": read_ceiling(gpu, stack, nb),
+            "read_ceiling": None if released else read_ceiling(gpu, stack, nb),  # it reads the GGUF-order bytes
             "stack": {"GBps_algorithmic": res[nb]["stack_GBps"], "frac_of_peak": res[nb]["stack_GBps"] / HBM_PEAK_GBS, "gpu_ms_per_step": res[nb]["gpu_ms_per_step"],
                       "mean_unique_experts": res[nb]["mean_U"], "bytes_per_step": res[nb]["bytes_per_step"]},
             "by_batch": {str(k): v for k, v in res.items()},

@@ -92,6 +92,12 @@ bool qw_gguf_tensor_at(const qw_gguf *f, const qw_gguf_tensor *t, qw_tensor *out
 /* The MoE weights of one layer (blk.<layer>.ffn_*), checked against each other; D, I, E receive the layer's sizes. */
 bool qw_gguf_moe_layer(const qw_gguf *f, int layer, qw_moe_layer *M, int *D, int *I, int *E, char *err, size_t errlen);
 
+/* Keep only the tile-major copies of the routed experts: frees the GGUF-order bytes of this handle's arena
+ * (qw_hip_buf_release_source, include/qw_hip_ext.h) once every layer's experts have been dispatched at least once. Only
+ * for a handle that loaded the routed expert matrices alone (parts = QW_GG_MOE): the other tensors are read as they are,
+ * so they belong to a second handle on the same directory. */
+bool qw_gguf_release_source(qw_gguf *f, char *err, size_t errlen);
+
 /* The weights of one hyper-connection (src/gguf.c:222-229, :250-252): which = 0 blk.<layer>.hc_attn_*, 1 blk.<layer>.hc_ffn_*,
  * 2 the output mixer (no inject rows; H->inject.buf stays NULL); D receives the width of a stream. The inject rows must be
  * exact in BF16 (they are converted as a small tensor), as the reference's kernel reads them as BF16. */

@@ -48,6 +48,16 @@ void *qw_hip_buf_devptr(const qw_buf *b);
  * environment, or qw_hip_set_repack(g, false), turns the copies off (kernels then read the GGUF rows directly). */
 void qw_hip_set_repack(qw_gpu *g, bool on);
 size_t qw_hip_packed_bytes(const qw_gpu *g);
+/* Keep only the tile-major copies of a weight buffer: frees the buffer's device bytes (the GGUF-order rows) once the
+ * copies that the kernels read have been made, i.e. after every matrix in it has been through a dispatch that makes one
+ * (moe_gu_gg, moe_dn_gg, moe_pf_gg and qmv_gg over IQ3_S rows; moe_dn_gg over IQ4_NL rows of 320 or 640). Residency of
+ * such a matrix drops from 2.018 to 1.018 times its bytes. Afterwards the buffer may only be bound as those weights:
+ * a dispatch that no existing copy serves (another shape or split, a matrix that was never dispatched, dq_test, any output
+ * role) fails the batch with a message, the explicit copy calls return false, qw_hip_buf_devptr gives NULL, and the
+ * buffer is otherwise freed as usual. Returns false (and frees nothing) when the buffer has no copy yet or is written by
+ * a batch still in flight. Keep shared-expert and router tensors in buffers of their own: they are read in GGUF order. */
+bool qw_hip_buf_release_source(qw_buf *b);
+size_t qw_hip_released_bytes(const qw_gpu *g);
 
 /* Optional: a batch whose launches (functions, grids, argument records) equal those of one of the last few batches —
  * a decode step over the same resident buffers — is instantiated as a HIP graph of kernel nodes and replayed from

@@ -66,6 +66,7 @@ typedef struct qw_hbuf {
     uint64_t out_seq; // the last batch that counted itself in pending_out
     struct qw_gpu *g;
     int npack;       // packed copies made from this buffer (dropped when its contents change)
+    bool released;   // the device bytes were freed (qw_hip_buf_release_source): dptr is only the key of its tile-major copies
 } qw_hbuf;
 
 // A tile-major copy of IQ3_S weight rows (layout: qwk_pack_args), made at the first use of a weight matrix.
@@ -105,6 +106,7 @@ struct qw_batch {
     qw_use *use;
     int nuse, capuse, done_use;
     bool noalloc;      // the device's static recorder (qw_hip_batch_begin_static): fixed storage, no tile-major copies made
+    bool allow_released; // set by a translator while it binds weights that a tile-major copy may stand in for
     hipStream_t xstream; // noalloc: the caller's stream (NULL: the device's)
     uint64_t seq;      // this batch's number (qw_hbuf.out_seq)
     qw_hbuf **outs;    // buffers whose pending_out this batch raised
@@ -173,7 +175,7 @@ struct qw_gpu {
     bool na_busy;
     float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
-    size_t pack_bytes;
+    size_t pack_bytes, released_bytes;
 };
 
 static void set_err(qw_gpu *g, const char *fmt, ...) {
@@ -621,7 +623,7 @@ void qw_buf_free(qw_buf *b) {
     if (!b || !b->handle) return;
     qw_hbuf *h = b->handle;
     packs_drop(h);
-    (void)hipFree(h->dptr);
+    if (!h->released) (void)hipFree(h->dptr);
     if (h->own_host) {
         if (h->pinned) (void)hipHostFree(h->host);
         else free(h->host);
@@ -636,7 +638,7 @@ void *qw_pool_push(void) { return NULL; }
 void qw_pool_pop(void *pool) { (void)pool; }
 
 void qw_hip_buf_mark_dirty(qw_buf *b) {
-    if (!b || !b->handle) return;
+    if (!b || !b->handle || ((qw_hbuf *)b->handle)->released) return; // a released buffer has nothing to refresh
     ((qw_hbuf *)b->handle)->dirty = true;
     packs_drop(b->handle);
 }
@@ -644,10 +646,23 @@ void qw_hip_set_repack(qw_gpu *g, bool on) { g->repack = on; }
 unsigned qw_hip_graph_launches(const qw_gpu *g) { return g->ngraph_launches; }
 void qw_hip_set_graphs(qw_gpu *g, bool on) { g->use_graphs = on; }
 size_t qw_hip_packed_bytes(const qw_gpu *g) { return g->pack_bytes; }
-void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle ? ((qw_hbuf *)b->handle)->dptr : NULL; }
-static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return off <= h->size && len <= h->size - off; }
+void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle && !((qw_hbuf *)b->handle)->released ? ((qw_hbuf *)b->handle)->dptr : NULL; }
+static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return !h->released && off <= h->size && len <= h->size - off; } // a released buffer has no bytes to copy
+// Free the device bytes of a weight buffer and keep its tile-major copies (include/qw_hip_ext.h).
+bool qw_hip_buf_release_source(qw_buf *b) {
+    qw_hbuf *h = b ? b->handle : NULL;
+    if (!h || h->released || !h->npack || h->pending_out) return false;
+    if (hipDeviceSynchronize() != hipSuccess) return false; // a batch in flight may still read the bytes
+    if (hipFree(h->dptr) != hipSuccess) { (void)hipGetLastError(); return false; }
+    h->released = true; // dptr stays as the key the copies were filed under; nothing dereferences it from here on
+    h->dirty = false;
+    h->g->released_bytes += h->size;
+    return true;
+}
+size_t qw_hip_released_bytes(const qw_gpu *g) { return g->released_bytes; }
 bool qw_hip_buf_upload(qw_buf *b, size_t off, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
+    if (h && h->released) return false;
     packs_drop(h);
     return h && h->host && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, (char *)h->host + off, len, hipMemcpyHostToDevice) == hipSuccess;
 }
@@ -657,6 +672,7 @@ bool qw_hip_buf_download(qw_buf *b, size_t off, size_t len) {
 }
 bool qw_hip_buf_write(qw_buf *b, size_t off, const void *src, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
+    if (h && h->released) return false;
     packs_drop(h);
     return h && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
 }
@@ -807,6 +823,8 @@ static bool bind_ptr(qw_batch *b, unsigned index, size_t need, bool out, const c
     const size_t off = b->buf[index].off;
     if (off > h->size || need > h->size - off) return fail(b, "%s: %s at index %u needs %zu bytes after offset %zu, buffer has %zu", b->k->name, what, index, need, off, h->size);
     if (out && h->wrapped) return fail(b, "%s: %s at index %u is a wrapped (read-only) buffer", b->k->name, what, index);
+    if (h->released && (out || !b->allow_released))
+        return fail(b, "%s: %s at index %u: the buffer's GGUF-order bytes were released (qw_hip_buf_release_source); only dispatches that a tile-major copy serves may bind it", b->k->name, what, index);
     if (out) packs_drop(h); // a kernel is about to write it
     *p = (char *)h->dptr + off;
     if (b->nuse == b->capuse) {
@@ -966,8 +984,10 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
     if (a.xstride < a.K || a.xstride % 8 || a.ystride < a.N) return fail(b, "qmv_gg: xstride %u (needs >= K, multiple of 8) / ystride %u (needs >= N)", a.xstride, a.ystride);
     if (b->buf[3].h && b->buf[3].off % 16) return fail(b, "qmv_gg: x offset %zu is not 16-byte aligned", b->buf[3].off);
     a.ntiles = cdiv(a.N, 16);
-    if (!bind_ptr(b, 0, (size_t)a.N * a.rowbytes, false, "W", (void **)&a.W) ||
-        !bind_ptr(b, 3, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x) ||
+    b->allow_released = true; // W may be a buffer of which only the tile-major copy is left
+    const bool bound = bind_ptr(b, 0, (size_t)a.N * a.rowbytes, false, "W", (void **)&a.W);
+    b->allow_released = false;
+    if (!bound || !bind_ptr(b, 3, ((size_t)(a.nb - 1) * a.xstride + a.K) * 2, false, "x", (void **)&a.x) ||
         !bind_ptr(b, 4, ((size_t)(a.nb - 1) * a.ystride + a.N) * (a.yfloat ? 4 : 2), true, "y", &a.y)) return false;
     char fn[48];
     int F = p->F;
@@ -976,6 +996,7 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
         const uint8_t *pk = get_pack(b, b->buf[0].h, a.W, NULL, NULL, a.N / 16, nblk, a.rowbytes, 16);
         if (pk) F = QW_F_PACKED, a.W = pk, a.rowbytes = nblk * QW_SLAB_BYTES;
     }
+    if (b->buf[0].h->released && F != QW_F_PACKED) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     if (p->valu) { // the VALU GEMV, for measurement against the matrix-core form
         if (F != QW_F_PACKED || p->K % 512 || p->NB > 4) return fail(b, "qmv_gg: the VALU form needs packed IQ3_S weights, K a multiple of 512 and NB <= 4");
         fname_fmt(fn, sizeof fn, "qwk_qmv_valu_n%d", p->NB <= 1 ? 1 : p->NB <= 2 ? 2 : 4);
@@ -1031,9 +1052,14 @@ static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf 
     if (!g->repack) return NULL;
     for (int i = 0; i < g->npacks; i++) {
         const qw_pack *p = &g->packs[i];
-        if (p->A == A && p->B == B && p->ntiles == ntiles && p->nblk == nblk && p->split == split) return p->dst;
+        if (p->A != A || p->B != B || p->ntiles != ntiles || p->nblk != nblk || p->split != split) continue;
+        // The addresses are the key (a view of the same memory under another handle finds the copy too) — unless the
+        // source was released: its address may since have been given to another allocation, so only its own handle matches.
+        const bool gone = (p->ha && p->ha->released) || (p->hb && p->hb->released);
+        if (!gone || (p->ha == ha && p->hb == hb)) return p->dst;
     }
     if (b->noalloc) return NULL; // a copy that exists was found above; none is made here
+    if ((ha && ha->released) || (hb && hb->released)) return NULL; // nothing left to copy from
     qw_hbuf *hs[2] = {ha, hb};
     for (int i = 0; i < 2; i++) {
         qw_hbuf *h = hs[i];
@@ -1081,8 +1107,10 @@ static bool fill_gu(qw_batch *b, qwk_gu_args *a, int F, unsigned iWg, unsigned i
     const size_t rb = fmt_rb(F, p->D), ne = shared ? 1 : (size_t)p->E;
     *a = (qwk_gu_args){.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = shared,
                        .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I, .glut = glut(b->g)};
-    if (!bind_ptr(b, iWg, ne * p->I * rb, false, "gate weights", (void **)&a->Wg) || !bind_ptr(b, iWu, ne * p->I * rb, false, "up weights", (void **)&a->Wu) ||
-        !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a->x) || !bind_ptr(b, iH, (size_t)a->hplane * 4, true, "H", (void **)&a->H)) return false;
+    b->allow_released = !shared; // the routed matrices may be buffers of which only the tile-major copy is left (the caller checks that one serves)
+    const bool bound = bind_ptr(b, iWg, ne * p->I * rb, false, "gate weights", (void **)&a->Wg) && bind_ptr(b, iWu, ne * p->I * rb, false, "up weights", (void **)&a->Wu);
+    b->allow_released = false;
+    if (!bound || !bind_ptr(b, ix, (size_t)nbr * p->D * 2, false, "x", (void **)&a->x) || !bind_ptr(b, iH, (size_t)a->hplane * 4, true, "H", (void **)&a->H)) return false;
     if (b->buf[ix].off % 16) return fail(b, "%s: x offset %zu is not 16-byte aligned", b->k->name, b->buf[ix].off);
     return true;
 }
@@ -1240,6 +1268,7 @@ static bool tr_gu(qw_batch *b) {
             if (fs == 21) fs = QW_F_PACKED, a.Wsg = ps, a.Wsu = NULL, a.sg_rowbytes = tileb;
         }
     }
+    if ((b->buf[0].h->released || b->buf[1].h->released) && fgu != QW_F_PACKED) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     char fn[64];
     if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", fgu, cg, fs, cs);
     else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", fgu, cg);
@@ -1267,7 +1296,11 @@ static bool tr_dn(qw_batch *b) {
     const size_t rb = fmt_rb(p->fd, p->I);
     qwk_dn_args a = {.D = (uint32_t)p->D, .I = (uint32_t)p->I, .rowbytes = (uint32_t)rb, .nbr = nbr, .topk = (uint32_t)p->topk, .gnb = (uint32_t)p->gnb, .shared = 0,
                      .hplane = (uint32_t)p->NB * (uint32_t)(p->topk + 1) * (uint32_t)p->I, .glut = glut(b->g)};
-    if (!bind_ptr(b, 0, (size_t)p->E * p->D * rb, false, "down weights", (void **)&a.Wd) || !bind_ptr(b, 2, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
+    b->allow_released = true; // Wd may be a buffer of which only the tile-major copy is left
+    const bool bound = bind_ptr(b, 0, (size_t)p->E * p->D * rb, false, "down weights", (void **)&a.Wd);
+    b->allow_released = false;
+    const bool rel = bound && b->buf[0].h->released;
+    if (!bound || !bind_ptr(b, 2, (size_t)a.hplane * 4, false, "H", (void **)&a.H) ||
         !bind_ptr(b, 9, (size_t)nbr * p->topk * p->D * 4, true, "Pg", (void **)&a.P) ||
         !bind_ptr(b, 3, QW_SEL_BYTES((size_t)p->gnb, (size_t)p->topk), false, "selection", (void **)&a.sel)) return false;
     int fs = 0;
@@ -1293,6 +1326,7 @@ static bool tr_dn(qw_batch *b) {
             if (fs == 21) fs = QW_F_PACKED, a.Wsd = ps, a.sd_rowbytes = tileb;
         }
     }
+    if (rel && fd != QW_F_PACKED && fd != 20) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
     // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
@@ -1320,6 +1354,7 @@ static bool tr_dn(qw_batch *b) {
                 return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
             }
         }
+        if (rel) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
         const int ch = p->I % 320 == 0 && !b->sw.nl_c4 ? 10 : 4; // blocks per chunk
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d_s%d_c%d", ch, fs, fs == 20 ? ch : 4);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f20_c%d", ch);
@@ -1345,6 +1380,7 @@ static bool tr_dn(qw_batch *b) {
     }
     // wider rows: one tile at a time, operand A from global memory
     fname_fmt(fn, sizeof fn, "qwk_dn_f%d_any%s", p->fd, sfx);
+    if (rel && fd != QW_F_PACKED) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     return add_launch(b, intern(fn), persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DN), 64 * QW_WAVES_DN, &a, sizeof a);
 }
 
@@ -1447,6 +1483,7 @@ static bool launch_pf(qw_batch *b, qwk_pf_args *a, int F, int E, qw_hbuf *hw, qw
         }
         if (wb) return false; // the caller launches the two matrices one by one
     }
+    if (hw && hw->released) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     if (F == 21) fname_fmt(fn, sizeof fn, "qwk_pf_f21_c%d", a->K % 512 == 0 ? 2 : 1);
     else fname_fmt(fn, sizeof fn, "qwk_pf_f%d_c4", F == 20 ? 20 : 8);
     // every entry can hold a tile: the grid covers the whole table, the kernel counts the entries in use
@@ -1467,7 +1504,10 @@ static bool tr_pf(qw_batch *b, unsigned gy) {
     if (gy > 2048) return fail(b, "moe_pf_gg: %u tile entries, this build takes at most 2048", gy);
     const size_t rb = fmt_rb(p->F, p->K);
     qwk_pf_args a = {.M = mn[0], .N = mn[1], .K = (uint32_t)p->K, .rowbytes = (uint32_t)rb, .max_tiles = gy, .tm = (uint32_t)p->tm, .glut = glut(b->g)};
-    if (!bind_ptr(b, 0, (size_t)a.M * p->K * 2, false, "X", (void **)&a.X) || !bind_ptr(b, 1, (size_t)p->E * a.N * rb, false, "weights", (void **)&a.W) ||
+    b->allow_released = true; // the weights may be a buffer of which only the tile-major copy is left (launch_pf checks that one serves)
+    const bool bound = bind_ptr(b, 1, (size_t)p->E * a.N * rb, false, "weights", (void **)&a.W);
+    b->allow_released = false;
+    if (!bound || !bind_ptr(b, 0, (size_t)a.M * p->K * 2, false, "X", (void **)&a.X) ||
         !bind_ptr(b, 4, (size_t)a.M * a.N * 2, true, "Y", (void **)&a.Y) || !bind_ptr(b, 6, (size_t)gy * 16, false, "tiles", (void **)&a.tiles)) return false;
     if (b->buf[0].off % 16 || b->buf[6].off % 16) return fail(b, "moe_pf_gg: X and the tile table must be 16-byte aligned");
     qw_hbuf *hw = b->buf[1].h, *hx = b->buf[0].h, *hy = b->buf[4].h;
@@ -1593,6 +1633,7 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     (void)gz; (void)tx; (void)ty; (void)tz;
     if (b->failed) return;
     if (!b->k) { fail(b, "qw_batch_dispatch without a kernel"); return; }
+    b->allow_released = false;
     const int first = b->nl;
     bool ok;
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
@@ -1718,6 +1759,7 @@ static bool submit_segment(qw_batch *b) {
         if (h->device_only || !h->host) continue;
         // A kernel of a batch that was submitted (or of an earlier segment of this one) and not yet waited for wrote
         // this buffer: HBM holds the newer contents, and the shadow must not overwrite them.
+        if (h->released) continue; // no device bytes: its tile-major copies are what the kernels read
         if (h->pending_out > 0 && !h->dirty) continue;
         if (h->dirty || (!h->wrapped && h->size <= QW_HIP_SMALL_BYTES)) {
             if (!HIPOK(g, hipMemcpyAsync(h->dptr, h->host, h->size, hipMemcpyHostToDevice, st))) { b->failed = true; return false; }

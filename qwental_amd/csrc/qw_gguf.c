@@ -34,6 +34,7 @@ struct qw_gguf {
     // residency
     qw_gpu *g;
     qw_buf arena;
+    bool only_experts; // the arena holds routed expert matrices and nothing else (qw_gguf_release_source)
     bool loaded;
     uint64_t *dev_off; // per tensor; valid when res_type >= 0
     size_t resident;
@@ -469,6 +470,9 @@ bool qw_gguf_load(qw_gguf *G, qw_gpu *g, unsigned parts, char *err, size_t errle
         nsel++;
     }
     if (!nsel) return fail(err, errlen, "GGUF: no tensor of parts 0x%x", parts);
+    G->only_experts = true;
+    for (int i = 0; i < G->nt; i++)
+        if (G->t[i].part && (G->t[i].part & parts) && G->t[i].kind != QW_GK_EXP) G->only_experts = false;
     if (!qw_hip_buf_new_device(g, (size_t)total, &G->arena)) return fail(err, errlen, "GGUF: cannot allocate %llu bytes of device memory: %s", (unsigned long long)total, qw_hip_last_error(g));
     G->g = g;
     G->loaded = true;
@@ -584,5 +588,14 @@ bool qw_gguf_hyper(const qw_gguf *G, int layer, int which, qw_hyper_w *H, int *D
         return fail(err, errlen, "GGUF: hyper-connection tensors must be resident as F32 norm and BF16 matrices (got %s, %s, %s, %s)", qw_ggml_name(H->hc_norm.type),
                     qw_ggml_name(H->mix_down.type), qw_ggml_name(H->mix_up.type), t[3] ? qw_ggml_name(H->inject.type) : "-");
     *D = (int)(hcd / QW_PATH_HC);
+    return true;
+}
+
+// Keep only the tile-major copies of the routed experts of this handle (qw_hip_buf_release_source on its arena).
+bool qw_gguf_release_source(qw_gguf *G, char *err, size_t errlen) {
+    if (err && errlen) err[0] = 0;
+    if (!G->loaded) return fail(err, errlen, "GGUF: nothing is resident");
+    if (!G->only_experts) return fail(err, errlen, "GGUF: this handle's arena also holds tensors that are read as they are; load the routed experts (part moe) through a handle of their own");
+    if (!qw_hip_buf_release_source(&G->arena)) return fail(err, errlen, "GGUF: no tile-major copy has been made from the arena yet (run every layer once), or a batch that writes it is in flight");
     return true;
 }

@@ -71,7 +71,7 @@ SYMBOLS = [
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
     ("qw_hip_buf_write_fd", _b, [_pb, _sz, _i, C.c_uint64, _sz]),
     ("qw_hip_set_repack", None, [_vp, _b]), ("qw_hip_graph_launches", C.c_uint, [_vp]), ("qw_hip_set_graphs", None, [_vp, _b]),
-    ("qw_hip_packed_bytes", _sz, [_vp]),
+    ("qw_hip_packed_bytes", _sz, [_vp]), ("qw_hip_buf_release_source", _b, [_pb]), ("qw_hip_released_bytes", _sz, [_vp]),
     ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
     ("qw_hip_last_error", C.c_char_p, [_vp]), ("qw_hip_cu_count", _i, [_vp]), ("qw_hip_arch", C.c_char_p, []),
     ("qw_hip_profile_mean", _d, [_vp, C.c_char_p, C.POINTER(_i)]),
@@ -100,6 +100,7 @@ SYMBOLS = [
     ("qw_gguf_shard_data_start", C.c_uint64, [_vp, _i]), ("qw_gguf_count", _i, [_vp]), ("qw_gguf_get", _pg, [_vp, _i]),
     ("qw_gguf_find", _pg, [_vp, C.c_char_p]), ("qw_gguf_host", _vp, [_vp, _pg]),
     ("qw_gguf_load", _b, [_vp, _vp, _u, C.c_char_p, _sz]), ("qw_gguf_resident_bytes", _sz, [_vp]), ("qw_gguf_load_seconds", _d, [_vp]),
+    ("qw_gguf_release_source", _b, [_vp, C.c_char_p, _sz]),
     ("qw_gguf_hyper", _b, [_vp, _i, _i, C.POINTER(QwHyperW), _pi, C.c_char_p, _sz]),
     ("qw_gguf_tensor_at", _b, [_vp, _pg, _pt]), ("qw_gguf_moe_layer", _b, [_vp, _i, _pm, _pi, _pi, _pi, C.c_char_p, _sz]),
     # qw_par.h
@@ -490,6 +491,11 @@ class Gguf:
         if not self.L.qw_gguf_moe_layer(self.f, layer, C.byref(M), C.byref(D), C.byref(I), C.byref(E), err, len(err)):
             raise ValueError(err.value.decode())
         return M, D.value, I.value, E.value
+
+    def release_source(self):
+        err = C.create_string_buffer(1024)
+        if not self.L.qw_gguf_release_source(self.f, err, len(err)):
+            raise ValueError(err.value.decode())
 
     def hyper(self, layer, which):
         """(HyperW, D) of blk.<layer>.hc_attn_* (which 0), hc_ffn_* (1) or the output mixer (2)."""

@@ -110,6 +110,16 @@ class MoeStack:
                                   self.lg_c, self.sel_c, self.out)
         return b.end()
 
+    def release_sources(self):
+        """Keep only the tile-major copies of the routed experts' matrices (made by the first step): frees the GGUF-order
+        bytes of every layer's routed weights. Returns the bytes freed. The weights can no longer be read back."""
+        before = self.gpu.L.qw_hip_released_bytes(self.gpu.g)
+        for l in range(self.L):
+            w = self.bufs[3 * l]
+            if not self.gpu.L.qw_hip_buf_release_source(w.ref()):
+                raise RuntimeError("layer %d: no tile-major copy to keep (run a step first)" % l)
+        return int(self.gpu.L.qw_hip_released_bytes(self.gpu.g) - before)
+
     def shared_bytes(self, l):
         f = self.shared_fmt[l]
         return self.I * (synth.row_bytes(f[0], self.D) + synth.row_bytes(f[1], self.D)) + self.D * synth.row_bytes(f[2], self.I)

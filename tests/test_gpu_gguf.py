@@ -339,3 +339,35 @@ def test_hyper_connections_from_files(gpu, oracle, tmp_path):
     pd.free()
     path.close()
     g.close()
+
+
+def test_expert_arena_released_after_first_use(gpu, oracle, model):
+    """Two handles on one directory: the routed experts in an arena of their own, everything else in another. After every
+    layer ran once the experts' GGUF-order bytes are freed; the layer computes the same bits from the tile-major copies."""
+    tmp, m, _, _ = model
+    ge, gr = q.Gguf(tmp), q.Gguf(tmp)
+    ge.load(gpu, "moe")
+    gr.load(gpu, "shared,router")
+    with pytest.raises(ValueError):
+        gr.release_source()  # holds tensors that are read as they are
+    with pytest.raises(ValueError):
+        ge.release_source()  # no copy made yet
+    # the layer's struct: routed matrices from the experts' handle, the rest from the other
+    from qwental_amd.gpu import QwMoeLayer, QwTensor
+    M = QwMoeLayer()
+    for name, src, key in (("gate", ge, "ffn_gate_exps"), ("up", ge, "ffn_up_exps"), ("down", ge, "ffn_down_exps"), ("router", gr, "ffn_gate_inp"),
+                           ("sh_gate_w", gr, "ffn_gate_inp_shexp"), ("sh_gate", gr, "ffn_gate_shexp"), ("sh_up", gr, "ffn_up_shexp"), ("sh_down", gr, "ffn_down_shexp")):
+        setattr(M, name, src.tensor_at(src.find("blk.%d.%s.weight" % (LAYER, key))))
+    path = q.Path(gpu, D, I, E, K, 16)
+    x = synth.activations(np.random.default_rng(80), 16, D)
+    before = {nb: run_moe(gpu, path, _Layer(M), x[:nb], nb)[0] for nb in (16, 2)}
+    resident = ge.resident_bytes()
+    freed0 = gpu.L.qw_hip_released_bytes(gpu.g)
+    ge.release_source()
+    assert gpu.L.qw_hip_released_bytes(gpu.g) - freed0 >= resident
+    for nb in (16, 2):
+        out = run_moe(gpu, path, _Layer(M), x[:nb], nb)[0]
+        assert np.array_equal(out.view(np.uint16), before[nb].view(np.uint16))
+    path.close()
+    ge.close()
+    gr.close()
