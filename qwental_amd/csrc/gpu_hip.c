@@ -921,10 +921,19 @@ static unsigned pick_split(unsigned chunks, unsigned tiles, unsigned slots) {
         if (chunks % s == 0 && tiles * s <= slots) return s;
     return 1;
 }
-static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a) {
+// hw: the buffers the matrices lie in (NULL: no tile-major copies are looked for)
+#define QW_Q6_PACK_MIN_ROWS 16384u
+static bool launch_qmvm(qw_batch *b, qwk_qmvm_args *a, qw_hbuf *const *hw) {
     unsigned tiles = 0;
     a->sums = 0;
     for (uint32_t j = 0; j < a->nmat; j++) {
+        // A large Q6_K matrix (the vocabulary projection, src/engine.c:658-704) is read from a tile-major copy made at
+        // its first use: five coalesced loads a block instead of seventeen 4-byte ones and seventeen cross-lane moves.
+        if (hw && a->fmt[j] == 14 && a->K % 256 == 0 && a->N[j] % 16 == 0 && a->N[j] >= QW_Q6_PACK_MIN_ROWS) {
+            const uint32_t nblk = a->K / 256;
+            const uint8_t *pk = get_pack(b, hw[j], a->W[j], NULL, NULL, a->N[j] / 16, nblk, a->rowbytes[j], QW_F_PACKED_Q6);
+            if (pk) a->W[j] = pk, a->fmt[j] = QW_F_PACKED_Q6, a->rowbytes[j] = nblk * QW_Q6_SLAB_BYTES;
+        }
         a->ntiles[j] = cdiv(a->N[j], 16);
         tiles += a->ntiles[j];
         if (a->fmt[j] == 12 || a->fmt[j] == 13) a->sums = 1;
@@ -960,7 +969,8 @@ static bool tr_qmvm(qw_batch *b) { // src/engine.c:752-771: 0..3 W, 4 x, 5..8 y,
             !bind_ptr(b, 5u + (unsigned)j, (size_t)a.nb * a.N[j] * (a.yfloat ? 4 : 2), true, "y", &a.y[j])) return false;
     }
     if (in.total != total) return fail(b, "qmv_ggm: total %u, the matrices have %u rows", in.total, total);
-    return launch_qmvm(b, &a);
+    qw_hbuf *hm[4] = {b->buf[0].h, b->buf[1].h, b->buf[2].h, b->buf[3].h};
+    return launch_qmvm(b, &a, hm);
 }
 
 static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, xstride, ystride, pad}
@@ -976,7 +986,8 @@ static bool tr_qmv(qw_batch *b) { // src/engine.c:717-723: 0 W, 3 x, 4 y, 5 {N, 
         if (!bind_ptr(b, 0, (size_t)m.N[0] * m.rowbytes[0], false, "W", (void **)&m.W[0]) ||
             !bind_ptr(b, 3, ((size_t)(m.nb - 1) * m.xstride + m.K) * 2, false, "x", (void **)&m.x) ||
             !bind_ptr(b, 4, ((size_t)(m.nb - 1) * m.ystride[0] + m.N[0]) * (m.yfloat ? 4 : 2), true, "y", &m.y[0])) return false;
-        return launch_qmvm(b, &m);
+        qw_hbuf *hm[4] = {b->buf[0].h};
+        return launch_qmvm(b, &m, hm);
     }
     qwk_qmv_args a = {.N = a4[0], .K = (uint32_t)p->K, .rowbytes = (uint32_t)p->RB, .xstride = a4[1], .ystride = a4[2], .nb = (uint32_t)p->NB, .yfloat = (uint32_t)p->yfloat,
                       .glut = glut(b->g)};
@@ -1074,10 +1085,10 @@ static const uint8_t *get_pack(qw_batch *b, qw_hbuf *ha, const void *A, qw_hbuf 
             h->dirty = false;
         }
     }
-    const bool nl = split == QW_F_PACKED_NL; // IQ4_NL rows: nblk counts chunks of ten blocks
-    hipFunction_t f = get_func(g, nl ? "qwk_pack_nl" : "qwk_pack_iq3");
+    const bool nl = split == QW_F_PACKED_NL, q6 = split == QW_F_PACKED_Q6; // IQ4_NL rows: nblk counts chunks of ten blocks; Q6_K rows: blocks
+    hipFunction_t f = get_func(g, nl ? "qwk_pack_nl" : q6 ? "qwk_pack_q6" : "qwk_pack_iq3");
     if (!f) return NULL;
-    const size_t bytes = (size_t)ntiles * nblk * (nl ? QW_NL_CHUNK_BYTES : QW_SLAB_BYTES);
+    const size_t bytes = (size_t)ntiles * nblk * (nl ? QW_NL_CHUNK_BYTES : q6 ? QW_Q6_SLAB_BYTES : QW_SLAB_BYTES);
     void *dst;
     if (hipMalloc(&dst, bytes) != hipSuccess) {
         (void)hipGetLastError();
@@ -1161,7 +1172,7 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
             if (m.fmt[j] == 12 || m.fmt[j] == 13) m.sums = 1;
         }
         if (!add_launch(b, "qwk_qmvm_swiglu", umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2)), 64 * QW_WAVES_GU, &m, sizeof m)) return false;
-    } else if (!launch_qmvm(b, &m) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
+    } else if (!launch_qmvm(b, &m, NULL) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
     if (b->sw.side == 1)
         for (int i = first; i < b->nl; i++) b->l[i].side = true;
     return true;

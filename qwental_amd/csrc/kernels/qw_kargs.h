@@ -183,6 +183,13 @@ typedef struct { /* read-pattern ceiling of a decode layer (the reference's kern
  * A wave reads a chunk with three fully coalesced loads plus 20 bytes of scales per lane. */
 #define QW_F_PACKED_NL 120
 #define QW_NL_CHUNK_BYTES 2880u
+/* Tile-major copy of Q6_K rows (format code QW_F_PACKED_Q6; qwk_pack_args with split = QW_F_PACKED_Q6, nblk = blocks a
+ * row): per (tile of 16 rows, block of 256 values) QW_Q6_SLAB_BYTES = 16 x 210 contiguous bytes in the lane order of the
+ * matrix instruction (lane = row & 15 | k-group << 4): [0, 3072) three planes of 16 bytes a lane holding the twelve
+ * dwords of ql and qh that the lane decodes (the r[0..11] of the Q6_K decoder), [3072, 3328) the sixteen int8 scales of
+ * every row (16 bytes a row, read by the row's four lanes), [3328, 3360) d of every row. Exactly the matrix's bytes. */
+#define QW_F_PACKED_Q6 114
+#define QW_Q6_SLAB_BYTES 3360u
 typedef struct {
     const uint8_t *A, *B;
     uint8_t *dst;

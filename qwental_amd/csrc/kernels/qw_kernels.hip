@@ -104,6 +104,27 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) 
     }
 }
 
+// The tile-major copy of Q6_K rows (layout: QW_F_PACKED_Q6 in qw_kargs.h); a wave per (tile, block). The twelve dwords a
+// lane takes are the ones qw_kq<14>::load reads for that lane's row and k-group.
+extern "C" __global__ __launch_bounds__(256) void qwk_pack_q6(qwk_pack_args a) {
+    const uint64_t nslab = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
+    for (uint64_t sl = (uint64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); sl < nslab; sl += step) {
+        const uint64_t tile = sl / a.nblk;
+        const uint8_t *src = a.A + (tile * 16 + n) * a.rowbytes + 210 * (sl % a.nblk);
+        uint8_t *dst = a.dst + sl * QW_Q6_SLAB_BYTES;
+        uint32_t r[12];
+#pragma unroll
+        for (int i = 0; i < 8; i++) r[i] = *(const u1a2 *)(src + 64 * (i >> 2) + 32 * ((i >> 1) & 1) + 16 * (i & 1) + 4 * kg);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[8 + i] = *(const u1a2 *)(src + 128 + 32 * (i >> 1) + 16 * (i & 1) + 4 * kg);
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) *(u4 *)(dst + 1024 * pl + 16 * lane) = u4{r[4 * pl], r[4 * pl + 1], r[4 * pl + 2], r[4 * pl + 3]};
+        *(uint32_t *)(dst + 3072 + 16 * n + 4 * kg) = *(const u1a2 *)(src + 192 + 4 * kg); // the row's four lanes write its sixteen scales
+        if (kg == 0) *(uint16_t *)(dst + 3328 + 2 * n) = *(const uint16_t *)(src + 208);
+    }
+}
+
 // The tile-major copy of IQ4_NL rows (layout: QW_F_PACKED_NL in qw_kargs.h); a wave per (tile, chunk of ten blocks).
 extern "C" __global__ __launch_bounds__(256) void qwk_pack_nl(qwk_pack_args a) {
     const uint64_t nchunk = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
@@ -212,7 +233,10 @@ template <int F, int NB> struct qmvm_tile {
     typedef qw_chunk_kq<F, NB> C;
     const qwk_qmvm_args &a;
     uint32_t j;
+    static constexpr bool TILED = F == QW_F_PACKED_Q6; // a tile-major copy: rowbytes = bytes of a tile, loads in matrix-core lane order
+    __device__ __forceinline__ uint32_t kl() const { return TILED ? qw_lane() : qw_lane() & 3; }
     __device__ __forceinline__ const uint8_t *rowp(uint32_t t) const {
+        if constexpr (TILED) return a.W[j] + (size_t)t * a.rowbytes[j];
         const uint32_t r = 16 * t + (qw_lane() >> 2);
         return a.W[j] + (size_t)(r < a.N[j] ? r : a.N[j] - 1) * a.rowbytes[j];
     }
@@ -234,7 +258,7 @@ template <int F, int NB> __device__ __forceinline__ void qmvm_matrix(const qwk_q
     const qmvm_tile<F, NB> T = {a, j};
     const uint32_t lane = qw_lane(), kg = lane >> 4, cpr = a.K / (C::BLK_K * NB);
     f4 acc = {0, 0, 0, 0};
-    qw_task_pipeline<C>(a.ntiles[j], t0, nw, cpr, NB * C::BLK_B, lane & 3, [&](uint32_t t) { return T.rowp(t); }, [&](uint32_t t, uint32_t ci, const C &c) {
+    qw_task_pipeline<C>(a.ntiles[j], t0, nw, cpr, NB * C::BLK_B, T.kl(), [&](uint32_t t) { return T.rowp(t); }, [&](uint32_t t, uint32_t ci, const C &c) {
         c.mac(tab, af, ci * NB * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         T.store(t, acc);
@@ -253,7 +277,7 @@ template <int F, int NB> __device__ __forceinline__ void qmvm_matrix_split(const
         const uint32_t t = wave / sp < tpg ? g * tpg + wave / sp : a.ntiles[j]; // waves past a whole number of tiles: none
         f4 acc = {0, 0, 0, 0};
         if (t < a.ntiles[j])
-            qw_task_pipeline<C>(1, 0, 1, cpp, NB * C::BLK_B, lane & 3, [&](uint32_t) { return T.rowp(t) + (size_t)part * cpp * NB * C::BLK_B; },
+            qw_task_pipeline<C>(1, 0, 1, cpp, NB * C::BLK_B, T.kl(), [&](uint32_t) { return T.rowp(t) + (size_t)part * cpp * NB * C::BLK_B; },
                                 [&](uint32_t, uint32_t ci, const C &c) { c.mac(tab, af, (part * cpp + ci) * NB * C::BLK_K, kg, acc); });
         red[wave * 64 + lane] = acc;
         __syncthreads();
@@ -369,6 +393,7 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args 
             case 12: qmvm_matrix_split<12, 1>(a, j, L.tab, af, L.red, g0, ng); break;
             case 13: qmvm_matrix_split<13, 1>(a, j, L.tab, af, L.red, g0, ng); break;
             case 14: qmvm_matrix_split<14, 1>(a, j, L.tab, af, L.red, g0, ng); break;
+            case QW_F_PACKED_Q6: qmvm_matrix_split<QW_F_PACKED_Q6, 1>(a, j, L.tab, af, L.red, g0, ng); break;
             case 23: qmvm_matrix_split<23, 1>(a, j, L.tab, af, L.red, g0, ng); break;
             case 20: qmvm_matrix_split<20, 8>(a, j, L.tab, af, L.red, g0, ng); break;
             case 1: qmvm_matrix_split<1, 8>(a, j, L.tab, af, L.red, g0, ng); break;
@@ -382,6 +407,7 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args 
         case 12: qmvm_matrix<12, 1>(a, j, L.tab, af, t0, nw); break;
         case 13: qmvm_matrix<13, 1>(a, j, L.tab, af, t0, nw); break;
         case 14: qmvm_matrix<14, 1>(a, j, L.tab, af, t0, nw); break;
+        case QW_F_PACKED_Q6: qmvm_matrix<QW_F_PACKED_Q6, 1>(a, j, L.tab, af, t0, nw); break;
         case 23: qmvm_matrix<23, 1>(a, j, L.tab, af, t0, nw); break;
         case 20: k256 ? qmvm_matrix<20, 8>(a, j, L.tab, af, t0, nw) : qmvm_matrix<20, 1>(a, j, L.tab, af, t0, nw); break;
         case 1: k256 ? qmvm_matrix<1, 8>(a, j, L.tab, af, t0, nw) : qmvm_matrix<1, 1>(a, j, L.tab, af, t0, nw); break;

@@ -455,3 +455,32 @@ template <int F, int NB> struct qw_chunk_kq {
         for (int i = 0; i < NB; i++) qw_kq_block<F>(b[i], tab, af, k0 + BLK_K * i, kg, acc);
     }
 };
+
+// The tile-major copy of Q6_K rows (QW_F_PACKED_Q6 in qw_kargs.h): the decoder's seventeen dwords arrive in matrix-core
+// lane order by five coalesced loads a block (three of 16 bytes a lane, the row's scales, its d), and nothing moves
+// between lanes. p is the wave-uniform address of the chunk's first slab, the second argument the lane. The arithmetic
+// is qw_kq<14>'s, so the results are those of the GGUF rows bit for bit.
+template <int NB> struct qw_chunk_kq<QW_F_PACKED_Q6, NB> {
+    static constexpr uint32_t BLK_K = 256, BLK_B = QW_Q6_SLAB_BYTES;
+    static constexpr int DEPTH = 3;
+    qw_kq<14> b[NB];
+    __device__ __forceinline__ void load(const uint8_t *p, uint32_t lane) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const uint8_t *sl = p + QW_Q6_SLAB_BYTES * i;
+#pragma unroll
+            for (int pl = 0; pl < 3; pl++) {
+                const u4 v = *(const u4 *)(sl + 1024 * pl + 16 * lane);
+                b[i].r[4 * pl] = v[0], b[i].r[4 * pl + 1] = v[1], b[i].r[4 * pl + 2] = v[2], b[i].r[4 * pl + 3] = v[3];
+            }
+            const u4 sc = *(const u4 *)(sl + 3072 + 16 * (lane & 15));
+            b[i].r[12] = sc[0], b[i].r[13] = sc[1], b[i].r[14] = sc[2], b[i].r[15] = sc[3];
+            b[i].r[16] = *(const uint16_t *)(sl + 3328 + 2 * (lane & 15));
+        }
+    }
+    __device__ __forceinline__ void transpose() {}
+    __device__ __forceinline__ void mac(const uint32_t *tab, const qw_afrag_kq &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int i = 0; i < NB; i++) qw_kq_block<14>(b[i], tab, af, k0 + BLK_K * i, kg, acc);
+    }
+};

@@ -194,3 +194,42 @@ def test_multi_matrix_largest_k_and_bad_calls(gpu, oracle):
     for bb in wbs + ybs + [xb, small]:
         bb.free()
     path.close()
+
+
+def test_large_q6k_matrix_from_its_tile_major_copy(gpu, oracle):
+    """A Q6_K matrix of vocabulary size (the reference's lm_head, src/engine.c:658-704) is read from a tile-major copy made
+    at its first use: the same bits as from the GGUF rows (copies switched off), through qmv_gg and as one of several
+    matrices of qmv_ggm, and the copy is exactly the matrix's bytes."""
+    N, K = 16384 + 32, 2048
+    rng = np.random.default_rng(14)
+    W = synth.matrix(rng, 14, N, K)
+    path = q.Path(gpu, 2048, 512, 512, 10, 16)
+    wb = gpu.buf_from(W, device_only=True)
+    small = synth.matrix(rng, 12, 64, K)
+    sb = gpu.buf_from(small, device_only=True)
+    res = {}
+    for copies in (False, True):
+        gpu.L.qw_hip_set_repack(gpu.g, copies)
+        before = gpu.L.qw_hip_packed_bytes(gpu.g)
+        for nb in (1, 7, 16):
+            x = synth.activations(np.random.default_rng(nb), nb, K)
+            xb, yb, y2, ys = gpu.buf_from(x), gpu.buf(nb * N * 4), gpu.buf(nb * N * 4), gpu.buf(nb * 64 * 4)
+            b = gpu.batch()
+            path.qmv_gg(b, q.Tensor(wb, 14), N, K, xb, yb, nb)
+            path.qmv_ggm(b, [q.Tensor(sb, 12), q.Tensor(wb, 14)], [64, N], K, xb, [ys, y2], nb)
+            assert b.end() >= 0, gpu.last_error()
+            y = yb.view(np.float32)[:nb * N].copy()
+            assert np.array_equal(y.view(np.uint32), y2.view(np.uint32)[:nb * N])
+            if copies:
+                assert np.array_equal(y.view(np.uint32), res[nb].view(np.uint32))
+            else:
+                res[nb] = y
+                if nb == 7:
+                    assert maxrel(y.reshape(nb, N).astype(np.float64), oracle.qmv(14, W, N, K, x, f64=True)) <= 1e-5
+            for bb in (xb, yb, y2, ys):
+                bb.free()
+        assert gpu.L.qw_hip_packed_bytes(gpu.g) - before == (W.nbytes if copies else 0)
+    gpu.L.qw_hip_set_repack(gpu.g, True)
+    for bb in (wb, sb):
+        bb.free()
+    path.close()
