@@ -1833,13 +1833,21 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
             hv[r] = a.h[(ts + 8 * r) * HCD + (size_t)sq * a.D + i];
             if (a.apply) ov[r] = qw_h2f(a.out[(size_t)(ts + 8 * r) * a.D + i]);
         }
+    // (before the middle step: its loads then share that step's round trip)
+    if (tid < a.nb * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
     if (GIVEN) {
-        for (uint32_t j = tid; j < a.nb * QW_HC_LR; j += blockDim.x) sx[j / QW_HC_LR][j % QW_HC_LR] = a.sx[j];
+        for (uint32_t j0 = tid; j0 < a.nb * QW_HC_LR; j0 += 8 * blockDim.x) { // eight loads in flight a thread
+            float v[8];
+#pragma unroll
+            for (uint32_t e = 0; e < 8; e++) v[e] = j0 + e * blockDim.x < a.nb * QW_HC_LR ? a.sx[j0 + e * blockDim.x] : 0.0f;
+#pragma unroll
+            for (uint32_t e = 0; e < 8; e++)
+                if (j0 + e * blockDim.x < a.nb * QW_HC_LR) (&sx[0][0])[j0 + e * blockDim.x] = v[e];
+        }
         if (tid < a.nb * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[tid];
     } else {
         hc_mid(a, 0, a.nb, &rs[0][0], &sx[0][0], blockIdx.x == 0 && a.want_inj ? a.injo : nullptr);
     }
-    if (tid < a.nb * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
     __syncthreads();
     float v[QW_HC][10];
 #pragma unroll
