@@ -26,6 +26,7 @@ static const unsigned char qw_code_object[] = {
 #embed "qw_kernels_gfx950.hsaco"
 };
 
+#define QW_DNQ_MIN_DEFAULT 3u // token count from which down + combine run as one launch of token quarters (qwk_dnq_*)
 enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 8192, QW_MAX_FUNCS = 256 };
 
 // ---------------------------------------------------------------- records
@@ -126,9 +127,9 @@ struct qw_batch {
     struct { bool valid; qwk_pf_args a; qw_hbuf *hw, *hx, *hy; int E; } pend_pf;
     // a down projection over a few tokens that waits for the combine of the same layer: both in one launch
     // (qwk_dnc_*); launched as it is at any other dispatch or at submit
-    struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid; } pend_dn;
+    struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid, fused_grid; bool quarters; } pend_dn;
     // measurement switches, read from the environment once when the batch begins
-    struct { unsigned dnc_nb; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select; } sw;
+    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select; } sw;
 };
 
 #define QW_LD_MAX 16
@@ -775,6 +776,8 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     const char *e = getenv("QW_HIP_DNC_NB"); // token count up to which down + combine run as one launch (0: never)
     b->sw.dnc_nb = e ? (unsigned)atoi(e) : 2;
     if (b->sw.dnc_nb > QW_DNC_MAXNB) b->sw.dnc_nb = QW_DNC_MAXNB;
+    e = getenv("QW_HIP_DNQ_MIN"); // token count from which down + combine run as one launch of token quarters (0: never)
+    b->sw.dnq_min = e ? (unsigned)atoi(e) : QW_DNQ_MIN_DEFAULT;
     e = getenv("QW_HIP_SIDE"); // the side stream for launches that depend on the step's input alone: 1 on
     b->sw.side = e && e[0] == '1';
     b->sw.dn_any = getenv("QW_HIP_DN_ANY") != NULL, b->sw.nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
@@ -1299,6 +1302,11 @@ static bool flush_dn(qw_batch *b) {
     return true;
 }
 
+// The fused down + combine launch (qwk_dnq_*) shares the tokens over two quarters up to 8 tokens and over four up to 16:
+// every quarter has four tokens at most, and with one tile of rows per workgroup for two quarters and two tiles for four
+// the launch has D / 8 workgroups either way.
+static unsigned dnq_quarters(unsigned nbr) { return nbr <= 8 ? 2 : 4; }
+
 // src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
 // The shared down tiles (remembered from moe_gu_gg) run in the same launch.
 static bool tr_dn(qw_batch *b) {
@@ -1359,7 +1367,7 @@ static bool tr_dn(qw_batch *b) {
                     fname_fmt(fu, sizeof fu, "qwk_dnc_f120_c10%s", tail);
                     b->pend_dn.valid = true;
                     b->pend_dn.a = a;
-                    b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid;
+                    b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid, b->pend_dn.fused_grid = (unsigned)p->D / 16, b->pend_dn.quarters = false;
                     return true;
                 }
                 return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
@@ -1384,7 +1392,21 @@ static bool tr_dn(qw_batch *b) {
             else fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d", fd, ch);
             b->pend_dn.valid = true;
             b->pend_dn.a = a;
-            b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid;
+            b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid, b->pend_dn.fused_grid = (unsigned)p->D / 16, b->pend_dn.quarters = false;
+            return true;
+        }
+        // More tokens: down + combine as one launch in which a workgroup owns one or two tiles of output rows and a
+        // quarter of the tokens (qwk_dnq_*), when the quarter's H rows fit in LDS beside the table: waits for the combine too.
+        const unsigned tpe = (unsigned)p->D / 16, nq = dnq_quarters(nbr), tpw = nq > 2 ? 2 : 1;
+        if (b->sw.dnq_min && nbr >= b->sw.dnq_min && nbr <= 16 && fd == QW_F_PACKED && (fs == 0 || fs == 8 || fs == QW_F_PACKED) && p->topk <= 10 && p->gnb * p->topk <= (int)QW_DNQ_MAXU &&
+            tpe % 16 == 0) {
+            char fu[48];
+            if (fs) fname_fmt(fu, sizeof fu, "qwk_dnq_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
+            else fname_fmt(fu, sizeof fu, "qwk_dnq_f%d_c%d", fd, ch);
+            a.nq = nq, a.tpw = tpw;
+            b->pend_dn.valid = true;
+            b->pend_dn.a = a;
+            b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid, b->pend_dn.fused_grid = tpe / tpw * nq, b->pend_dn.quarters = true;
             return true;
         }
         return add_launch(b, intern(fn), grid, 64 * QW_WAVES_DNR, &a, sizeof a);
@@ -1412,7 +1434,11 @@ static bool tr_cmb(qw_batch *b) {
             d->nbr = nbr;
             d->out = a.out;
             d->Psh = (float *)a.Psh;
-            return add_launch(b, b->pend_dn.fused, a.D / 16, 64 * QW_WAVES_DNR, d, sizeof *d);
+            if (b->pend_dn.quarters) { // the quarters and the tiles per workgroup follow the bound token count, not the compiled one
+                d->nq = dnq_quarters(nbr), d->tpw = d->nq > 2 ? 2 : 1;
+                b->pend_dn.fused_grid = a.D / 16 / d->tpw * d->nq;
+            }
+            return add_launch(b, b->pend_dn.fused, b->pend_dn.fused_grid, 64 * QW_WAVES_DNR, d, sizeof *d);
         }
         if (!flush_dn(b)) return false;
     }
@@ -1933,6 +1959,7 @@ qw_batch *qw_hip_batch_begin_static(qw_gpu *g, void *stream) {
     qw_use *use = b->use;
     memset(b, 0, sizeof *b);
     *b = (qw_batch){.g = g, .seq = ++g->batch_seq, .stream = g->cur_stream, .noalloc = true, .xstream = (hipStream_t)stream, .l = l, .capl = 64, .use = use, .capuse = 1024};
+    b->sw.dnq_min = QW_DNQ_MIN_DEFAULT;
     b->sw.dnc_nb = 2; // the defaults of qw_batch_begin; the measurement switches of the environment do not apply here
     g->na_busy = true;
     g->err[0] = 0;

@@ -405,7 +405,7 @@ template <int NB> struct qw_chunk<21, NB> {
         }
     }
     // The same arithmetic with operand A gathered from global memory four steps at a time (qw_afrag_gather).
-    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+    template <class AF> __device__ __forceinline__ void mac_gather(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const uint32_t kb = k0 + 256 * b + 64 * kg;
@@ -558,7 +558,7 @@ template <int NB> struct qw_chunk<8, NB> {
         }
     }
     // operand A gathered four blocks at a time (NB a multiple of 4)
-    __device__ __forceinline__ void mac_gather(const u2 *, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+    template <class AF> __device__ __forceinline__ void mac_gather(const u2 *, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
         if constexpr (NB % 4 != 0) { // block by block
 #pragma unroll
             for (int b = 0; b < NB; b++) {
@@ -724,12 +724,13 @@ __device__ __forceinline__ void qw_lds_arrive() { __builtin_amdgcn_s_waitcnt(0);
 // Issue the copy of the 64 KB table into LDS (direct loads, a wave takes 64 entries at a time). Every workgroup of a
 // launch starts at a different place of the table (a rotation by its index), so that at any moment the workgroups
 // ask different memory channels. The caller runs qw_lds_arrive() and a barrier before the table is read.
-__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut) {
+// With skip > 0 the first skip waves of the workgroup take no part (they must not call this).
+__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut, uint32_t skip = 0) {
     const u4 *src = (const u4 *)glut;
     u4 *dst = (u4 *)lut;
     constexpr uint32_t N = QW_LUT_BYTES / 16;
     const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63;
-    for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i < N; i += blockDim.x) {
+    for (uint32_t i = ((uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) - skip) * 64; i < N; i += blockDim.x - 64 * skip) {
         const uint32_t j = (i + rot) & (N - 1); // a multiple of 64, the same in every lane
         qw_load_to_lds(src + j + lane, dst + j);
     }

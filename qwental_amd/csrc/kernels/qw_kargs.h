@@ -110,7 +110,12 @@ typedef struct {
     /* down + combine in one launch (qwk_dnc_*, at most QW_DNC_MAXNB tokens): the layer's output [nbr][D] binary16;
      * Psh is then also read when the launch carries no shared expert */
     uint16_t *out;
+    /* qwk_dnq_*: quarters of four tokens (nq of them) and weight tiles per workgroup (tpw: 1 or 2) */
+    uint32_t nq, tpw;
 } qwk_dn_args;
+/* Down + combine with a quarter of the tokens per workgroup (qwk_dnq_*): limits of the staged H rows */
+#define QW_DNQ_ROWS 44u /* 4 tokens x (topk + 1) rows, topk <= 10 */
+#define QW_DNQ_MAXU 160u
 #define QW_DNC_MAXNB 4
 
 /* front part of a layer: router rows on the first nrouter workgroups; when g.Wsg != NULL the shared expert's gate/up

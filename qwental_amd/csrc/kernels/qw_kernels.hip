@@ -1365,6 +1365,202 @@ QW_DNC(121, 1, 0, 1, qwk_dnc_f121_c1) QW_DNC(121, 1, 121, 1, qwk_dnc_f121_c1_s12
 QW_DNC(8, 4, 0, 1, qwk_dnc_f8_c4) QW_DNC(8, 4, 8, 4, qwk_dnc_f8_c4_s8_c4)
 QW_DNC(120, 10, 0, 10, qwk_dnc_f120_c10) QW_DNC(120, 10, 120, 10, qwk_dnc_f120_c10_s120_c10) QW_DNC(120, 10, 8, 4, qwk_dnc_f120_c10_s8_c4) // tile-major IQ4_NL rows of 640
 
+// Down + combine in one launch for 3 to 16 tokens. The range form above needs a second launch because the products
+// that make up one output row are spread over all workgroups. Here a workgroup owns tpw tiles of 16 output rows and a
+// quarter of the tokens (four): it stages all H rows of its tokens in LDS once (4 x (topk + 1) rows, both planes),
+// lists the unique experts that its tokens picked, and its waves stream those experts' tiles (the shared expert's
+// first) through the same pipeline and the same arithmetic as the range form; the partial results meet in LDS by (token,
+// slot, row) and are added in rank order, the shared expert last, exactly as the combine kernel does. An expert picked
+// by tokens of several quarters is read once per quarter (about 1.15 times the unique experts' bytes at 16 tokens);
+// the quarters of a tile group are placed on one XCD so that the repeats hit its L2. Pg and Psh are still written.
+struct qw_dnq_lds {
+    u4 hrows[2 * 64 * QW_DNQ_ROWS]; // [plane][8 k-values][row], 16 bytes each: row = local token * (topk + 1) + slot
+    float part[4 * 11 * 32];        // [local token][slot][row of the group]
+    float wl[4 * 11];               // gating weights of the quarter's tokens
+    uint32_t ue[QW_DNQ_MAXU], slot4[QW_DNQ_MAXU]; // expert of unique index u; the slot bytes of the quarter's four tokens
+    uint16_t mask[QW_DNQ_MAXU], vlist[48];        // token mask of u; the unique indices this quarter needs
+    uint32_t U, nv;
+};
+// Operand A from the staged rows, in the manner of qw_afrag_gather: lane m < 4 is local token m, its row chosen per
+// expert; four fragments per plane at a time inside one predicated region, into registers the caller keeps (and has
+// zeroed once), so that the lanes that are off (12 of every 16 at least) cost LDS nothing.
+struct qw_afrag_rows {
+    const u4 *hi_, *lo_; // this lane's row in the two planes
+    bool on;
+    h8 (&hi)[4];
+    h8 (&lo)[4];
+    static constexpr bool has_lo = true;
+    __device__ __forceinline__ void fetch4(uint32_t koff, uint32_t kstep) const {
+        if (on) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                hi[i] = __builtin_bit_cast(h8, hi_[((koff + i * kstep) >> 3) * QW_DNQ_ROWS]);
+                lo[i] = __builtin_bit_cast(h8, lo_[((koff + i * kstep) >> 3) * QW_DNQ_ROWS]);
+            }
+        }
+    }
+};
+// The tiles of `nv` experts (shared: the one shared expert) for this workgroup's tpw tiles, dealt to its waves.
+template <int F, int CH, bool SHARED, class S>
+__device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, qw_dnq_lds &L, uint32_t g, uint32_t t0, uint32_t nt, uint32_t nv, uint32_t dealt, S ready) {
+    typedef qw_chunk<F, CH> C;
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, tpe = a.D / 16, tpw = a.tpw, cpr = a.I / (C::BLK_K * CH), rw = 16 * tpw;
+    const uint32_t ts = (uint32_t)__builtin_ctz(tpw), tm = tpw - 1; // tpw is a power of two
+    const uint32_t m = n; // operand A row of this lane
+    f4 acc = {0, 0, 0, 0};
+    const u4 *const lo0 = L.hrows + a.I / 8 * QW_DNQ_ROWS;
+    h8 xhi[4] = {}, xlo[4] = {};
+    qw_afrag_rows af = {L.hrows, lo0, false, xhi, xlo};
+    auto expert = [&](uint32_t task) { return SHARED ? 0u : (uint32_t)L.vlist[task >> ts]; };
+    const uint32_t nw = blockDim.x >> 6, w0 = (qw_wave() + nw - dealt % nw) % nw; // the deal goes on where the last one (dealt tiles) stopped
+    qw_task_stream<C>(nv * tpw, w0, nw, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
+        [&](uint32_t task) {
+            const uint32_t tile = g * tpw + (task & tm);
+            const uint8_t *W = SHARED ? a.Wsd : a.Wd + (size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)L.ue[expert(task)]) * (qw_tiled(F) ? tpe : a.D) * a.rowbytes;
+            const uint32_t rb = SHARED ? a.sd_rowbytes : a.rowbytes;
+            if constexpr (qw_tiled(F)) return W + (size_t)tile * rb; // rowbytes = bytes of a tile
+            else return W + (size_t)(16 * tile + (lane >> 2)) * rb;
+        },
+        [&](uint32_t task, uint32_t ci, const C &c) {
+            const uint32_t u = expert(task);
+            if (ci == 0) { // this lane's operand A row for the task's expert
+                const uint32_t tl = m & 3, mk = SHARED ? qw_all_tokens(a.snbr) >> t0 : (uint32_t)L.mask[u] >> t0;
+                const uint32_t r = tl * (K + 1) + (SHARED ? K : (L.slot4[u] >> (8 * tl)) & 255);
+                af.on = m < nt && ((mk >> m) & 1);
+                af.hi_ = L.hrows + r, af.lo_ = lo0 + r; // (read only where on: one of the 44 rows then)
+                // a lane that is off keeps the fragments of an earlier expert: they feed output rows that are never
+                // stored (a matrix-core output row depends on its own operand A row only)
+            }
+            c.mac_gather(lut, af, ci * CH * C::BLK_K, kg, acc);
+            if (ci + 1 != cpr) return;
+            // lanes of k-group 0 hold local tokens 0 .. 3 of row n
+            const uint32_t mk = SHARED ? qw_all_tokens(a.snbr) >> t0 : (uint32_t)L.mask[u] >> t0, col = 16 * (task & tm) + n, r = 16 * (g * tpw + (task & tm)) + n;
+            if (kg == 0) {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; j++) {
+                    if (j < nt && ((mk >> j) & 1)) {
+                        const uint32_t s = SHARED ? K : (L.slot4[u] >> (8 * j)) & 255;
+                        L.part[(j * (K + 1) + s) * rw + col] = acc[j];
+                        qw_store_f32(SHARED ? a.Psh + (size_t)(t0 + j) * a.D + r : a.P + ((size_t)(t0 + j) * K + s) * a.D + r, acc[j]);
+                    }
+                }
+            }
+            acc = f4{0, 0, 0, 0};
+        },
+        ready, qw_has_lut(F) ? (const uint8_t *)a.glut : nullptr);
+}
+template <int F, int CH, int FSD, int CHSD>
+__device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_lds &L) {
+    const uint32_t K = a.topk, gnb = a.gnb, tid = threadIdx.x, lane = qw_lane(), nq = a.nq, tpw = a.tpw, rw = 16 * tpw;
+    uint32_t GU = gnb * K;
+    if (GU > QW_DNQ_MAXU) GU = QW_DNQ_MAXU; // (the host admits topk <= 10: 160 at most)
+    // workgroup -> (tile group g, quarter q): the quarters of a group are eight workgroups apart, which puts them on one XCD.
+    // The nq quarters (2 or 4) share the tokens evenly: sizes differ by one at most, four at most each.
+    const uint32_t hi8 = blockIdx.x >> 3, g = (hi8 / nq) * 8 + (blockIdx.x & 7), q = hi8 % nq;
+    const uint32_t base = a.nbr / nq, rem = a.nbr % nq, t0 = q * base + (q < rem ? q : rem);
+    uint32_t nt = base + (q < rem ? 1 : 0);
+    if (nt > 4) nt = 4; // (the host admits 16 tokens in four quarters, 8 in two)
+    // one memory round trip: the record (U, experts, masks, this quarter's slot bytes and gating weights) and the table,
+    // through registers (a workgroup has nothing else to do meanwhile, and plain loads move more bytes per clock
+    // than the direct ones)
+    {
+        const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mk = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
+        const uint8_t *sl = a.sel + QW_SEL_OFF_SLOT(gnb, K);
+        const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K)) + t0 * (K + 1);
+        constexpr uint32_t N = QW_LUT_BYTES / 16, PER = (N + QW_WG_DN - 1) / QW_WG_DN;
+        const uint32_t rot = blockIdx.x * 320u; // every workgroup starts at another place of the table
+        u4 tab[PER];
+        if (qw_has_lut(F) || qw_has_lut(FSD)) {
+#pragma unroll
+            for (uint32_t it = 0; it < PER; it++) {
+                const uint32_t i = tid + it * QW_WG_DN;
+                if (i < N) tab[it] = ((const u4 *)a.glut)[(i + rot) & (N - 1)];
+            }
+        }
+        for (uint32_t i = tid; i < GU; i += blockDim.x) {
+            uint32_t s4 = 0;
+            for (uint32_t j = 0; j < nt; j++) s4 |= (uint32_t)sl[i * gnb + t0 + j] << (8 * j);
+            L.ue[i] = ue[i], L.mask[i] = (uint16_t)mk[i], L.slot4[i] = s4;
+        }
+        for (uint32_t i = tid; i < nt * (K + 1); i += blockDim.x) L.wl[i] = wg[i];
+        if (tid == 0) L.U = *(const uint32_t *)a.sel;
+        if (qw_has_lut(F) || qw_has_lut(FSD)) {
+#pragma unroll
+            for (uint32_t it = 0; it < PER; it++) {
+                const uint32_t i = tid + it * QW_WG_DN;
+                if (i < N) ((u4 *)lut)[(i + rot) & (N - 1)] = tab[it];
+            }
+        }
+    }
+    __syncthreads();
+    // the unique experts this quarter's tokens picked, in record order: every wave makes the whole list (all write the
+    // same values to the same places), so that none waits for another before it asks for its first weights
+    uint32_t nv = 0;
+    {
+        uint32_t U = L.U;
+        if (U > GU) U = GU;
+        const uint32_t want = (1u << nt) - 1;
+        for (uint32_t u0 = 0; u0 < U; u0 += 64) {
+            const uint32_t u = u0 + lane;
+            const bool on = u < U && (((uint32_t)L.mask[u] >> t0) & want);
+            const unsigned long long bal = __ballot(on);
+            const uint32_t at = nv + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0));
+            if (on && at < 48) L.vlist[at] = (uint16_t)u;
+            nv += (uint32_t)__popcll(bal);
+        }
+        if (nv > 48) nv = 48; // (four tokens of ten experts: 40 at most)
+    }
+    const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0;
+    bool staged = false;
+    // once per wave, behind its first weight loads: every H row of the quarter's tokens into LDS in fragment order.
+    // A wave's load takes 8 rows x 128 bytes (whole cache lines), lanes 0 .. 31 the first 64 bytes of a row, 32 .. 63 the rest
+    auto ready = [&] {
+        if (staged) return;
+        staged = true;
+        const uint32_t upr = a.I / 8, cbs = upr / 8, used = nt * (K + 1), nrb = (used + 7) / 8, nunits = 2 * nrb * cbs, wv = qw_wave();
+        constexpr uint32_t NW = QW_WG_DN / 64, PER = (2 * 6 * 8 + NW - 1) / NW; // 2 planes x 6 row blocks x 8 column blocks at most
+        u4 t[PER];
+        uint32_t at[PER];
+#pragma unroll
+        for (uint32_t it = 0; it < PER; it++) {
+            const uint32_t unit = wv + it * NW, cb = unit % cbs, rest = unit / cbs, rb = rest % nrb, pl = rest / nrb;
+            const uint32_t r = 8 * rb + ((lane >> 2) & 7), c = 8 * cb + 4 * (lane >> 5) + (lane & 3);
+            at[it] = unit < nunits && r < used ? (pl * upr + c) * QW_DNQ_ROWS + r : ~0u;
+            if (at[it] != ~0u) t[it] = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t0 * (K + 1) + r) * a.I + 8 * c);
+        }
+#pragma unroll
+        for (uint32_t it = 0; it < PER; it++)
+            if (at[it] != ~0u) L.hrows[at[it]] = t[it];
+        __syncthreads();
+    };
+    // the routed experts first (every wave has tiles there, so every wave's first weights are on their way before the
+    // rows are asked for); the shared expert's tiles go to the waves that the routed deal gave one tile fewer
+    dnq_run<F, CH, false>(a, lut, L, g, t0, nt, nv, 0, ready);
+    if (FSD != 0) {
+        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true>(a, lut, L, g, t0, nt, 1, nv * tpw, ready);
+    }
+    ready(); // (for symmetry only: both runs call it, with or without tiles)
+    __syncthreads();
+    for (uint32_t j = tid; j < nt * rw; j += blockDim.x) { // rank order, then the shared expert (qwk_cmb's arithmetic)
+        const uint32_t t = j >> (4 + __builtin_ctz(tpw)), i = j & (rw - 1), r = g * rw + i;
+        const float *w = L.wl + t * (K + 1), *p = L.part + t * (K + 1) * rw + i;
+        float o = 0;
+        for (uint32_t s = 0; s < K; s++) o = __builtin_fmaf(w[s], p[s * rw], o);
+        float sh;
+        if (nsh) sh = p[K * rw];
+        else sh = a.Psh[(size_t)(t0 + t) * a.D + r]; // the caller's own shared product
+        o = __builtin_fmaf(w[K], sh, o);
+        a.out[(size_t)(t0 + t) * a.D + r] = qw_f2h(o);
+    }
+}
+#define QW_DNQ(F, CH, FSD, CHSD, NAME)                                                              \
+    extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                    \
+        __shared__ struct { u2 lut[QW_LUT_ENTRIES]; qw_dnq_lds d; } L;                               \
+        dnq_body<F, CH, FSD, CHSD>(a, L.lut, L.d);                                                  \
+    }
+QW_DNQ(121, 2, 0, 1, qwk_dnq_f121_c2) QW_DNQ(121, 2, 121, 2, qwk_dnq_f121_c2_s121_c2) QW_DNQ(121, 2, 8, 4, qwk_dnq_f121_c2_s8_c4)
+QW_DNQ(121, 1, 0, 1, qwk_dnq_f121_c1) QW_DNQ(121, 1, 121, 1, qwk_dnq_f121_c1_s121_c1) QW_DNQ(121, 1, 8, 4, qwk_dnq_f121_c1_s8_c4)
+
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
     typedef qw_chunk<F, 1> C;

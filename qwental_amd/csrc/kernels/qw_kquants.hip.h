@@ -367,7 +367,7 @@ template <int NB> struct qw_chunk<20, NB> {
             }
         }
     }
-    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+    template <class AF> __device__ __forceinline__ void mac_gather(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const uint32_t kb = k0 + 32 * b + 4 * kg;
@@ -416,7 +416,7 @@ template <> struct qw_chunk<QW_F_PACKED_NL, 10> {
     }
     template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     // operand A gathered from the two H planes in global memory by the lanes whose token is in use
-    __device__ __forceinline__ void mac_gather(const u2 *lut, const qw_afrag_gather &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+    template <class AF> __device__ __forceinline__ void mac_gather(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < 10; b++) {
             const uint32_t kb = k0 + 32 * b + 4 * kg;

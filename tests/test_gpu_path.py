@@ -604,6 +604,46 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
     dl.free()
 
 
+@pytest.mark.parametrize("nb", [3, 5, 8, 9, 13, 16])
+@pytest.mark.parametrize("fshd,I,E", [(21, 512, 64), (8, 512, 64), (21, 256, 16)])
+def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E):
+    """From five tokens on, down + combine run as one launch in which a workgroup owns one or two tiles of output rows and
+    four of the tokens (qwk_dnq_*). Output, Pg and Psh must equal bit for bit what the range-form down launch and the
+    combine launch leave (QW_HIP_DNQ_MIN=0), for token counts that fill the last quarter and that do not."""
+    if os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
+    D, K = 2048, 10
+    rng = np.random.default_rng(700 + nb + fshd + I)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21 if fshd == 21 else 8, fshd=fshd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    x[nb - 1] = x[0]  # two tokens of different quarters on the same experts
+    dl = DeviceLayer(gpu, m, device_only=True)
+    old = os.environ.get("QW_HIP_DNQ_MIN")
+    res = {}
+    try:
+        for lim in (0, 3):
+            os.environ["QW_HIP_DNQ_MIN"] = str(lim)
+            path = q.Path(gpu, D, I, E, K, 16)
+            gpu.profile(True)
+            out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            res[lim] = (out, lg, path.scratch(2).view(np.float32)[:nb * D].copy(), path.scratch(3).view(np.float32)[:nb * K * D].copy(), names)
+            path.close()
+    finally:
+        if old is None:
+            os.environ.pop("QW_HIP_DNQ_MIN", None)
+        else:
+            os.environ["QW_HIP_DNQ_MIN"] = old
+    a, b = res[0], res[3]
+    assert any(n.startswith("qwk_dnq_") for n in b[4]) and "qwk_cmb" not in b[4] and "qwk_cmb" in a[4], (a[4], b[4])
+    assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
+    assert np.array_equal(a[2].view(np.uint32), b[2].view(np.uint32)) and np.array_equal(a[3].view(np.uint32), b[3].view(np.uint32))
+    assert maxrel(b[0], oracle.moe_layer_f64(m, b[1], x)) <= TOL
+    dl.free()
+
+
 @pytest.mark.parametrize("nb,valu", [(1, False), (3, False), (16, False), (1, True), (2, True), (4, True)])
 def test_qmv_packed_and_valu_forms(gpu, oracle, nb, valu):
     """Weights in a device-only buffer take the tile-major copy; with QW_VALU in the block the VALU GEMV runs instead of
