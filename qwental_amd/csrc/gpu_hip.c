@@ -26,7 +26,7 @@ static const unsigned char qw_code_object[] = {
 #embed "qw_kernels_gfx950.hsaco"
 };
 
-#define QW_DNQ_MIN_DEFAULT 3u // token count from which down + combine run as one launch of token quarters (qwk_dnq_*)
+#define QW_DNQ_MIN_DEFAULT 2u // token count from which down + combine run as one launch of token quarters (qwk_dnq_*)
 enum { QW_MAX_ARGS = 256, QW_MAX_KERNELS = 4096, QW_MAX_BIND = 32, QW_MAX_BYTES = 256, QW_PROF_MAX = 8192, QW_MAX_FUNCS = 256 };
 
 // ---------------------------------------------------------------- records
@@ -1384,9 +1384,14 @@ static bool tr_dn(qw_batch *b) {
         if (fs) fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
         else fname_fmt(fn, sizeof fn, "qwk_dnr_f%d_c%d", fd, ch);
         const unsigned grid = persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DNR);
+        // Down + combine as one launch in which a workgroup owns one or two tiles of output rows and a share of the
+        // tokens (qwk_dnq_*): for tile-major IQ3_S rows when a share's H rows fit in LDS beside the table.
+        const unsigned tpe = (unsigned)p->D / 16, nq = dnq_quarters(nbr), tpw = nq > 2 ? 2 : 1;
+        const bool by_shares = b->sw.dnq_min && nbr >= b->sw.dnq_min && nbr <= 16 && fd == QW_F_PACKED && (fs == 0 || fs == 8 || fs == QW_F_PACKED) && p->topk <= 10 &&
+                               p->gnb * p->topk <= (int)QW_DNQ_MAXU && tpe % 16 == 0;
         // a few tokens: wait for the combine, the two run as one launch (tile-major IQ3_S or Q8_0 routed rows; a shared
         // expert in either of these)
-        if (nbr <= b->sw.dnc_nb && (fd == QW_F_PACKED || fd == 8) && (fs == 0 || fs == 8 || (fs == QW_F_PACKED && fd == QW_F_PACKED))) {
+        if (!by_shares && nbr <= b->sw.dnc_nb && (fd == QW_F_PACKED || fd == 8) && (fs == 0 || fs == 8 || (fs == QW_F_PACKED && fd == QW_F_PACKED))) {
             char fu[48];
             if (fs) fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
             else fname_fmt(fu, sizeof fu, "qwk_dnc_f%d_c%d", fd, ch);
@@ -1395,11 +1400,7 @@ static bool tr_dn(qw_batch *b) {
             b->pend_dn.fname = intern(fn), b->pend_dn.fused = intern(fu), b->pend_dn.kname = b->k->name, b->pend_dn.grid = grid, b->pend_dn.fused_grid = (unsigned)p->D / 16, b->pend_dn.quarters = false;
             return true;
         }
-        // More tokens: down + combine as one launch in which a workgroup owns one or two tiles of output rows and a
-        // quarter of the tokens (qwk_dnq_*), when the quarter's H rows fit in LDS beside the table: waits for the combine too.
-        const unsigned tpe = (unsigned)p->D / 16, nq = dnq_quarters(nbr), tpw = nq > 2 ? 2 : 1;
-        if (b->sw.dnq_min && nbr >= b->sw.dnq_min && nbr <= 16 && fd == QW_F_PACKED && (fs == 0 || fs == 8 || fs == QW_F_PACKED) && p->topk <= 10 && p->gnb * p->topk <= (int)QW_DNQ_MAXU &&
-            tpe % 16 == 0) {
+        if (by_shares) { // waits for the combine too
             char fu[48];
             if (fs) fname_fmt(fu, sizeof fu, "qwk_dnq_f%d_c%d_s%d_c%d", fd, ch, fs, fs == 8 ? 4 : p->I / 256);
             else fname_fmt(fu, sizeof fu, "qwk_dnq_f%d_c%d", fd, ch);

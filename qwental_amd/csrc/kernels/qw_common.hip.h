@@ -724,13 +724,12 @@ __device__ __forceinline__ void qw_lds_arrive() { __builtin_amdgcn_s_waitcnt(0);
 // Issue the copy of the 64 KB table into LDS (direct loads, a wave takes 64 entries at a time). Every workgroup of a
 // launch starts at a different place of the table (a rotation by its index), so that at any moment the workgroups
 // ask different memory channels. The caller runs qw_lds_arrive() and a barrier before the table is read.
-// With skip > 0 the first skip waves of the workgroup take no part (they must not call this).
-__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut, uint32_t skip = 0) {
+__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut) {
     const u4 *src = (const u4 *)glut;
     u4 *dst = (u4 *)lut;
     constexpr uint32_t N = QW_LUT_BYTES / 16;
     const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63;
-    for (uint32_t i = ((uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) - skip) * 64; i < N; i += blockDim.x - 64 * skip) {
+    for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i < N; i += blockDim.x) {
         const uint32_t j = (i + rot) & (N - 1); // a multiple of 64, the same in every lane
         qw_load_to_lds(src + j + lane, dst + j);
     }

@@ -580,6 +580,8 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
         x[nb - 1] = x[0]  # two tokens on the same experts: one product serves both
     dl = DeviceLayer(gpu, m, device_only=dev)
     old = os.environ.get("QW_HIP_DNC_NB")
+    oldq = os.environ.get("QW_HIP_DNQ_MIN")
+    os.environ["QW_HIP_DNQ_MIN"] = "0"  # the one-launch form by token shares would take these layers from two tokens on
     res = {}
     try:
         for lim in (0, limit):
@@ -596,6 +598,10 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
             os.environ.pop("QW_HIP_DNC_NB", None)
         else:
             os.environ["QW_HIP_DNC_NB"] = old
+        if oldq is None:
+            os.environ.pop("QW_HIP_DNQ_MIN", None)
+        else:
+            os.environ["QW_HIP_DNQ_MIN"] = oldq
     a, b = res[0], res[limit]
     assert any(n.startswith("qwk_dnc_") for n in b[4]) and not any(n.startswith("qwk_dnc_") for n in a[4]), (a[4], b[4])
     assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
@@ -604,12 +610,13 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
     dl.free()
 
 
-@pytest.mark.parametrize("nb", [3, 5, 8, 9, 13, 16])
+@pytest.mark.parametrize("nb", [2, 3, 5, 8, 9, 13, 16])
 @pytest.mark.parametrize("fshd,I,E", [(21, 512, 64), (8, 512, 64), (21, 256, 16)])
 def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E):
-    """From five tokens on, down + combine run as one launch in which a workgroup owns one or two tiles of output rows and
-    four of the tokens (qwk_dnq_*). Output, Pg and Psh must equal bit for bit what the range-form down launch and the
-    combine launch leave (QW_HIP_DNQ_MIN=0), for token counts that fill the last quarter and that do not."""
+    """From two tokens on, down + combine run as one launch in which a workgroup owns one or two tiles of output rows and
+    a share of the tokens, four at most (qwk_dnq_*). Output, Pg and Psh must equal bit for bit what the range-form down
+    launch and the combine launch leave (QW_HIP_DNQ_MIN=0 and QW_HIP_DNC_NB=0), for token counts that split evenly over
+    the two or four shares and that do not."""
     if os.environ.get("QW_HIP_REPACK") == "0":
         pytest.skip("tile-major copies are switched off in this environment")
     D, K = 2048, 10
@@ -620,9 +627,11 @@ def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E):
     x[nb - 1] = x[0]  # two tokens of different quarters on the same experts
     dl = DeviceLayer(gpu, m, device_only=True)
     old = os.environ.get("QW_HIP_DNQ_MIN")
+    oldc = os.environ.get("QW_HIP_DNC_NB")
+    os.environ["QW_HIP_DNC_NB"] = "0"
     res = {}
     try:
-        for lim in (0, 3):
+        for lim in (0, 2):
             os.environ["QW_HIP_DNQ_MIN"] = str(lim)
             path = q.Path(gpu, D, I, E, K, 16)
             gpu.profile(True)
@@ -636,7 +645,11 @@ def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E):
             os.environ.pop("QW_HIP_DNQ_MIN", None)
         else:
             os.environ["QW_HIP_DNQ_MIN"] = old
-    a, b = res[0], res[3]
+        if oldc is None:
+            os.environ.pop("QW_HIP_DNC_NB", None)
+        else:
+            os.environ["QW_HIP_DNC_NB"] = oldc
+    a, b = res[0], res[2]
     assert any(n.startswith("qwk_dnq_") for n in b[4]) and "qwk_cmb" not in b[4] and "qwk_cmb" in a[4], (a[4], b[4])
     assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
     assert np.array_equal(a[2].view(np.uint32), b[2].view(np.uint32)) and np.array_equal(a[3].view(np.uint32), b[3].view(np.uint32))
