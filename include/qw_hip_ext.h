@@ -75,6 +75,8 @@ unsigned qw_hip_graph_launches(const qw_gpu *g);
  *   QW_HIP_DNC_NB=n           token count up to which moe_dn_gg + moe_cmb_gg run as one launch (default 2, at most 4; 0: never)
  *   QW_HIP_DNQ_MIN=n          token count from which (up to 16) they run as the one launch by token shares, for tile-major IQ3_S
  *                             down rows (default 2; 0: never)
+ *   QW_HIP_PK_SPLIT           the packing sequence (p_zero, moe_count, moe_plan_t, moe_scatter, moe_pf_gg x 2, p_act2) one launch per
+ *                             dispatch instead of one launch for the first four and SwiGLU inside the gate / up launch
  *   QW_HIP_SIDE=1             a shared expert's gate/up in the K-quant / IQ4 / plain formats runs on a side stream beside the router
  *   QW_HIP_DN_ANY             IQ4_NL down rows take the any-shape kernel instead of the range kernel
  *   QW_HIP_NL_C4              IQ4_NL down rows from GGUF order in chunks of four blocks instead of ten

@@ -125,11 +125,15 @@ struct qw_batch {
     // a grouped product over IQ3_S rows that waits for its twin (gate, then up over the same packed rows: one launch
     // over the tile-major copy that holds both); launched alone at the next other dispatch or at submit
     struct { bool valid; qwk_pf_args a; qw_hbuf *hw, *hx, *hy; int E; } pend_pf;
+    // a gate / up pair of grouped products that runs as one launch, waiting for the p_act2 dispatch that may ride in it
+    struct { bool valid; qwk_pf_args f, second; qw_hbuf *hw, *hwb; int E; const char *kname; } pend_tw;
+    // p_zero, moe_count and moe_plan(_t) waiting for the moe_scatter dispatch with which they run as one launch (stage = how many wait)
+    struct { int stage; qwk_zero_args z; qwk_count_args c; qwk_plan_args pl; const char *kn[3]; } pend_pk;
     // a down projection over a few tokens that waits for the combine of the same layer: both in one launch
     // (qwk_dnc_*); launched as it is at any other dispatch or at submit
     struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid, fused_grid; bool quarters; } pend_dn;
     // measurement switches, read from the environment once when the batch begins
-    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select; } sw;
+    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split; } sw;
 };
 
 #define QW_LD_MAX 16
@@ -783,6 +787,7 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     b->sw.dn_any = getenv("QW_HIP_DN_ANY") != NULL, b->sw.nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
     b->sw.no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, b->sw.shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
     b->sw.split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
+    b->sw.pk_split = getenv("QW_HIP_PK_SPLIT") != NULL; // the packing sequence one launch per dispatch
     return b;
 }
 
@@ -1447,14 +1452,41 @@ static bool tr_cmb(qw_batch *b) {
 }
 
 // ---------------------------------------------------------------- ragged packing (kernels/moe_prefill.metal; src/engine.c:4133-4224)
+// The sequence p_zero (the counters), moe_count, moe_plan(_t), moe_scatter of a step with at most QW_PREP_MAXP pairs runs as
+// one launch (qwk_moe_prep): each of the first three dispatches waits for the next one as long as it continues the
+// sequence on the same buffers; anything else launches what waits, one kernel per dispatch (QW_HIP_PK_SPLIT: always).
+static bool add_named(qw_batch *b, const char *kname, const char *fname, unsigned gx, unsigned bx, const void *args, size_t argsz) {
+    const int first = b->nl;
+    if (!add_launch(b, fname, gx, bx, args, argsz)) return false;
+    if (b->nl > first) b->l[b->nl - 1].kname = kname, b->l[b->nl - 1].last_of_dispatch = true;
+    return true;
+}
+static bool flush_pk(qw_batch *b) {
+    const int st = b->pend_pk.stage;
+    b->pend_pk.stage = 0;
+    if (st >= 1 && !add_named(b, b->pend_pk.kn[0], "qwk_zero", cdiv(b->pend_pk.z.n, 256), 256, &b->pend_pk.z, sizeof b->pend_pk.z)) return false;
+    if (st >= 2 && !add_named(b, b->pend_pk.kn[1], "qwk_moe_count", cdiv(b->pend_pk.c.P, 256), 256, &b->pend_pk.c, sizeof b->pend_pk.c)) return false;
+    if (st >= 3 && !add_named(b, b->pend_pk.kn[2], "qwk_moe_plan", 1, 1024, &b->pend_pk.pl, sizeof b->pend_pk.pl)) return false;
+    return true;
+}
 static bool tr_pk_count(qw_batch *b) { // 0 ids, 1 counts, 2 P
     qwk_count_args a = {.E = (uint32_t)b->k->p.E};
     if (!bind_bytes(b, 2, &a.P, 4, "P") || !bind_ptr(b, 0, (size_t)a.P * 4, false, "ids", (void **)&a.ids) || !bind_ptr(b, 1, (size_t)a.E * 4, true, "counts", (void **)&a.counts)) return false;
+    if (b->pend_pk.stage == 1 && b->pend_pk.z.x == a.counts && b->pend_pk.z.n == a.E && a.E <= 1024 && a.P <= QW_PREP_MAXP) {
+        b->pend_pk.stage = 2, b->pend_pk.c = a, b->pend_pk.kn[1] = b->k->name;
+        return true;
+    }
+    if (!flush_pk(b)) return false;
     return add_launch(b, "qwk_moe_count", cdiv(a.P, 256), 256, &a, sizeof a);
 }
 static bool tr_pk_zero(qw_batch *b) { // kernels/prefill.metal:601-603: 0 x, 1 n (dwords to clear)
     qwk_zero_args a = {0};
     if (!bind_bytes(b, 1, &a.n, 4, "n") || !bind_ptr(b, 0, (size_t)a.n * 4, true, "x", (void **)&a.x)) return false;
+    if (!flush_pk(b)) return false;
+    if (!b->sw.pk_split) {
+        b->pend_pk.stage = 1, b->pend_pk.z = a, b->pend_pk.kn[0] = b->k->name;
+        return true;
+    }
     return add_launch(b, "qwk_zero", cdiv(a.n, 256), 256, &a, sizeof a);
 }
 static bool tr_pk_plan(qw_batch *b, bool tm_bound) { // 0 counts, 1 offs, 2 cursor, 3 tiles, 4 max_tiles (, 5 tm)
@@ -1465,6 +1497,11 @@ static bool tr_pk_plan(qw_batch *b, bool tm_bound) { // 0 counts, 1 offs, 2 curs
     if (!bind_ptr(b, 0, (size_t)a.E * 4, false, "counts", (void **)&a.counts) || !bind_ptr(b, 1, (size_t)a.E * 4, true, "offs", (void **)&a.offs) ||
         !bind_ptr(b, 2, (size_t)a.E * 4, true, "cursor", (void **)&a.cursor) || !bind_ptr(b, 3, (size_t)a.max_tiles * 16, true, "tiles", (void **)&a.tiles)) return false;
     if (b->buf[3].off % 16) return fail(b, "%s: tile table offset %zu is not 16-byte aligned", b->k->name, b->buf[3].off);
+    if (b->pend_pk.stage == 2 && b->pend_pk.c.counts == a.counts && b->pend_pk.c.E == a.E) {
+        b->pend_pk.stage = 3, b->pend_pk.pl = a, b->pend_pk.kn[2] = b->k->name;
+        return true;
+    }
+    if (!flush_pk(b)) return false;
     return add_launch(b, "qwk_moe_plan", 1, 1024, &a, sizeof a);
 }
 static bool tr_pk_scatter(qw_batch *b, unsigned gx) { // 0 X, 1 ids, 2 cursor, 3 Xs, 4 pos_of; grid x = P
@@ -1475,6 +1512,14 @@ static bool tr_pk_scatter(qw_batch *b, unsigned gx) { // 0 X, 1 ids, 2 cursor, 3
         !bind_ptr(b, 2, (size_t)p->E * 4, true, "cursor", (void **)&a.cursor) || !bind_ptr(b, 3, (size_t)gx * p->K * 2, true, "Xs", (void **)&a.Xs) ||
         !bind_ptr(b, 4, (size_t)gx * 4, true, "pos_of", (void **)&a.pos_of)) return false;
     if (b->buf[0].off % 16 || b->buf[3].off % 16) return fail(b, "moe_scatter: row buffers must be 16-byte aligned");
+    if (b->pend_pk.stage == 3 && b->pend_pk.pl.cursor == a.cursor && b->pend_pk.c.ids == a.ids && b->pend_pk.c.P == a.P && b->pend_pk.c.E == a.E && a.KD % 8 == 0) {
+        const qwk_plan_args *pl = &b->pend_pk.pl;
+        const qwk_prep_args f = {.ids = a.ids, .counts = b->pend_pk.c.counts, .offs = pl->offs, .cursor = pl->cursor, .tiles = pl->tiles, .pos_of = a.pos_of, .X = a.X, .Xs = a.Xs,
+                                 .P = a.P, .E = a.E, .topk = a.topk, .KD = a.KD, .tm = pl->tm, .max_tiles = pl->max_tiles};
+        b->pend_pk.stage = 0;
+        return add_launch(b, "qwk_moe_prep", a.P, 256, &f, sizeof f);
+    }
+    if (!flush_pk(b)) return false;
     return add_launch(b, "qwk_moe_scatter", gx, 256, &a, sizeof a);
 }
 static bool tr_pk_act(qw_batch *b) { // 0 G [P][2 I], 1 H [P][I], 2 P
@@ -1485,10 +1530,18 @@ static bool tr_pk_act(qw_batch *b) { // 0 G [P][2 I], 1 H [P][I], 2 P
     if (!bind_ptr(b, 0, (size_t)a.n * 4, false, "G", (void **)&a.G) || !bind_ptr(b, 1, (size_t)a.n * 2, true, "H", (void **)&a.H)) return false;
     return add_launch(b, "qwk_moe_act", cdiv(a.n, 256), 256, &a, sizeof a);
 }
+static bool flush_tw(qw_batch *b, uint16_t *H, bool *acted);
 static bool tr_pk_act2(qw_batch *b) { // kernels/prefill.metal:485-488: 0 G, 1 U, 2 H, 3 n
     qwk_act_args a = {0};
     if (!bind_bytes(b, 3, &a.n, 4, "n")) return false;
     if (!bind_ptr(b, 0, (size_t)a.n * 2, false, "G", (void **)&a.G) || !bind_ptr(b, 1, (size_t)a.n * 2, false, "U", (void **)&a.U) || !bind_ptr(b, 2, (size_t)a.n * 2, true, "H", (void **)&a.H)) return false;
+    if (b->pend_tw.valid) { // SwiGLU of exactly what the waiting gate / up launch writes: it rides at that launch's end
+        const qwk_pf_args *f = &b->pend_tw.f;
+        const bool rides = !b->sw.pk_split && f->Y == a.G && f->Y1 == a.U && (uint64_t)f->M * f->N == a.n && a.H != f->Y && a.H != f->Y1 && (const uint16_t *)a.H != f->X;
+        bool acted = false;
+        if (!flush_tw(b, rides ? a.H : NULL, &acted)) return false;
+        if (acted) return true;
+    }
     return add_launch(b, "qwk_moe_act", cdiv(a.n, 256), 256, &a, sizeof a);
 }
 static bool tr_pk_combine(qw_batch *b, unsigned gy) { // 0 D, 1 pos_of, 2 w, 3 Y; grid = (KD / 4 / 64, T)
@@ -1505,6 +1558,7 @@ static bool tr_pk_combine(qw_batch *b, unsigned gy) { // 0 D, 1 pos_of, 2 w, 3 Y
 // matrix of a gate / up pair (tiles of 8 + 8 rows, outputs a->Y and a->Y1), else a single matrix (tiles of 16 rows).
 static bool launch_pf(qw_batch *b, qwk_pf_args *a, int F, int E, qw_hbuf *hw, qw_hbuf *hwb, const uint8_t *wb) {
     a->split = 16, a->ntn = a->N / 16;
+    if (!wb) a->H = NULL, a->Y1 = NULL; // SwiGLU rides only in a launch that holds both matrices
     char fn[32];
     if (F == 21 && a->K % 256 == 0) {
         const uint32_t nblk = a->K / 256, split = wb ? 8 : 16;
@@ -1533,6 +1587,26 @@ static bool flush_pf(qw_batch *b) {
     b->pend_pf.valid = false;
     return launch_pf(b, &b->pend_pf.a, 21, b->pend_pf.E, b->pend_pf.hw, NULL, NULL);
 }
+// The waiting gate / up pair: one launch over the tile-major copy of both (H: SwiGLU of the two results at its end, *acted
+// tells whether it was done), or the two matrices one by one when there is no such copy (small buffers, copies switched off).
+static bool flush_tw(qw_batch *b, uint16_t *H, bool *acted) {
+    if (acted) *acted = false;
+    if (!b->pend_tw.valid) return true;
+    b->pend_tw.valid = false;
+    const int first = b->nl;
+    qwk_pf_args f = b->pend_tw.f;
+    f.H = H;
+    bool ok = launch_pf(b, &f, 21, b->pend_tw.E, b->pend_tw.hw, b->pend_tw.hwb, b->pend_tw.second.W);
+    if (ok) {
+        if (acted) *acted = H != NULL;
+    } else {
+        if (b->failed) return false;
+        qwk_pf_args one = b->pend_tw.f, two = b->pend_tw.second;
+        ok = launch_pf(b, &one, 21, b->pend_tw.E, b->pend_tw.hw, NULL, NULL) && launch_pf(b, &two, 21, b->pend_tw.E, b->pend_tw.hwb, NULL, NULL);
+    }
+    for (int i = first; ok && i < b->nl; i++) b->l[i].kname = b->pend_tw.kname;
+    return ok;
+}
 
 static bool tr_pf(qw_batch *b, unsigned gy) {
     const qw_kparams *p = &b->k->p;
@@ -1554,14 +1628,12 @@ static bool tr_pf(qw_batch *b, unsigned gy) {
         const qwk_pf_args *q = &b->pend_pf.a;
         const bool twin = p->F == 21 && q->X == a.X && q->tiles == a.tiles && q->M == a.M && q->N == a.N && q->K == a.K && q->max_tiles == a.max_tiles &&
                           q->W != a.W && q->Y != a.Y && b->pend_pf.E == p->E && hy != b->pend_pf.hx && b->pend_pf.hy != hx && b->pend_pf.hy != hy;
-        if (twin) {
-            qwk_pf_args f = *q;
-            f.Y1 = a.Y;
+        if (twin) { // launched at the next dispatch (flush_tw): a p_act2 over the two results rides in the same launch
             b->pend_pf.valid = false;
-            if (launch_pf(b, &f, 21, p->E, b->pend_pf.hw, hw, a.W)) return true;
-            if (b->failed) return false;
-            qwk_pf_args first = *q; // no tile-major copy (small buffers, copies switched off): one by one
-            return launch_pf(b, &first, 21, p->E, b->pend_pf.hw, NULL, NULL) && launch_pf(b, &a, 21, p->E, hw, NULL, NULL);
+            b->pend_tw.valid = true;
+            b->pend_tw.f = *q, b->pend_tw.f.Y1 = a.Y, b->pend_tw.second = a;
+            b->pend_tw.hw = b->pend_pf.hw, b->pend_tw.hwb = hw, b->pend_tw.E = p->E, b->pend_tw.kname = b->k->name;
+            return true;
         }
         if (!flush_pf(b)) return false;
     }
@@ -1675,8 +1747,10 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     const int first = b->nl;
     bool ok;
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
+    if (b->k->fam != FAM_PK_ACT2 && !flush_tw(b, NULL, NULL)) return;
     if (b->k->fam != FAM_PF && !flush_pf(b)) return;
     if (b->k->fam != FAM_CMB && !flush_dn(b)) return;
+    if (b->k->fam != FAM_PK_ZERO && b->k->fam != FAM_PK_COUNT && b->k->fam != FAM_PK_PLAN && b->k->fam != FAM_PK_PLAN_T && b->k->fam != FAM_PK_SCATTER && !flush_pk(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
     case FAM_QMV_GGM: ok = tr_qmvm(b); break;
@@ -1786,7 +1860,7 @@ static int graph_run(qw_batch *b, hipStream_t st) {
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
-    if (b->failed || !flush_select(b) || !flush_pf(b) || !flush_dn(b)) return false;
+    if (b->failed || !flush_select(b) || !flush_tw(b, NULL, NULL) || !flush_pf(b) || !flush_dn(b) || !flush_pk(b)) return false;
     if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
     // host -> device for what this segment binds
     const unsigned mark = ++g->mark;
@@ -1969,7 +2043,7 @@ qw_batch *qw_hip_batch_begin_static(qw_gpu *g, void *stream) {
 bool qw_hip_batch_launch_static(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = b->xstream ? b->xstream : g->stream[b->stream];
-    bool ok = !b->failed && flush_select(b) && flush_pf(b) && flush_dn(b) && !b->failed;
+    bool ok = !b->failed && flush_select(b) && flush_tw(b, NULL, NULL) && flush_pf(b) && flush_dn(b) && flush_pk(b) && !b->failed;
     for (int i = 0; ok && i < b->nl; i++) {
         qw_launch *l = &b->l[i];
         void *params[] = {l->args};

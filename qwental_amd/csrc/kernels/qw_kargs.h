@@ -249,7 +249,18 @@ typedef struct { /* Y[m][n] = X[m] . W[expert][n] for the rows m of every tile e
                            * matrix B (-> Y1), N rows each; ntn = tiles per expert (N / 16 or N / 8) */
     const void *glut;
     uint16_t *Y1;
+    uint16_t *H;          /* split 8 only, may be null: [M][N] = SiLU(Y) * Y1 from the rounded values, as qwk_moe_act leaves it */
 } qwk_pf_args;
+/* count + prefix sums + tile table + rows to packed order in one launch of P workgroups (P <= QW_PREP_MAXP, E <= 1024) */
+#define QW_PREP_MAXP 4096u
+typedef struct {
+    const uint32_t *ids;                  /* [P] */
+    uint32_t *counts, *offs, *cursor;     /* [E]: as qwk_zero + qwk_moe_count, qwk_moe_plan and qwk_moe_scatter leave them */
+    uint32_t *tiles, *pos_of;
+    const uint16_t *X;
+    uint16_t *Xs;
+    uint32_t P, E, topk, KD, tm, max_tiles;
+} qwk_prep_args;
 
 typedef struct { /* synthetic weights: nblocks GGUF blocks of one type, scale d = binary16(|N(0, sigma)|), the rest uniform */
     uint8_t *dst;

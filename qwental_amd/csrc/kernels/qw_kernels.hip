@@ -1660,6 +1660,74 @@ extern "C" __global__ __launch_bounds__(256) void qwk_moe_scatter(qwk_scatter_ar
     u4 *dst = (u4 *)(a.Xs + (size_t)pos * a.KD);
     for (uint32_t i = threadIdx.x; i < a.KD / 8; i += blockDim.x) dst[i] = src[i];
 }
+// The four launches above as one, for a step of a few thousand pairs at most: a workgroup per pair, and every workgroup
+// counts all pairs itself (LDS atomics over the P ids), which gives it its own packed row without a hand-over: the rows
+// of the experts below its own plus the earlier pairs of its own expert. The order inside an expert is therefore the
+// order of the pairs (the cursor form leaves whatever order the atomics came in; both are permutations the grouped
+// product and the combine do not care about). Workgroup 0 also leaves counts, offsets, cursors (where the scatter
+// would have left them) and the tile table.
+extern "C" __global__ __launch_bounds__(256) void qwk_moe_prep(qwk_prep_args a) {
+    __shared__ uint32_t cnt[1024], red[4], wr[4], wt[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, p = blockIdx.x;
+    const uint32_t ep = (uint32_t)__builtin_amdgcn_readfirstlane((int)a.ids[p]);
+    for (uint32_t e = tid; e < a.E; e += 256) cnt[e] = 0;
+    __syncthreads();
+    uint32_t mine = 0; // earlier pairs of this pair's expert
+    for (uint32_t q = tid; q < a.P; q += 256) {
+        const uint32_t e = a.ids[q];
+        if (e < a.E) atomicAdd(&cnt[e], 1u);
+        mine += e == ep && q < p;
+    }
+    __syncthreads();
+    if (ep < a.E)
+        for (uint32_t e = tid; e < ep; e += 256) mine += cnt[e]; // rows of the experts below
+#pragma unroll
+    for (int o = 32; o; o >>= 1) mine += __shfl_xor(mine, o);
+    if (lane == 0) red[wave] = mine;
+    __syncthreads();
+    const uint32_t pos = ep < a.E ? red[0] + red[1] + red[2] + red[3] : 0xffffffffu; // an expert id outside the table: the pair is dropped
+    if (tid == 0) a.pos_of[p] = pos;
+    if (pos < a.P) {
+        const u4 *src = (const u4 *)(a.X + (size_t)(p / a.topk) * a.KD);
+        u4 *dst = (u4 *)(a.Xs + (size_t)pos * a.KD);
+        for (uint32_t i = tid; i < a.KD / 8; i += 256) dst[i] = src[i];
+    }
+    if (blockIdx.x != 0) return;
+    // the tables (qwk_moe_plan's arithmetic): thread t has experts 4 t .. 4 t + 3
+    uint32_t c[4], nt[4], sr = 0, st = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        const uint32_t e = 4 * tid + i;
+        c[i] = e < a.E ? cnt[e] : 0, nt[i] = (c[i] + a.tm - 1) / a.tm;
+        sr += c[i], st += nt[i];
+    }
+    uint32_t pr = sr, pt = st; // inclusive scans inside the wave
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t ur = __shfl_up(pr, o), ut = __shfl_up(pt, o);
+        if (lane >= (uint32_t)o) pr += ur, pt += ut;
+    }
+    if (lane == 63) wr[wave] = pr, wt[wave] = pt;
+    __syncthreads();
+    uint32_t row0 = pr - sr, tile0 = pt - st, total_t = 0;
+    for (uint32_t w = 0; w < 4; w++) {
+        if (w < wave) row0 += wr[w], tile0 += wt[w];
+        total_t += wt[w];
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        const uint32_t e = 4 * tid + i;
+        if (e < a.E) {
+            a.counts[e] = c[i], a.offs[e] = row0, a.cursor[e] = row0 + c[i];
+            for (uint32_t t = 0; t < nt[i]; t++) {
+                const uint32_t r = row0 + t * a.tm;
+                if (tile0 + t < a.max_tiles) *(u4 *)(a.tiles + 4 * (tile0 + t)) = u4{e, r, r + a.tm < row0 + c[i] ? r + a.tm : row0 + c[i], 0};
+            }
+        }
+        row0 += c[i], tile0 += nt[i];
+    }
+    for (uint32_t t = total_t + tid; t < a.max_tiles; t += 256) *(u4 *)(a.tiles + 4 * t) = u4{0, 0, 0, 0}; // unused entries
+}
 // H = SiLU(gate) * up, binary16 in and out, the product rounded once (kernels/moe_prefill.metal:95-103, kernels/prefill.metal:485-488)
 extern "C" __global__ __launch_bounds__(256) void qwk_moe_act(qwk_act_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -1691,6 +1759,13 @@ extern "C" __global__ __launch_bounds__(64) void qwk_moe_combine(qwk_combine_arg
     *(u2 *)(a.Y + (size_t)t * a.KD + 4 * c4) = o;
 }
 
+// SwiGLU at the end of a tile of 8 gate + 8 up rows (a.H given): lane n < 8 has the gate value of a packed row and a
+// column, lane n + 8 the up value of the same two; both as the binary16 the G and U buffers hold, the product rounded
+// once, exactly as qwk_moe_act computes it from those buffers. Called by all lanes.
+__device__ __forceinline__ void qw_pf_act(const qwk_pf_args &a, uint16_t y, uint32_t m, bool store, uint32_t col) {
+    const float g = qw_h2f(y), u = qw_h2f((uint16_t)__shfl_xor((int)y, 8));
+    if (store) a.H[(size_t)m * a.N + col] = qw_f2h(g / (1.0f + __expf(-g)) * u);
+}
 // Grouped product over the packed rows (kernels/moe_gg.metal:761-838): task = (tile entry, 16 weight rows); the
 // weights of a task are decoded once and multiplied into up to four groups of 16 packed rows of the entry
 // (tm <= 64). The non-empty entries are the first ones of the table; their number is counted here.
@@ -1752,7 +1827,9 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
 #pragma unroll
                 for (uint32_t j = 0; j < 4; j++) {
                     const uint32_t m = m0 + 16 * g + 4 * kg + j;
-                    if (m < m1) Y[(size_t)m * a.N + col] = qw_f2h(acc[g][j]);
+                    const uint16_t y = qw_f2h(acc[g][j]);
+                    if (m < m1) Y[(size_t)m * a.N + col] = y;
+                    if (a.H) qw_pf_act(a, y, m, m < m1 && !second, col);
                 }
                 acc[g] = f4{0, 0, 0, 0};
             }
@@ -1775,7 +1852,7 @@ template <int CH> __device__ __forceinline__ void pf_range_body(const qwk_pf_arg
     typedef qw_chunk<QW_F_PACKED, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, nwv = blockDim.x >> 6;
     if (threadIdx.x == 0) *cnt = 0;
-    qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_lut_copy_issue(lut, (const u2 *)a.glut); // lands while the table of entries is read: one memory round trip for both
     __syncthreads();
     uint32_t mine = 0; // the non-empty entries are the first ones of the table
     for (uint32_t t = threadIdx.x; t < a.max_tiles; t += blockDim.x) {
@@ -1783,6 +1860,7 @@ template <int CH> __device__ __forceinline__ void pf_range_body(const qwk_pf_arg
         mine += e.z > e.y;
     }
     if (mine) atomicAdd(cnt, mine);
+    qw_lds_arrive();
     __syncthreads();
     const uint32_t used = *cnt, ntn = a.ntn, total = used * ntn, cpr = a.K / (C::BLK_K * CH);
     const uint32_t per = (total + gridDim.x - 1) / gridDim.x;
@@ -1812,7 +1890,9 @@ template <int CH> __device__ __forceinline__ void pf_range_body(const qwk_pf_arg
 #pragma unroll
                 for (uint32_t j = 0; j < 4; j++) {
                     const uint32_t m = m0 + 4 * kg + j;
-                    if (m < m1) Y[(size_t)m * a.N + col] = qw_f2h(acc[j]);
+                    const uint16_t y = qw_f2h(acc[j]);
+                    if (m < m1) Y[(size_t)m * a.N + col] = y;
+                    if (a.H) qw_pf_act(a, y, m, m < m1 && !second, col);
                 }
                 acc = f4{0, 0, 0, 0};
             }, ready);

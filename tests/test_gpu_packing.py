@@ -166,3 +166,63 @@ def test_ragged_step_decode_groups_equal_packing_path(gpu, oracle):
         bb.free()
     dl.free()
     path.close()
+
+
+@pytest.mark.parametrize("dev,tm,T", [(True, 16, 40), (True, 64, 40), (False, 16, 24), (True, 16, 130)])
+def test_packing_fused_launches_equal_one_per_dispatch(gpu, oracle, dev, tm, T):
+    """p_zero + moe_count + moe_plan_t + moe_scatter run as one launch (qwk_moe_prep), and p_act2 rides at the end of the
+    gate / up launch when that one runs over the tile-major copy. Against one launch per dispatch (QW_HIP_PK_SPLIT):
+    counts, offsets and tile table equal, every pair's packed x and H rows equal bit for bit, the output equal bit for
+    bit; the packed order inside an expert is the order of the pairs."""
+    if dev and os.environ.get("QW_HIP_REPACK") == "0":
+        pytest.skip("tile-major copies are switched off in this environment")
+    E, K, D, I = 32, 4, 512, 512
+    rng = np.random.default_rng(300 + tm + T)
+    m = synth.moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21)
+    x = synth.activations(rng, T, D)
+    ids = synth.zipf_ids(rng, T, E, K)
+    w = rng.uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    dl = DeviceLayer(gpu, m, device_only=dev)
+    P = T * K
+    old = os.environ.get("QW_HIP_PK_SPLIT")
+    res = {}
+    try:
+        for split in (True, False):
+            if split:
+                os.environ["QW_HIP_PK_SPLIT"] = "1"
+            else:
+                os.environ.pop("QW_HIP_PK_SPLIT", None)
+            path = q.Path(gpu, D, I, E, K, 16)
+            path.pf_reserve(T, tm)
+            xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.ravel()), gpu.buf(T * D * 2)
+            gpu.profile(True)
+            b = gpu.batch()
+            path.pf_moe(b, dl.layer, T, xb, ib, wb, ob)
+            assert b.end() >= 0, gpu.last_error()
+            names = [n for n, _ in gpu.profile_entries()]
+            gpu.profile(False)
+            mt = path.pf_max_tiles()
+            res[split] = dict(names=names, out=ob.view(np.uint16)[:T * D].copy(), cnt=path.pf_scratch(0, np.uint32)[:E].copy(), offs=path.pf_scratch(1, np.uint32)[:E].copy(),
+                              tiles=path.pf_scratch(2, np.uint32)[:4 * mt].copy(), pos=path.pf_scratch(3, np.uint32)[:P].copy(),
+                              Xs=path.pf_scratch(4, np.uint16)[:P * D].reshape(P, D).copy(), H=path.pf_scratch(5, np.uint16)[:P * I].reshape(P, I).copy())
+            for bb in (xb, ib, wb, ob):
+                bb.free()
+            path.close()
+    finally:
+        if old is None:
+            os.environ.pop("QW_HIP_PK_SPLIT", None)
+        else:
+            os.environ["QW_HIP_PK_SPLIT"] = old
+    a, f = res[True], res[False]
+    assert "qwk_moe_prep" in f["names"] and not any(n in f["names"] for n in ("qwk_zero", "qwk_moe_count", "qwk_moe_plan", "qwk_moe_scatter")), f["names"]
+    assert "qwk_moe_prep" not in a["names"] and "qwk_moe_scatter" in a["names"] and "qwk_moe_act" in a["names"], a["names"]
+    assert ("qwk_moe_act" not in f["names"]) == dev, f["names"]  # it rides only in the launch over the tile-major copy of gate and up
+    for key in ("cnt", "offs", "tiles", "out"):
+        assert np.array_equal(a[key], f[key]), key
+    assert sorted(f["pos"].tolist()) == list(range(P))
+    flat = ids.ravel()
+    for e in range(E):  # inside an expert: the order of the pairs
+        pe = f["pos"][flat == e]
+        assert np.array_equal(pe, f["offs"][e] + np.arange(len(pe)))
+    assert np.array_equal(a["Xs"][a["pos"]], f["Xs"][f["pos"]]) and np.array_equal(a["H"][a["pos"]], f["H"][f["pos"]])
+    dl.free()
