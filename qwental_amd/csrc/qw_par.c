@@ -24,20 +24,28 @@ void qw_par_observe(qw_par *p, int b, double ms) {
 double qw_par_group_cost(const qw_par *p, int b) { return b >= 1 && b <= QW_PAR_VBMAX ? p->cost[b] : 0; }
 
 // Sizes never measured, filled in on the line through the smallest and the largest measured size (one size: flat).
+// Two measured sizes close together can give the line any slope (a launch's time varies by a few per cent): a falling
+// line is taken as flat at the cheapest measured size, and no size is estimated below half of that, so that an estimate is never
+// zero or negative (a step cut into many groups that "cost nothing").
 static bool fill_line(const double *c, int n, double *out) {
     int lo = 0, hi = 0;
+    double least = 0;
     for (int b = 1; b <= n; b++)
         if (c[b] > 0) {
             if (!lo) lo = b;
             hi = b;
+            if (least == 0 || c[b] < least) least = c[b];
         }
     if (!lo) return false;
-    double a = c[lo], k = 0;
-    if (hi > lo) {
+    double a = hi > lo ? least : c[lo], k = 0;
+    if (hi > lo && c[hi] > c[lo]) {
         k = (c[hi] - c[lo]) / (hi - lo);
         a = c[lo] - k * lo;
     }
-    for (int b = 1; b <= n; b++) out[b] = c[b] > 0 ? c[b] : a + k * b;
+    for (int b = 1; b <= n; b++) {
+        out[b] = c[b] > 0 ? c[b] : a + k * b;
+        if (out[b] < 0.5 * least) out[b] = 0.5 * least;
+    }
     return true;
 }
 

@@ -52,6 +52,22 @@ def test_estimate_fills_unmeasured_sizes_on_a_line():
     p.free()
 
 
+def test_estimate_is_never_zero_or_negative():
+    """Two measured sizes close together whose times fall with the size (a launch's time varies by a few per cent): the
+    line is taken as flat and no estimate goes below half of the cheapest measured size."""
+    p = q.Par()
+    feed(p, 14, [0.30])
+    feed(p, 16, [0.216])
+    assert p.cost(1) == pytest.approx(0.216) and p.cost(8) == pytest.approx(0.216)  # flat at the cheapest measured size
+    assert p.cost(46) == pytest.approx(3 * 0.216)
+    p.free()
+    p = q.Par()
+    feed(p, 15, [1.0])
+    feed(p, 16, [2.0])  # a steep rising line through two neighbours would cross zero at 14
+    assert p.cost(1) == pytest.approx(0.5) and p.cost(3) == pytest.approx(0.5)
+    p.free()
+
+
 def brute(cost, B):
     """Cheapest sum over every multiset of group sizes 1..16 that adds up to B."""
     @functools.lru_cache(None)
