@@ -65,6 +65,7 @@ RATIOS = [
     ("tcp_pending_stall_frac", "TCP_PENDING_STALL_CYCLES_sum", "TCP_GATE_EN1_sum", "cycles the vector L1 stalled on a pending request / cycles it was clocked"),
     ("l1_miss_frac", "TCP_TCC_READ_REQ_sum", "TCP_TOTAL_CACHE_ACCESSES_sum", "read requests the vector L1 sent to L2 / its accesses"),
     ("wait_frac", "SQ_WAIT_INST_ANY", "SQ_WAVE_CYCLES", "quad-cycles waves waited for any instruction's result / quad-cycles waves were resident"),
+    ("icache_miss_frac", "SQC_ICACHE_MISSES", "SQC_ICACHE_REQ", "instruction cache misses / requests"),
 ]
 
 
