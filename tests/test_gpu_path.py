@@ -611,16 +611,15 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
 
 
 @pytest.mark.parametrize("nb", [2, 3, 5, 8, 9, 13, 16])
-@pytest.mark.parametrize("fshd,I,E", [(21, 512, 64), (8, 512, 64), (21, 256, 16)])
-def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E):
+@pytest.mark.parametrize("fshd,I,E,K,D", [(21, 512, 64, 10, 2048), (8, 512, 64, 10, 2048), (21, 256, 16, 10, 2048), (21, 512, 64, 8, 1024), (8, 256, 32, 4, 2560)])
+def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E, K, D):
     """From two tokens on, down + combine run as one launch in which a workgroup owns one or two tiles of output rows and
     a share of the tokens, four at most (qwk_dnq_*). Output, Pg and Psh must equal bit for bit what the range-form down
     launch and the combine launch leave (QW_HIP_DNQ_MIN=0 and QW_HIP_DNC_NB=0), for token counts that split evenly over
     the two or four shares and that do not."""
     if os.environ.get("QW_HIP_REPACK") == "0":
         pytest.skip("tile-major copies are switched off in this environment")
-    D, K = 2048, 10
-    rng = np.random.default_rng(700 + nb + fshd + I)
+    rng = np.random.default_rng(700 + nb + fshd + I + K)
     m = synth.moe_layer(rng, D, I, E, fgu=21, fd=21, fsh=21 if fshd == 21 else 8, fshd=fshd)
     m["topk"] = K
     x = synth.activations(rng, nb, D)
