@@ -226,3 +226,115 @@ def test_packing_fused_launches_equal_one_per_dispatch(gpu, oracle, dev, tm, T):
         assert np.array_equal(pe, f["offs"][e] + np.arange(len(pe)))
     assert np.array_equal(a["Xs"][a["pos"]], f["Xs"][f["pos"]]) and np.array_equal(a["H"][a["pos"]], f["H"][f["pos"]])
     dl.free()
+
+
+def _pk_kernels(gpu, tag, E, K, KD, I, tm):
+    ks = {}
+    for base in ("p_zero", "moe_count", "moe_plan_t", "moe_scatter"):
+        name = "%s_%s" % (base, tag)
+        ok, err = gpu.compile("#define %s %s\n#define E %d\n#define TOPK %d\n#define KD %d\n#define I %d\n#define TM %d\n" % (base, name, E, K, KD, I, tm))
+        assert ok, err
+        ks[base] = gpu.kernel(name)
+        assert ks[base]
+    return ks
+
+
+def _pk_dispatch(b, ks, which, **a):
+    """One dispatch of the packing sequence with the reference's binding indices (src/engine.c:4137-4144, 4201-4227)."""
+    b.kernel(ks[which])
+    if which == "p_zero":
+        b.buf(0, a["x"])
+        b.bytes(1, np.uint32([a["n"]]))
+        b.dispatch((a["n"] + 255) // 256, tx=256)
+    elif which == "moe_count":
+        b.buf(0, a["ids"])
+        b.buf(1, a["counts"])
+        b.bytes(2, np.uint32([a["P"]]))
+        b.dispatch((a["P"] + 255) // 256, tx=256)
+    elif which == "moe_plan_t":
+        for i, key in enumerate(("counts", "offs", "cursor", "tiles")):
+            b.buf(i, a[key])
+        b.bytes(4, np.uint32([a["max_tiles"]]))
+        b.bytes(5, np.uint32([a["tm"]]))
+        b.dispatch(1, tx=a["E"])
+    else:
+        for i, key in enumerate(("X", "ids", "cursor", "Xs", "pos_of")):
+            b.buf(i, a[key])
+        b.dispatch(a["P"], tx=256)
+
+
+def test_packing_sequence_that_breaks_the_pattern(gpu, oracle):
+    """p_zero, moe_count and moe_plan_t wait for the next dispatch of the sequence; a dispatch that does not continue it
+    on the same buffers (or the end of the batch) launches what waited, one kernel per dispatch, in order. Every case
+    must leave what the dispatches say, whichever launches carry them."""
+    E, K, KD, I, tm, T = 32, 4, 512, 512, 16, 20
+    P = T * K
+    ks = _pk_kernels(gpu, "brk", E, K, KD, I, tm)
+    rng = np.random.default_rng(81)
+    ids = synth.zipf_ids(rng, T, E, K).astype(np.uint32).ravel()
+    x = synth.activations(rng, T, KD)
+    mt = (P + tm - 1) // tm + E
+    counts, offs, _, tiles, _ = oracle.moe_pack(ids, E, tm, mt)
+    idb, idb2, xb = gpu.buf_from(ids), gpu.buf_from(ids), gpu.buf_from(x)
+    mk = lambda n: gpu.buf_from(np.full(n, 7, np.uint32))  # stale contents everywhere
+    gpu.profile(True)
+
+    def names():
+        return [n for n, _ in gpu.profile_entries()]
+
+    # 1. the counters cleared are not the counters counted into: two launches, both effects
+    A, B = mk(E), mk(E)
+    b = gpu.batch()
+    _pk_dispatch(b, ks, "p_zero", x=A, n=E)
+    _pk_dispatch(b, ks, "moe_count", ids=idb, counts=B, P=P)
+    b.end()
+    assert names() == ["qwk_zero", "qwk_moe_count"]
+    assert not A.view(np.uint32)[:E].any() and np.array_equal(B.view(np.uint32)[:E], 7 + counts)
+    # 2. the batch ends after the count: the two that waited are launched
+    b = gpu.batch()
+    _pk_dispatch(b, ks, "p_zero", x=A, n=E)
+    _pk_dispatch(b, ks, "moe_count", ids=idb, counts=A, P=P)
+    b.end()
+    assert names() == ["qwk_zero", "qwk_moe_count"] and np.array_equal(A.view(np.uint32)[:E], counts)
+    # 3. fewer dwords cleared than there are counters: no part of the pattern
+    b = gpu.batch()
+    _pk_dispatch(b, ks, "p_zero", x=B, n=E // 2)
+    _pk_dispatch(b, ks, "moe_count", ids=idb, counts=B, P=P)
+    b.end()
+    assert names() == ["qwk_zero", "qwk_moe_count"]
+    assert np.array_equal(B.view(np.uint32)[:E], np.concatenate([counts[:E // 2], 7 + 2 * counts[E // 2:]]))
+    # 4. the scatter reads other ids than the count did (the same values at another address): three launches, then the scatter
+    offb, curb, tilb, posb, Xs = mk(E), mk(E), mk(4 * mt), mk(P), gpu.buf(P * KD * 2)
+    seq = dict(counts=A, offs=offb, cursor=curb, tiles=tilb, max_tiles=mt, tm=tm, E=E, X=xb, Xs=Xs, pos_of=posb, P=P)
+    b = gpu.batch()
+    _pk_dispatch(b, ks, "p_zero", x=A, n=E)
+    _pk_dispatch(b, ks, "moe_count", ids=idb, **seq)
+    _pk_dispatch(b, ks, "moe_plan_t", **seq)
+    _pk_dispatch(b, ks, "moe_scatter", ids=idb2, **seq)
+    b.end()
+    assert names() == ["qwk_zero", "qwk_moe_count", "qwk_moe_plan", "qwk_moe_scatter"]
+
+    def check():
+        assert np.array_equal(A.view(np.uint32)[:E], counts) and np.array_equal(offb.view(np.uint32)[:E], offs)
+        assert np.array_equal(curb.view(np.uint32)[:E], offs + counts) and np.array_equal(tilb.view(np.uint32)[:4 * mt], tiles.ravel())
+        pos = posb.view(np.uint32)[:P]
+        assert sorted(pos.tolist()) == list(range(P)) and all(offs[ids[p]] <= pos[p] < offs[ids[p]] + counts[ids[p]] for p in range(P))
+        rows = Xs.view(np.uint16)[:P * KD].reshape(P, KD)
+        assert all(np.array_equal(rows[pos[p]], x[p // K].view(np.uint16)) for p in range(P))
+
+    check()
+    # 5. the whole sequence twice in one batch, on the same buffers: one launch each, the same contents
+    for bb in (A, offb, curb, posb):
+        bb.fill(np.full(bb.view(np.uint32).size, 9, np.uint32))
+    b = gpu.batch()
+    for _ in range(2):
+        _pk_dispatch(b, ks, "p_zero", x=A, n=E)
+        _pk_dispatch(b, ks, "moe_count", ids=idb, **seq)
+        _pk_dispatch(b, ks, "moe_plan_t", **seq)
+        _pk_dispatch(b, ks, "moe_scatter", ids=idb, **seq)
+    b.end()
+    assert names() == ["qwk_moe_prep", "qwk_moe_prep"]
+    check()
+    gpu.profile(False)
+    for bb in (idb, idb2, xb, A, B, offb, curb, tilb, posb, Xs):
+        bb.free()
