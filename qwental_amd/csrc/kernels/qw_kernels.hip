@@ -789,6 +789,11 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     }
     issued(); // the waves without a token
     __syncthreads();
+    if (a.nbr == 1) { // one token: its picks are the unique experts, in rank order (what the steps below would leave)
+        if (tid < K) c.ue[tid] = s.ids[tid], c.mask[tid] = 1, c.slot[tid * gnb] = (uint8_t)tid;
+        if (tid == 0) c.U = K;
+        __syncthreads();
+    } else {
     if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid); // first flat index of every picked expert
     __syncthreads();
     // lead = this pair is its expert's first; every wave leaves the ballot of its leads (UM <= 256: four waves)
@@ -820,6 +825,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         c.U = U;
     }
     __syncthreads();
+    }
     if (!store) return;
     // the record, in one pass of dword stores: U | ue[GU] | mask[GU] | slot[GU][gnb] | w[gnb][K + 1]
     uint32_t *out = (uint32_t *)a.sel;
