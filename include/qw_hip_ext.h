@@ -81,6 +81,7 @@ unsigned qw_hip_graph_launches(const qw_gpu *g);
  *   QW_HIP_DN_ANY             IQ4_NL down rows take the any-shape kernel instead of the range kernel
  *   QW_HIP_NL_C4              IQ4_NL down rows from GGUF order in chunks of four blocks instead of ten
  *   QW_HIP_NO_SWIGLU_MATVEC   such a shared expert's gate/up as two launches (matvec, then SwiGLU) instead of one
+ *   QW_HIP_KQ_OWN_LAUNCH      such a shared expert's gate/up as a launch of its own instead of on the workgroups behind the router's
  *   QW_HIP_SHARED_IN_GU       an IQ3_S / Q8_0 shared expert's gate/up inside the gate/up launch instead of the front launch
  *   QW_HIP_SPLIT_SELECT       the selection as a launch of its own instead of inside the gate/up launch
  * QW_HIP_REPACK=0 and QW_HIP_GRAPH=1 are read once, by qw_gpu_open() (see above); QW_HIP_LOAD_THREADS by qw_hip_buf_write_fd();

@@ -133,7 +133,7 @@ struct qw_batch {
     // (qwk_dnc_*); launched as it is at any other dispatch or at submit
     struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid, fused_grid; bool quarters; } pend_dn;
     // measurement switches, read from the environment once when the batch begins
-    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split; } sw;
+    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split, kq_own; } sw;
 };
 
 #define QW_LD_MAX 16
@@ -788,6 +788,7 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     b->sw.no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, b->sw.shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
     b->sw.split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
     b->sw.pk_split = getenv("QW_HIP_PK_SPLIT") != NULL; // the packing sequence one launch per dispatch
+    b->sw.kq_own = getenv("QW_HIP_KQ_OWN_LAUNCH") != NULL; // a K-quant / IQ4 / plain shared expert's gate/up as a launch of its own
     return b;
 }
 
@@ -849,6 +850,7 @@ static bool bind_bytes(qw_batch *b, unsigned index, void *dst, size_t len, const
     return true;
 }
 
+_Static_assert(sizeof(qwk_prekq_args) <= QW_MAX_ARGS, "argument record");
 _Static_assert(sizeof(qwk_pre_args) <= QW_MAX_ARGS && sizeof(qwk_gu_args) <= QW_MAX_ARGS && sizeof(qwk_dn_args) <= QW_MAX_ARGS && sizeof(qwk_qmv_args) <= QW_MAX_ARGS,
                "a kernel argument record is larger than the launch record's copy of it");
 
@@ -1154,8 +1156,11 @@ static bool tr_sel(qw_batch *b) { // src/engine.c:609-614: 0 logits, 1 sel, 2 nb
 // A shared expert whose gate and up rows are in the other format family (Q4_K gate and IQ4_XS up in the reference's
 // model, bench/moe_bw.c:19-20): the multi-format matvec over the two matrices, then SwiGLU into H.
 #define QW_SHGU_MAXI 4096
-static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t *h) {
+// front: the router's arguments when the caller is the front launch, which then takes this work onto the workgroups
+// after the router's (one launch, qwk_pre_w1_kq) when it can; *rode tells whether it did.
+static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t *h, const qwk_pre_args *front, bool *rode) {
     const qw_kparams *p = &b->k->p;
+    if (rode) *rode = false;
     if (p->I > QW_SHGU_MAXI) return fail(b, "moe_pre_gg: I %d too wide for shared gate/up types %d/%d", p->I, p->fsg, p->fsu);
     if (b->buf[2].off % 16 || b->buf[6].off % 16 || b->buf[7].off % 16) return fail(b, "moe_pre_gg: x and shared gate/up offsets must be 16-byte aligned for types %d/%d", p->fsg, p->fsu);
     float *gy = b->g->shgu + (size_t)b->stream * 2 * 16 * QW_SHGU_MAXI, *uy = gy + (size_t)16 * p->I;
@@ -1179,7 +1184,14 @@ static bool shared_gu_kq(qw_batch *b, uint32_t nbr, const uint16_t *x, uint16_t 
             m.ntiles[j] = cdiv((unsigned)p->I, 16);
             if (m.fmt[j] == 12 || m.fmt[j] == 13) m.sums = 1;
         }
-        if (!add_launch(b, "qwk_qmvm_swiglu", umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2)), 64 * QW_WAVES_GU, &m, sizeof m)) return false;
+        const unsigned wgs = umin((unsigned)b->g->ncu, cdiv(m.ntiles[0], QW_WAVES_GU / sw / 2));
+        if (front && p->rwf == 1 && b->sw.side != 1 && !b->sw.kq_own) { // binary16 router: its workgroups first, then these
+            qwk_prekq_args f = {.r = front->r, .nrouter = front->nrouter, .m = m};
+            if (!add_launch(b, "qwk_pre_w1_kq", f.nrouter + wgs, 64 * QW_WAVES_GU, &f, sizeof f)) return false;
+            *rode = true;
+            return true;
+        }
+        if (!add_launch(b, "qwk_qmvm_swiglu", wgs, 64 * QW_WAVES_GU, &m, sizeof m)) return false;
     } else if (!launch_qmvm(b, &m, NULL) || !add_launch(b, "qwk_sh_act", cdiv(nbr * (unsigned)p->I, 256), 256, &sa, sizeof sa)) return false;
     if (b->sw.side == 1)
         for (int i = first; i < b->nl; i++) b->l[i].side = true;
@@ -1206,7 +1218,7 @@ static bool tr_pre(qw_batch *b) {
     b->pend_sg.nbr = nbr;
     if (!p->rbf) { // router and selection come as dispatches of their own
         const uint16_t *x;
-        return !kq_ok(p->fsg) || (bind_ptr(b, 2, (size_t)nbr * p->D * 2, false, "x", (void **)&x) && shared_gu_kq(b, nbr, x, h));
+        return !kq_ok(p->fsg) || (bind_ptr(b, 2, (size_t)nbr * p->D * 2, false, "x", (void **)&x) && shared_gu_kq(b, nbr, x, h, NULL, NULL));
     }
     // router rows per workgroup: 16 on the matrix cores (binary16 router), 8 on the vector units (bf16 router)
     qwk_pre_args a = {.nrouter = cdiv((unsigned)p->E + 1, p->rwf == 1 ? 16 : 8)};
@@ -1233,8 +1245,9 @@ static bool tr_pre(qw_batch *b) {
         }
     }
     // the counter buffer of the reference's hand-over (index 4) is not used
-    if (kq_ok(p->fsg) && !shared_gu_kq(b, nbr, a.r.x, h)) return false; // first: side launches fork where they stand in the batch
-    if (!add_launch(b, intern(fn), grid, 512, &a, sizeof a)) return false;
+    bool rode = false;
+    if (kq_ok(p->fsg) && !shared_gu_kq(b, nbr, a.r.x, h, &a, &rode)) return false; // first: side launches fork where they stand in the batch
+    if (!rode && !add_launch(b, intern(fn), grid, 512, &a, sizeof a)) return false;
     if (!fill_select(b, &b->pend_sel.a, 3, 5, nbr)) return false;
     b->pend_sel.valid = true; // made by the gate/up launch if one follows for the same record, else by its own launch
     return true;

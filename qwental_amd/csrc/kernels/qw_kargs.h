@@ -125,6 +125,13 @@ typedef struct {
     uint32_t nrouter, pad;
     qwk_gu_args g;
 } qwk_pre_args;
+/* the front launch when the shared expert's gate/up rows are in the K-quant / IQ4 / plain family (qwk_pre_w1_kq):
+ * m as for qwk_qmvm_swiglu, on the workgroups after the router's */
+typedef struct {
+    qwk_router_args r;
+    uint32_t nrouter, pad;
+    qwk_qmvm_args m;
+} qwk_prekq_args;
 
 typedef struct { /* out[t][row] = half(sum_s w[t][s] * Pg[t][s][row] + w[t][topk] * Psh[t][row]) */
     const float *Pg, *Psh;

@@ -303,8 +303,9 @@ template <int F, int NB> __device__ __forceinline__ f4 qmvm_part(const qwk_qmvm_
 // matrix 0 holds the gate rows, matrix 1 the up rows, each of its own format. A workgroup takes 12 / split / 2 pairs of
 // tiles (gate tile t and up tile t side by side), split waves a tile as in qwk_qmvm; the partial sums meet in LDS, and
 // the first wave of a gate tile adds up both tiles in part order, applies SwiGLU and stores H's two planes.
-extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmvm_args a) {
-    __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; } L;
+// bid of nblk: the workgroup's number among those that do this work (the front launch puts the router's workgroups first).
+struct qw_qmvm_lds { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; };
+__device__ __forceinline__ void qmvm_swiglu_body(const qwk_qmvm_args &a, qw_qmvm_lds &L, uint32_t bid, uint32_t nblk) {
     qw_kq_tab_build(L.tab);
     qw_stage_x(L.xf, a.x, a.xstride, a.K, a.nb);
     __syncthreads();
@@ -326,7 +327,7 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmv
     const qw_afrag_kq af = {L.xf, L.xs, n, kg};
     const uint32_t pairs = (QW_WG_QMVM / 64) / sp / 2, slot = wave / sp, part = wave % sp, which = slot & 1, ntiles = a.ntiles[0];
     const uint32_t ngroups = (ntiles + pairs - 1) / pairs;
-    for (uint32_t g = blockIdx.x; g < ngroups; g += gridDim.x) {
+    for (uint32_t g = bid; g < ngroups; g += nblk) {
         const uint32_t t = slot < 2 * pairs ? g * pairs + slot / 2 : ntiles; // waves past a whole number of pairs: none
         f4 acc = {0, 0, 0, 0};
         if (t < ntiles) {
@@ -361,6 +362,10 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmv
         }
         __syncthreads();
     }
+}
+extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmvm_args a) {
+    __shared__ qw_qmvm_lds L;
+    qmvm_swiglu_body(a, L, blockIdx.x, gridDim.x);
 }
 
 extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args a) {
@@ -988,15 +993,16 @@ template <int WF> __device__ __forceinline__ void pre_router(const qwk_pre_args 
 // Binary16 router on the matrix cores: a workgroup takes 16 router rows (row E is the shared-expert gate vector), its
 // waves split K among themselves (256 values = 8 matrix instructions a wave per pass), the partial sums meet in LDS
 // and wave 0 adds them in wave order. A token's logits do not depend on the other token columns.
-__device__ __forceinline__ void pre_router_mfma(const qwk_pre_args &pa, u4 *xf, f4 *part) {
-    const qwk_router_args &a = pa.r;
-    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, wave = qw_wave(), nwv = blockDim.x >> 6;
+// Eight waves take part whatever the workgroup's size: the split of K and the order of the final sum, hence the bits
+// of the logits, are the same in every kernel that holds this router.
+__device__ __forceinline__ void pre_router_mfma(const qwk_router_args &a, u4 *xf, f4 *part) {
+    const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, wave = qw_wave(), nwv = QW_WG / 64;
     const uint32_t row = 16 * blockIdx.x + n;
     const uint16_t *wrow = row < a.E ? (const uint16_t *)a.Wr + (size_t)row * a.D : (const uint16_t *)a.Wsg; // rows past E repeat the gate vector; not stored
     f4 acc = {0, 0, 0, 0};
     // the first pass's weights are in flight while x is staged
     u4 w[8];
-    uint32_t k0 = 256 * wave;
+    uint32_t k0 = wave < nwv ? 256 * wave : a.D; // (waves past the eighth: nothing)
     if (k0 < a.D)
 #pragma unroll
         for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 32 * j + 8 * kg);
@@ -1063,13 +1069,20 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {                           \
         __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[(QW_WG / 64) * 64]; } L; \
         if (blockIdx.x < a.nrouter) {                                                                   \
-            if (WF == 1) pre_router_mfma(a, L.xf, L.part);                                              \
+            if (WF == 1) pre_router_mfma(a.r, L.xf, L.part);                                            \
             else pre_router<WF>(a, L.xf);                                                               \
         }                                                                                               \
         else if (F != 0) pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part);                              \
     }
 QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
 QW_PRE(1, 121, 2, qwk_pre_w1_s121_c2) QW_PRE(30, 121, 2, qwk_pre_w30_s121_c2) QW_PRE(1, 8, 16, qwk_pre_w1_s8_c16) QW_PRE(30, 8, 16, qwk_pre_w30_s8_c16)
+// The same front launch for a shared expert whose gate/up rows are in the K-quant / IQ4 / plain family: the binary16
+// router on the first workgroups, the multi-format product with SwiGLU (qwk_qmvm_swiglu's work) on those after them.
+extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_pre_w1_kq(qwk_prekq_args a) {
+    __shared__ qw_qmvm_lds L;
+    if (blockIdx.x < a.nrouter) pre_router_mfma(a.r, L.xf, L.red);
+    else qmvm_swiglu_body(a.m, L, blockIdx.x - a.nrouter, gridDim.x - a.nrouter);
+}
 
 // SwiGLU of the shared expert (kernels/moe_gg.metal:563-573) after a matvec of its gate and up rows in another format
 // family: the arithmetic and the two-plane store of pre_shared. One thread per (token, column).

@@ -524,7 +524,8 @@ def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd
     out, lg, selraw, _ = run_moe(gpu, path, dl, x, nb)
     names = [n for n, _ in gpu.profile_entries()]
     gpu.profile(False)
-    assert "qwk_qmvm_swiglu" in names or ("qwk_qmvm" in names and "qwk_sh_act" in names), names
+    # rows of several chunks: inside the front launch, behind the router's workgroups; a single chunk: matvec, then SwiGLU
+    assert ("qwk_pre_w1_kq" in names and "qwk_pre_w1" not in names) or ("qwk_qmvm" in names and "qwk_sh_act" in names), names
     gnb = 8 if nb <= 8 else 16
     ref = oracle.moe_layer_f64(m, lg, x)
     assert np.isfinite(out.astype(np.float64)).all()
@@ -721,6 +722,7 @@ def test_packed_copy_follows_the_source(gpu, oracle):
     ("QW_HIP_SHARED_IN_GU", (2048, 512, 64, 10, 16, 21, 21, 21, 21, None), "qwk_gu_f121_c2_s121_c2"),    # shared gate/up inside the gate/up launch
     ("QW_HIP_NL_C4", (1024, 640, 32, 10, 6, 21, 20, 8, 20, None), "qwk_dnr_f20_c4_s20_c4"),              # IQ4_NL down in chunks of four blocks
     ("QW_HIP_NO_SWIGLU_MATVEC", (2560, 640, 32, 10, 4, 21, 20, 12, 20, 23), "qwk_sh_act"),               # shared gate/up: matvec, then SwiGLU
+    ("QW_HIP_KQ_OWN_LAUNCH", (2560, 640, 32, 10, 9, 21, 20, 12, 20, 23), "qwk_qmvm_swiglu"),              # shared gate/up: a launch of its own beside the front launch
 ])
 def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, oracle, switch, shape, want):
     """The environment switches that qw_batch_begin reads (include/qw_hip_ext.h) route a layer through kernels that other
@@ -751,7 +753,7 @@ def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, or
         os.environ.pop(switch, None)
         if old is not None:
             os.environ[switch] = old
-    if switch in ("QW_HIP_SPLIT_SELECT", "QW_HIP_NO_SWIGLU_MATVEC"):  # the same products in the same order (the shared gate/up inside
+    if switch in ("QW_HIP_SPLIT_SELECT", "QW_HIP_NO_SWIGLU_MATVEC", "QW_HIP_KQ_OWN_LAUNCH"):  # the same products in the same order (the shared gate/up inside
         # the gate/up launch adds a row's blocks one after the other, the front launch per chunk first)
         assert np.array_equal(outs[False].view(np.uint16), outs[True].view(np.uint16))
     dl.free()
