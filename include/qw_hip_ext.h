@@ -29,7 +29,9 @@ bool qw_hip_buf_new_device(qw_gpu *g, size_t size, qw_buf *out);
 /* The host changed a large buffer after its first use: copy it again at the next submit. */
 void qw_hip_buf_mark_dirty(qw_buf *b);
 /* Explicit copies (synchronous). upload/download move [offset, offset + len) between the shadow and HBM;
- * write/read move between caller memory and HBM (the only way to fill or inspect a device-only buffer). */
+ * write/read move between caller memory and HBM (the only way to fill or inspect a device-only buffer). write and
+ * write_fd also store the bytes in the host side of a buffer that has one (not a wrapped one: that memory is the
+ * caller's), so that the upload at the buffer's next bind carries them. */
 bool qw_hip_buf_upload(qw_buf *b, size_t offset, size_t len);
 bool qw_hip_buf_download(qw_buf *b, size_t offset, size_t len);
 bool qw_hip_buf_write(qw_buf *b, size_t offset, const void *src, size_t len);
@@ -69,9 +71,19 @@ size_t qw_hip_released_bytes(const qw_gpu *g);
 void qw_hip_set_graphs(qw_gpu *g, bool on);
 unsigned qw_hip_graph_launches(const qw_gpu *g);
 
-/* Measurement switches, read from the environment by every qw_batch_begin(). Each routes a layer through kernels that
- * other shapes or formats reach by themselves, so that both forms can be timed on one shape; results do not change
- * (tests/test_gpu_path.py runs a layer with each of them set).
+/* Measurement switches, read from the environment ONCE, by qw_gpu_open(); a batch takes the device's switches as they
+ * are when it begins, and nothing reads the environment afterwards. A program that changes a variable while it holds
+ * a device (the tests and the benchmark do, to time two forms on one shape) calls qw_hip_reload_switches() to have
+ * them read again. Each switch routes a layer through kernels that other shapes or formats reach by themselves;
+ * results do not change (tests/test_gpu_path.py runs a layer with each of them set).
+ *   QW_HIP_FUSE=1             routed gate/up, down and combine of a layer run as one launch whose workgroups meet at a barrier
+ *                             (qwk_gud_*: tile-major IQ3_S rows with D <= 2048, I = 512, top-k <= 10, on stream 0). Off by
+ *                             default: the hand-over inside the launch costs what the two launch boundaries cost
+ *   QW_HIP_SPIN_LIMIT=n       polls of the barrier word after which a workgroup of that launch stops waiting for the others
+ *                             (default 65536, some tenths of a second). A launch that gives up fails its batch with a message
+ *                             (negative time from qw_batch_end); the device then keeps its layers as separate launches until
+ *                             qw_hip_reload_switches() is called. All workgroups of such a launch must be resident at once:
+ *                             it is used on stream 0 only and never by qw_path_gg_moe_noalloc (the caller's stream).
  *   QW_HIP_DNC_NB=n           token count up to which moe_dn_gg + moe_cmb_gg run as one launch (default 2, at most 4; 0: never)
  *   QW_HIP_DNQ_MIN=n          token count from which (up to 16) they run as the one launch by token shares, for tile-major IQ3_S
  *                             down rows (default 2; 0: never)
@@ -84,8 +96,13 @@ unsigned qw_hip_graph_launches(const qw_gpu *g);
  *   QW_HIP_KQ_OWN_LAUNCH      such a shared expert's gate/up as a launch of its own instead of on the workgroups behind the router's
  *   QW_HIP_SHARED_IN_GU       an IQ3_S / Q8_0 shared expert's gate/up inside the gate/up launch instead of the front launch
  *   QW_HIP_SPLIT_SELECT       the selection as a launch of its own instead of inside the gate/up launch
- * QW_HIP_REPACK=0 and QW_HIP_GRAPH=1 are read once, by qw_gpu_open() (see above); QW_HIP_LOAD_THREADS by qw_hip_buf_write_fd();
- * QW_HIP_VERBOSE prints every error text to stderr as it is set, QW_HIP_QUIET keeps qw_batch_wait from printing one. */
+ * Read at the same two places: QW_HIP_LOAD_THREADS (threads of qw_hip_buf_write_fd), QW_HIP_VERBOSE (every error text
+ * goes to stderr as it is set) and QW_HIP_QUIET (qw_batch_wait prints none). QW_HIP_REPACK=0 and QW_HIP_GRAPH=1 are
+ * read by qw_gpu_open() only (see above); afterwards qw_hip_set_repack / qw_hip_set_graphs change them. */
+void qw_hip_reload_switches(qw_gpu *g);
+/* The device's synchronisation words (the first 384 are the barrier's: all zero between launches except word 0, the
+ * generation; word 352 is the error word), copied to dst after a device synchronisation. For tests. */
+bool qw_hip_sync_words(qw_gpu *g, uint32_t *dst, size_t nwords);
 
 /* The define-block front end of qw_gpu_compile() without a device: parses src as qw_gpu_compile would, and on
  * success writes the names of the kernels it would register to names (comma separated). For host-side tests. */

@@ -22,6 +22,7 @@ extern "C" {
 
 enum { QW_PAR_VBMAX = 16, QW_PAR_MAX = 64 }; /* rows of one group; rows of one step (src/engine.h:79) */
 enum { QW_PAR_PACK_MAX = 256 };             /* rows the packed form is tracked for */
+enum { QW_PAR_SLICE_MAX = 3 };              /* conversations up to which time slices are weighed against a joint step (tools/serve.c:1252) */
 
 typedef struct qw_par qw_par;
 
@@ -44,6 +45,14 @@ double qw_par_packed_cost(const qw_par *p, int rows);
  * rows <= QW_PAR_MAX, else ngroups = 0 and the caller cuts into full groups). The packing path is chosen only when
  * both forms have estimates and its estimate is lower. */
 bool qw_par_choose(const qw_par *p, int rows, int *groups, int *ngroups);
+/* The server's rule between time slices and a joint step for n decoding conversations (tools/serve.c:1715-1729 of the
+ * reference, want_slice): true = one conversation at a time. n <= 1: true; n > QW_PAR_SLICE_MAX: false. sliced_rate: the
+ * measured total rate of n conversations taking turns, switches included (0: not measured; then the mean of solo_rate[i],
+ * each conversation's rate inside its own slice, solo_default standing in for a 0 or for solo_rate == NULL).
+ * batched_rate: the measured total rate of a joint step of n rows (0: not measured; then n rows per qw_par_cost(p, n)).
+ * Without a figure on either side: false. Otherwise the mode changes only when the other one is five per cent faster:
+ * slicing_now keeps slices while sliced > 0.95 batched, a joint step goes over to slices only when sliced > 1.05 batched. */
+bool qw_par_want_slice(const qw_par *p, int n, bool slicing_now, double sliced_rate, const double *solo_rate, double solo_default, double batched_rate);
 
 #ifdef __cplusplus
 }

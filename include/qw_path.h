@@ -140,7 +140,9 @@ bool qw_path_hyper_moe_stack(qw_path *p, qw_batch *b, const qw_hyper_w *H, const
  * `stream` (a hipStream_t; NULL = the stream qw_gpu_set_stream selected) and returns without waiting: no device or pinned
  * memory is allocated or freed, no event or stream is made, nothing is copied, and a tile-major copy of the weights is
  * used when an earlier allocating call made one, never made here (the GGUF rows are read directly otherwise; same
- * results). Every call on a device uses the same array, which keeps the last call's contents (nothing in it has to
+ * results). The first call for a shape registers that shape's kernel names with the device (a few small host
+ * allocations and look-ups in the code object, nothing on the device): a caller that must not even do that makes one
+ * call per shape beforehand. Every call on a device uses the same array, which keeps the last call's contents (nothing in it has to
  * start from zero): calls that overlap on one device, on any streams, race. */
 #define QW_NOALLOC_MAX_NB 16
 #define QW_NOALLOC_MAX_D 2560

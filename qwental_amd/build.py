@@ -3,7 +3,8 @@
     python -m qwental_amd.build
 
 Three steps, all cross-compile without a GPU:
-  1. hipcc --genco: csrc/kernels/qw_kernels.hip -> csrc/qw_kernels_gfx950.hsaco
+  1. hipcc --genco: csrc/kernels/qw_kernels.hip -> csrc/qw_kernels_gfx950.hsaco (one code object: the same kernels spread over
+     several measured 3 % slower on the 48-layer step)
   2. hipcc -c: csrc/qw_noalloc.hip (host + device: the per-device scratch array of the entry point that allocates nothing) -> csrc/qw_noalloc.o
   3. clang -std=c23: csrc/gpu_hip.c (embeds the code object) + csrc/qw_path.c + csrc/qw_gguf.c + csrc/qw_par.c + qw_noalloc.o -> qwental_amd/libqwgpu_hip.so
 """
@@ -18,9 +19,17 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 CLANG = os.path.join(ROCM, "llvm", "bin", "clang")
 LIB = os.path.join(HERE, "libqwgpu_hip.so")
-HSACO = os.path.join(CSRC, "qw_kernels_gfx950.hsaco")
+# Experiments: QW_BUILD_TAG=<tag> makes a second build beside the product's, libqwgpu_hip_<tag>.so with its objects in
+# csrc/_<tag>/ (QW_HIP_LIB selects it at run time); QW_BUILD_DEFS adds compiler flags, e.g. -DQW_PARTS=0x37 for a code
+# object that holds only some groups of kernels (a short compile).
+TAG = os.environ.get("QW_BUILD_TAG", "")
+OBJDIR = os.path.join(CSRC, "_" + TAG) if TAG else CSRC
+if TAG:
+    os.makedirs(OBJDIR, exist_ok=True)
+    LIB = os.path.join(HERE, "libqwgpu_hip_%s.so" % TAG)
+HSACO = os.path.join(OBJDIR, "qw_kernels_gfx950.hsaco")
 # -packed-fp32-ops: packed FP32 instructions are kept out of every kernel of this library
-HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + os.environ.get("QW_BUILD_DEFS", "").split()
 
 
 def _run(cmd):
@@ -35,17 +44,18 @@ def _run(cmd):
 def build(verbose=False, kernels=True):
     """kernels=False keeps the code object of the last build (host-side iterations: `python -m qwental_amd.build --host-only`)."""
     if kernels or not os.path.exists(HSACO):
-        out = _run([HIPCC] + HIPFLAGS + ["--genco", "-I", os.path.join(CSRC, "kernels"), "-o", HSACO,
-                                        os.path.join(CSRC, "kernels", "qw_kernels.hip")])
+        out = _run([HIPCC] + HIPFLAGS + ["--genco", "-I", os.path.join(CSRC, "kernels"), "-o", HSACO, os.path.join(CSRC, "kernels", "qw_kernels.hip")])
         if verbose and out.strip():
             print(out)
-    noalloc_o = os.path.join(CSRC, "qw_noalloc.o")
+    noalloc_o = os.path.join(OBJDIR, "qw_noalloc.o")
     _run([HIPCC] + HIPFLAGS + ["-fPIC", "-I", CSRC, "-I", os.path.join(ROOT, "include"), "-c", os.path.join(CSRC, "qw_noalloc.hip"), "-o", noalloc_o])
-    out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+    out = _run([CLANG, "-std=c23", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "--embed-dir=" + OBJDIR] + [f for f in os.environ.get("QW_BUILD_DEFS", "").split() if f.startswith("-D")] + ["-I", os.path.join(ROOT, "include"), "-I", CSRC,
                 "-I", os.path.join(ROCM, "include"), os.path.join(CSRC, "gpu_hip.c"), os.path.join(CSRC, "qw_path.c"), os.path.join(CSRC, "qw_gguf.c"), os.path.join(CSRC, "qw_par.c"), noalloc_o, "-pthread", "-o", LIB,
                 "-L", os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib")])
     if verbose and out.strip():
         print(out)
+    if TAG:
+        return LIB
     # command-line tool with the reference's dqtest contract
     _run([CLANG, "-std=c23", "-O2", "-Wall", "-I", os.path.join(ROOT, "include"), os.path.join(CSRC, "tools", "dqhip.c"), "-o",
           os.path.join(HERE, "dqhip"), "-L", HERE, "-lqwgpu_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + os.path.join(ROCM, "lib")])

@@ -94,6 +94,9 @@ typedef struct {
 
 typedef struct { qw_hbuf *b; bool out; } qw_use;
 
+// measurement switches: read from the environment by qw_gpu_open (and again by qw_hip_reload_switches), never per batch
+typedef struct { unsigned dnc_nb, dnq_min, spin_limit; int side, load_threads; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split, kq_own, no_fuse, verbose, quiet; } qw_switches;
+
 struct qw_batch {
     qw_gpu *g;
     int stream;
@@ -132,8 +135,11 @@ struct qw_batch {
     // a down projection over a few tokens that waits for the combine of the same layer: both in one launch
     // (qwk_dnc_*); launched as it is at any other dispatch or at submit
     struct { bool valid; qwk_dn_args a; const char *fname, *fused, *kname; unsigned grid, fused_grid; bool quarters; } pend_dn;
-    // measurement switches, read from the environment once when the batch begins
-    struct { unsigned dnc_nb, dnq_min; int side; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split, kq_own; } sw;
+    // a routed gate/up launch that waits for the down projection and the combine of the same layer: the three run as one
+    // launch (qwk_gud_*) when the down dispatch qualifies for the form by token shares; launched as it is otherwise
+    struct { bool valid; qwk_gu_args a; const char *fname, *kname; unsigned grid; } pend_gu;
+    bool uses_sync;    // some launch of this batch has its workgroups wait for one another: the error word is read back at the end
+    qw_switches sw; // the device's switches when the batch began (no_fuse also set for what must not wait for its workgroups)
 };
 
 #define QW_LD_MAX 16
@@ -178,6 +184,10 @@ struct qw_gpu {
     const char *na_err;
     struct qw_batch *na_batch; // its recorder, with fixed storage (made by qw_gpu_open)
     bool na_busy;
+    qw_switches sw;
+    uint32_t *sync;      // QW_SYNC_BYTES: synchronisation words of launches whose workgroups wait for one another (stream 0 only)
+    uint32_t *sync_host; // pinned: the error word of those launches, copied back when a batch is waited for
+    bool fuse_broken;    // such a launch gave up once: the layers stay separate launches from then on
     float *shgu;         // [2 streams][2][16][QW_SHGU_MAXI] gate and up results of a shared expert in the K-quant format family
     bool repack;         // make packed copies (QW_HIP_REPACK=0 in the environment or qw_hip_set_repack turn it off)
     size_t pack_bytes, released_bytes;
@@ -188,7 +198,7 @@ static void set_err(qw_gpu *g, const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g->err, sizeof g->err, fmt, ap);
     va_end(ap);
-    if (getenv("QW_HIP_VERBOSE")) fprintf(stderr, "[qw_hip] %s\n", g->err);
+    if (g->sw.verbose) fprintf(stderr, "[qw_hip] %s\n", g->err);
 }
 #define HIPOK(g, call) (hip_ok((g), (call), #call))
 static bool hip_ok(qw_gpu *g, hipError_t e, const char *what) {
@@ -201,6 +211,44 @@ double qw_now(void) {
     struct timespec ts;
     clock_gettime(CLOCK_MONOTONIC, &ts);
     return (double)ts.tv_sec + (double)ts.tv_nsec * 1e-9;
+}
+
+static void read_switches(qw_gpu *g) {
+    qw_switches *w = &g->sw;
+    const char *e = getenv("QW_HIP_DNC_NB"); // token count up to which down + combine run as one launch (0: never)
+    w->dnc_nb = e ? (unsigned)atoi(e) : 2;
+    if (w->dnc_nb > QW_DNC_MAXNB) w->dnc_nb = QW_DNC_MAXNB;
+    e = getenv("QW_HIP_DNQ_MIN"); // token count from which down + combine run as one launch of token shares (0: never)
+    w->dnq_min = e ? (unsigned)atoi(e) : QW_DNQ_MIN_DEFAULT;
+    e = getenv("QW_HIP_SIDE"); // the side stream for launches that depend on the step's input alone: 1 on
+    w->side = e && e[0] == '1';
+    w->dn_any = getenv("QW_HIP_DN_ANY") != NULL, w->nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
+    w->no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, w->shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
+    w->split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
+    w->pk_split = getenv("QW_HIP_PK_SPLIT") != NULL; // the packing sequence one launch per dispatch
+    w->kq_own = getenv("QW_HIP_KQ_OWN_LAUNCH") != NULL; // a K-quant / IQ4 / plain shared expert's gate/up as a launch of its own
+    e = getenv("QW_HIP_FUSE"); // 1: routed gate/up, down and combine of a layer as one launch (off unless asked for: measured as no gain)
+    w->no_fuse = !(e && e[0] == '1');
+    e = getenv("QW_HIP_SPIN_LIMIT"); // polls after which a workgroup of a fused launch stops waiting for the others
+    w->spin_limit = e ? (unsigned)strtoul(e, NULL, 10) : 1u << 16;
+    e = getenv("QW_HIP_LOAD_THREADS");
+    w->load_threads = e && atoi(e) > 0 ? (atoi(e) > QW_LD_MAX ? QW_LD_MAX : atoi(e)) : 4;
+    w->verbose = getenv("QW_HIP_VERBOSE") != NULL, w->quiet = getenv("QW_HIP_QUIET") != NULL;
+}
+bool qw_hip_sync_words(qw_gpu *g, uint32_t *dst, size_t nwords) {
+    if (nwords * 4 > QW_SYNC_ALLOC) return false;
+    return hipDeviceSynchronize() == hipSuccess && hipMemcpy(dst, g->sync, nwords * 4, hipMemcpyDeviceToHost) == hipSuccess;
+}
+void qw_hip_reload_switches(qw_gpu *g) {
+    read_switches(g);
+    g->fuse_broken = false; // fused launches are tried again
+}
+
+static hipFunction_t find_func(qw_gpu *g, const char *fname) {
+    hipFunction_t f;
+    if (hipModuleGetFunction(&f, g->mod, fname) == hipSuccess) return f;
+    (void)hipGetLastError();
+    return NULL;
 }
 
 // ---------------------------------------------------------------- device
@@ -227,8 +275,9 @@ qw_gpu *qw_gpu_open(void) {
     for (int i = 0; i < 2; i++)
         if (hipStreamCreateWithFlags(&g->stream[i], hipStreamNonBlocking) != hipSuccess) { free(g); return NULL; }
     g->kernels = calloc(QW_MAX_KERNELS, sizeof *g->kernels);
+    read_switches(g);
     {
-        const char *e = getenv("QW_HIP_REPACK");
+        const char *e = getenv("QW_HIP_REPACK"); // these two have setters of their own; the environment gives the start value
         g->repack = !(e && e[0] == '0');
         e = getenv("QW_HIP_GRAPH"); // off unless asked for: measured as no gain on this path (the steps are bound by the GPU)
         g->use_graphs = e && e[0] == '1';
@@ -239,7 +288,9 @@ qw_gpu *qw_gpu_open(void) {
         void *params[] = {&ta};
         if (hipMalloc(&g->tabs, QW_TAB_BYTES) != hipSuccess || hipMemset(g->tabs, 0, QW_TAB_BYTES) != hipSuccess ||
             hipMalloc((void **)&g->shgu, (size_t)2 * 2 * 16 * 4096 * 4) != hipSuccess ||
-            hipModuleGetFunction(&f, g->mod, "qwk_tab_init") != hipSuccess) { free(g->kernels); free(g); return NULL; }
+            hipMalloc((void **)&g->sync, QW_SYNC_ALLOC) != hipSuccess || hipMemset(g->sync, 0, QW_SYNC_ALLOC) != hipSuccess ||
+            hipHostMalloc((void **)&g->sync_host, 64, hipHostMallocDefault) != hipSuccess ||
+            !(f = find_func(g, "qwk_tab_init"))) { free(g->kernels); free(g); return NULL; }
         ta = (qwk_tab_args){.tab = g->tabs, .slot_order = 1};
         if (hipDeviceSynchronize() != hipSuccess || hipModuleLaunchKernel(f, 32, 1, 1, 256, 1, 1, 0, g->stream[0], params, NULL) != hipSuccess ||
             hipStreamSynchronize(g->stream[0]) != hipSuccess) {
@@ -251,6 +302,14 @@ qw_gpu *qw_gpu_open(void) {
     }
     // the entry point that allocates nothing: its scratch array's address on this device and its recorder, made now
     if (!qw_noalloc_scratch(g->dev, &g->na_scratch, &g->na_bytes, &g->na_err)) g->na_scratch = NULL;
+#ifdef QW_STAMPS // working builds: the kernels' time stamps go behind the synchronisation words
+    {
+        hipDeviceptr_t p;
+        size_t sz;
+        if (hipModuleGetGlobal(&p, &sz, g->mod, "qw_stamp_ptr") == hipSuccess) (void)hipMemcpy((void *)p, &g->sync, sizeof g->sync, hipMemcpyHostToDevice);
+        else (void)hipGetLastError();
+    }
+#endif
     g->na_batch = calloc(1, sizeof *g->na_batch);
     if (g->na_batch) {
         g->na_batch->capl = 64, g->na_batch->l = calloc(64, sizeof(qw_launch));
@@ -286,6 +345,8 @@ void qw_gpu_close(qw_gpu *g) {
         free(g->graphs[i].key);
     }
     (void)hipFree(g->shgu);
+    (void)hipFree(g->sync);
+    (void)hipHostFree(g->sync_host);
     if (g->na_batch) { free(g->na_batch->l); free(g->na_batch->use); free(g->na_batch); }
     (void)hipModuleUnload(g->mod);
     free(g->kernels);
@@ -302,8 +363,8 @@ static hipFunction_t get_func(qw_gpu *g, const char *fname) {
     for (int i = 0; i < g->nfuncs; i++)
         if (!strcmp(g->funcs[i].name, fname)) return g->funcs[i].f;
     if (g->nfuncs >= QW_MAX_FUNCS) return NULL;
-    hipFunction_t f;
-    if (!HIPOK(g, hipModuleGetFunction(&f, g->mod, fname))) return NULL;
+    hipFunction_t f = find_func(g, fname);
+    if (!f) { set_err(g, "no entry point %s in the code objects", fname); return NULL; }
     snprintf(g->funcs[g->nfuncs].name, sizeof g->funcs[0].name, "%s", fname);
     g->funcs[g->nfuncs].f = f;
     return g->funcs[g->nfuncs++].f;
@@ -678,8 +739,12 @@ bool qw_hip_buf_download(qw_buf *b, size_t off, size_t len) {
 bool qw_hip_buf_write(qw_buf *b, size_t off, const void *src, size_t len) {
     qw_hbuf *h = b ? b->handle : NULL;
     if (h && h->released) return false;
+    if (!h || !range_ok(h, off, len)) return false;
     packs_drop(h);
-    return h && range_ok(h, off, len) && hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
+    // A buffer with a host side keeps it in step: a later upload of the shadow (a new or marked buffer is sent whole at
+    // its next bind, a small one at every submit) then carries these bytes instead of wiping them out.
+    if (h->host && !h->wrapped) memcpy((char *)h->host + off, src, len);
+    return hipMemcpy((char *)h->dptr + off, src, len, hipMemcpyHostToDevice) == hipSuccess;
 }
 // File -> HBM through pinned staging. Chunk c of the range belongs to lane c % nth; a lane is two pinned buffers, a
 // stream (default priority) and two events, kept by the device handle from their first use: the pread() of a lane's
@@ -706,6 +771,7 @@ static void *fd_worker(void *arg) {
             if (r <= 0) ok = false; // an error, or the file ends inside the range
             else got += (size_t)r;
         }
+        if (ok && j->h->host && !j->h->wrapped) memcpy((char *)j->h->host + j->off + c, L->pin[slot], n); // the host side keeps in step (qw_hip_buf_write)
         ok = ok && hipMemcpyAsync((char *)j->h->dptr + j->off + c, L->pin[slot], n, hipMemcpyHostToDevice, L->st) == hipSuccess;
         ok = ok && hipEventRecord(L->ev[slot], L->st) == hipSuccess;
         used[slot] = true;
@@ -739,9 +805,7 @@ bool qw_hip_buf_write_fd(qw_buf *b, size_t off, int fd, uint64_t foff, size_t le
     if (!h || !range_ok(h, off, len) || fd < 0) return false;
     packs_drop(h);
     if (!len) return true;
-    int nth = 4;
-    const char *e = getenv("QW_HIP_LOAD_THREADS");
-    if (e && atoi(e) > 0) nth = atoi(e) > QW_LD_MAX ? QW_LD_MAX : atoi(e);
+    int nth = h->g->sw.load_threads;
     const size_t nchunk = (len + QW_FD_CHUNK - 1) / QW_FD_CHUNK;
     if ((size_t)nth > nchunk) nth = (int)nchunk;
     if (!ld_lanes(h->g, nth)) return false;
@@ -759,8 +823,7 @@ bool qw_hip_buf_write_fd(qw_buf *b, size_t off, int fd, uint64_t foff, size_t le
         ok = ok && job[i].ok;
     }
     if (!ok) set_err(h->g, "qw_hip_buf_write_fd: read or copy failed");
-    if (h->host && !h->wrapped) h->dirty = false; // HBM is now newer than the shadow; the shadow is not refreshed
-    return ok;
+    return ok; // (a host side got the same bytes; whether it still holds others that HBM lacks stays as it was)
 }
 bool qw_hip_buf_read(const qw_buf *b, size_t off, void *dst, size_t len) {
     const qw_hbuf *h = b ? b->handle : NULL;
@@ -777,18 +840,8 @@ qw_batch *qw_batch_begin(qw_gpu *g, bool concurrent) {
     b->stream = g->cur_stream;
     b->prof = g->prof;
     g->err[0] = 0;
-    const char *e = getenv("QW_HIP_DNC_NB"); // token count up to which down + combine run as one launch (0: never)
-    b->sw.dnc_nb = e ? (unsigned)atoi(e) : 2;
-    if (b->sw.dnc_nb > QW_DNC_MAXNB) b->sw.dnc_nb = QW_DNC_MAXNB;
-    e = getenv("QW_HIP_DNQ_MIN"); // token count from which down + combine run as one launch of token quarters (0: never)
-    b->sw.dnq_min = e ? (unsigned)atoi(e) : QW_DNQ_MIN_DEFAULT;
-    e = getenv("QW_HIP_SIDE"); // the side stream for launches that depend on the step's input alone: 1 on
-    b->sw.side = e && e[0] == '1';
-    b->sw.dn_any = getenv("QW_HIP_DN_ANY") != NULL, b->sw.nl_c4 = getenv("QW_HIP_NL_C4") != NULL;
-    b->sw.no_swiglu_matvec = getenv("QW_HIP_NO_SWIGLU_MATVEC") != NULL, b->sw.shared_in_gu = getenv("QW_HIP_SHARED_IN_GU") != NULL;
-    b->sw.split_select = getenv("QW_HIP_SPLIT_SELECT") != NULL;
-    b->sw.pk_split = getenv("QW_HIP_PK_SPLIT") != NULL; // the packing sequence one launch per dispatch
-    b->sw.kq_own = getenv("QW_HIP_KQ_OWN_LAUNCH") != NULL; // a K-quant / IQ4 / plain shared expert's gate/up as a launch of its own
+    b->sw = g->sw;
+    b->sw.no_fuse = g->sw.no_fuse || g->fuse_broken || b->stream != 0; // launches that wait for all their workgroups: one stream only
     return b;
 }
 
@@ -820,7 +873,7 @@ static bool fail(qw_batch *b, const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(b->g->err, sizeof b->g->err, fmt, ap);
     va_end(ap);
-    if (getenv("QW_HIP_VERBOSE")) fprintf(stderr, "[qw_hip] %s\n", b->g->err);
+    if (b->g->sw.verbose) fprintf(stderr, "[qw_hip] %s\n", b->g->err);
     b->failed = true;
     return false;
 }
@@ -1308,7 +1361,33 @@ static bool tr_gu(qw_batch *b) {
     // With few tiles (one or two tokens: 640 to 1280 of them) every compute unit still gets a workgroup: the waves are
     // numbered wave-major, so the tiles spread over all compute units instead of filling the waves of the first
     // workgroups (48-layer step at one token: gate/up launch 18.3 -> 13.4 us, 615 -> 715 tokens/s).
-    return add_launch(b, intern(fn), umin((unsigned)b->g->ncu, tasks), 64 * QW_WAVES_GU, &a, sizeof a);
+    const unsigned grid = umin((unsigned)b->g->ncu, tasks);
+    // Tile-major IQ3_S rows of the shape the fused launch is built for: wait for the down dispatch (qwk_gud_*)
+    if (!b->sw.no_fuse && b->sw.side != 1 && fgu == QW_F_PACKED && cg == 2 && !fs && p->D <= 2048 && p->I == 512 && p->topk <= 10 && p->gnb * p->topk <= (int)QW_DNQ_MAXU &&
+        b->buf[6].off % 4 == 0) {
+        b->pend_gu.valid = true;
+        b->pend_gu.a = a;
+        b->pend_gu.fname = intern(fn), b->pend_gu.kname = b->k->name, b->pend_gu.grid = grid;
+        return true;
+    }
+    return add_launch(b, intern(fn), grid, 64 * QW_WAVES_GU, &a, sizeof a);
+}
+
+// The gate/up launch that waited for a down dispatch to join it, on its own after all.
+static bool flush_gu(qw_batch *b) {
+    if (!b->pend_gu.valid) return true;
+    b->pend_gu.valid = false;
+    const int first = b->nl;
+    if (!add_launch(b, b->pend_gu.fname, b->pend_gu.grid, 64 * QW_WAVES_GU, &b->pend_gu.a, sizeof b->pend_gu.a)) return false;
+    if (b->nl > first) b->l[b->nl - 1].kname = b->pend_gu.kname, b->l[b->nl - 1].last_of_dispatch = true;
+    return true;
+}
+// Shares of the tokens and tiles per workgroup of the fused launch's down phase: at most QW_GUD_SHARE tokens a share.
+static void gud_shape(unsigned nbr, unsigned *nq, unsigned *tpw) {
+    unsigned q = 1;
+    while (q < 8 && (nbr == 1 ? q < 1 : cdiv(nbr, q) > QW_GUD_SHARE || q < 2)) q *= 2;
+    *nq = q;
+    *tpw = q > 2 ? q / 2 : 1;
 }
 
 static bool flush_dn(qw_batch *b) {
@@ -1327,7 +1406,28 @@ static unsigned dnq_quarters(unsigned nbr) { return nbr <= 8 ? 2 : 4; }
 
 // src/engine.c:633-639: 0 Wd, 2 H, 3 sel, 7 tables, 9 Pg. The token count is not bound: the masks carry it.
 // The shared down tiles (remembered from moe_gu_gg) run in the same launch.
+static bool tr_dn_inner(qw_batch *b);
 static bool tr_dn(qw_batch *b) {
+    const int first = b->nl;
+    if (!tr_dn_inner(b)) return false;
+    if (!b->pend_gu.valid) return true;
+    // a gate/up launch waits: it stays only if this dispatch became a down + combine by token shares over its H and record
+    const qwk_gu_args *gu = &b->pend_gu.a;
+    const qwk_dn_args *d = &b->pend_dn.a;
+    if (b->pend_dn.valid && b->pend_dn.quarters && b->nl == first && d->H == gu->H && d->sel == gu->sel && d->D == gu->D && d->I == gu->I && d->topk == gu->topk && d->gnb == gu->gnb &&
+        d->hplane == gu->hplane) return true;
+    // otherwise it goes in front of what this dispatch launched
+    const int n = b->nl - first;
+    if (!flush_gu(b)) return false;
+    if (n > 0 && b->nl == first + n + 1) {
+        const qw_launch gl = b->l[b->nl - 1];
+        memmove(&b->l[first + 1], &b->l[first], sizeof(qw_launch) * (size_t)n);
+        b->l[first] = gl;
+        b->l[first].last_of_dispatch = true;
+    }
+    return true;
+}
+static bool tr_dn_inner(qw_batch *b) {
     const qw_kparams *p = &b->k->p;
     const uint32_t nbr = (uint32_t)p->NB;
     const size_t rb = fmt_rb(p->fd, p->I);
@@ -1405,7 +1505,8 @@ static bool tr_dn(qw_batch *b) {
         // Down + combine as one launch in which a workgroup owns one or two tiles of output rows and a share of the
         // tokens (qwk_dnq_*): for tile-major IQ3_S rows when a share's H rows fit in LDS beside the table.
         const unsigned tpe = (unsigned)p->D / 16, nq = dnq_quarters(nbr), tpw = nq > 2 ? 2 : 1;
-        const bool by_shares = b->sw.dnq_min && nbr >= b->sw.dnq_min && nbr <= 16 && fd == QW_F_PACKED && (fs == 0 || fs == 8 || fs == QW_F_PACKED) && p->topk <= 10 &&
+        // (a gate/up launch that waits to be joined asks for this form at any token count)
+        const bool by_shares = (b->pend_gu.valid || (b->sw.dnq_min && nbr >= b->sw.dnq_min)) && nbr <= 16 && fd == QW_F_PACKED && (fs == 0 || fs == 8 || fs == QW_F_PACKED) && p->topk <= 10 &&
                                p->gnb * p->topk <= (int)QW_DNQ_MAXU && tpe % 16 == 0;
         // a few tokens: wait for the combine, the two run as one launch (tile-major IQ3_S or Q8_0 routed rows; a shared
         // expert in either of these)
@@ -1453,14 +1554,30 @@ static bool tr_cmb(qw_batch *b) {
             d->nbr = nbr;
             d->out = a.out;
             d->Psh = (float *)a.Psh;
+            if (b->pend_gu.valid && b->pend_dn.quarters && b->pend_gu.a.nbr == nbr && (!d->Wsd || d->snbr == nbr)) { // gate/up, down and combine as one launch
+                unsigned nq, tpw;
+                gud_shape(nbr, &nq, &tpw);
+                const unsigned grid = (unsigned)b->g->ncu, tpe = a.D / 16;
+                if (tpe % (8 * tpw) == 0 && tpe / tpw * nq <= grid && grid % 8 == 0) {
+                    b->pend_gu.valid = false;
+                    qwk_gud_args f = {.gu = b->pend_gu.a, .dn = *d, .sync = b->g->sync, .spin_limit = b->sw.spin_limit};
+                    f.dn.nq = nq, f.dn.tpw = tpw;
+                    char fu[48];
+                    fname_fmt(fu, sizeof fu, "qwk_gud%s", b->pend_dn.fused + 7); // the same formats as the qwk_dnq_* launch
+                    b->uses_sync = true;
+                    return add_launch(b, intern(fu), grid, 64 * QW_WAVES_GU, &f, sizeof f);
+                }
+            }
+            if (!flush_gu(b)) return false;
             if (b->pend_dn.quarters) { // the quarters and the tiles per workgroup follow the bound token count, not the compiled one
                 d->nq = dnq_quarters(nbr), d->tpw = d->nq > 2 ? 2 : 1;
                 b->pend_dn.fused_grid = a.D / 16 / d->tpw * d->nq;
             }
             return add_launch(b, b->pend_dn.fused, b->pend_dn.fused_grid, 64 * QW_WAVES_DNR, d, sizeof *d);
         }
-        if (!flush_dn(b)) return false;
+        if (!flush_gu(b) || !flush_dn(b)) return false;
     }
+    if (!flush_gu(b)) return false;
     return add_launch(b, "qwk_cmb", cdiv(nbr * (unsigned)p->D, 256), 256, &a, sizeof a);
 }
 
@@ -1762,7 +1879,8 @@ void qw_batch_dispatch(qw_batch *b, unsigned gx, unsigned gy, unsigned gz, unsig
     if (b->k->fam != FAM_GU && b->k->fam != FAM_PRE && !flush_select(b)) return;
     if (b->k->fam != FAM_PK_ACT2 && !flush_tw(b, NULL, NULL)) return;
     if (b->k->fam != FAM_PF && !flush_pf(b)) return;
-    if (b->k->fam != FAM_CMB && !flush_dn(b)) return;
+    // a gate/up launch waits for the down dispatch of its layer, a down launch for the combine; anything else sends them off
+    if (b->k->fam != FAM_CMB && (b->k->fam != FAM_DN || b->pend_dn.valid) && (!flush_gu(b) || !flush_dn(b))) return;
     if (b->k->fam != FAM_PK_ZERO && b->k->fam != FAM_PK_COUNT && b->k->fam != FAM_PK_PLAN && b->k->fam != FAM_PK_PLAN_T && b->k->fam != FAM_PK_SCATTER && !flush_pk(b)) return;
     switch (b->k->fam) {
     case FAM_DQ_TEST: ok = tr_dq_test(b, gx); break;
@@ -1873,7 +1991,7 @@ static int graph_run(qw_batch *b, hipStream_t st) {
 static bool submit_segment(qw_batch *b) {
     qw_gpu *g = b->g;
     hipStream_t st = g->stream[b->stream];
-    if (b->failed || !flush_select(b) || !flush_tw(b, NULL, NULL) || !flush_pf(b) || !flush_dn(b) || !flush_pk(b)) return false;
+    if (b->failed || !flush_select(b) || !flush_tw(b, NULL, NULL) || !flush_pf(b) || !flush_gu(b) || !flush_dn(b) || !flush_pk(b)) return false;
     if (b->nseg >= 9) return fail(b, "too many flushes in one batch");
     // host -> device for what this segment binds
     const unsigned mark = ++g->mark;
@@ -1975,7 +2093,7 @@ double qw_batch_wait(qw_batch *b) {
     if (b->failed) {
         (void)hipStreamSynchronize(st);
         if (!g->err[0]) set_err(g, "batch failed");
-        if (!getenv("QW_HIP_QUIET")) fprintf(stderr, "qw_batch: %s\n", g->err);
+        if (!g->sw.quiet) fprintf(stderr, "qw_batch: %s\n", g->err);
         batch_free(b);
         return -1;
     }
@@ -1989,7 +2107,14 @@ double qw_batch_wait(qw_batch *b) {
         if (h->device_only || !h->host || h->wrapped || h->size > QW_HIP_BIG_OUT_BYTES) continue;
         ok = HIPOK(g, hipMemcpyAsync(h->host, h->dptr, h->size, hipMemcpyDeviceToHost, st));
     }
+    if (ok && b->uses_sync) ok = HIPOK(g, hipMemcpyAsync(g->sync_host, g->sync + QW_SYNC_ERR_WORD, 4, hipMemcpyDeviceToHost, st));
     ok = ok && HIPOK(g, hipStreamSynchronize(st));
+    if (ok && b->uses_sync && g->sync_host[0]) { // a launch whose workgroups wait for one another gave up: its results are not valid
+        (void)hipMemset(g->sync, 0, QW_SYNC_BYTES);
+        g->fuse_broken = true;
+        set_err(g, "a fused layer launch timed out waiting for its workgroups (are other kernels running on this device?); layers run as separate launches from now on");
+        ok = false;
+    }
     if (ok) {
         secs = 0;
         for (int s = 0; s < b->nseg; s++) {
@@ -2009,7 +2134,7 @@ double qw_batch_wait(qw_batch *b) {
         }
     }
     if (!ok) {
-        if (!getenv("QW_HIP_QUIET")) fprintf(stderr, "qw_batch: %s\n", g->err);
+        if (!g->sw.quiet) fprintf(stderr, "qw_batch: %s\n", g->err);
         secs = -1;
     }
     batch_free(b);
@@ -2048,15 +2173,16 @@ qw_batch *qw_hip_batch_begin_static(qw_gpu *g, void *stream) {
     memset(b, 0, sizeof *b);
     *b = (qw_batch){.g = g, .seq = ++g->batch_seq, .stream = g->cur_stream, .noalloc = true, .xstream = (hipStream_t)stream, .l = l, .capl = 64, .use = use, .capuse = 1024};
     b->sw.dnq_min = QW_DNQ_MIN_DEFAULT;
-    b->sw.dnc_nb = 2; // the defaults of qw_batch_begin; the measurement switches of the environment do not apply here
+    b->sw.dnc_nb = 2; // the defaults; the measurement switches of the environment do not apply here
+    b->sw.no_fuse = true; // the caller's stream may run beside other work of this device: no launch that waits for all of its workgroups
     g->na_busy = true;
     g->err[0] = 0;
     return b;
 }
-bool qw_hip_batch_launch_static(qw_batch *b) {
+bool qw_hip_batch_launch_static(qw_batch *b, bool recorded) {
     qw_gpu *g = b->g;
     hipStream_t st = b->xstream ? b->xstream : g->stream[b->stream];
-    bool ok = !b->failed && flush_select(b) && flush_tw(b, NULL, NULL) && flush_pf(b) && flush_dn(b) && flush_pk(b) && !b->failed;
+    bool ok = recorded && !b->failed && flush_select(b) && flush_tw(b, NULL, NULL) && flush_pf(b) && flush_gu(b) && flush_dn(b) && flush_pk(b) && !b->failed;
     for (int i = 0; ok && i < b->nl; i++) {
         qw_launch *l = &b->l[i];
         void *params[] = {l->args};

@@ -178,6 +178,64 @@ __device__ __forceinline__ h8 qw_q8_cvt(u2 q) {
 __device__ __forceinline__ void qw_store_u16(uint16_t *p, uint16_t v) { asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"((uint32_t)v) : "memory"); }
 __device__ __forceinline__ void qw_store_f32(float *p, float v) { asm volatile("global_store_dword %0, %1, off" : : "v"(p), "v"(v) : "memory"); }
 
+// ---------------------------------------------------------------- data handed between workgroups of one launch
+// The eight XCDs of the device have an L2 each, coherent with one another only at the boundaries of a kernel. What one
+// workgroup writes and another reads inside one launch therefore goes around those caches: stores and loads of device
+// ("agent") scope (cache policy sc1), which the hardware carries out at the memory side. No fences: a release fence
+// writes back a whole L2 and an acquire fence drops one (tens of microseconds per hand-over). A store of device scope
+// that its wave has waited for (s_waitcnt) is visible to every load of device scope issued after it.
+__device__ __forceinline__ void qw_st_coh(uint32_t *p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ uint32_t qw_ld_coh(const uint32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// Seven 16-byte loads of device scope, issued together and awaited (every outstanding memory operation of the wave is):
+// one statement, so that the compiler never touches a destination register before the wait.
+__device__ __forceinline__ void qw_ld_coh7(u4 (&v)[7], const u4 *const (&p)[7]) {
+    asm volatile("global_load_dwordx4 %0, %7, off sc1\n\t"
+                 "global_load_dwordx4 %1, %8, off sc1\n\t"
+                 "global_load_dwordx4 %2, %9, off sc1\n\t"
+                 "global_load_dwordx4 %3, %10, off sc1\n\t"
+                 "global_load_dwordx4 %4, %11, off sc1\n\t"
+                 "global_load_dwordx4 %5, %12, off sc1\n\t"
+                 "global_load_dwordx4 %6, %13, off sc1\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6])
+                 : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6])
+                 : "memory");
+}
+
+// Synchronisation words of a launch whose workgroups wait for one another (QW_SYNC_BYTES of device memory owned by
+// the backend, zero between launches except the generation). Such a launch has at most one workgroup per compute unit,
+// so all of them are resident at once and a wait ends as soon as the others arrive; every wait is bounded all the same
+// (limit = number of polls): a workgroup that gives up sets the error word, everybody winds down without waiting
+// again, and the host fails the batch.
+//   word 0: generation, raised by one by the workgroup that completes a barrier     word 32: arrivals at the top level
+//   word 64 + 32 g: arrivals of group g (workgroup index & 7: one XCD)              word 352: error
+enum { QW_SYNC_GEN = 0, QW_SYNC_TOP = 32, QW_SYNC_GROUP = 64, QW_SYNC_ERR = QW_SYNC_ERR_WORD };
+__device__ __forceinline__ uint32_t qw_sync_add(uint32_t *p) { return __hip_atomic_fetch_add(p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// One thread per workgroup calls this, after a __syncthreads() behind which every thread of the workgroup has waited
+// for its own stores. gen0: the generation read when the launch began (no barrier can complete before every workgroup
+// has read it); k: number of this barrier in the launch, from 1; G: workgroups of the launch. The last to arrive clears
+// the counters for the next use and only then raises the generation. False: the wait gave up.
+__device__ __forceinline__ bool qw_grid_barrier(uint32_t *sync, uint32_t gen0, uint32_t k, uint32_t G, uint32_t limit) {
+    const uint32_t g = blockIdx.x & 7, per = (G + 7 - g) >> 3, groups = G < 8 ? G : 8;
+    if (qw_sync_add(sync + QW_SYNC_GROUP + 32 * g) + 1 == per) {
+        qw_st_coh(sync + QW_SYNC_GROUP + 32 * g, 0);
+        __builtin_amdgcn_s_waitcnt(0); // cleared before anybody can be released into a later barrier
+        if (qw_sync_add(sync + QW_SYNC_TOP) + 1 == groups) {
+            qw_st_coh(sync + QW_SYNC_TOP, 0);
+            __builtin_amdgcn_s_waitcnt(0);
+            qw_st_coh(sync + QW_SYNC_GEN, gen0 + k);
+        }
+    }
+    for (uint32_t spins = 0; qw_ld_coh(sync + QW_SYNC_GEN) - gen0 < k; spins++) {
+        if (spins >= limit || ((spins & 63) == 63 && qw_ld_coh(sync + QW_SYNC_ERR))) {
+            qw_st_coh(sync + QW_SYNC_ERR, 1);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------- activation fragment providers (operand A)
 // Fragment order in LDS: chunk c (8 consecutive k-values) of token m lives at xf[c * 16 + m], 16 bytes, so that the
 // 16 lanes of a k-group read 256 contiguous bytes. Tokens >= nb are stored as zeros.

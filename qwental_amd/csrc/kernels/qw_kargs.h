@@ -118,6 +118,26 @@ typedef struct {
 #define QW_DNQ_MAXU 160u
 #define QW_DNC_MAXNB 4
 
+/* Synchronisation words of launches whose workgroups wait for one another (layout: QW_SYNC_* in qw_common.hip.h). */
+#define QW_SYNC_BYTES 1536u
+#define QW_SYNC_ALLOC 32768u /* what the backend allocates: the words above, the rest for working builds that leave time stamps */
+#define QW_SYNC_ERR_WORD 352u
+/* Routed gate/up, down and combine of a layer as one launch (qwk_gud_*: tile-major IQ3_S routed rows, D <= 2048 a
+ * multiple of 512, I = 512, topk <= 10, 1 to 16 tokens): the argument records of the launches it stands for. The grid
+ * is one workgroup per compute unit; all of them stream gate/up tiles, leave their SwiGLU values in H through stores
+ * of device scope, meet at one barrier over the grid, and then run the down projection and the combine as qwk_dnq_*
+ * does, with shares of at most QW_GUD_SHARE tokens: dn.nq shares, dn.tpw tiles of 16 output rows per workgroup,
+ * D / 16 / dn.tpw * dn.nq <= grid workgroups take part in that phase. */
+#define QW_GUD_SHARE 3u
+#define QW_GUD_ROWS 33u /* staged H rows per workgroup: QW_GUD_SHARE tokens x (topk + 1) */
+#define QW_GUD_HCAP 192u /* (tile, token) results of the gate/up phase a workgroup keeps in LDS; more go to memory directly */
+typedef struct {
+    qwk_gu_args gu;
+    qwk_dn_args dn;
+    uint32_t *sync;
+    uint32_t spin_limit, pad; /* polls of the generation word after which a waiting workgroup gives up */
+} qwk_gud_args;
+
 /* front part of a layer: router rows on the first nrouter workgroups; when g.Wsg != NULL the shared expert's gate/up
  * on the workgroups after them (g: its arguments, shared = 1), one chunk of a tile per wave, summed through LDS. */
 typedef struct {

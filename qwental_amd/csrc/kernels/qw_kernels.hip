@@ -8,6 +8,22 @@
 #include "qw_common.hip.h"
 #include "qw_kquants.hip.h"
 
+// The entry points come in groups, QW_IN_PART(k) around each: a build with -DQW_PARTS=<bit mask> holds only the groups
+// whose bit is set (experiments that need a few kernels and a short compile); the product build holds all of them, in
+// one code object (the same kernels spread over several code objects measured 3 % slower on the 48-layer step).
+#ifdef QW_PARTS
+#define QW_IN_PART(k) ((QW_PARTS >> (k)) & 1)
+#else
+#define QW_IN_PART(k) 1
+#endif
+#ifdef QW_STAMPS // working builds only: time stamps (10 ns units) of thread 0 of every workgroup, 16 words a workgroup, where the host points this
+extern "C" __device__ uint32_t *qw_stamp_ptr;
+__device__ uint32_t *qw_stamp_ptr;
+#define QW_DSTAMP(k) do { if (threadIdx.x == 0 && qw_stamp_ptr) qw_stamp_ptr[512 + 16 * blockIdx.x + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define QW_DSTAMP(k) do {} while (0)
+#endif
+
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
 #define QW_WG_DN 768       // down range kernels: 12 waves
 #define QW_WG_GU 768       // gate/up and dense matvec: 12 waves, three per SIMD (a wave issues at most one instruction in ~6 cycles)
@@ -44,6 +60,7 @@ template <int F> __device__ __forceinline__ void dq_test_body(const qwk_dq_args 
     }
 }
 
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f21(qwk_dq_args a) {
     __shared__ u2 lut[QW_LUT_ENTRIES];
     qw_lut_build(lut);
@@ -51,6 +68,7 @@ extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f21(qwk_dq_args a) 
     dq_test_body<21>(a, lut);
 }
 extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_f8(qwk_dq_args a) { dq_test_body<8>(a, nullptr); }
+#endif
 
 // The formats of qw_kquants.hip.h: every lane decodes the slice of a block it would supply to the matrix instruction
 // and writes the values as the reference computes them (scale * integer - min in float). Grid: rows x 64.
@@ -64,6 +82,7 @@ template <int F> __device__ __forceinline__ void dq_test_kq(const qwk_dq_args &a
         qw_kq_values<F>(b, tab, kg, y + (size_t)qw_kq<F>::BLK_K * blk);
     }
 }
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_kq(qwk_dq_args a) {
     __shared__ uint32_t tab[QW_KQ_TAB];
     qw_kq_tab_build(tab);
@@ -78,16 +97,20 @@ extern "C" __global__ __launch_bounds__(64) void qwk_dq_test_kq(qwk_dq_args a) {
     case 30: dq_test_kq<30>(a, tab); break;
     }
 }
+#endif
 
 // ================================================================ lookup-table buffer (kernels/moe_gg.metal:495-515)
 // Only the IQ3_S section is produced; the sections of formats without a gfx950 build stay zero. Grid: 32 x 256.
+#if QW_IN_PART(0)
 extern "C" __global__ void qwk_tab_init(qwk_tab_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < QW_LUT_ENTRIES) ((u2 *)(a.tab + QW_TAB_IQ3SS))[a.slot_order ? qw_lut_slot(i) : i] = qw_lut_entry(i);
 }
+#endif
 
 // ================================================================ packing of IQ3_S rows (layout: qwk_pack_args)
 // One thread per (slab, lane), grid-stride over the slabs; run once per weight matrix, at its first use.
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) {
     const uint64_t nslab = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
     const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
@@ -103,9 +126,11 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_iq3(qwk_pack_args a) 
         *(uint32_t *)(dst + 1536 + 4 * lane) = qh | sc << 16 | db << 24;
     }
 }
+#endif
 
 // The tile-major copy of Q6_K rows (layout: QW_F_PACKED_Q6 in qw_kargs.h); a wave per (tile, block). The twelve dwords a
 // lane takes are the ones qw_kq<14>::load reads for that lane's row and k-group.
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(256) void qwk_pack_q6(qwk_pack_args a) {
     const uint64_t nslab = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
     const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
@@ -124,8 +149,10 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_q6(qwk_pack_args a) {
         if (kg == 0) *(uint16_t *)(dst + 3328 + 2 * n) = *(const uint16_t *)(src + 208);
     }
 }
+#endif
 
 // The tile-major copy of IQ4_NL rows (layout: QW_F_PACKED_NL in qw_kargs.h); a wave per (tile, chunk of ten blocks).
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(256) void qwk_pack_nl(qwk_pack_args a) {
     const uint64_t nchunk = a.ntiles * a.nblk, step = (uint64_t)gridDim.x * (blockDim.x >> 6);
     const uint32_t lane = threadIdx.x & 63, n = lane & 15, kg = lane >> 4;
@@ -144,6 +171,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_pack_nl(qwk_pack_args a) {
             for (int b = 0; b < 10; b++) *(uint16_t *)(dst + 2560 + 20 * n + 2 * b) = *(const uint16_t *)(src + 18 * b);
     }
 }
+#endif
 
 // ================================================================ dense matvec (kernels/qmv_gg.metal:17-39)
 // y[b][row] = sum_k W[row][k] x[b][k] for up to 16 activations; the weights are streamed once for all of them.
@@ -219,8 +247,10 @@ template <int F, int CH, bool XLDS> __device__ __forceinline__ void qmv_body(con
         __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[XLDS ? QW_XF_MAXK * 2 : 1]; f4 red[QW_WG_GU]; } L; /* table first: LDS address 0 */ \
         qmv_body<F, CH, XLDS>(a, L.lut, L.xf, L.red);                                                   \
     }
+#if QW_IN_PART(0)
 QW_QMV(21, 2, true, _c2) QW_QMV(21, 1, true, _c1) QW_QMV(21, 1, false, _c1g)
 QW_QMV(121, 2, true, _c2) QW_QMV(121, 1, true, _c1) // packed IQ3_S: a.rowbytes = bytes of a 16-row tile
+#endif
 
 // ---- the other formats, one to four matrices a launch (kernels/qmv_ggm.metal:232-262).
 // split == 1: the 16-row tiles of all matrices form one list dealt round-robin to the waves of a persistent grid; a
@@ -363,11 +393,14 @@ __device__ __forceinline__ void qmvm_swiglu_body(const qwk_qmvm_args &a, qw_qmvm
         __syncthreads();
     }
 }
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm_swiglu(qwk_qmvm_args a) {
     __shared__ qw_qmvm_lds L;
     qmvm_swiglu_body(a, L, blockIdx.x, gridDim.x);
 }
+#endif
 
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args a) {
     __shared__ struct { u4 xf[QW_KQ_MAXK * 2]; float xs[QW_KQ_MAXK / 2]; uint32_t tab[QW_KQ_TAB]; f4 red[QW_WG_QMVM]; } L;
     qw_kq_tab_build(L.tab);
@@ -421,6 +454,7 @@ extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_qmvm(qwk_qmvm_args 
         toff += a.ntiles[j];
     }
 }
+#endif
 
 // The VALU GEMV the matrix-core kernels are measured against (1, 2 or 4 activations, K a multiple of 512 up to 2560,
 // packed IQ3_S): the same streaming and decoding, v_dot2_f32_f16 instead of the matrix instruction, and a sum over
@@ -460,8 +494,10 @@ template <int NT> __device__ __forceinline__ void qmv_valu_body(const qwk_qmv_ar
         __shared__ struct { u2 lut[QW_LUT_ENTRIES]; u4 xf[QW_XF_MAXK * 2]; } L;                          \
         qmv_valu_body<NT>(a, L.lut, L.xf);                                                               \
     }
+#if QW_IN_PART(0)
 QW_QMV_VALU(1) QW_QMV_VALU(2) QW_QMV_VALU(4)
 QW_QMV(8, 16, true, _c16) QW_QMV(8, 1, true, _c1) QW_QMV(8, 1, false, _c1g)
+#endif
 
 // ================================================================ router (kernels/moe_gg.metal:25-41)
 // logits[t][r] = Wr[r] . x[t] in binary32, one wave per row; a token's sum order does not depend on nb: explicit
@@ -541,8 +577,10 @@ template <int WF> __device__ __forceinline__ void router_rows(const qwk_router_a
     else if (a.nb <= 8) router_row<WF, 8>(a, r, lane);
     else router_row<WF, 16>(a, r, lane);
 }
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(256) void qwk_router_w1(qwk_router_args a) { router_rows<1>(a, blockIdx.x * 4 + qw_wave(), qw_lane()); }
 extern "C" __global__ __launch_bounds__(256) void qwk_router_w30(qwk_router_args a) { router_rows<30>(a, blockIdx.x * 4 + qw_wave(), qw_lane()); }
+#endif
 
 // ================================================================ selection + dedupe (kernels/moe_gg.metal:123-189)
 // Per token (one wave): top-k by repeated maximum with ties to the lowest expert index, softmax over the picked logits
@@ -632,6 +670,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
 #pragma unroll
         for (int j = 0; j < PER; j++) k[t][j] = __builtin_bit_cast(uint32_t, logits[(size_t)tok[t] * (E + 1) + lane * PER + j]);
     issued();
+    QW_DSTAMP(13);
 #pragma unroll
     for (int t = 0; t < T; t++) {
         M[t] = 0;
@@ -677,6 +716,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
         for (int j = 0; j < PER; j++)
             if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], lane * PER + j};
     }
+    QW_DSTAMP(14);
     uint32_t mk[T], me[T], rank[T];
 #pragma unroll
     for (int t = 0; t < T; t++) {
@@ -749,8 +789,10 @@ __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 ||
 
 // The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
 // floats per wave (288 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
+// store: this workgroup writes the record; need_w: it wants the gating weights in s.w (store implies it).
 template <class H>
-__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued) {
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued, bool need_w = false) {
+    need_w = need_w || store;
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
@@ -772,11 +814,11 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
             const uint32_t t1[1] = {tk[0]};
             uint32_t fail;
             switch (E) {
-            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
-            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
-            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
-            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, store, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
-            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, store, issued); break;
+            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
+            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
+            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
+            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
+            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
             }
             for (uint32_t i = 0; i < 2; i++) { // more than 64 keys tie at the bound: the repeated maximum instead
                 if (!((fail >> i) & 1) || (i == 1 && !two)) continue;
@@ -793,6 +835,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
     issued(); // the waves without a token
+    QW_DSTAMP(15);
     __syncthreads();
     if (a.nbr == 1) { // one token: its picks are the unique experts, in rank order (what the steps below would leave)
         if (tid < K) c.ue[tid] = s.ids[tid], c.mask[tid] = 1, c.slot[tid * gnb] = (uint8_t)tid;
@@ -847,12 +890,14 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     __syncthreads(); // the caller may reuse the scratch
 }
 
+#if QW_IN_PART(0)
 extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a) {
     __shared__ qw_sel_scratch s;
     __shared__ qw_sel_cache c;
     __shared__ float lgs[16 * 1024];
     select_all(a, s, c, lgs, true, [] {});
 }
+#endif
 
 // ================================================================ gate/up + SwiGLU (kernels/moe_gg.metal:428-447, 563-573, 600-631)
 // A tile holds gate rows j0..j0+7 (n < 8) and up rows j0..j0+7 (n >= 8) of one expert; the up results move over by
@@ -866,8 +911,21 @@ __device__ __forceinline__ void qw_sel_load(qw_sel_cache &c, const uint8_t *sel,
     if (threadIdx.x == 0) c.U = *(const uint32_t *)sel;
 }
 
-template <int F, int CH, class S>
-__device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw, S ready) {
+// Where the SwiGLU values of a tile go. The plain form: the two planes of H in global memory, for a later launch.
+struct qw_h_global {
+    uint16_t *H;
+    uint32_t hplane;
+    // a tile is done: m = the tokens that picked its expert (wave-uniform)
+    __device__ __forceinline__ void tile(uint32_t) const {}
+    __device__ __forceinline__ void stamp(uint32_t k) const { QW_DSTAMP(k); }
+    // column j0 + n of (token, slot): o = its offset in a plane
+    __device__ __forceinline__ void put(uint32_t, uint32_t, size_t o, uint16_t hi, uint16_t lo) const {
+        qw_store_u16(H + o, hi);
+        qw_store_u16(H + o + hplane, lo);
+    }
+};
+template <int F, int CH, class S, class HS>
+__device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw, S ready, HS &hs) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
     const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
@@ -884,18 +942,18 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
         c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
-        const uint32_t m = a.shared ? qw_all_tokens(a.nbr) : sc->mask[u];
+        const uint32_t m = (a.shared ? 0xffffffffu : sc->mask[u]) & qw_all_tokens(a.nbr);
+        hs.tile(m);
 #pragma unroll
         for (uint32_t j = 0; j < 4; j++) {
             const float up = __shfl_xor(acc[j], 8), g = acc[j];
             const uint32_t tok = 4 * kg + j;
-            if (n < 8 && tok < a.nbr && ((m >> tok) & 1)) {
+            if (n < 8 && ((m >> tok) & 1)) {
                 const uint32_t s = a.shared ? K : sc->slot[u * gnb + tok];
                 const float h = g / (1.0f + __expf(-g)) * up;
                 const _Float16 hi = (_Float16)h, lo = (_Float16)(h - (float)hi);
                 const size_t o = ((size_t)tok * (K + 1) + s) * a.I + j0 + n;
-                qw_store_u16(a.H + o, __builtin_bit_cast(uint16_t, hi));
-                qw_store_u16(a.H + o + a.hplane, __builtin_bit_cast(uint16_t, lo));
+                hs.put(m, tok, o, __builtin_bit_cast(uint16_t, hi), __builtin_bit_cast(uint16_t, lo));
             }
         }
         acc = f4{0, 0, 0, 0};
@@ -907,14 +965,18 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 // addresses depend on it); then every wave issues its first weight loads, and only then the table copy, the activation
 // staging and the second barrier follow, overlapping that first round trip to HBM. When the selection is made here,
 // the table and the activations are fetched under it instead (direct global-to-LDS loads: no registers are held).
-template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss) {
+// hs: where the SwiGLU values go (qw_h_global, or the fused launch's LDS buffer). all_w: every workgroup wants the gating
+// weights in ss->w, not only the one that writes the record. selected(): called by every thread once the selection
+// cache *sc (and ss->w) is complete and published, before any tile is taken; ss may be reused after a barrier of its own.
+template <int FGU, int CHGU, int FSG, int CHSG, class HS, class SEL>
+__device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss, HS &hs, bool all_w, SEL selected) {
     bool staged = false, tabled = false;
+    QW_DSTAMP(0);
     if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
         if (qw_select_fast_e(a.E)) {
-            // Neither the table nor the activations depend on the selection: their direct-to-LDS loads are issued right
-            // behind those of the logits and land while the selection is made. The selection's scratch lies behind
-            // the staged activations when D leaves room there (D <= 2048), else in their place (they follow in ready()).
+            // The selection's scratch lies behind the staged activations when D leaves room there (D <= 2048), else in
+            // their place (they follow in ready()).
             constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
             const bool early = a.D * 2 + (QW_WG_GU / 64) * 288 / 4 <= QW_XF_MAXK * 2;
             bool fetched = false;
@@ -923,19 +985,30 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
                 fetched = true;
                 if (lutp) qw_lut_copy_issue(lut, (const u2 *)a.glut);
                 if (early) qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
-            });
+            }, all_w);
             qw_lds_arrive();
             __syncthreads();
-            tabled = true;
+            hs.stamp(10);
             staged = early;
+            tabled = true;
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
             qw_sel_scratch &so = *(qw_sel_scratch *)xf;
-            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [] {});
+            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [] {}, all_w);
+            if (all_w) { // (the caller reads the weights from ss)
+                for (uint32_t i = threadIdx.x; i < a.gnb * (a.topk + 1); i += blockDim.x) ss->w[i] = so.w[i];
+                __syncthreads();
+            }
         }
     } else {
         if (!a.shared) qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+        if (all_w) {
+            const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(a.gnb, a.topk));
+            for (uint32_t i = threadIdx.x; i < a.gnb * (a.topk + 1); i += blockDim.x) ss->w[i] = wg[i];
+        }
         __syncthreads();
     }
+    selected();
+    QW_DSTAMP(1);
     auto ready = [&] {
         if (staged) return;
         staged = true;
@@ -954,27 +1027,33 @@ template <int FGU, int CHGU, int FSG, int CHSG> __device__ __forceinline__ void 
             sa.Wu = a.Wsu;
             sa.rowbytes = a.sg_rowbytes;
             sa.shared = 1;
-            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready);
+            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready, hs);
         }
     }
     // the waves that did a shared tile come last in the routed deal, so that the work stays level
-    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready);
+    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready, hs);
+    QW_DSTAMP(2);
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
         __shared__ struct { u2 lut[(qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; qw_sel_scratch ss; } L; \
-        gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc, &L.ss);                                             \
+        qw_h_global hs = {a.H, a.hplane};                                                                      \
+        gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc, &L.ss, hs, false, [] {});                           \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
+#if QW_IN_PART(1)
 QW_GU(21, 2, 0, 1, qwk_gu_f21_c2) QW_GU(21, 1, 0, 1, qwk_gu_f21_c1)
 QW_GU(8, 16, 0, 1, qwk_gu_f8_c16) QW_GU(8, 1, 0, 1, qwk_gu_f8_c1)
 QW_GU(21, 2, 21, 2, qwk_gu_f21_c2_s21_c2) QW_GU(21, 2, 8, 16, qwk_gu_f21_c2_s8_c16)
 QW_GU(21, 1, 21, 1, qwk_gu_f21_c1_s21_c1) QW_GU(21, 1, 8, 1, qwk_gu_f21_c1_s8_c1)
 QW_GU(8, 16, 8, 16, qwk_gu_f8_c16_s8_c16) QW_GU(8, 16, 21, 2, qwk_gu_f8_c16_s21_c2)
 QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_s8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_s21_c1)
+#endif
 // packed IQ3_S routed experts (and shared expert, when it is IQ3_S too)
+#if QW_IN_PART(1)
 QW_GU(121, 2, 0, 1, qwk_gu_f121_c2) QW_GU(121, 2, 121, 2, qwk_gu_f121_c2_s121_c2) QW_GU(121, 2, 8, 16, qwk_gu_f121_c2_s8_c16)
 QW_GU(121, 1, 0, 1, qwk_gu_f121_c1) QW_GU(121, 1, 121, 1, qwk_gu_f121_c1_s121_c1) QW_GU(121, 1, 8, 1, qwk_gu_f121_c1_s8_c1)
+#endif
 
 // ================================================================ front part of a layer (kernels/moe_gg.metal:534-590)
 // Router rows with the activations copied into LDS once per workgroup (8 rows per workgroup) on the first
@@ -1074,18 +1153,23 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
         }                                                                                               \
         else if (F != 0) pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part);                              \
     }
+#if QW_IN_PART(2)
 QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
 QW_PRE(1, 121, 2, qwk_pre_w1_s121_c2) QW_PRE(30, 121, 2, qwk_pre_w30_s121_c2) QW_PRE(1, 8, 16, qwk_pre_w1_s8_c16) QW_PRE(30, 8, 16, qwk_pre_w30_s8_c16)
+#endif
 // The same front launch for a shared expert whose gate/up rows are in the K-quant / IQ4 / plain family: the binary16
 // router on the first workgroups, the multi-format product with SwiGLU (qwk_qmvm_swiglu's work) on those after them.
+#if QW_IN_PART(2)
 extern "C" __global__ __launch_bounds__(QW_WG_QMVM) void qwk_pre_w1_kq(qwk_prekq_args a) {
     __shared__ qw_qmvm_lds L;
     if (blockIdx.x < a.nrouter) pre_router_mfma(a.r, L.xf, L.red);
     else qmvm_swiglu_body(a.m, L, blockIdx.x - a.nrouter, gridDim.x - a.nrouter);
 }
+#endif
 
 // SwiGLU of the shared expert (kernels/moe_gg.metal:563-573) after a matvec of its gate and up rows in another format
 // family: the arithmetic and the two-plane store of pre_shared. One thread per (token, column).
+#if QW_IN_PART(2)
 extern "C" __global__ __launch_bounds__(256) void qwk_sh_act(qwk_shact_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= a.nb * a.I) return;
@@ -1096,6 +1180,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_sh_act(qwk_shact_args a) {
     a.H[o] = __builtin_bit_cast(uint16_t, hi);
     a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
 }
+#endif
 
 // ================================================================ down (kernels/moe_gg.metal:456-483, 606-617, 639-652)
 // The shared expert's down projection rides in the same launch: tiles of 16 rows, operand A = H[t][topk] (hi + lo
@@ -1278,22 +1363,30 @@ template <int F, int CH, int FSD, int CHSD> __device__ __forceinline__ void dn_r
         __shared__ struct { u2 lut[QW_KQ_TAB / 2]; uint16_t arows[2 * 16 * 2 * 640]; qw_sel_cache sc; } L; \
         dn_range_body<20, CH, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                               \
     }
+#if QW_IN_PART(3)
 QW_DN_RANGE_NL(4, 0, 1, qwk_dnr_f20_c4) QW_DN_RANGE_NL(4, 20, 4, qwk_dnr_f20_c4_s20_c4) QW_DN_RANGE_NL(4, 8, 4, qwk_dnr_f20_c4_s8_c4)
+#endif
 #define QW_DN_RANGE_NLP(FSD, CHSD, NAME)                                                          \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                  \
         __shared__ struct { u2 lut[QW_KQ_TAB / 2]; uint16_t arows[2 * 16 * 2 * 640]; qw_sel_cache sc; } L; \
         dn_range_body<QW_F_PACKED_NL, 10, FSD, CHSD>(a, L.lut, L.arows, &L.sc);                   \
     }
 // the tile-major copy: rows of 320 or 640
+#if QW_IN_PART(3)
 QW_DN_RANGE_NLP(0, 10, qwk_dnr_f120_c10) QW_DN_RANGE_NLP(QW_F_PACKED_NL, 10, qwk_dnr_f120_c10_s120_c10) QW_DN_RANGE_NLP(8, 4, qwk_dnr_f120_c10_s8_c4)
+#endif
 // rows of 320 or 640: chunks of ten blocks (a row of 640 in two), 5760 bytes a tile in flight per wave
+#if QW_IN_PART(3)
 QW_DN_RANGE_NL(10, 0, 1, qwk_dnr_f20_c10) QW_DN_RANGE_NL(10, 20, 10, qwk_dnr_f20_c10_s20_c10) QW_DN_RANGE_NL(10, 8, 4, qwk_dnr_f20_c10_s8_c4)
+#endif
 // I = 512: a row is one chunk of 2 IQ3_S blocks or four chunks of 4 Q8_0 blocks; I = 256: one IQ3_S block, two Q8_0 chunks
+#if QW_IN_PART(3)
 QW_DN_RANGE(21, 2, 0, 1, qwk_dnr_f21_c2) QW_DN_RANGE(21, 2, 21, 2, qwk_dnr_f21_c2_s21_c2) QW_DN_RANGE(21, 2, 8, 4, qwk_dnr_f21_c2_s8_c4)
 QW_DN_RANGE(21, 1, 0, 1, qwk_dnr_f21_c1) QW_DN_RANGE(21, 1, 21, 1, qwk_dnr_f21_c1_s21_c1) QW_DN_RANGE(21, 1, 8, 4, qwk_dnr_f21_c1_s8_c4)
 QW_DN_RANGE(121, 2, 0, 1, qwk_dnr_f121_c2) QW_DN_RANGE(121, 2, 121, 2, qwk_dnr_f121_c2_s121_c2) QW_DN_RANGE(121, 2, 8, 4, qwk_dnr_f121_c2_s8_c4)
 QW_DN_RANGE(121, 1, 0, 1, qwk_dnr_f121_c1) QW_DN_RANGE(121, 1, 121, 1, qwk_dnr_f121_c1_s121_c1) QW_DN_RANGE(121, 1, 8, 4, qwk_dnr_f121_c1_s8_c4)
 QW_DN_RANGE(8, 4, 0, 1, qwk_dnr_f8_c4) QW_DN_RANGE(8, 4, 8, 4, qwk_dnr_f8_c4_s8_c4) QW_DN_RANGE(8, 4, 21, 2, qwk_dnr_f8_c4_s21_c2) QW_DN_RANGE(8, 4, 21, 1, qwk_dnr_f8_c4_s21_c1)
+#endif
 
 // Down + combine in one launch for a few tokens (at most QW_DNC_MAXNB; kernels/moe_gg.metal:639-663 in one pass).
 // With one or two tokens the layer is bound by its launches, and the combine is a launch that only adds up what the
@@ -1379,10 +1472,12 @@ __device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *p
         __shared__ struct { u2 lut[(qw_has_lut(F) || qw_has_lut(FSD)) ? QW_LUT_ENTRIES : (F == QW_F_PACKED_NL || FSD == QW_F_PACKED_NL) ? QW_KQ_TAB / 2 : 1]; float part[QW_DNC_MAXNB * 17 * 16], wl[QW_DNC_MAXNB * 17]; qw_sel_cache sc; } L; \
         dnc_body<F, CH, FSD, CHSD>(a, L.lut, L.part, L.wl, &L.sc);                                  \
     }
+#if QW_IN_PART(4)
 QW_DNC(121, 2, 0, 1, qwk_dnc_f121_c2) QW_DNC(121, 2, 121, 2, qwk_dnc_f121_c2_s121_c2) QW_DNC(121, 2, 8, 4, qwk_dnc_f121_c2_s8_c4)
 QW_DNC(121, 1, 0, 1, qwk_dnc_f121_c1) QW_DNC(121, 1, 121, 1, qwk_dnc_f121_c1_s121_c1) QW_DNC(121, 1, 8, 4, qwk_dnc_f121_c1_s8_c4)
 QW_DNC(8, 4, 0, 1, qwk_dnc_f8_c4) QW_DNC(8, 4, 8, 4, qwk_dnc_f8_c4_s8_c4)
 QW_DNC(120, 10, 0, 10, qwk_dnc_f120_c10) QW_DNC(120, 10, 120, 10, qwk_dnc_f120_c10_s120_c10) QW_DNC(120, 10, 8, 4, qwk_dnc_f120_c10_s8_c4) // tile-major IQ4_NL rows of 640
+#endif
 
 // Down + combine in one launch for 3 to 16 tokens. The range form above needs a second launch because the products
 // that make up one output row are spread over all workgroups. Here a workgroup owns tpw tiles of 16 output rows and a
@@ -1403,7 +1498,7 @@ struct qw_dnq_lds {
 // Operand A from the staged rows, in the manner of qw_afrag_gather: lane m < 4 is local token m, its row chosen per
 // expert; four fragments per plane at a time inside one predicated region, into registers the caller keeps (and has
 // zeroed once), so that the lanes that are off (12 of every 16 at least) cost LDS nothing.
-struct qw_afrag_rows {
+template <uint32_t ROWS> struct qw_afrag_rows {
     const u4 *hi_, *lo_; // this lane's row in the two planes
     bool on;
     h8 (&hi)[4];
@@ -1413,23 +1508,30 @@ struct qw_afrag_rows {
         if (on) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                hi[i] = __builtin_bit_cast(h8, hi_[((koff + i * kstep) >> 3) * QW_DNQ_ROWS]);
-                lo[i] = __builtin_bit_cast(h8, lo_[((koff + i * kstep) >> 3) * QW_DNQ_ROWS]);
+                hi[i] = __builtin_bit_cast(h8, hi_[((koff + i * kstep) >> 3) * ROWS]);
+                lo[i] = __builtin_bit_cast(h8, lo_[((koff + i * kstep) >> 3) * ROWS]);
             }
         }
     }
 };
+// What dnq_run reads and writes in LDS (the two kernels that hold it lay their LDS out differently).
+struct qw_dnq_view {
+    const u4 *hrows;       // [plane][8 k-values][row], 16 bytes each, ROWS rows: row = local token * (topk + 1) + slot
+    float *part;           // [local token][slot][row of the group]
+    const uint32_t *ue, *slot4;
+    const uint16_t *mask, *vlist;
+};
 // The tiles of `nv` experts (shared: the one shared expert) for this workgroup's tpw tiles, dealt to its waves.
-template <int F, int CH, bool SHARED, class S>
-__device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, qw_dnq_lds &L, uint32_t g, uint32_t t0, uint32_t nt, uint32_t nv, uint32_t dealt, S ready) {
+template <int F, int CH, bool SHARED, uint32_t ROWS, class S>
+__device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, const qw_dnq_view &L, uint32_t g, uint32_t t0, uint32_t nt, uint32_t nv, uint32_t dealt, S ready) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, tpe = a.D / 16, tpw = a.tpw, cpr = a.I / (C::BLK_K * CH), rw = 16 * tpw;
     const uint32_t ts = (uint32_t)__builtin_ctz(tpw), tm = tpw - 1; // tpw is a power of two
     const uint32_t m = n; // operand A row of this lane
     f4 acc = {0, 0, 0, 0};
-    const u4 *const lo0 = L.hrows + a.I / 8 * QW_DNQ_ROWS;
+    const u4 *const lo0 = L.hrows + a.I / 8 * ROWS;
     h8 xhi[4] = {}, xlo[4] = {};
-    qw_afrag_rows af = {L.hrows, lo0, false, xhi, xlo};
+    qw_afrag_rows<ROWS> af = {L.hrows, lo0, false, xhi, xlo};
     auto expert = [&](uint32_t task) { return SHARED ? 0u : (uint32_t)L.vlist[task >> ts]; };
     const uint32_t nw = blockDim.x >> 6, w0 = (qw_wave() + nw - dealt % nw) % nw; // the deal goes on where the last one (dealt tiles) stopped
     qw_task_stream<C>(nv * tpw, w0, nw, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
@@ -1554,9 +1656,10 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
     };
     // the routed experts first (every wave has tiles there, so every wave's first weights are on their way before the
     // rows are asked for); the shared expert's tiles go to the waves that the routed deal gave one tile fewer
-    dnq_run<F, CH, false>(a, lut, L, g, t0, nt, nv, 0, ready);
+    const qw_dnq_view V = {L.hrows, L.part, L.ue, L.slot4, L.mask, L.vlist};
+    dnq_run<F, CH, false, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, nv, 0, ready);
     if (FSD != 0) {
-        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true>(a, lut, L, g, t0, nt, 1, nv * tpw, ready);
+        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, 1, nv * tpw, ready);
     }
     ready(); // (for symmetry only: both runs call it, with or without tiles)
     __syncthreads();
@@ -1577,8 +1680,188 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         __shared__ struct { u2 lut[QW_LUT_ENTRIES]; qw_dnq_lds d; } L;                               \
         dnq_body<F, CH, FSD, CHSD>(a, L.lut, L.d);                                                  \
     }
+#if QW_IN_PART(4)
 QW_DNQ(121, 2, 0, 1, qwk_dnq_f121_c2) QW_DNQ(121, 2, 121, 2, qwk_dnq_f121_c2_s121_c2) QW_DNQ(121, 2, 8, 4, qwk_dnq_f121_c2_s8_c4)
 QW_DNQ(121, 1, 0, 1, qwk_dnq_f121_c1) QW_DNQ(121, 1, 121, 1, qwk_dnq_f121_c1_s121_c1) QW_DNQ(121, 1, 8, 4, qwk_dnq_f121_c1_s8_c4)
+#endif
+
+// ================================================================ routed gate/up, down and combine as one launch
+// (kernels/moe_gg.metal:600-663 in one pass.) Three launches a layer each pay their own start: the launch itself, the
+// table and the record into LDS, the first round trip to memory. Here the persistent workgroups of the gate/up launch go
+// on into the down projection: the table and the selection stay in LDS, and every wave asks for its first down tiles
+// before it waits for the others. What the two phases hand over is H, produced column by column all over the grid and
+// consumed row by row: the SwiGLU values of a workgroup's tiles are kept in LDS while it streams (a store of device
+// scope among the weight loads would hold up every wait for them) and leave in one burst of device-scope stores at the
+// end; then one barrier over the grid; then every workgroup stages the H rows of its share of the tokens with loads
+// of device scope and runs the down projection and the combine exactly as qwk_dnq_* does. Pg, Psh, H and the record
+// are left in memory as the separate launches leave them.
+struct qw_h_lds { // the gate/up phase's SwiGLU values in LDS: entry = one (tile, token), eight columns
+    uint32_t *count, *off, *val; // val: hi | lo << 16
+    uint16_t *H;
+    uint32_t hplane, base;
+    __device__ __forceinline__ void stamp(uint32_t k) const { QW_DSTAMP(k); }
+    __device__ __forceinline__ void tile(uint32_t m) {
+        uint32_t b = 0;
+        if (qw_lane() == 0) b = atomicAdd(count, (uint32_t)__builtin_popcount(m));
+        base = (uint32_t)__builtin_amdgcn_readfirstlane((int)b);
+    }
+    __device__ __forceinline__ void put(uint32_t m, uint32_t tok, size_t o, uint16_t hi, uint16_t lo) const {
+        const uint32_t idx = base + (uint32_t)__builtin_popcount(m & ((1u << tok) - 1)), n = qw_lane() & 7;
+        if (idx < QW_GUD_HCAP) {
+            val[idx * 8 + n] = (uint32_t)hi | (uint32_t)lo << 16;
+            if (n == 0) off[idx] = (uint32_t)o;
+        } else { // (more results than the buffer holds: straight to memory)
+            __hip_atomic_store(H + o, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(H + o + hplane, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+};
+struct qw_gud_lds {
+    u2 lut[QW_LUT_ENTRIES];
+    union {
+        u4 xf[QW_XF_MAXK * 2];                 // gate/up phase: the activations (and the selection's per-wave scratch behind them)
+        u4 hrows[2 * 64 * QW_GUD_ROWS];        // down phase: the H rows of the share's tokens
+    } big;
+    qw_sel_cache sc;
+    union {
+        qw_sel_scratch ss;                                                    // while the selection is made
+        struct { uint32_t off[QW_GUD_HCAP], val[QW_GUD_HCAP * 8]; } hb;       // gate/up phase
+        float part[2 * 11 * 64];                                              // down phase: [local token][slot][row of the group]
+    } u;
+    float wl[QW_GUD_SHARE * 11];
+    uint32_t ue[QW_DNQ_MAXU], slot4[QW_DNQ_MAXU];
+    uint16_t mask[QW_DNQ_MAXU], vlist[32];
+    uint32_t hcount, bail;
+};
+static_assert(sizeof(qw_gud_lds) <= 160 * 1024, "LDS of the fused launch");
+static_assert(QW_GUD_SHARE * 11 * 32 <= 2 * 11 * 64, "part holds three tokens by two tiles or two tokens by four");
+#define QW_STAMP(k) QW_DSTAMP(k)
+template <int FSD, int CHSD> __device__ __forceinline__ void gud_body(const qwk_gud_args &ga, qw_gud_lds &L) {
+    constexpr int F = QW_F_PACKED, CH = 2; // tile-major IQ3_S, D a multiple of 512, I = 512
+    const qwk_gu_args &a = ga.gu;
+    const qwk_dn_args &d = ga.dn;
+    const uint32_t K = d.topk, gnb = d.gnb, tid = threadIdx.x, lane = qw_lane(), nq = d.nq, tpw = d.tpw, rw = 16 * tpw;
+    uint32_t gen0 = 0;
+    QW_STAMP(0);
+    if (tid == 0) gen0 = qw_ld_coh(ga.sync + QW_SYNC_GEN);
+    // the down phase's place of this workgroup: tile group g, share q of the tokens (the shares of a group are eight
+    // workgroups apart: one XCD); workgroups past the last group only take part in the gate/up phase
+    const uint32_t hi8 = blockIdx.x >> 3, g = (hi8 / nq) * 8 + (blockIdx.x & 7), q = hi8 % nq;
+    const bool active = g < d.D / 16 / tpw;
+    const uint32_t base = d.nbr / nq, rem = d.nbr % nq, t0 = q * base + (q < rem ? q : rem);
+    uint32_t nt = base + (q < rem ? 1 : 0);
+    if (nt > QW_GUD_SHARE) nt = QW_GUD_SHARE; // (the host keeps the shares that small)
+    uint32_t nv = 0;
+    qw_h_lds hs = {&L.hcount, L.u.hb.off, L.u.hb.val, a.H, a.hplane, 0};
+    gu_body<F, CH, 0, 1>(a, L.lut, L.big.xf, &L.sc, &L.u.ss, hs, true, [&] {
+        // the down phase's lists, made while everything they come from is in LDS: gating weights of the share's tokens,
+        // experts, masks, the share's slot bytes, and the unique experts its tokens picked in record order (every wave
+        // makes the whole list: all write the same values)
+        uint32_t GU = gnb * K;
+        if (GU > QW_DNQ_MAXU) GU = QW_DNQ_MAXU;
+        for (uint32_t i = tid; i < nt * (K + 1); i += blockDim.x) L.wl[i] = L.u.ss.w[t0 * (K + 1) + i];
+        for (uint32_t i = tid; i < GU; i += blockDim.x) {
+            uint32_t s4 = 0;
+            for (uint32_t j = 0; j < nt; j++) s4 |= (uint32_t)L.sc.slot[i * gnb + t0 + j] << (8 * j);
+            L.ue[i] = L.sc.ue[i], L.mask[i] = (uint16_t)L.sc.mask[i], L.slot4[i] = s4;
+        }
+        if (tid == 0) L.hcount = 0, L.bail = 0;
+        uint32_t U = L.sc.U;
+        if (U > GU) U = GU;
+        const uint32_t want = (1u << nt) - 1;
+        for (uint32_t u0 = 0; u0 < U; u0 += 64) {
+            const uint32_t u = u0 + lane;
+            const bool on = active && u < U && ((L.sc.mask[u] >> t0) & want);
+            const unsigned long long bal = __ballot(on);
+            const uint32_t at = nv + __builtin_amdgcn_mbcnt_hi((uint32_t)(bal >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bal, 0));
+            if (on && at < 32) L.vlist[at] = (uint16_t)u;
+            nv += (uint32_t)__popcll(bal);
+        }
+        if (nv > 32) nv = 32; // (three tokens of ten experts: 30 at most)
+        __syncthreads(); // the selection's scratch becomes the buffer of SwiGLU values
+    });
+    const uint32_t nsh = (FSD != 0 && d.Wsd) ? 1 : 0;
+    bool met = false;
+    // Once per wave, behind its first down loads (or straight away for a workgroup without a share): the hand-over.
+    auto meet = [&] {
+        if (met) return;
+        met = true;
+        QW_STAMP(3);
+        __syncthreads(); // every wave of the workgroup has left the gate/up phase
+        QW_STAMP(4);
+        uint32_t cnt = L.hcount;
+        if (cnt > QW_GUD_HCAP) cnt = QW_GUD_HCAP;
+        for (uint32_t i = tid; i < cnt * 4; i += blockDim.x) { // two columns a thread, a dword a plane
+            const uint32_t e = i >> 2, c = 2 * (i & 3), v0 = L.u.hb.val[e * 8 + c], v1 = L.u.hb.val[e * 8 + c + 1];
+            uint32_t *p = (uint32_t *)(a.H + L.u.hb.off[e] + c);
+            qw_st_coh(p, (v0 & 0xffffu) | (v1 << 16));
+            qw_st_coh(p + a.hplane / 2, (v0 >> 16) | (v1 & 0xffff0000u));
+        }
+        __builtin_amdgcn_s_waitcnt(0); // this wave's stores (and its first down loads) have completed
+        __syncthreads();
+        QW_STAMP(5);
+        if (tid == 0 && !qw_grid_barrier(ga.sync, gen0, 1, gridDim.x, ga.spin_limit)) L.bail = 1;
+        __syncthreads();
+        QW_STAMP(6);
+        if (!active || L.bail) return;
+        // every H row of the share's tokens into LDS in fragment order: a wave's load takes 8 rows x 128 bytes (whole
+        // cache lines), lanes 0 .. 31 the first 64 bytes of a row, 32 .. 63 the rest
+        const uint32_t upr = d.I / 8, cbs = upr / 8, used = nt * (K + 1), nrb = (used + 7) / 8, nunits = 2 * nrb * cbs, wv = qw_wave();
+        constexpr uint32_t NW = QW_WG_GU / 64, PER = (2 * ((QW_GUD_ROWS + 7) / 8) * 8 + NW - 1) / NW; // 2 planes x 5 row blocks x 8 column blocks at most
+        static_assert(PER == 7, "qw_ld_coh7 takes seven loads");
+        u4 t[PER];
+        const u4 *src[PER];
+        uint32_t at[PER];
+#pragma unroll
+        for (uint32_t it = 0; it < PER; it++) {
+            const uint32_t unit = wv + it * NW, cb = unit % cbs, rest = unit / cbs, rb = rest % nrb, pl = rest / nrb;
+            const uint32_t r = 8 * rb + ((lane >> 2) & 7), c = 8 * cb + 4 * (lane >> 5) + (lane & 3);
+            const bool on = unit < nunits && r < used;
+            at[it] = on ? (pl * upr + c) * QW_GUD_ROWS + r : ~0u;
+            src[it] = (const u4 *)(on ? d.H + pl * (size_t)d.hplane + ((size_t)t0 * (K + 1) + r) * d.I + 8 * c : d.H); // (off: a valid address, not kept)
+        }
+        qw_ld_coh7(t, src);
+#pragma unroll
+        for (uint32_t it = 0; it < PER; it++)
+            if (at[it] != ~0u) L.big.hrows[at[it]] = t[it];
+        __syncthreads();
+        QW_STAMP(7);
+    };
+    if (!active) {
+        meet();
+        return;
+    }
+    const qw_dnq_view V = {L.big.hrows, L.u.part, L.ue, L.slot4, L.mask, L.vlist};
+    // the routed experts first; the shared expert's tiles go to the waves that the routed deal gave one tile fewer
+    dnq_run<F, CH, false, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, nv, 0, meet);
+    if (FSD != 0) {
+        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, 1, nv * tpw, meet);
+    }
+    meet();
+    QW_STAMP(8);
+    __syncthreads();
+    QW_STAMP(9);
+    if (L.bail) return;
+    for (uint32_t j = tid; j < nt * rw; j += blockDim.x) { // rank order, then the shared expert (qwk_cmb's arithmetic)
+        const uint32_t t = j >> (4 + __builtin_ctz(tpw)), i = j & (rw - 1), r = g * rw + i;
+        const float *w = L.wl + t * (K + 1), *p = L.u.part + t * (K + 1) * rw + i;
+        float o = 0;
+        for (uint32_t s = 0; s < K; s++) o = __builtin_fmaf(w[s], p[s * rw], o);
+        float sh;
+        if (nsh) sh = p[K * rw];
+        else sh = d.Psh[(size_t)(t0 + t) * d.D + r]; // the caller's own shared product
+        o = __builtin_fmaf(w[K], sh, o);
+        d.out[(size_t)(t0 + t) * d.D + r] = qw_f2h(o);
+    }
+}
+#define QW_GUD(FSD, CHSD, NAME)                                                                     \
+    extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gud_args a) {                   \
+        __shared__ qw_gud_lds L;                                                                    \
+        gud_body<FSD, CHSD>(a, L);                                                                  \
+    }
+#if QW_IN_PART(4)
+QW_GUD(0, 1, qwk_gud_f121_c2) QW_GUD(121, 2, qwk_gud_f121_c2_s121_c2) QW_GUD(8, 4, qwk_gud_f121_c2_s8_c4)
+#endif
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
 template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
@@ -1616,16 +1899,21 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
         __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : (F == 20 || FSD == 20) ? QW_KQ_TAB / 2 : 1]; qw_sel_cache sc; } L; \
         dn_any_body<F, FSD>(a, L.lut, &L.sc);                                         \
     }
+#if QW_IN_PART(2)
 QW_DN_ANY(21, 0, qwk_dn_f21_any) QW_DN_ANY(21, 21, qwk_dn_f21_any_s21) QW_DN_ANY(21, 8, qwk_dn_f21_any_s8)
 QW_DN_ANY(8, 0, qwk_dn_f8_any) QW_DN_ANY(8, 21, qwk_dn_f8_any_s21) QW_DN_ANY(8, 8, qwk_dn_f8_any_s8)
+#endif
 // IQ4_NL down rows (the routed and shared down projections of a layer with I = 640, bench/moe_bw.c:22-24 of the reference)
+#if QW_IN_PART(2)
 QW_DN_ANY(20, 0, qwk_dn_f20_any) QW_DN_ANY(20, 20, qwk_dn_f20_any_s20) QW_DN_ANY(20, 8, qwk_dn_f20_any_s8)
+#endif
 
 // ================================================================ ragged packing (kernels/moe_prefill.metal:15-119)
 // P (token, expert) pairs -> per-expert counts -> exclusive prefix sums (first packed row of every expert, tile table)
 // -> rows copied to packed order -> grouped product -> gathered, weighted sum. Integer work; bit-exact.
 // The counters are cleared on the device, inside the recorded sequence (kernels/prefill.metal:601-603): a batch may hold
 // the packing sequence several times, and all of it is recorded before any of it runs.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_zero(qwk_zero_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < a.n) a.x[i] = 0;
@@ -1634,8 +1922,10 @@ extern "C" __global__ __launch_bounds__(256) void qwk_moe_count(qwk_count_args a
     const uint32_t p = blockIdx.x * blockDim.x + threadIdx.x;
     if (p < a.P && a.ids[p] < a.E) atomicAdd(&a.counts[a.ids[p]], 1u);
 }
+#endif
 // One workgroup of 1024 threads, thread e = expert e (E <= 1024): two exclusive scans (rows, tiles) by ballot-free
 // wave scans (DPP row shifts through __shfl_up) and one pass over the sixteen wave totals.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(1024) void qwk_moe_plan(qwk_plan_args a) {
     __shared__ uint32_t wr[16], wt[16];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1664,7 +1954,9 @@ extern "C" __global__ __launch_bounds__(1024) void qwk_moe_plan(qwk_plan_args a)
     }
     for (uint32_t t = total_t + tid; t < a.max_tiles; t += blockDim.x) *(u4 *)(a.tiles + 4 * t) = u4{0, 0, 0, 0}; // unused entries
 }
+#endif
 // One workgroup per pair: take the next row of the pair's expert, remember it, copy the token's row there.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_moe_scatter(qwk_scatter_args a) {
     __shared__ uint32_t pos;
     const uint32_t p = blockIdx.x;
@@ -1679,12 +1971,14 @@ extern "C" __global__ __launch_bounds__(256) void qwk_moe_scatter(qwk_scatter_ar
     u4 *dst = (u4 *)(a.Xs + (size_t)pos * a.KD);
     for (uint32_t i = threadIdx.x; i < a.KD / 8; i += blockDim.x) dst[i] = src[i];
 }
+#endif
 // The four launches above as one, for a step of a few thousand pairs at most: a workgroup per pair, and every workgroup
 // counts all pairs itself (LDS atomics over the P ids), which gives it its own packed row without a hand-over: the rows
 // of the experts below its own plus the earlier pairs of its own expert. The order inside an expert is therefore the
 // order of the pairs (the cursor form leaves whatever order the atomics came in; both are permutations the grouped
 // product and the combine do not care about). Workgroup 0 also leaves counts, offsets, cursors (where the scatter
 // would have left them) and the tile table.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_moe_prep(qwk_prep_args a) {
     __shared__ uint32_t cnt[1024], red[4], wr[4], wt[4];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, p = blockIdx.x;
@@ -1747,7 +2041,9 @@ extern "C" __global__ __launch_bounds__(256) void qwk_moe_prep(qwk_prep_args a) 
     }
     for (uint32_t t = total_t + tid; t < a.max_tiles; t += 256) *(u4 *)(a.tiles + 4 * t) = u4{0, 0, 0, 0}; // unused entries
 }
+#endif
 // H = SiLU(gate) * up, binary16 in and out, the product rounded once (kernels/moe_prefill.metal:95-103, kernels/prefill.metal:485-488)
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_moe_act(qwk_act_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= a.n) return;
@@ -1759,7 +2055,9 @@ extern "C" __global__ __launch_bounds__(256) void qwk_moe_act(qwk_act_args a) {
     }
     a.H[i] = qw_f2h(g / (1.0f + __expf(-g)) * u);
 }
+#endif
 // y[t][c] = sum_s w[t][s] * D[pos_of[t][s]][c] in rank order; one thread per (token, 4 columns).
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(64) void qwk_moe_combine(qwk_combine_args a) {
     const uint32_t c4 = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
     if (c4 >= a.KD / 4 || t >= a.T) return;
@@ -1777,6 +2075,7 @@ extern "C" __global__ __launch_bounds__(64) void qwk_moe_combine(qwk_combine_arg
     o.y = (uint32_t)qw_f2h(acc[2]) | (uint32_t)qw_f2h(acc[3]) << 16;
     *(u2 *)(a.Y + (size_t)t * a.KD + 4 * c4) = o;
 }
+#endif
 
 // SwiGLU at the end of a tile of 8 gate + 8 up rows (a.H given): lane n < 8 has the gate value of a packed row and a
 // column, lane n + 8 the up value of the same two; both as the binary16 the G and U buffers hold, the product rounded
@@ -1859,9 +2158,11 @@ template <int F, int CH> __device__ __forceinline__ void pf_body(const qwk_pf_ar
         __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : F == 20 ? QW_KQ_TAB / 2 : 1]; u4 tl[2048]; uint32_t cnt; } L; \
         pf_body<F, CH>(a, L.lut, L.tl, &L.cnt);                                                  \
     }
+#if QW_IN_PART(5)
 QW_PF(21, 2, qwk_pf_f21_c2) QW_PF(21, 1, qwk_pf_f21_c1) QW_PF(8, 4, qwk_pf_f8_c4)
 QW_PF(20, 4, qwk_pf_f20_c4) // IQ4_NL rows (the down projection of the reference model's layer: K = 640)
 QW_PF(121, 2, qwk_pf_f121_c2) QW_PF(121, 1, qwk_pf_f121_c1) // tile-major IQ3_S: one matrix, or gate and up rows side by side
+#endif
 
 // The same product for entries of at most 16 packed rows over tile-major weights, the way the decode kernels work:
 // a workgroup takes a contiguous range of (entry, weight tile) tasks - the tiles of one entry, or the end of one and
@@ -1923,10 +2224,13 @@ template <int CH> __device__ __forceinline__ void pf_range_body(const qwk_pf_arg
         __shared__ struct { u2 lut[QW_LUT_ENTRIES]; u4 xf[QW_XF_MAXK * 2]; uint32_t cnt; } L;     \
         pf_range_body<CH>(a, L.lut, L.xf, &L.cnt);                                                \
     }
+#if QW_IN_PART(5)
 QW_PFR(2, qwk_pfr_f121_c2) QW_PFR(1, qwk_pfr_f121_c1)
+#endif
 
 // ================================================================ combine (kernels/moe_gg.metal:655-663)
 // Rank order, then the shared expert. One thread per (token, row).
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_cmb(qwk_cmb_args a) {
     const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= a.nbr * a.D) return;
@@ -1942,10 +2246,12 @@ extern "C" __global__ __launch_bounds__(256) void qwk_cmb(qwk_cmb_args a) {
     o = __builtin_fmaf(w[K], a.Psh[(size_t)t * a.D + row], o);
     a.out[(size_t)t * a.D + row] = qw_f2h(o);
 }
+#endif
 
 // ================================================================ memory helpers
 // Pure-read ceiling: every thread folds 16-byte loads into an XOR sink the compiler cannot drop
 // (the method of the reference's kernels/ceiling_mem.metal:10-71). Grid-stride over n 16-byte units.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_bw_read(qwk_mem_args a) {
     const u4 *p = (const u4 *)a.src;
     u4 s = {0, 0, 0, 0};
@@ -1958,6 +2264,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_bw_read(qwk_mem_args a) {
     for (; i < a.n; i += step) s ^= p[i];
     if ((s.x ^ s.y ^ s.z ^ s.w) == 0x9e3779b9u && a.seed == 0x1234) ((u4 *)a.dst)[0] = s; // practically never taken
 }
+#endif
 // ================================================================ hyper-connection, GGUF profile (kernels/hyper_gg.metal:94-233)
 // Everything in binary32, as there. Two launches a hyper-connection whatever the token count: a launch boundary costs
 // more here than recomputing nb x 320 activations per workgroup, which is what the reference's third kernel avoids.
@@ -2055,6 +2362,7 @@ template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_
         else if (rb == 0) pd[QW_HC_LR + QW_HC] = sum;
     }
 }
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r4(qwk_hc_args a) {
     __shared__ float part[8][QW_HC_TG][17]; // [wave][token][row | squares]
     hc_down_body<4>(a, part);
@@ -2063,6 +2371,7 @@ extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r16(qwk_hc_args a)
     __shared__ float part[8][QW_HC_TG][17];
     hc_down_body<16>(a, part);
 }
+#endif
 // What follows the down kernel for tokens t0 .. t0 + nt - 1, by the threads of one workgroup: the streams' 1 / rms,
 // silu of the normalised mix_down sums, and (injo given) the inject sums in the caller's format
 // (kernels/hyper_gg.metal:165-181, 312-340). rs [nt][HC] and sx [nt][LR] are in LDS; ends with a barrier.
@@ -2095,6 +2404,7 @@ __device__ __forceinline__ void hc_mid(const qwk_hc_args &a, uint32_t t0, uint32
     __syncthreads();
 }
 // The middle kernel of the three-kernel form (kernels/hyper_gg.metal:312-340): a workgroup a token.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(320) void qwk_hc_mid(qwk_hc_args a) {
     __shared__ float rs[QW_HC], sx[QW_HC_LR];
     const uint32_t t = blockIdx.x;
@@ -2102,6 +2412,7 @@ extern "C" __global__ __launch_bounds__(320) void qwk_hc_mid(qwk_hc_args a) {
     for (uint32_t r = threadIdx.x; r < QW_HC_LR; r += blockDim.x) a.sx[t * QW_HC_LR + r] = sx[r];
     if (threadIdx.x < QW_HC) a.rs[t * QW_HC + threadIdx.x] = rs[threadIdx.x];
 }
+#endif
 // Up: mix_up, the gates and the mix over the streams, the write-back of h (kernels/hyper_gg.metal:141-233, 344-).
 // A workgroup of 256 threads takes eight output columns i, one per group of 32 lanes; a lane holds ten low-rank columns
 // of the four mix_up rows s D + i (20 bytes each). GIVEN: sx and rs come from qwk_hc_mid instead of being made here.
@@ -2186,8 +2497,10 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
         if (t < a.nb && sq == 0) a.x[(size_t)t * a.D + i] = qw_f2h(m / QW_HC);
     }
 }
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_hc_up(qwk_hc_args a) { hc_up_body<false>(a); }
 extern "C" __global__ __launch_bounds__(256) void qwk_hc_upv(qwk_hc_args a) { hc_up_body<true>(a); }
+#endif
 
 // Read pattern of a decode layer without the decoding (kernels/moe_bw.metal:7-26): workgroup (x, c) reads slice x
 // (SL 16-byte units) of chunk c, every thread LD independent loads a round, folded into an XOR sink.
@@ -2215,6 +2528,7 @@ template <int LD> __device__ __forceinline__ void bw_chunks_body(const qwk_bwpat
     const uint32_t r = s.x ^ s.y ^ s.z ^ s.w;
     if (r == 0x9e3779b9u) a.out[tid] = r; // practically never taken
 }
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(1024) void qwk_bw_chunks(qwk_bwpat_args a) {
     switch (a.ld) {
     case 1: bw_chunks_body<1>(a); break;
@@ -2223,9 +2537,11 @@ extern "C" __global__ __launch_bounds__(1024) void qwk_bw_chunks(qwk_bwpat_args 
     default: bw_chunks_body<8>(a); break; // the host admits 1, 2, 4, 8
     }
 }
+#endif
 // The row pattern (kernels/moe_bw.metal:30-41): a group of 32 lanes takes one row of RB bytes and reads it two bytes
 // at a time, a unit of UB bytes per lane and step; workgroup (x, c) takes rows 8 x .. 8 x + 7 of chunk c. The
 // reference's group is the 32-lane SIMD group of its hardware: here it is half of a wave, the same rows and loads.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_bw_rows(qwk_bwpat_args a) {
     const uint32_t sg = threadIdx.x >> 5, lane = threadIdx.x & 31;
     const uint64_t off = (uint64_t)a.chunks[2 * blockIdx.y] * 16 + ((uint64_t)blockIdx.x * 8 + sg) * a.rb;
@@ -2236,18 +2552,22 @@ extern "C" __global__ __launch_bounds__(256) void qwk_bw_rows(qwk_bwpat_args a) 
         for (uint32_t j = 0; j < a.ub; j += 2) acc ^= *(const uint16_t *)(row + (size_t)u * a.ub + j);
     if (acc == 0x9e3779b9u) a.out[lane] = acc; // practically never taken
 }
+#endif
 // Plain copy of n 16-byte units (the known-size kernel the hardware traffic counters are scaled against).
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_copy(qwk_mem_args a) {
     const u4 *p = (const u4 *)a.src;
     u4 *q = (u4 *)a.dst;
     const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += step) q[i] = p[i];
 }
+#endif
 // Fill n 16-byte units with a counter-based hash of (seed, index): uniform random bytes.
 __device__ __forceinline__ uint32_t qw_mix(uint64_t x) {
     x ^= x >> 33; x *= 0xff51afd7ed558ccdull; x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ull; x ^= x >> 33;
     return (uint32_t)x;
 }
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_fill_random(qwk_mem_args a) {
     u4 *q = (u4 *)a.dst;
     const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
@@ -2256,9 +2576,11 @@ extern "C" __global__ __launch_bounds__(256) void qwk_fill_random(qwk_mem_args a
         q[i] = u4{qw_mix(c), qw_mix(c + 1), qw_mix(c + 2), qw_mix(c + 3)};
     }
 }
+#endif
 
 // Synthetic GGUF blocks, one thread per block: d = binary16(|N(0, sigma)|) by Box-Muller over two hashed uniforms,
 // every other byte uniform (IQ3_S, IQ4_NL), or int8 uniform in [-127, 127] (Q8_0). Blocks are 2-byte aligned: 16-bit stores.
+#if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_fill_blocks(qwk_fill_args a) {
     const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
     const uint32_t bb = a.type == 21 ? 110 : a.type == 20 ? 18 : 34; // IQ4_NL: d and sixteen uniform bytes
@@ -2278,3 +2600,4 @@ extern "C" __global__ __launch_bounds__(256) void qwk_fill_blocks(qwk_fill_args 
         }
     }
 }
+#endif

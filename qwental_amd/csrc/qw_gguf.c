@@ -163,46 +163,71 @@ static char *map_name(const char *g, unsigned *part, int *kind) {
     return strdup("");
 }
 
-// ---------------------------------------------------------------- parsing (src/gguf.c:73-173)
-static bool rdn(FILE *f, void *p, size_t n) { return fread(p, 1, n, f) == n; }
-static char *rstr(FILE *f) {
-    uint64_t n;
-    if (!rdn(f, &n, 8) || n > (1u << 24)) return NULL;
-    char *s = malloc(n + 1);
-    if (!s) return NULL;
-    if (!rdn(f, s, n)) {
-        free(s);
+// ---------------------------------------------------------------- parsing
+// What the header of a file holds and which files are refused follows the reference's parser (src/gguf.c:73-173): GGUF
+// version 2 or later, strings of at most 16 MiB, tensors of at most four dimensions, no arrays of arrays, of the metadata
+// only general.alignment kept (default 32), the data start rounded up to the alignment. Here the file is mapped first
+// and the header is walked in the mapping by a cursor that can never leave it: a read past the end yields zero and
+// marks the cursor, and the caller looks at the mark when a section is done.
+typedef struct {
+    const uint8_t *base;
+    uint64_t size, at;
+    bool overrun;
+} cursor;
+// n bytes at the cursor, or NULL (and the mark) when fewer are left
+static const uint8_t *cur_take(cursor *c, uint64_t n) {
+    if (c->overrun || n > c->size - c->at) {
+        c->overrun = true;
         return NULL;
     }
-    s[n] = 0;
-    return s;
+    const uint8_t *p = c->base + c->at;
+    c->at += n;
+    return p;
 }
-// Skip one metadata value of GGUF value type t; a scalar under the key general.alignment is kept.
-static bool skip_value(FILE *f, uint32_t t, uint32_t *align, const char *key) {
-    static const int sz[] = {1, 1, 2, 2, 4, 4, 4, 1, 0, 0, 8, 8, 8}; // u8 i8 u16 i16 u32 i32 f32 bool str arr u64 i64 f64
-    if (t == 8) {
-        char *s = rstr(f);
-        const bool ok = s != NULL;
-        free(s);
-        return ok;
-    }
-    if (t == 9) {
-        uint32_t at;
-        uint64_t n;
-        if (!rdn(f, &at, 4) || !rdn(f, &n, 8)) return false;
-        if (at == 8) {
-            for (uint64_t i = 0; i < n; i++)
-                if (!skip_value(f, 8, NULL, NULL)) return false;
-            return true;
-        }
-        if (at > 12 || at == 9) return false; // arrays of arrays are not accepted
-        return fseeko(f, (off_t)(n * (uint64_t)sz[at]), SEEK_CUR) == 0;
-    }
-    if (t > 12) return false;
+// a little-endian unsigned integer of 1 to 8 bytes
+static uint64_t cur_uint(cursor *c, unsigned width) {
+    const uint8_t *p = cur_take(c, width);
     uint64_t v = 0;
-    if (!rdn(f, &v, (size_t)sz[t])) return false;
-    if (align && key && !strcmp(key, "general.alignment")) *align = (uint32_t)v;
-    return true;
+    for (unsigned i = 0; p && i < width; i++) v |= (uint64_t)p[i] << (8 * i);
+    return v;
+}
+// a string (u64 length, then the bytes): pointer into the mapping and its length; longer than 16 MiB counts as damage
+static const char *cur_text(cursor *c, uint64_t *len) {
+    *len = cur_uint(c, 8);
+    if (*len > ((uint64_t)1 << 24)) c->overrun = true;
+    return (const char *)cur_take(c, *len);
+}
+enum { GV_STRING = 8, GV_ARRAY = 9, GV_TYPES = 13 };
+// bytes of a scalar of each GGUF value type: u8 i8 u16 i16 u32 i32 f32 bool | string array | u64 i64 f64
+static const uint8_t GV_WIDTH[GV_TYPES] = {1, 1, 2, 2, 4, 4, 4, 1, 0, 0, 8, 8, 8};
+// Step over one metadata value of type vt. A scalar's integer value goes to *scalar when the caller wants it.
+static void cur_skip_value(cursor *c, uint32_t vt, uint64_t *scalar) {
+    uint64_t n;
+    if (vt == GV_STRING) {
+        (void)cur_text(c, &n);
+    } else if (vt == GV_ARRAY) {
+        const uint32_t et = (uint32_t)cur_uint(c, 4);
+        n = cur_uint(c, 8);
+        if (et == GV_ARRAY || et >= GV_TYPES) c->overrun = true; // (arrays of arrays are not accepted)
+        else if (et == GV_STRING)
+            for (uint64_t i = 0; i < n && !c->overrun; i++) {
+                uint64_t l;
+                (void)cur_text(c, &l);
+            }
+        else if (n > (c->size - c->at) / GV_WIDTH[et]) c->overrun = true;
+        else (void)cur_take(c, n * GV_WIDTH[et]);
+    } else if (vt < GV_TYPES) {
+        const uint64_t v = cur_uint(c, GV_WIDTH[vt]);
+        if (scalar) *scalar = v;
+    } else c->overrun = true;
+}
+static char *text_dup(const char *p, uint64_t len) {
+    char *s = malloc(len + 1);
+    if (s) {
+        memcpy(s, p, len);
+        s[len] = 0;
+    }
+    return s;
 }
 
 // rows, rowbytes and nbytes of a tensor (nbytes 0 for a type that is not in the table); false when a product of its
@@ -222,84 +247,64 @@ static bool tensor_bytes(qw_gguf_tensor *t) {
 
 static bool parse_shard(qw_gguf *G, int si, const char *path, char *err, size_t errlen) {
     shard *s = &G->sh[si];
-    s->fd = -1;
     s->path = strdup(path);
-    FILE *f = fopen(path, "rb");
-    if (!f) return fail(err, errlen, "GGUF: cannot open %s", path);
-    struct stat sb;
-    if (fstat(fileno(f), &sb)) {
-        fclose(f);
-        return fail(err, errlen, "GGUF: cannot stat %s", path);
-    }
-    s->fsize = (uint64_t)sb.st_size;
-    char magic[4];
-    uint32_t ver, align = 32;
-    uint64_t nt, nkv;
-    if (!rdn(f, magic, 4) || memcmp(magic, "GGUF", 4) || !rdn(f, &ver, 4) || !rdn(f, &nt, 8) || !rdn(f, &nkv, 8) || ver < 2) {
-        fclose(f);
-        return fail(err, errlen, "GGUF: %s is not GGUF v2+", path);
-    }
-    // every metadata entry takes at least 12 bytes and every tensor entry at least 24: a count beyond that is damage
-    if (nkv > s->fsize / 12 || nt > s->fsize / 24) {
-        fclose(f);
-        return fail(err, errlen, "GGUF: %s: metadata is damaged", path);
-    }
-    for (uint64_t i = 0; i < nkv; i++) {
-        char *k = rstr(f);
-        uint32_t t;
-        const bool ok = k && rdn(f, &t, 4) && skip_value(f, t, &align, k);
-        free(k);
-        if (!ok) {
-            fclose(f);
-            return fail(err, errlen, "GGUF: %s: metadata is damaged", path);
-        }
-    }
-    if (align == 0) {
-        fclose(f);
-        return fail(err, errlen, "GGUF: %s: metadata is damaged", path);
-    }
-    qw_gguf_tensor *nt_arr = realloc(G->t, sizeof *G->t * (size_t)(G->nt + (int)nt + 1));
-    if (!nt_arr) {
-        fclose(f);
-        return fail(err, errlen, "GGUF: out of memory");
-    }
-    G->t = nt_arr;
-    const int t0 = G->nt;
-    for (uint64_t i = 0; i < nt; i++) {
-        qw_gguf_tensor *t = &G->t[G->nt];
-        memset(t, 0, sizeof *t);
-        char *name = rstr(f);
-        bool ok = name && rdn(f, &t->nd, 4) && t->nd <= 4;
-        for (uint32_t d = 0; ok && d < t->nd; d++) ok = rdn(f, &t->dims[d], 8);
-        ok = ok && rdn(f, &t->type, 4) && rdn(f, &t->offset, 8);
-        if (!ok) {
-            free(name);
-            fclose(f);
-            return fail(err, errlen, "GGUF: %s: tensor table is damaged", path);
-        }
-        t->name = name;
-        t->shard = si;
-        t->res_type = -1;
-        t->model = map_name(name, &t->part, &t->kind);
-        G->nt++;
-    }
-    s->version = ver;
-    s->align = align;
-    s->data0 = ((uint64_t)ftello(f) + align - 1) / align * align;
-    fclose(f);
-    for (int i = t0; i < G->nt; i++) { // offsets in the table are relative to the data start
-        qw_gguf_tensor *t = &G->t[i];
-        if (!tensor_bytes(t) || __builtin_add_overflow(t->offset, s->data0, &t->offset)) return fail(err, errlen, "GGUF: %s: tensor table is damaged", path);
-        if (t->offset > s->fsize || t->nbytes > s->fsize - t->offset) return fail(err, errlen, "GGUF: %s: tensor %s lies beyond the end of the file", path, t->name);
-    }
     s->fd = open(path, O_RDONLY);
     if (s->fd < 0) return fail(err, errlen, "GGUF: cannot open %s", path);
+    struct stat sb;
+    if (fstat(s->fd, &sb)) return fail(err, errlen, "GGUF: cannot stat %s", path);
+    s->fsize = (uint64_t)sb.st_size;
     if (s->fsize) {
         s->map = mmap(NULL, s->fsize, PROT_READ, MAP_SHARED, s->fd, 0);
         if (s->map == MAP_FAILED) {
             s->map = NULL;
             return fail(err, errlen, "GGUF: mmap of %s failed", path);
         }
+    }
+    cursor c = {.base = s->map, .size = s->fsize};
+    const uint8_t *magic = cur_take(&c, 4);
+    const uint32_t ver = (uint32_t)cur_uint(&c, 4);
+    const uint64_t ntensors = cur_uint(&c, 8), nmeta = cur_uint(&c, 8);
+    if (c.overrun || memcmp(magic, "GGUF", 4) || ver < 2) return fail(err, errlen, "GGUF: %s is not GGUF v2+", path);
+    // every metadata entry takes at least 12 bytes and every tensor entry at least 24: a count beyond that is damage
+    if (nmeta > s->fsize / 12 || ntensors > s->fsize / 24) return fail(err, errlen, "GGUF: %s: metadata is damaged", path);
+    uint64_t align = 32;
+    static const char ALIGN_KEY[] = "general.alignment";
+    for (uint64_t i = 0; i < nmeta && !c.overrun; i++) {
+        uint64_t klen;
+        const char *key = cur_text(&c, &klen);
+        const uint32_t vt = (uint32_t)cur_uint(&c, 4);
+        const bool is_align = key && klen == sizeof ALIGN_KEY - 1 && !memcmp(key, ALIGN_KEY, klen);
+        cur_skip_value(&c, vt, is_align ? &align : NULL);
+    }
+    align &= 0xffffffffu;
+    if (c.overrun || align == 0) return fail(err, errlen, "GGUF: %s: metadata is damaged", path);
+    qw_gguf_tensor *grown = realloc(G->t, sizeof *G->t * (size_t)(G->nt + (int)ntensors + 1));
+    if (!grown) return fail(err, errlen, "GGUF: out of memory");
+    G->t = grown;
+    const int first = G->nt;
+    for (uint64_t i = 0; i < ntensors; i++) {
+        qw_gguf_tensor *t = &G->t[G->nt];
+        memset(t, 0, sizeof *t);
+        uint64_t nlen;
+        const char *name = cur_text(&c, &nlen);
+        t->nd = (uint32_t)cur_uint(&c, 4);
+        if (t->nd > 4) c.overrun = true;
+        for (uint32_t d = 0; d < t->nd && !c.overrun; d++) t->dims[d] = cur_uint(&c, 8);
+        t->type = (uint32_t)cur_uint(&c, 4);
+        t->offset = cur_uint(&c, 8); // relative to the data start until the loop below
+        if (c.overrun || !(t->name = text_dup(name, nlen))) return fail(err, errlen, "GGUF: %s: tensor table is damaged", path);
+        t->shard = si;
+        t->res_type = -1;
+        t->model = map_name(t->name, &t->part, &t->kind);
+        G->nt++;
+    }
+    s->version = ver;
+    s->align = (uint32_t)align;
+    s->data0 = (c.at + align - 1) / align * align;
+    for (int i = first; i < G->nt; i++) {
+        qw_gguf_tensor *t = &G->t[i];
+        if (!tensor_bytes(t) || __builtin_add_overflow(t->offset, s->data0, &t->offset)) return fail(err, errlen, "GGUF: %s: tensor table is damaged", path);
+        if (t->offset > s->fsize || t->nbytes > s->fsize - t->offset) return fail(err, errlen, "GGUF: %s: tensor %s lies beyond the end of the file", path, t->name);
     }
     return true;
 }

@@ -27,8 +27,9 @@ QW_INTERNAL bool qw_hip_noalloc_scratch(qw_gpu *g, void **ptr, size_t *bytes);
  * it is in use. stream: a hipStream_t, or NULL for the stream qw_gpu_set_stream selected. */
 QW_INTERNAL qw_batch *qw_hip_batch_begin_static(qw_gpu *g, void *stream);
 /* Launches what was recorded, in order, on the recorder's stream and releases the recorder; no copies, no events, no
- * synchronisation. false + qw_hip_last_error if a dispatch was refused (then nothing was launched) or a launch failed. */
-QW_INTERNAL bool qw_hip_batch_launch_static(qw_batch *b);
+ * synchronisation. recorded: whether the caller's recording went through; when it did not, or when a dispatch was
+ * refused, nothing is launched. false + qw_hip_last_error in those cases and when a launch failed. */
+QW_INTERNAL bool qw_hip_batch_launch_static(qw_batch *b, bool recorded);
 
 #ifdef __cplusplus
 }

@@ -49,35 +49,36 @@ static bool fill_line(const double *c, int n, double *out) {
     return true;
 }
 
-double qw_par_cost(const qw_par *p, int B) { // src/engine.c:8764-8781
-    if (B < 1) return 0;
-    double c[QW_PAR_VBMAX + 1], best[QW_PAR_MAX + 1];
-    if (!fill_line(p->cost, QW_PAR_VBMAX, c)) return 0;
-    if (B > QW_PAR_MAX) B = QW_PAR_MAX;
-    best[0] = 0;
+// One dynamic programme serves both questions (src/engine.c:8764-8797). cheapest[n]: least total of group costs c[]
+// that covers n rows; last[n]: the size of the group that completes it. Among equal totals the larger group wins.
+static void cover(const double *c, int B, double *cheapest, int *last) {
+    cheapest[0] = 0;
     for (int n = 1; n <= B; n++) {
-        best[n] = 1e30;
-        for (int b = 1; b <= QW_PAR_VBMAX && b <= n; b++)
-            if (best[n - b] + c[b] < best[n]) best[n] = best[n - b] + c[b];
+        cheapest[n] = 1e30;
+        last[n] = 1;
+        for (int b = 1; b <= QW_PAR_VBMAX && b <= n; b++) {
+            const double total = cheapest[n - b] + c[b];
+            if (total <= cheapest[n]) cheapest[n] = total, last[n] = b;
+        }
     }
-    return best[B];
 }
 
-int qw_par_split(const qw_par *p, int B, int *g) { // src/engine.c:8783-8797
+double qw_par_cost(const qw_par *p, int B) { // the estimate: sizes never measured lie on the line through the measured ones
+    if (B < 1) return 0;
+    double c[QW_PAR_VBMAX + 1], cheapest[QW_PAR_MAX + 1];
+    int last[QW_PAR_MAX + 1];
+    if (!fill_line(p->cost, QW_PAR_VBMAX, c)) return 0;
+    if (B > QW_PAR_MAX) B = QW_PAR_MAX;
+    cover(c, B, cheapest, last);
+    return cheapest[B];
+}
+
+int qw_par_split(const qw_par *p, int B, int *g) { // the cut: a size never measured costs 0, so that it gets tried
     if (B < 1 || B > QW_PAR_MAX) return 0;
-    double best[QW_PAR_MAX + 1];
-    int arg[QW_PAR_MAX + 1], ng = 0;
-    best[0] = 0;
-    for (int n = 1; n <= B; n++) {
-        best[n] = 1e30;
-        arg[n] = 1;
-        for (int b = 1; b <= QW_PAR_VBMAX && b <= n; b++) // "<=": at equal cost the larger group wins; a size never measured costs 0
-            if (best[n - b] + p->cost[b] <= best[n]) {
-                best[n] = best[n - b] + p->cost[b];
-                arg[n] = b;
-            }
-    }
-    for (int n = B; n > 0; n -= arg[n]) g[ng++] = arg[n];
+    double cheapest[QW_PAR_MAX + 1];
+    int last[QW_PAR_MAX + 1], ng = 0;
+    cover(p->cost, B, cheapest, last);
+    for (int n = B; n > 0; n -= last[n]) g[ng++] = last[n];
     return ng;
 }
 
@@ -105,4 +106,25 @@ bool qw_par_choose(const qw_par *p, int rows, int *groups, int *ngroups) {
     }
     const double packed = qw_par_packed_cost(p, rows);
     return packed > 0 && packed < grouped;
+}
+
+// tools/serve.c:1715-1729 of the reference. Two ways to serve n conversations that are decoding: one at a time in time
+// slices (each runs at its own speed, speculative decoding included, and pays for the switches), or all together as one
+// step of n rows. Rates in tokens per second; 0 = not measured.
+bool qw_par_want_slice(const qw_par *p, int n, bool slicing_now, double sliced_rate, const double *solo_rate, double solo_default, double batched_rate) {
+    if (n <= 1) return true;
+    if (n > QW_PAR_SLICE_MAX) return false;
+    double rs = sliced_rate;
+    if (rs <= 0) { // never measured with the switches in: the mean of what each conversation reaches inside its own slice
+        rs = 0;
+        for (int i = 0; i < n; i++) rs += solo_rate && solo_rate[i] > 0 ? solo_rate[i] : solo_default;
+        rs /= n;
+    }
+    double rb = batched_rate;
+    if (rb <= 0) { // never measured: n rows per estimated step
+        const double ms = qw_par_cost(p, n);
+        rb = ms > 0 ? n * 1e3 / ms : 0;
+    }
+    if (rs <= 0 || rb <= 0) return false; // no figures: together (with two or more that is usually the faster way)
+    return rs > rb * (slicing_now ? 0.95 : 1.05); // five per cent either way before the mode changes
 }

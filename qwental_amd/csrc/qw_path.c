@@ -619,7 +619,7 @@ bool qw_path_gg_moe_noalloc(qw_gpu *g, int D, int I, int E, int topk, const qw_m
         return false;
     }
     const bool rec = gg_moe(&p, b, &M, nb, &xb, &s[1], &s[2], &ob, false);
-    const bool ok = qw_hip_batch_launch_static(b) && rec; // also releases the recorder when the recording failed (nothing is launched then)
+    const bool ok = qw_hip_batch_launch_static(b, rec); // also releases the recorder; nothing is launched when the recording failed
     if (!ok) fprintf(stderr, "qw_path_gg_moe_noalloc: %s\n", qw_hip_last_error(g));
     return ok;
 }

@@ -2,6 +2,7 @@
 the host side of the path (include/qw_path.h), the GGUF reader (include/qw_gguf.h) and the step planner
 (include/qw_par.h). Thin by design: one Python
 method per C function."""
+import contextlib
 import ctypes as C
 import os
 
@@ -70,6 +71,7 @@ SYMBOLS = [
     ("qw_hip_buf_upload", _b, [_pb, _sz, _sz]), ("qw_hip_buf_download", _b, [_pb, _sz, _sz]),
     ("qw_hip_buf_write", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_read", _b, [_pb, _sz, _vp, _sz]), ("qw_hip_buf_devptr", _vp, [_pb]),
     ("qw_hip_buf_write_fd", _b, [_pb, _sz, _i, C.c_uint64, _sz]),
+    ("qw_hip_reload_switches", None, [_vp]), ("qw_hip_sync_words", _b, [_vp, _vp, _sz]),
     ("qw_hip_set_repack", None, [_vp, _b]), ("qw_hip_graph_launches", C.c_uint, [_vp]), ("qw_hip_set_graphs", None, [_vp, _b]),
     ("qw_hip_packed_bytes", _sz, [_vp]), ("qw_hip_buf_release_source", _b, [_pb]), ("qw_hip_released_bytes", _sz, [_vp]),
     ("qw_hip_compile_check", _b, [C.c_char_p, _sz, C.c_char_p, _sz, C.c_char_p, _sz]),
@@ -107,6 +109,7 @@ SYMBOLS = [
     ("qw_par_new", _vp, []), ("qw_par_free", None, [_vp]), ("qw_par_observe", None, [_vp, _i, _d]), ("qw_par_group_cost", _d, [_vp, _i]),
     ("qw_par_cost", _d, [_vp, _i]), ("qw_par_split", _i, [_vp, _i, _pi]), ("qw_par_observe_packed", None, [_vp, _i, _d]),
     ("qw_par_packed_cost", _d, [_vp, _i]), ("qw_par_choose", _b, [_vp, _i, _pi, _pi]),
+    ("qw_par_want_slice", _b, [_vp, _i, _b, _d, C.POINTER(_d), _d, _d]),
 ]
 
 
@@ -119,6 +122,8 @@ def load_lib():
         raise RuntimeError("libqwgpu_hip.so is not built: run `python -m qwental_amd.build` (needs hipcc and clang from ROCm)")
     L = C.CDLL(lib_path())
     for name, res, args in SYMBOLS:
+        if os.environ.get("QW_HIP_LIB") and not hasattr(L, name):
+            continue  # another build of the library (experiments) may predate a symbol
         f = getattr(L, name)  # AttributeError if the library lacks a declared symbol
         f.restype = res
         f.argtypes = args
@@ -294,6 +299,30 @@ class Gpu:
 
     def profile(self, on):
         self.L.qw_profile_enable(self.g, on)
+
+    @contextlib.contextmanager
+    def switches(self, **env):
+        """Measurement switches of include/qw_hip_ext.h for the batches begun inside the block: QW_HIP_<NAME> is set to the
+        value given (None: unset), the device reads its switches again, and both are put back afterwards. The library
+        reads the environment only when a device is opened or asked to."""
+        old = {}
+        for k, v in env.items():
+            name = "QW_HIP_" + k.upper()
+            old[name] = os.environ.get(name)
+            if v is None:
+                os.environ.pop(name, None)
+            else:
+                os.environ[name] = str(v)
+        self.L.qw_hip_reload_switches(self.g)
+        try:
+            yield
+        finally:
+            for name, v in old.items():
+                if v is None:
+                    os.environ.pop(name, None)
+                else:
+                    os.environ[name] = v
+            self.L.qw_hip_reload_switches(self.g)
 
     def profile_entries(self, entry_points=True):
         """(name, microseconds) per launch of the last profiled batch; entry-point names, or the callers' kernel names."""
@@ -564,3 +593,8 @@ class Par:
         g, n = (C.c_int * 64)(), C.c_int()
         packed = self.L.qw_par_choose(self.p, rows, g, C.byref(n))
         return bool(packed), list(g[:n.value])
+
+    def want_slice(self, n, slicing_now, sliced_rate=0.0, solo_rates=None, solo_default=0.0, batched_rate=0.0):
+        """Time slices (True) or a joint step (False) for n decoding conversations; rates in tokens/s, 0 = not measured."""
+        arr = (C.c_double * max(n, 1))(*(list(solo_rates) + [0.0] * n)[:max(n, 1)]) if solo_rates is not None else None
+        return bool(self.L.qw_par_want_slice(self.p, n, slicing_now, sliced_rate, arr, solo_default, batched_rate))

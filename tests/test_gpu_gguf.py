@@ -85,19 +85,9 @@ def model(tmp_path_factory):
 @pytest.mark.parametrize("threads", ["1", "3", None])
 def test_resident_bytes_are_the_files_bytes(gpu, model, threads):
     tmp, m, lm, small = model
-    old = os.environ.get("QW_HIP_LOAD_THREADS")
-    if threads is None:
-        os.environ.pop("QW_HIP_LOAD_THREADS", None)
-    else:
-        os.environ["QW_HIP_LOAD_THREADS"] = threads  # one thread: a 28 MB tensor passes four times through two staging buffers
-    try:
+    with gpu.switches(load_threads=threads):  # one thread: a 28 MB tensor passes four times through two staging buffers
         g = q.Gguf(tmp)
         g.load(gpu, "moe,shared,router,lm,lin,attn")
-    finally:
-        if old is None:
-            os.environ.pop("QW_HIP_LOAD_THREADS", None)
-        else:
-            os.environ["QW_HIP_LOAD_THREADS"] = old
     total = 0
     for i in range(len(g)):
         t = g.get(i)

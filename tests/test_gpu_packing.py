@@ -184,14 +184,9 @@ def test_packing_fused_launches_equal_one_per_dispatch(gpu, oracle, dev, tm, T):
     w = rng.uniform(0.05, 1.0, (T, K)).astype(np.float32)
     dl = DeviceLayer(gpu, m, device_only=dev)
     P = T * K
-    old = os.environ.get("QW_HIP_PK_SPLIT")
     res = {}
-    try:
-        for split in (True, False):
-            if split:
-                os.environ["QW_HIP_PK_SPLIT"] = "1"
-            else:
-                os.environ.pop("QW_HIP_PK_SPLIT", None)
+    for split in (True, False):
+        with gpu.switches(pk_split="1" if split else None):
             path = q.Path(gpu, D, I, E, K, 16)
             path.pf_reserve(T, tm)
             xb, ib, wb, ob = gpu.buf_from(x), gpu.buf_from(ids.astype(np.uint32).ravel()), gpu.buf_from(w.ravel()), gpu.buf(T * D * 2)
@@ -208,11 +203,6 @@ def test_packing_fused_launches_equal_one_per_dispatch(gpu, oracle, dev, tm, T):
             for bb in (xb, ib, wb, ob):
                 bb.free()
             path.close()
-    finally:
-        if old is None:
-            os.environ.pop("QW_HIP_PK_SPLIT", None)
-        else:
-            os.environ["QW_HIP_PK_SPLIT"] = old
     a, f = res[True], res[False]
     assert "qwk_moe_prep" in f["names"] and not any(n in f["names"] for n in ("qwk_zero", "qwk_moe_count", "qwk_moe_plan", "qwk_moe_scatter")), f["names"]
     assert "qwk_moe_prep" not in a["names"] and "qwk_moe_scatter" in a["names"] and "qwk_moe_act" in a["names"], a["names"]

@@ -356,12 +356,8 @@ def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
     m["topk"] = K
     x = synth.activations(rng, nb, D)
     dl = DeviceLayer(gpu, m)  # host-shadowed buffers: no tile-major copies
-    old = os.environ.get("QW_HIP_DN_ANY")
-    try:
-        for env, want in ((None, "qwk_dnr_f20_c10_s20_c10"), ("1", "qwk_dn_f20_any_s20")):
-            os.environ.pop("QW_HIP_DN_ANY", None)
-            if env:
-                os.environ["QW_HIP_DN_ANY"] = env
+    for env, want in ((None, "qwk_dnr_f20_c10_s20_c10"), ("1", "qwk_dn_f20_any_s20")):
+        with gpu.switches(dn_any=env):
             path = q.Path(gpu, D, I, E, K, 16)
             gpu.profile(True)
             out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
@@ -370,10 +366,6 @@ def test_iq4_nl_down_in_the_any_shape_kernel(gpu, oracle):
             assert want in names, names
             assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
             path.close()
-    finally:
-        os.environ.pop("QW_HIP_DN_ANY", None)
-        if old is not None:
-            os.environ["QW_HIP_DN_ANY"] = old
     dl.free()
 
 
@@ -539,9 +531,7 @@ def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd
     # with QW_HIP_SIDE=1 (and no profiling) the shared expert's launches run on a side stream beside the router and the routed gate/up: three layers
     # in one batch (three forks and joins), twice, against the same launches kept in line
     def three(side):
-        old = os.environ.pop("QW_HIP_SIDE", None)
-        os.environ["QW_HIP_SIDE"] = "1" if side else "0"  # off by default
-        try:
+        with gpu.switches(side="1" if side else "0"):  # off by default
             xb = gpu.buf_from(x)
             lgs, sels, outs = [gpu.buf(path.logits_bytes(nb)) for _ in range(3)], [gpu.buf(path.sel_bytes(nb)) for _ in range(3)], [gpu.buf(nb * D * 2) for _ in range(3)]
             b = gpu.batch()
@@ -552,10 +542,6 @@ def test_shared_expert_in_other_formats(gpu, oracle, nb, D, I, fsg, fsu, fsd, fd
             for bb in [xb] + lgs + sels + outs:
                 bb.free()
             return res
-        finally:
-            os.environ.pop("QW_HIP_SIDE", None)
-            if old is not None:
-                os.environ["QW_HIP_SIDE"] = old
     inline = three(False)
     assert all(np.array_equal(r, out.view(np.uint16).ravel()) for r in inline)
     for _ in range(2):
@@ -580,13 +566,9 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
     if nb > 1:
         x[nb - 1] = x[0]  # two tokens on the same experts: one product serves both
     dl = DeviceLayer(gpu, m, device_only=dev)
-    old = os.environ.get("QW_HIP_DNC_NB")
-    oldq = os.environ.get("QW_HIP_DNQ_MIN")
-    os.environ["QW_HIP_DNQ_MIN"] = "0"  # the one-launch form by token shares would take these layers from two tokens on
     res = {}
-    try:
-        for lim in (0, limit):
-            os.environ["QW_HIP_DNC_NB"] = str(lim)
+    for lim in (0, limit):
+        with gpu.switches(dnq_min=0, dnc_nb=lim):  # (the one-launch form by token shares would take these layers from two tokens on)
             path = q.Path(gpu, D, I, E, K, 16)
             gpu.profile(True)
             out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
@@ -594,15 +576,6 @@ def test_down_and_combine_in_one_launch(gpu, oracle, nb, limit, fd, fshd, dev, I
             gpu.profile(False)
             res[lim] = (out, lg, path.scratch(2).view(np.float32)[:nb * D].copy(), path.scratch(3).view(np.float32)[:nb * K * D].copy(), names)
             path.close()
-    finally:
-        if old is None:
-            os.environ.pop("QW_HIP_DNC_NB", None)
-        else:
-            os.environ["QW_HIP_DNC_NB"] = old
-        if oldq is None:
-            os.environ.pop("QW_HIP_DNQ_MIN", None)
-        else:
-            os.environ["QW_HIP_DNQ_MIN"] = oldq
     a, b = res[0], res[limit]
     assert any(n.startswith("qwk_dnc_") for n in b[4]) and not any(n.startswith("qwk_dnc_") for n in a[4]), (a[4], b[4])
     assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
@@ -626,13 +599,9 @@ def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E, K, D):
     x = synth.activations(rng, nb, D)
     x[nb - 1] = x[0]  # two tokens of different quarters on the same experts
     dl = DeviceLayer(gpu, m, device_only=True)
-    old = os.environ.get("QW_HIP_DNQ_MIN")
-    oldc = os.environ.get("QW_HIP_DNC_NB")
-    os.environ["QW_HIP_DNC_NB"] = "0"
     res = {}
-    try:
-        for lim in (0, 2):
-            os.environ["QW_HIP_DNQ_MIN"] = str(lim)
+    for lim in (0, 2):
+        with gpu.switches(dnc_nb=0, dnq_min=lim, fuse=0):  # (shapes of the fused layer launch would not reach qwk_dnq_*)
             path = q.Path(gpu, D, I, E, K, 16)
             gpu.profile(True)
             out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
@@ -640,15 +609,6 @@ def test_down_and_combine_by_token_quarters(gpu, oracle, nb, fshd, I, E, K, D):
             gpu.profile(False)
             res[lim] = (out, lg, path.scratch(2).view(np.float32)[:nb * D].copy(), path.scratch(3).view(np.float32)[:nb * K * D].copy(), names)
             path.close()
-    finally:
-        if old is None:
-            os.environ.pop("QW_HIP_DNQ_MIN", None)
-        else:
-            os.environ["QW_HIP_DNQ_MIN"] = old
-        if oldc is None:
-            os.environ.pop("QW_HIP_DNC_NB", None)
-        else:
-            os.environ["QW_HIP_DNC_NB"] = oldc
     a, b = res[0], res[2]
     assert any(n.startswith("qwk_dnq_") for n in b[4]) and "qwk_cmb" not in b[4] and "qwk_cmb" in a[4], (a[4], b[4])
     assert np.array_equal(a[0].view(np.uint16), b[0].view(np.uint16))
@@ -717,6 +677,46 @@ def test_packed_copy_follows_the_source(gpu, oracle):
         bb.free()
 
 
+def test_explicit_write_to_a_host_shadowed_buffer_survives_its_first_bind(gpu, oracle):
+    """A new buffer with a host side is uploaded whole when it is first bound. Bytes put into it through qw_hip_buf_write
+    (or from a file) before that must be what the kernel then reads: the explicit writes keep the host side in step."""
+    N, K, nb = 4096, 2048, 2   # 3.6 MB of weights: more than the size that is uploaded at every submit anyway
+    rng = np.random.default_rng(78)
+    W = synth.matrix(rng, 21, N, K)
+    x = synth.activations(rng, nb, K)
+    rb = synth.row_bytes(21, K)
+    ok, err = gpu.compile("#define qmv_gg qmv_gg_written\n#define GF 21\n#define KD %d\n#define RB %d\n#define NB %d\n#define YT float\n" % (K, rb, nb))
+    assert ok, err
+    import tempfile
+    for how in ("write", "write_fd"):
+        wb = gpu.buf(W.size + (5 << 20))  # host-shadowed, never touched through its host pointer
+        assert wb.size > (4 << 20)
+        src = np.ascontiguousarray(W)
+        if how == "write":
+            assert gpu.L.qw_hip_buf_write(wb.ref(), 0, src.ctypes.data, src.nbytes)
+        else:
+            with tempfile.NamedTemporaryFile() as f:
+                f.write(src.tobytes())
+                f.flush()
+                fd = os.open(f.name, os.O_RDONLY)
+                try:
+                    assert gpu.L.qw_hip_buf_write_fd(wb.ref(), 0, fd, 0, src.nbytes)
+                finally:
+                    os.close(fd)
+        xb, yb = gpu.buf_from(x), gpu.buf(nb * N * 4)
+        b = gpu.batch()
+        b.kernel(gpu.kernel("qmv_gg_written"))
+        b.buf(0, wb)
+        b.buf(3, xb)
+        b.buf(4, yb)
+        b.bytes(5, np.array([N, K, N, 0], np.uint32))
+        b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
+        assert b.end() >= 0, gpu.last_error()
+        assert maxrel(yb.view(np.float32)[:nb * N].reshape(nb, N), oracle.qmv(21, W, N, K, x, f64=True)) <= 1e-5, how
+        for bb in (wb, xb, yb):
+            bb.free()
+
+
 @pytest.mark.parametrize("switch,shape,want", [
     ("QW_HIP_SPLIT_SELECT", (2048, 512, 64, 10, 16, 21, 21, 21, 21, None), "qwk_select"),                 # the selection as a launch of its own
     ("QW_HIP_SHARED_IN_GU", (2048, 512, 64, 10, 16, 21, 21, 21, 21, None), "qwk_gu_f121_c2_s121_c2"),    # shared gate/up inside the gate/up launch
@@ -725,7 +725,7 @@ def test_packed_copy_follows_the_source(gpu, oracle):
     ("QW_HIP_KQ_OWN_LAUNCH", (2560, 640, 32, 10, 9, 21, 20, 12, 20, 23), "qwk_qmvm_swiglu"),              # shared gate/up: a launch of its own beside the front launch
 ])
 def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, oracle, switch, shape, want):
-    """The environment switches that qw_batch_begin reads (include/qw_hip_ext.h) route a layer through kernels that other
+    """The environment switches that qw_gpu_open / qw_hip_reload_switches read (include/qw_hip_ext.h) route a layer through kernels that other
     shapes reach by themselves; with a switch set the named kernel runs and the layer still meets the float64 oracle."""
     D, I, E, K, nb, fgu, fd, fsh, fshd, fshu = shape
     rng = np.random.default_rng(len(switch) + D)
@@ -733,13 +733,9 @@ def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, or
     m["topk"] = K
     x = synth.activations(rng, nb, D)
     dl = DeviceLayer(gpu, m, device_only=switch != "QW_HIP_NL_C4")  # host-shadowed rows: no tile-major copy of the IQ4_NL matrix
-    old = os.environ.get(switch)
     outs = {}
-    try:
-        for on in (False, True):
-            os.environ.pop(switch, None)
-            if on:
-                os.environ[switch] = "1"
+    for on in (False, True):
+        with gpu.switches(**{switch[len("QW_HIP_"):].lower(): "1" if on else None}):
             path = q.Path(gpu, D, I, E, K, 16)
             gpu.profile(True)
             out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
@@ -749,10 +745,6 @@ def test_measurement_switches_select_other_kernels_with_the_same_results(gpu, or
             assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
             outs[on] = out
             path.close()
-    finally:
-        os.environ.pop(switch, None)
-        if old is not None:
-            os.environ[switch] = old
     if switch in ("QW_HIP_SPLIT_SELECT", "QW_HIP_NO_SWIGLU_MATVEC", "QW_HIP_KQ_OWN_LAUNCH"):  # the same products in the same order (the shared gate/up inside
         # the gate/up launch adds a row's blocks one after the other, the front launch per chunk first)
         assert np.array_equal(outs[False].view(np.uint16), outs[True].view(np.uint16))

@@ -137,3 +137,36 @@ def test_groups_or_packing_path():
     assert all(not s.choose(r)[0] for r in (1, 16, 40, 64, 200))
     s.free()
     p.free()
+
+
+def test_time_slices_or_a_joint_step():
+    """qw_par_want_slice, the rule of the reference's tools/serve.c:1715-1729: the trivial counts, the figures it falls
+    back on, and the five per cent either way before the mode changes."""
+    p = q.Par()
+    # one conversation: slices, whatever the figures; more than QW_PAR_SLICE_MAX = 3: a joint step, whatever the figures
+    assert p.want_slice(1, False) and p.want_slice(0, False, batched_rate=1e9)
+    assert not p.want_slice(4, True, sliced_rate=1e9, batched_rate=1.0)
+    # no figure on one side: together
+    assert not p.want_slice(2, True, sliced_rate=100.0)
+    assert not p.want_slice(2, True, batched_rate=100.0)
+    assert not p.want_slice(2, True)
+    # both measured: slices stay while they reach 95 % of the joint rate, and are taken up only above 105 %
+    for n in (2, 3):
+        assert p.want_slice(n, True, sliced_rate=96.0, batched_rate=100.0)
+        assert not p.want_slice(n, True, sliced_rate=94.0, batched_rate=100.0)
+        assert not p.want_slice(n, False, sliced_rate=104.0, batched_rate=100.0)
+        assert p.want_slice(n, False, sliced_rate=106.0, batched_rate=100.0)
+        assert not p.want_slice(n, True, sliced_rate=95.0, batched_rate=100.0)   # the comparison is strict
+    # slices never measured: the mean of the conversations' own rates, the default standing in for a missing one
+    assert p.want_slice(2, False, solo_rates=[150.0, 70.0], solo_default=40.0, batched_rate=100.0)       # mean 110
+    assert not p.want_slice(2, False, solo_rates=[150.0, 0.0], solo_default=40.0, batched_rate=100.0)    # mean 95
+    assert p.want_slice(2, True, solo_rates=[150.0, 0.0], solo_default=42.0, batched_rate=100.0)         # mean 96, already slicing
+    assert p.want_slice(3, False, solo_default=120.0, batched_rate=100.0)                                # nothing per conversation
+    assert not p.want_slice(3, False, solo_default=0.0, batched_rate=100.0)
+    # the joint step never measured: n rows per estimated step from the table of group times
+    feed(p, 2, [10.0])   # a group of two rows takes 10 ms: 200 tokens/s together
+    assert p.cost(2) == 10.0
+    assert p.want_slice(2, False, sliced_rate=211.0) and not p.want_slice(2, False, sliced_rate=209.0)
+    assert p.want_slice(2, True, sliced_rate=191.0) and not p.want_slice(2, True, sliced_rate=189.0)
+    assert p.want_slice(3, False, sliced_rate=3e3 / p.cost(3) * 1.06) and not p.want_slice(3, False, sliced_rate=3e3 / p.cost(3) * 1.04)
+    p.free()
