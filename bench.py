@@ -79,6 +79,21 @@ def model_shape_leg(gpu, layers, steps, warmup, cpu_check):
     return res
 
 
+def ablation_leg(gpu, stack, x, nb, full_us):
+    """Where the dominant launch's time goes, measured in this run: the launch as it is (full_us), the same launch without
+    its arithmetic (QW_HIP_ABLATE: selection, table and activation staging, loads and stores stay; the decoding and the
+    matrix instructions go; its results are meaningless and nothing here looks at them), and — from read_ceiling — a
+    kernel that only reads the same bytes. Microseconds per launch, HIP events around every launch of one step."""
+    with gpu.switches(ablate="1"):
+        stack.step(x, nb)  # (warm: first use of that entry point)
+        gpu.profile(True)
+        stack.step(x, nb)
+        gpu.profile(False)
+        t, n = gpu.profile_mean("qwk_gu_f122")
+    stack.step(x, nb)  # leaves the buffers as a real step leaves them
+    return {"full_us": full_us, "without_arithmetic_us": t * 1e6 if n else None, "launches": n}
+
+
 def committed_traffic():
     """HBM bytes per launch of the dominant kernel as the committed counter summary states them (two rocprofv3
     --pmc runs of this file with --copy-calib, FETCH_SIZE and WRITE_SIZE, scaled by the copy kernel); None without it."""
@@ -550,20 +565,26 @@ def main():
         per_kernel.setdefault(name, []).append(us)
     roof = {"bound": "hbm", "kernel": DOMINANT, "achieved": gu_bytes / mean_s / 1e9 if mean_s > 0 else None, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": gu_bytes / mean_s / 1e9 / HBM_PEAK_GBS if mean_s > 0 else None, "traffic": a.traffic if a.traffic is not None else committed_traffic(),
+            "traffic_source": "--traffic argument (counter runs of this command)" if a.traffic is not None else
+                              "constant from the committed counter summary profiles/moe_stack_b16_hbm_traffic.txt, not measured in this run",
             "launches": n_l, "mean_launch_us": mean_s * 1e6, "algorithmic_bytes_per_launch": gu_bytes}
     line = {"metric": "batched IQ3_S MoE decode tokens/s at B=16 (48-layer FFN stack); achieved HBM GB/s", "value": res[nb]["tokens_per_s"], "unit": "tokens/s",
             "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": res[nb]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "u8 blocks -> f16 matrix-core operands, f32 accumulate", "data": "synthetic (seeded, generated on device)",
+            "vs_baseline": None, "dtype": "u8 blocks -> f16 matrix-core operands, f32 accumulate", "data": "synthetic (seeded, generated on device); block scales d drawn as BASELINE states them times %g (synth.MOE_D_SCALE: the stated |N(0, 0.02)| "
+                    "overflows the binary16 layer output; bytes and work are unchanged)" % synth.MOE_D_SCALE,
             "config": {"workload": "configs[4]: %d-layer MoE FFN stack decode, B=%d, D=2048 I=512 E=512 top-10, IQ3_S experts, shared expert Q8_0 every 4th layer; "
                                    "every layer reads the same x and overwrites one out, launched in order on one stream (a bandwidth bench: no overlap between layers is used)" % (stack.L, nb),
                        "resident_weight_bytes": int(stack.weight_bytes), "packed_copy_bytes": int(gpu.L.qw_hip_packed_bytes(gpu.g)), "released_source_bytes": released, "device": gpu.name()},
             "roofline": roof,
             "read_ceiling": None if released else read_ceiling(gpu, stack, nb),  # it reads the GGUF-order bytes
+            "ablation": ablation_leg(gpu, stack, x, nb, mean_s * 1e6),
             "stack": {"GBps_algorithmic": res[nb]["stack_GBps"], "frac_of_peak": res[nb]["stack_GBps"] / HBM_PEAK_GBS, "gpu_ms_per_step": res[nb]["gpu_ms_per_step"],
                       "mean_unique_experts": res[nb]["mean_U"], "bytes_per_step": res[nb]["bytes_per_step"]},
             "by_batch": {str(k): v for k, v in res.items()},
             "kernel_us_mean": {k: float(np.mean(v)) for k, v in per_kernel.items()},
             "setup_s": setup_s}
+    if line["read_ceiling"]:
+        line["ablation"]["pure_read_of_the_same_bytes_us"] = line["read_ceiling"]["us_per_launch"]
     if not a.quick:
         line["hyper_ffn_step"] = hyper_ffn_leg(gpu, stack, min(a.steps, 10), a.warmup)
         line["ragged_step"] = ragged_steps(gpu, stack)

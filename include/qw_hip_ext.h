@@ -56,8 +56,9 @@ size_t qw_hip_packed_bytes(const qw_gpu *g);
  * such a matrix drops from 2.018 to 1.018 times its bytes. Afterwards the buffer may only be bound as those weights:
  * a dispatch that no existing copy serves (another shape or split, a matrix that was never dispatched, dq_test, any output
  * role) fails the batch with a message, the explicit copy calls return false, qw_hip_buf_devptr gives NULL, and the
- * buffer is otherwise freed as usual. Returns false (and frees nothing) when the buffer has no copy yet or is written by
- * a batch still in flight. Keep shared-expert and router tensors in buffers of their own: they are read in GGUF order. */
+ * buffer is otherwise freed as usual. Returns false (and frees nothing, with a text in qw_hip_last_error) while copies
+ * stand in for only a part of the buffer's bytes (a matrix in it has not been dispatched yet), or when the buffer is
+ * written by a batch still in flight. Keep shared-expert and router tensors in buffers of their own: they are read in GGUF order. */
 bool qw_hip_buf_release_source(qw_buf *b);
 size_t qw_hip_released_bytes(const qw_gpu *g);
 
@@ -79,6 +80,10 @@ unsigned qw_hip_graph_launches(const qw_gpu *g);
  *   QW_HIP_FUSE=1             routed gate/up, down and combine of a layer run as one launch whose workgroups meet at a barrier
  *                             (qwk_gud_*: tile-major IQ3_S rows with D <= 2048, I = 512, top-k <= 10, on stream 0). Off by
  *                             default: the hand-over inside the launch costs what the two launch boundaries cost
+ *   QW_HIP_ABLATE             MEASUREMENT ONLY, results are meaningless: the routed gate/up launch over tile-major IQ3_S rows runs
+ *                             without decoding and matrix instructions (qwk_gu_f122_c2: same selection, staging, loads and
+ *                             stores), so that bench.py can state what the launch costs without its arithmetic
+ *   QW_HIP_HC_ROWS=4|8|16     mix_down rows per workgroup of the hyper-connection's down launch (default: 4 up to twelve tokens, else 8)
  *   QW_HIP_SPIN_LIMIT=n       polls of the barrier word after which a workgroup of that launch stops waiting for the others
  *                             (default 65536, some tenths of a second). A launch that gives up fails its batch with a message
  *                             (negative time from qw_batch_end); the device then keeps its layers as separate launches until

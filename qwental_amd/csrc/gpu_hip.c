@@ -95,7 +95,7 @@ typedef struct {
 typedef struct { qw_hbuf *b; bool out; } qw_use;
 
 // measurement switches: read from the environment by qw_gpu_open (and again by qw_hip_reload_switches), never per batch
-typedef struct { unsigned dnc_nb, dnq_min, spin_limit; int side, load_threads; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split, kq_own, no_fuse, verbose, quiet; } qw_switches;
+typedef struct { unsigned dnc_nb, dnq_min, spin_limit, hc_rows; int side, load_threads; bool dn_any, nl_c4, no_swiglu_matvec, shared_in_gu, split_select, pk_split, kq_own, no_fuse, ablate, verbose, quiet; } qw_switches;
 
 struct qw_batch {
     qw_gpu *g;
@@ -229,6 +229,9 @@ static void read_switches(qw_gpu *g) {
     w->kq_own = getenv("QW_HIP_KQ_OWN_LAUNCH") != NULL; // a K-quant / IQ4 / plain shared expert's gate/up as a launch of its own
     e = getenv("QW_HIP_FUSE"); // 1: routed gate/up, down and combine of a layer as one launch (off unless asked for: measured as no gain)
     w->no_fuse = !(e && e[0] == '1');
+    w->ablate = getenv("QW_HIP_ABLATE") != NULL; // measurement: the routed gate/up launch without its arithmetic (results are meaningless)
+    e = getenv("QW_HIP_HC_ROWS"); // mix_down rows per workgroup of the hyper-connection's down launch: 4, 8 or 16 (0: by token count)
+    w->hc_rows = e ? (unsigned)atoi(e) : 0;
     e = getenv("QW_HIP_SPIN_LIMIT"); // polls after which a workgroup of a fused launch stops waiting for the others
     w->spin_limit = e ? (unsigned)strtoul(e, NULL, 10) : 1u << 16;
     e = getenv("QW_HIP_LOAD_THREADS");
@@ -675,6 +678,9 @@ static void packs_drop(qw_hbuf *h) {
     for (int i = 0; i < g->npacks; i++) {
         qw_pack *p = &g->packs[i];
         if (p->ha == h || p->hb == h) {
+            qw_hbuf *other = p->ha == h ? p->hb : p->ha;
+            if (other && other != h && other->released)
+                fprintf(stderr, "qw_hip: a tile-major copy is dropped whose other source buffer was released: that buffer's matrix can no longer be dispatched\n");
             (void)hipFree(p->dst);
             g->pack_bytes -= p->bytes;
             if (p->ha && p->ha != h) p->ha->npack--;
@@ -715,9 +721,41 @@ size_t qw_hip_packed_bytes(const qw_gpu *g) { return g->pack_bytes; }
 void *qw_hip_buf_devptr(const qw_buf *b) { return b && b->handle && !((qw_hbuf *)b->handle)->released ? ((qw_hbuf *)b->handle)->dptr : NULL; }
 static bool range_ok(const qw_hbuf *h, size_t off, size_t len) { return !h->released && off <= h->size && len <= h->size - off; } // a released buffer has no bytes to copy
 // Free the device bytes of a weight buffer and keep its tile-major copies (include/qw_hip_ext.h).
+// Bytes of h that some tile-major copy was made from: the union of the copies' source ranges inside the buffer.
+static size_t packed_source_bytes(const qw_hbuf *h) {
+    const qw_gpu *g = h->g;
+    enum { MAXIV = 256 };
+    size_t lo[MAXIV], hi[MAXIV];
+    int n = 0;
+    for (int i = 0; i < g->npacks && n + 2 <= MAXIV; i++) {
+        const qw_pack *p = &g->packs[i];
+        const bool nl = p->split == QW_F_PACKED_NL, q6 = p->split == QW_F_PACKED_Q6;
+        const size_t rowb = (size_t)p->nblk * (nl ? 180u : q6 ? 210u : 110u), rows_a = nl || q6 ? 16 : p->split, rows_b = nl || q6 ? 0 : 16 - p->split;
+        if (p->ha == h && p->A) lo[n] = (size_t)((const char *)p->A - (const char *)h->dptr), hi[n] = lo[n] + (size_t)p->ntiles * rows_a * rowb, n++;
+        if (p->hb == h && p->B && rows_b) lo[n] = (size_t)((const char *)p->B - (const char *)h->dptr), hi[n] = lo[n] + (size_t)p->ntiles * rows_b * rowb, n++;
+    }
+    for (int i = 1; i < n; i++) // by start (few intervals: insertion sort)
+        for (int j = i; j > 0 && lo[j] < lo[j - 1]; j--) {
+            const size_t a = lo[j], c = hi[j];
+            lo[j] = lo[j - 1], hi[j] = hi[j - 1], lo[j - 1] = a, hi[j - 1] = c;
+        }
+    size_t total = 0, end = 0;
+    for (int i = 0; i < n; i++) {
+        const size_t from = lo[i] > end ? lo[i] : end;
+        if (hi[i] > from) total += hi[i] - from, end = hi[i];
+    }
+    return total;
+}
 bool qw_hip_buf_release_source(qw_buf *b) {
     qw_hbuf *h = b ? b->handle : NULL;
     if (!h || h->released || !h->npack || h->pending_out) return false;
+    // Every byte of the buffer must have a copy to stand in for it (up to the alignment gaps of an arena: 256 bytes a
+    // copy): a matrix without one could never be dispatched again.
+    const size_t covered = packed_source_bytes(h);
+    if (covered + (size_t)256 * (size_t)h->npack * 2 < h->size) {
+        set_err(h->g, "qw_hip_buf_release_source: tile-major copies stand in for %zu of the buffer's %zu bytes; run every matrix of it once first", covered, h->size);
+        return false;
+    }
     if (hipDeviceSynchronize() != hipSuccess) return false; // a batch in flight may still read the bytes
     if (hipFree(h->dptr) != hipSuccess) { (void)hipGetLastError(); return false; }
     h->released = true; // dptr stays as the key the copies were filed under; nothing dereferences it from here on
@@ -1361,9 +1399,10 @@ static bool tr_gu(qw_batch *b) {
     // With few tiles (one or two tokens: 640 to 1280 of them) every compute unit still gets a workgroup: the waves are
     // numbered wave-major, so the tiles spread over all compute units instead of filling the waves of the first
     // workgroups (48-layer step at one token: gate/up launch 18.3 -> 13.4 us, 615 -> 715 tokens/s).
+    if (b->sw.ablate && fgu == QW_F_PACKED && cg == 2 && !fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c2", QW_F_ABLATE);
     const unsigned grid = umin((unsigned)b->g->ncu, tasks);
     // Tile-major IQ3_S rows of the shape the fused launch is built for: wait for the down dispatch (qwk_gud_*)
-    if (!b->sw.no_fuse && b->sw.side != 1 && fgu == QW_F_PACKED && cg == 2 && !fs && p->D <= 2048 && p->I == 512 && p->topk <= 10 && p->gnb * p->topk <= (int)QW_DNQ_MAXU &&
+    if (!b->sw.no_fuse && !b->sw.ablate && b->sw.side != 1 && fgu == QW_F_PACKED && cg == 2 && !fs && p->D <= 2048 && p->I == 512 && p->topk <= 10 && p->gnb * p->topk <= (int)QW_DNQ_MAXU &&
         b->buf[6].off % 4 == 0) {
         b->pend_gu.valid = true;
         b->pend_gu.a = a;
@@ -1820,8 +1859,11 @@ static bool tr_hc(qw_batch *b) {
     if (f == FAM_HC_DOWN) {
         if (!bind_ptr(b, 4, QW_HC_LR * HCD * 2, false, "mix_down", (void **)&a.Wd) || !bind_ptr(b, 6, nb * QW_HC * QW_HC_PDS * 4, true, "partial sums", (void **)&a.pd)) return false;
         if (a.want_inj && !bind_ptr(b, 5, QW_HC * HCD * 2, false, "inject", (void **)&a.Wi)) return false;
-        const unsigned R = nb <= 4 ? 4 : 16; // rows per workgroup: many workgroups at a few tokens, less re-reading of h at many
-        if (!add_launch(b, R == 4 ? "qwk_hc_down_r4" : "qwk_hc_down_r16", QW_HC_LR / R + (a.want_inj ? 1 : 0), (unsigned)(D / 8), &a, sizeof a)) return false;
+        // rows per workgroup. Measured per launch at D = 2048 (4 / 8 / 16 rows): 6.2 / 6.5 / 7.9 us at one token, 10.0 / 11.7 /
+        // 13.6 at eight, 12.5 / 12.3 / 14.1 at sixteen: many small workgroups beat fewer re-reads of h up to about a dozen tokens
+        unsigned R = nb <= 12 ? 4 : 8;
+        if (b->sw.hc_rows == 4 || b->sw.hc_rows == 8 || b->sw.hc_rows == 16) R = b->sw.hc_rows;
+        if (!add_launch(b, R == 4 ? "qwk_hc_down_r4" : R == 8 ? "qwk_hc_down_r8" : "qwk_hc_down_r16", QW_HC_LR / R + (a.want_inj ? 1 : 0), (unsigned)(D / 8), &a, sizeof a)) return false;
         b->l[b->nl - 1].gy = QW_HC;
         b->l[b->nl - 1].gz = (unsigned)(nb + QW_HC_TG - 1) / QW_HC_TG; // tokens four at a time
         return true;
@@ -1832,7 +1874,9 @@ static bool tr_hc(qw_batch *b) {
         if (a.want_inj && !bind_ptr(b, 7, nb * QW_HC * QW_HC * 4, true, "new inject sums", (void **)&a.injo)) return false;
     } else if (!bind_ptr(b, 5, nb * QW_HC_LR * 4, false, "sx", (void **)&a.sx) || !bind_ptr(b, 6, nb * QW_HC * 4, false, "rs", (void **)&a.rs) ||
                !bind_ptr(b, 7, nb * D * 2, true, "x", (void **)&a.x)) return false;
-    return add_launch(b, f == FAM_HC_UP ? "qwk_hc_up" : "qwk_hc_upv", (unsigned)(D / 8), 256, &a, sizeof a);
+    if (!add_launch(b, f == FAM_HC_UP ? "qwk_hc_up" : "qwk_hc_upv", (unsigned)(D / 8), 256, &a, sizeof a)) return false;
+    b->l[b->nl - 1].gy = (unsigned)(nb + QW_HC_TG - 1) / QW_HC_TG; // tokens four at a time
+    return true;
 }
 
 // bench/moe_bw.c:82-91, 106-112: 0 arena, 1 chunk records at the dispatch's first chunk, 2 sink; grid (slices or row groups, chunks)

@@ -174,7 +174,8 @@ __device__ __forceinline__ h8 qw_q8_cvt(u2 q) {
 // issued as assembly that this bookkeeping does not see. That is safe in the direction that matters: an outstanding
 // store only makes the hardware counter larger than the number of outstanding loads, so "at most N outstanding" still
 // implies that all but the N youngest loads have returned. A store reads its data registers when it is issued, and it
-// has completed when the kernel ends, which is when its readers start.
+// has completed when the kernel ends, which is when its readers start. INVARIANT for every user: what is stored this way
+// is never read back from memory inside the same kernel (the compiler would not wait for the store before such a read).
 __device__ __forceinline__ void qw_store_u16(uint16_t *p, uint16_t v) { asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"((uint32_t)v) : "memory"); }
 __device__ __forceinline__ void qw_store_f32(float *p, float v) { asm volatile("global_store_dword %0, %1, off" : : "v"(p), "v"(v) : "memory"); }
 
@@ -569,6 +570,19 @@ template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
             this->s[b].d = qw_h2f((uint16_t)(odd ? (other | mine << 8) : (mine | other << 8)));
             this->s[b].sc = (w >> 16) & 255;
             this->s[b].qh = w & 0xffff;
+        }
+    }
+};
+
+// QW_F_ABLATE: the same loads and lane moves, no decoding and no matrix instructions (a measurement; see qw_kargs.h).
+template <int NB> struct qw_chunk<QW_F_ABLATE, NB> : qw_chunk<QW_F_PACKED, NB> {
+    static constexpr uint32_t BLK_K = 256, BLK_B = QW_SLAB_BYTES;
+    static constexpr int DEPTH = 3;
+    template <class AF> __device__ __forceinline__ void mac_lean(const u2 *, const AF &, uint32_t, uint32_t, f4 &acc) const {
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const qw_iq3_slice &s = this->s[b];
+            acc[0] += __builtin_bit_cast(float, (s.qs[0] ^ s.qs[1] ^ s.qs[2] ^ s.qs[3] ^ s.sg.x ^ s.sg.y ^ s.qh ^ s.sc) & 0x007fffffu) + s.d;
         }
     }
 };

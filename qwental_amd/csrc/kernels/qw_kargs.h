@@ -206,6 +206,10 @@ typedef struct { /* read-pattern ceiling of a decode layer (the reference's kern
  * (row tile * (16 - split) + n - split): split 16 = one matrix, split 8 = gate rows and up rows side by side. */
 #define QW_SLAB_BYTES 1792u
 #define QW_F_PACKED 121
+/* Measurement only (QW_HIP_ABLATE): the tile-major IQ3_S stream of QW_F_PACKED with the decoding and the matrix
+ * instructions left out - the loaded registers are merely folded into the result, which is therefore meaningless. Times
+ * what the gate/up launch costs without its arithmetic (same selection, table and activation staging, loads, stores). */
+#define QW_F_ABLATE 122
 /* Tile-major copy of IQ4_NL rows (format code QW_F_PACKED_NL; qwk_pack_args with split = QW_F_PACKED_NL, nblk = chunks
  * of ten blocks per row, so the row length is a multiple of 320): every (tile of 16 rows, chunk) becomes
  * QW_NL_CHUNK_BYTES = 16 x 180 contiguous bytes in the lane order of the matrix instruction (lane = row & 15 | k-group

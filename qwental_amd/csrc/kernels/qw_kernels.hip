@@ -32,7 +32,7 @@ __device__ uint32_t *qw_stamp_ptr;
 // wave index in the workgroup, as a scalar (so that task indices and row bases stay in scalar registers)
 __device__ __forceinline__ uint32_t qw_wave() { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 __device__ __forceinline__ uint32_t qw_lane() { return threadIdx.x & 63; }
-constexpr bool qw_has_lut(int f) { return f == 21 || f == QW_F_PACKED; } // formats decoded through the LDS table
+constexpr bool qw_has_lut(int f) { return f == 21 || f == QW_F_PACKED || f == QW_F_ABLATE; } // formats decoded through the LDS table (the ablation copies it too)
 __device__ __forceinline__ uint32_t qw_all_tokens(uint32_t nbr) { return nbr >= 32 ? 0xffffffffu : (1u << nbr) - 1; }
 
 // ================================================================ dq_test (kernels/moe_iq.metal:208-217)
@@ -920,6 +920,7 @@ struct qw_h_global {
     __device__ __forceinline__ void stamp(uint32_t k) const { QW_DSTAMP(k); }
     // column j0 + n of (token, slot): o = its offset in a plane
     __device__ __forceinline__ void put(uint32_t, uint32_t, size_t o, uint16_t hi, uint16_t lo) const {
+        // (stores the compiler does not track: nothing in this kernel may read H back from memory)
         qw_store_u16(H + o, hi);
         qw_store_u16(H + o + hplane, lo);
     }
@@ -933,12 +934,12 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
     const qw_afrag_lds af = {xf, n};
     const uint32_t nl = lane >> 2; // (row, k-group) this lane loads from GGUF rows: (lane >> 2, lane & 3)
     auto rowp = [&](uint32_t task) {
-        const uint32_t u = task / tpe, e = a.shared ? 0 : sc->ue[u];
-        if constexpr (F == QW_F_PACKED) return a.Wg + ((size_t)e * tpe + task % tpe) * a.rowbytes; // the tile's slabs; rowbytes = bytes of a tile
+        const uint32_t u = task / tpe, e = a.shared ? 0 : (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->ue[u]); // (wave-uniform: the row base stays in scalar registers)
+        if constexpr (F == QW_F_PACKED || F == QW_F_ABLATE) return a.Wg + ((size_t)e * tpe + task % tpe) * a.rowbytes; // the tile's slabs; rowbytes = bytes of a tile
         else return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + 8 * (task % tpe) + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
-    qw_task_stream<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
+    qw_task_stream<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED || F == QW_F_ABLATE ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
         c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
@@ -1052,6 +1053,7 @@ QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_s8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_s21_c1)
 // packed IQ3_S routed experts (and shared expert, when it is IQ3_S too)
 #if QW_IN_PART(1)
 QW_GU(121, 2, 0, 1, qwk_gu_f121_c2) QW_GU(121, 2, 121, 2, qwk_gu_f121_c2_s121_c2) QW_GU(121, 2, 8, 16, qwk_gu_f121_c2_s8_c16)
+QW_GU(QW_F_ABLATE, 2, 0, 1, qwk_gu_f122_c2) // measurement: the launch above without its arithmetic
 QW_GU(121, 1, 0, 1, qwk_gu_f121_c1) QW_GU(121, 1, 121, 1, qwk_gu_f121_c1_s121_c1) QW_GU(121, 1, 8, 1, qwk_gu_f121_c1_s8_c1)
 #endif
 
@@ -1253,7 +1255,7 @@ template <int F, int CH, class S> __device__ __forceinline__ void dn_range_run(c
 #pragma unroll
             for (uint32_t j = 0; j < 4; j++) {
                 const uint32_t o = second ? off1[j] : off0[j];
-                if (o != ~0u) qw_store_f32(P + o + r, acc[j]);
+                if (o != ~0u) qw_store_f32(P + o + r, acc[j]); // (untracked store: Pg and Psh are never read back in this kernel)
             }
             acc = f4{0, 0, 0, 0};
         },
@@ -1562,6 +1564,7 @@ __device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, con
                     if (j < nt && ((mk >> j) & 1)) {
                         const uint32_t s = SHARED ? K : (L.slot4[u] >> (8 * j)) & 255;
                         L.part[(j * (K + 1) + s) * rw + col] = acc[j];
+                        // (untracked store: the combine below reads L.part, never Pg or Psh of this launch from memory)
                         qw_store_f32(SHARED ? a.Psh + (size_t)(t0 + j) * a.D + r : a.P + ((size_t)(t0 + j) * K + s) * a.D + r, acc[j]);
                     }
                 }
@@ -2367,6 +2370,10 @@ extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r4(qwk_hc_args a) 
     __shared__ float part[8][QW_HC_TG][17]; // [wave][token][row | squares]
     hc_down_body<4>(a, part);
 }
+extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r8(qwk_hc_args a) {
+    __shared__ float part[8][QW_HC_TG][17];
+    hc_down_body<8>(a, part);
+}
 extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r16(qwk_hc_args a) {
     __shared__ float part[8][QW_HC_TG][17];
     hc_down_body<16>(a, part);
@@ -2414,11 +2421,14 @@ extern "C" __global__ __launch_bounds__(320) void qwk_hc_mid(qwk_hc_args a) {
 }
 #endif
 // Up: mix_up, the gates and the mix over the streams, the write-back of h (kernels/hyper_gg.metal:141-233, 344-).
-// A workgroup of 256 threads takes eight output columns i, one per group of 32 lanes; a lane holds ten low-rank columns
-// of the four mix_up rows s D + i (20 bytes each). GIVEN: sx and rs come from qwk_hc_mid instead of being made here.
+// A workgroup of 256 threads takes eight output columns i, one per group of 32 lanes, and QW_HC_TG tokens (grid y: the
+// token groups; with all tokens in one workgroup a compute unit held four waves that walked sixteen tokens one after
+// the other, and every workgroup repeated the middle step for all of them); a lane holds ten low-rank columns of the
+// four mix_up rows s D + i (20 bytes each). GIVEN: sx and rs come from qwk_hc_mid instead of being made here.
 template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_args &a) {
-    __shared__ float sx[16][QW_HC_LR], rs[16][QW_HC], js[16][QW_HC];
-    const uint32_t tid = threadIdx.x, l32 = tid & 31, i = blockIdx.x * 8 + (tid >> 5);
+    __shared__ float sx[QW_HC_TG][QW_HC_LR], rs[QW_HC_TG][QW_HC], js[QW_HC_TG][QW_HC];
+    const uint32_t tid = threadIdx.x, l32 = tid & 31, i = blockIdx.x * 8 + (tid >> 5), t0 = blockIdx.y * QW_HC_TG;
+    const uint32_t nt = a.nb - t0 < QW_HC_TG ? a.nb - t0 : QW_HC_TG;
     const size_t HCD = (size_t)QW_HC * a.D;
     // the weights first: their round trip overlaps what follows
     uint32_t u[QW_HC][5];
@@ -2428,31 +2438,30 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
 #pragma unroll
         for (int k = 0; k < 5; k++) u[q][k] = wr[k];
     }
-    // lane l of a group owns token l / 4 (and that plus 8) and the stream qw_sum4 leaves with it: its h, out and norm weight
-    // are asked for now as well
+    // lane l < 4 QW_HC_TG of a group owns token l / 4 of the workgroup's and the stream qw_sum4 leaves with it: its h, out
+    // and norm weight are asked for now as well
     const uint32_t ts = l32 / QW_HC, sq = 2 * (l32 & 1) + ((l32 >> 1) & 1);
+    const bool mine = ts < nt;
     const float wn = a.w[(size_t)sq * a.D + i];
-    float hv[2] = {0, 0}, ov[2] = {0, 0};
-#pragma unroll
-    for (uint32_t r = 0; r < 2; r++)
-        if (ts + 8 * r < a.nb) {
-            hv[r] = a.h[(ts + 8 * r) * HCD + (size_t)sq * a.D + i];
-            if (a.apply) ov[r] = qw_h2f(a.out[(size_t)(ts + 8 * r) * a.D + i]);
-        }
+    float hv = 0, ov = 0;
+    if (mine) {
+        hv = a.h[(t0 + ts) * HCD + (size_t)sq * a.D + i];
+        if (a.apply) ov = qw_h2f(a.out[(size_t)(t0 + ts) * a.D + i]);
+    }
     // (before the middle step: its loads then share that step's round trip)
-    if (tid < a.nb * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
+    if (tid < nt * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (t0 + tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
     if (GIVEN) {
-        for (uint32_t j0 = tid; j0 < a.nb * QW_HC_LR; j0 += 8 * blockDim.x) { // eight loads in flight a thread
+        for (uint32_t j0 = tid; j0 < nt * QW_HC_LR; j0 += 8 * blockDim.x) { // eight loads in flight a thread
             float v[8];
 #pragma unroll
-            for (uint32_t e = 0; e < 8; e++) v[e] = j0 + e * blockDim.x < a.nb * QW_HC_LR ? a.sx[j0 + e * blockDim.x] : 0.0f;
+            for (uint32_t e = 0; e < 8; e++) v[e] = j0 + e * blockDim.x < nt * QW_HC_LR ? a.sx[t0 * QW_HC_LR + j0 + e * blockDim.x] : 0.0f;
 #pragma unroll
             for (uint32_t e = 0; e < 8; e++)
-                if (j0 + e * blockDim.x < a.nb * QW_HC_LR) (&sx[0][0])[j0 + e * blockDim.x] = v[e];
+                if (j0 + e * blockDim.x < nt * QW_HC_LR) (&sx[0][0])[j0 + e * blockDim.x] = v[e];
         }
-        if (tid < a.nb * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[tid];
+        if (tid < nt * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[t0 * QW_HC + tid];
     } else {
-        hc_mid(a, 0, a.nb, &rs[0][0], &sx[0][0], blockIdx.x == 0 && a.want_inj ? a.injo : nullptr);
+        hc_mid(a, t0, nt, &rs[0][0], &sx[0][0], blockIdx.x == 0 && a.want_inj ? a.injo : nullptr);
     }
     __syncthreads();
     float v[QW_HC][10];
@@ -2462,8 +2471,8 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
         for (int k = 0; k < 5; k++) v[q][2 * k] = __builtin_bit_cast(float, u[q][k] << 16), v[q][2 * k + 1] = __builtin_bit_cast(float, u[q][k] & 0xffff0000u);
     // mix_up: for every token four dot products of ten, summed over the group's 32 lanes; the lanes of the token's quad
     // keep the sums of their streams
-    float uv[2] = {0, 0};
-    for (uint32_t t = 0; t < a.nb; t++) {
+    float uv = 0;
+    for (uint32_t t = 0; t < nt; t++) {
         float xv[10];
 #pragma unroll
         for (int k = 0; k < 10; k++) xv[k] = sx[t][l32 * 10 + k];
@@ -2475,27 +2484,21 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
             for (int k = 0; k < 10; k++) d[q] = fmaf(v[q][k], xv[k], d[q]);
         }
         const float f = qw_sum4<32>(d[0], d[1], d[2], d[3], l32); // this lane's stream, summed over the group
-        const bool own = ts == (t & 7);
-        uv[0] = own && t < 8 ? f : uv[0];
-        uv[1] = own && t >= 8 ? f : uv[1];
+        uv = ts == t ? f : uv;
     }
     // the gates and the mix over the streams: the four streams of a token are neighbouring lanes
-#pragma unroll
-    for (uint32_t r = 0; r < 2; r++) {
-        const uint32_t t = ts + 8 * r;
-        float m = 0;
-        if (t < a.nb) {
-            float hq = hv[r];
-            if (a.apply) {
-                hq = fmaf(ov[r], js[t][sq], hq);
-                a.h[t * HCD + (size_t)sq * a.D + i] = hq;
-            }
-            m = (hq * rs[t][sq]) * wn / (1.0f + __expf(-uv[r]));
+    float m = 0;
+    if (mine) {
+        float hq = hv;
+        if (a.apply) {
+            hq = fmaf(ov, js[ts][sq], hq);
+            a.h[(t0 + ts) * HCD + (size_t)sq * a.D + i] = hq;
         }
-        m += __shfl_xor(m, 1);
-        m += __shfl_xor(m, 2);
-        if (t < a.nb && sq == 0) a.x[(size_t)t * a.D + i] = qw_f2h(m / QW_HC);
+        m = (hq * rs[ts][sq]) * wn / (1.0f + __expf(-uv));
     }
+    m += __shfl_xor(m, 1);
+    m += __shfl_xor(m, 2);
+    if (mine && sq == 0) a.x[(size_t)(t0 + ts) * a.D + i] = qw_f2h(m / QW_HC);
 }
 #if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_hc_up(qwk_hc_args a) { hc_up_body<false>(a); }

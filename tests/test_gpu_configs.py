@@ -80,6 +80,32 @@ def test_config4_every_layer_of_the_mixed_stack(gpu, oracle, stack8):
     x.free()
 
 
+def test_config4_all_48_layers_at_full_size(gpu, oracle):
+    """BASELINE configs[4] at its full size: the 48-layer stack (about 33 GB resident, every fourth layer's shared expert in
+    Q8_0) at B = 16, every one of the 48 layers against the float32 oracle on the layer's own resident bytes, top-k
+    identical everywhere. (The benchmark's CPU leg makes the same comparison on the layers its time budget reaches.)"""
+    from qwental_amd.stack import MoeStack
+    nb = 16
+    stack = MoeStack(gpu, layers=48, nbmax=16)
+    xh = synth.activations(np.random.default_rng(2024), nb, D)
+    x = gpu.buf_from(xh, device_only=True)
+    assert [f[0] for f in stack.shared_fmt] == [21, 21, 21, 8] * 12
+    worst = 0.0
+    for l in range(stack.L):
+        stack.step(x, nb, nlayers=l + 1)
+        m = stack.layer_weights_host(l)
+        lg = layer_logits(stack, l, nb)
+        assert np.array_equal(oracle.topk_ids(lg, K), oracle.topk_ids(oracle.router(m["Wr"], m["wsg"], xh), K)), l
+        out32, _, _ = oracle.moe_layer_f32(m, lg, xh, 16)
+        err = maxrel(layer_out(stack, nb), out32)
+        worst = max(worst, err)
+        assert err <= TOL, (l, err)
+        del m
+    print("48 layers, worst layer error %.2e" % worst)
+    x.free()
+    stack.free()
+
+
 def test_config3_continuous_batching_step(gpu, oracle, stack8):
     """BASELINE configs[3]: 16 slots with seeded row counts in 1..16 (64 rows), Zipf(1.1) routing forced through the
     logits. The rows go through the decode path in groups of 16 (every group against the float64 layer) and through

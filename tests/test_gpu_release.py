@@ -61,3 +61,39 @@ def test_release_keeps_results_and_refuses_the_rest(gpu):
     for bb in (y, yb, x):
         bb.free()
     stack.free()
+
+
+def test_release_waits_until_every_matrix_of_the_buffer_has_a_copy(gpu, oracle):
+    """Two matrices in one buffer: with a tile-major copy of only the first, the release is refused (the second could never
+    be dispatched again) and says why; once both have been through a dispatch it goes through and both still compute."""
+    import qwental_amd as q
+    from qwental_amd import Tensor
+    from helpers import maxrel
+    L = gpu.L
+    N, K, nb = 512, 1024, 3
+    rng = np.random.default_rng(31)
+    Wa, Wb = synth.matrix(rng, 21, N, K), synth.matrix(rng, 21, N, K)
+    x = synth.activations(rng, nb, K)
+    wb = gpu.buf_from(np.concatenate([Wa.ravel(), Wb.ravel()]), device_only=True)
+    xb, ya, yb = gpu.buf_from(x), gpu.buf(nb * N * 4), gpu.buf(nb * N * 4)
+    path = q.Path(gpu, 2048, 512, 8, 2, 16)
+
+    def run(which):
+        b = gpu.batch()
+        if which in ("a", "both"):
+            path.qmv_gg(b, Tensor(wb, 21), N, K, xb, ya, nb)
+        if which in ("b", "both"):
+            path.qmv_gg(b, Tensor(wb, 21, Wa.size), N, K, xb, yb, nb)
+        assert b.end() >= 0, gpu.last_error()
+
+    run("a")
+    assert not L.qw_hip_buf_release_source(wb.ref())
+    assert "stand in for" in gpu.last_error()
+    run("b")
+    assert L.qw_hip_buf_release_source(wb.ref()), gpu.last_error()
+    run("both")
+    for y, W in ((ya, Wa), (yb, Wb)):
+        assert maxrel(y.view(np.float32)[:nb * N].reshape(nb, N), oracle.qmv(21, W, N, K, x, f64=True)) <= 1e-5
+    for bb in (wb, xb, ya, yb):
+        bb.free()
+    path.close()
