@@ -23,7 +23,7 @@
 #include <unistd.h>
 
 static const unsigned char qw_code_object[] = {
-#embed "qw_kernels_gfx950.hsaco"
+#embed <qw_kernels_gfx950.hsaco>
 };
 
 #define QW_DNQ_MIN_DEFAULT 2u // token count from which down + combine run as one launch of token quarters (qwk_dnq_*)
@@ -420,6 +420,9 @@ static bool def_int(const qw_def *d, int n, const char *name, int *out) {
 static bool fmt_ok(int f) { return f == 8 || f == 21; } // formats of the MoE kernels
 // formats of the multi-format dense matvec: binary16, Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS, bfloat16 (src/gguf.c:15-25)
 static bool kq_ok(int f) { return f == 1 || f == 12 || f == 13 || f == 14 || f == 20 || f == 23 || f == 30; }
+// the other quantised types the reference's MoE kernels take (kernels/moe_gg.metal:336-395): served by the kernels whose
+// type is an argument (qwk_gu_rt*, qwk_dn_rt)
+static bool rt_ok(int f) { return f == 12 || f == 13 || f == 14 || f == 20 || f == 23; }
 static int fmt_qb(int f) { return f == 1 || f == 30 || f == 8 || f == 20 ? 32 : 256; } // values per decoding unit (plain rows: 32 at a time)
 static int fmt_bb(int f) {
     switch (f) {
@@ -533,13 +536,13 @@ bool qw_gpu_compile(qw_gpu *g, const char *src, size_t len, char *err, size_t er
             if (!reg_kernel(g, d, n, "moe_pre_gg", FAM_PRE, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 2) {
             if (!def_int(d, n, "FGU", &p.fgu) || !def_int(d, n, "FSD", &p.fsd)) FAIL("moe_gu_gg: FGU, FSD missing");
-            if (!fmt_ok(p.fgu) || !(fmt_ok(p.fsd) || p.fsd == 20)) FAIL("moe_gu_gg: types %d/%d have no gfx950 build (have 8, 21; shared down also 20)", p.fgu, p.fsd);
-            if (p.fsd == 21 && p.I % 256) FAIL("moe_gu_gg: I %d does not fit IQ3_S shared down rows", p.I);
+            if (!(fmt_ok(p.fgu) || rt_ok(p.fgu)) || !(fmt_ok(p.fsd) || rt_ok(p.fsd))) FAIL("moe_gu_gg: types %d/%d have no gfx950 build (have 8, 12, 13, 14, 20, 21, 23)", p.fgu, p.fsd);
+            if (p.I % fmt_qb(p.fsd)) FAIL("moe_gu_gg: I %d does not fit shared down rows of type %d", p.I, p.fsd);
             if (!reg_kernel(g, d, n, "moe_gu_gg", FAM_GU, &p, err, errlen)) { ok = false; goto out; }
         } else if (part == 3) {
             if (!def_int(d, n, "FD", &p.fd)) FAIL("moe_dn_gg: FD missing");
-            if (!fmt_ok(p.fd) && p.fd != 20) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 20, 21)", p.fd);
-            if (p.fd == 21 && p.I % 256) FAIL("moe_dn_gg: I %d does not fit IQ3_S rows", p.I);
+            if (!fmt_ok(p.fd) && !rt_ok(p.fd)) FAIL("moe_dn_gg: type %d has no gfx950 build (have 8, 12, 13, 14, 20, 21, 23)", p.fd);
+            if (p.I % fmt_qb(p.fd)) FAIL("moe_dn_gg: I %d does not fit rows of type %d", p.I, p.fd);
             if (!reg_kernel(g, d, n, "moe_dn_gg", FAM_DN, &p, err, errlen) || !reg_kernel(g, d, n, "moe_cmb_gg", FAM_CMB, &p, err, errlen)) { ok = false; goto out; }
         } else if (part != 5) FAIL("moe_gg: GG_PART %d has no gfx950 build (have 0..3, 5 and GG_ROUTER)", part);
     }
@@ -1381,6 +1384,12 @@ static bool tr_gu(qw_batch *b) {
         b->pend_sel.valid = false;
     } else if (!flush_select(b)) return false;
     int fgu = p->fgu;
+    const bool rt = rt_ok(fgu); // a type the kernel takes as an argument: one block a chunk, the shared expert's rows in GGUF order
+    if (rt) {
+        if (fs && fs != 8 && fs != 21) return fail(b, "moe_gu_gg: gate/up types %d (routed) / %d (shared) have no common gfx950 kernel", fgu, fs);
+        a.fgu = (uint32_t)fgu;
+        cg = cs = 1;
+    }
     if (fgu == 21) { // tile-major copies of the IQ3_S rows, made at first use
         const uint32_t nblk = (uint32_t)p->D / 256, tileb = nblk * QW_SLAB_BYTES;
         const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wg, b->buf[1].h, a.Wu, (uint64_t)p->E * (uint64_t)(p->I / 8), nblk, a.rowbytes, 8);
@@ -1393,7 +1402,10 @@ static bool tr_gu(qw_batch *b) {
     }
     if ((b->buf[0].h->released || b->buf[1].h->released) && fgu != QW_F_PACKED) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     char fn[64];
-    if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", fgu, cg, fs, cs);
+    if (rt) {
+        if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_rt_s%d_c1", fs);
+        else fname_fmt(fn, sizeof fn, "qwk_gu_rt");
+    } else if (fs) fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d_s%d_c%d", fgu, cg, fs, cs);
     else fname_fmt(fn, sizeof fn, "qwk_gu_f%d_c%d", fgu, cg);
     const unsigned tasks = umin((unsigned)p->E, nbr * (unsigned)p->topk) * (unsigned)(p->I / 8) + (fs ? (unsigned)p->I / 8 : 0);
     // With few tiles (one or two tokens: 640 to 1280 of them) every compute unit still gets a workgroup: the waves are
@@ -1492,6 +1504,14 @@ static bool tr_dn_inner(qw_batch *b) {
     }
     const unsigned umax = umin((unsigned)p->E, nbr * (unsigned)p->topk);
     int fd = p->fd;
+    // A pair of types without a build of its own (Q4_K, Q5_K, Q6_K or IQ4_XS on either side; IQ4_NL beside IQ3_S): the
+    // kernel that takes both types as arguments, rows in GGUF order.
+    const bool kq_d = rt_ok(fd) && fd != 20, kq_s = rt_ok(fs) && fs != 20;
+    if (kq_d || kq_s || ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8)))) {
+        if (rel) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
+        a.fd = (uint32_t)fd, a.fsd = (uint32_t)fs;
+        return add_launch(b, "qwk_dn_rt", persistent_grid(b->g, umax * (unsigned)(p->D / 16) + (unsigned)p->D / 16, QW_WAVES_DN), 64 * QW_WAVES_DN, &a, sizeof a);
+    }
     if (fd == 21 && p->I <= 512) {
         const uint32_t nblk = (uint32_t)p->I / 256, tileb = nblk * QW_SLAB_BYTES;
         const uint8_t *pk = get_pack(b, b->buf[0].h, a.Wd, NULL, NULL, (uint64_t)p->E * (uint64_t)(p->D / 16), nblk, a.rowbytes, 16);
@@ -1505,8 +1525,7 @@ static bool tr_dn_inner(qw_batch *b) {
     if (rel && fd != QW_F_PACKED && fd != 20) return fail(b, "%s: the GGUF-order bytes of the weights were released and no tile-major copy serves this dispatch", b->k->name);
     char fn[48], sfx[16] = "";
     if (fs) fname_fmt(sfx, sizeof sfx, "_s%d", fs);
-    // IQ4_NL routed rows: the shared expert's may be IQ4_NL or Q8_0 beside them
-    if ((fd == 20 || fs == 20) && (fd != 20 || (fs != 0 && fs != 20 && fs != 8))) return fail(b, "moe_dn_gg: down types %d (routed) / %d (shared) have no common gfx950 kernel", fd, fs);
+    // (IQ4_NL routed rows from here on have no shared expert beside them, or one in IQ4_NL or Q8_0)
     if (fd == 20 && p->I <= 640 && !b->sw.dn_any) { // the range kernel with rows of up to 640 staged
         if (p->I % 320 == 0) { // tile-major copies, as for IQ3_S rows (the shared expert's only together with the routed ones)
             const uint32_t nch = (uint32_t)p->I / 320, tileb = nch * QW_NL_CHUNK_BYTES;

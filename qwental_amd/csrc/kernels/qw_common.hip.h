@@ -246,6 +246,8 @@ struct qw_afrag_lds {
     static constexpr bool has_lo = false;
     __device__ __forceinline__ h8 hi(uint32_t koff) const { return __builtin_bit_cast(h8, xf[(koff >> 3) * 16 + m]); }
     __device__ __forceinline__ h8 lo(uint32_t) const { return h8{}; }
+    __device__ __forceinline__ h4 hi4(uint32_t koff) const { return __builtin_bit_cast(h4, ((const u2 *)xf)[((koff >> 3) * 16 + m) * 2 + ((koff >> 2) & 1)]); } // koff a multiple of 4
+    __device__ __forceinline__ h4 lo4(uint32_t) const { return h4{}; }
 };
 
 // Two planes (hi + lo) staged the same way.

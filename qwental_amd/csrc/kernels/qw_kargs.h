@@ -93,6 +93,8 @@ typedef struct {
     /* logits != NULL: the selection has not been made yet; every workgroup makes it from the logits [nbr][E + 1] for
      * itself and workgroup 0 also writes the record to sel (the later kernels of the layer read it from there) */
     const float *logits;
+    /* qwk_gu_rt*: the routed rows' ggml type (12, 13, 14, 20 or 23), chosen when the kernel runs */
+    uint32_t fgu, pad_fgu;
 } qwk_gu_args;
 
 /* down projection. routed: Pg[t][slot][row] for the tokens in mask[u]; shared != 0: Psh[t][row] from slot topk. */
@@ -112,6 +114,9 @@ typedef struct {
     uint16_t *out;
     /* qwk_dnq_*: quarters of four tokens (nq of them) and weight tiles per workgroup (tpw: 1 or 2) */
     uint32_t nq, tpw;
+    /* qwk_dn_rt: the ggml types of the routed and of the shared down rows (0: no shared expert in this launch),
+     * chosen when the kernel runs */
+    uint32_t fd, fsd;
 } qwk_dn_args;
 /* Down + combine with a quarter of the tokens per workgroup (qwk_dnq_*): limits of the staged H rows */
 #define QW_DNQ_ROWS 44u /* 4 tokens x (topk + 1) rows, topk <= 10 */
@@ -218,6 +223,8 @@ typedef struct { /* read-pattern ceiling of a decode layer (the reference's kern
  *   [2048, 2560) blocks 8..9:  8 bytes per lane      [2560, 2880)  d of the ten blocks, 20 bytes per row
  * A wave reads a chunk with three fully coalesced loads plus 20 bytes of scales per lane. */
 #define QW_F_PACKED_NL 120
+/* Template argument of the kernels whose routed format is chosen when they run (qwk_gu_rt*: qwk_gu_args.fgu): not a format. */
+#define QW_F_RT 99
 #define QW_NL_CHUNK_BYTES 2880u
 /* Tile-major copy of Q6_K rows (format code QW_F_PACKED_Q6; qwk_pack_args with split = QW_F_PACKED_Q6, nblk = blocks a
  * row): per (tile of 16 rows, block of 256 values) QW_Q6_SLAB_BYTES = 16 x 210 contiguous bytes in the lane order of the

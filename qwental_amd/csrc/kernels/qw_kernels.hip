@@ -19,9 +19,21 @@
 #ifdef QW_STAMPS // working builds only: time stamps (10 ns units) of thread 0 of every workgroup, 16 words a workgroup, where the host points this
 extern "C" __device__ uint32_t *qw_stamp_ptr;
 __device__ uint32_t *qw_stamp_ptr;
+#if QW_STAMPS == 2 // only the routed gate/up launch: every wave's end (slots 0 .. 11), the workgroup's entry (12) and selection (13)
+#define QW_DSTAMP(k) do {} while (0)
+#define QW_WSTAMP(k) do { if (qw_stamp_ptr && (threadIdx.x & 63) == 0) qw_stamp_ptr[512 + 16 * blockIdx.x + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#else
 #define QW_DSTAMP(k) do { if (threadIdx.x == 0 && qw_stamp_ptr) qw_stamp_ptr[512 + 16 * blockIdx.x + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#define QW_WSTAMP(k) do {} while (0)
+#endif
 #else
 #define QW_DSTAMP(k) do {} while (0)
+#define QW_WSTAMP(k) do {} while (0)
+#endif
+#ifdef QW_STAMPS
+#define QW_WG_END_STAMP(k) do { __syncthreads(); QW_DSTAMP(k); } while (0)
+#else
+#define QW_WG_END_STAMP(k) do {} while (0)
 #endif
 
 #define QW_WG 512          // threads per workgroup of the down and front kernels (8 waves)
@@ -669,6 +681,7 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
     for (int t = 0; t < T; t++)
 #pragma unroll
         for (int j = 0; j < PER; j++) k[t][j] = __builtin_bit_cast(uint32_t, logits[(size_t)tok[t] * (E + 1) + lane * PER + j]);
+    QW_DSTAMP(12);
     issued();
     QW_DSTAMP(13);
 #pragma unroll
@@ -716,7 +729,6 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
         for (int j = 0; j < PER; j++)
             if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], lane * PER + j};
     }
-    QW_DSTAMP(14);
     uint32_t mk[T], me[T], rank[T];
 #pragma unroll
     for (int t = 0; t < T; t++) {
@@ -802,6 +814,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
     if (tid < 8) s.lead[tid] = 0;
     for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
+    QW_DSTAMP(11);
     if (fast) { // two tokens per wave at a time when there are more tokens than waves; lgs gives a wave 288 dwords
         uint32_t *ws = (uint32_t *)lgs + 288 * wave;
         const uint32_t trot = a.nbr ? blockIdx.x % a.nbr : 0; // the workgroups of a launch read the tokens' logits in different orders
@@ -972,7 +985,9 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 template <int FGU, int CHGU, int FSG, int CHSG, class HS, class SEL>
 __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss, HS &hs, bool all_w, SEL selected) {
     bool staged = false, tabled = false;
+    if (threadIdx.x == 0) QW_WSTAMP(12);
     QW_DSTAMP(0);
+    if constexpr (FGU == QW_F_RT) qw_kq_tab_build((uint32_t *)(lut + (qw_has_lut(FSG) ? QW_LUT_ENTRIES : 0))); // (published by the barriers below)
     if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
         if (qw_select_fast_e(a.E)) {
@@ -989,7 +1004,6 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
             }, all_w);
             qw_lds_arrive();
             __syncthreads();
-            hs.stamp(10);
             staged = early;
             tabled = true;
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
@@ -1009,6 +1023,7 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
         __syncthreads();
     }
     selected();
+    if (threadIdx.x == 0) QW_WSTAMP(13);
     QW_DSTAMP(1);
     auto ready = [&] {
         if (staged) return;
@@ -1032,14 +1047,26 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
         }
     }
     // the waves that did a shared tile come last in the routed deal, so that the work stays level
-    gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready, hs);
+    if constexpr (FGU == QW_F_RT) { // the other GGUF types, one block a chunk; their byte table lies behind the IQ3_S table
+        const u2 *tab = lut + (qw_has_lut(FSG) ? QW_LUT_ENTRIES : 0);
+        switch (a.fgu) {
+        case 12: gu_tasks<12, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        case 13: gu_tasks<13, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        case 14: gu_tasks<14, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        case 20: gu_tasks<20, 8>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        case 23: gu_tasks<23, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        default: break; // (the host launches this kernel for these five only)
+        }
+    } else gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready, hs);
+    QW_WSTAMP(qw_wave());
     QW_DSTAMP(2);
 }
 #define QW_GU(FGU, CHGU, FSG, CHSG, NAME)                                                                 \
     extern "C" __global__ __launch_bounds__(QW_WG_GU) void NAME(qwk_gu_args a) {                             \
-        __shared__ struct { u2 lut[(qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; qw_sel_scratch ss; } L; \
+        __shared__ struct { u2 lut[((qw_has_lut(FGU) || qw_has_lut(FSG)) ? QW_LUT_ENTRIES : 0) + (FGU == QW_F_RT ? QW_KQ_TAB / 2 : 1)]; u4 xf[QW_XF_MAXK * 2]; qw_sel_cache sc; qw_sel_scratch ss; } L; \
         qw_h_global hs = {a.H, a.hplane};                                                                      \
         gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc, &L.ss, hs, false, [] {});                           \
+        QW_WG_END_STAMP(10);                                                                                    \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
 #if QW_IN_PART(1)
@@ -1055,6 +1082,10 @@ QW_GU(8, 1, 8, 1, qwk_gu_f8_c1_s8_c1) QW_GU(8, 1, 21, 1, qwk_gu_f8_c1_s21_c1)
 QW_GU(121, 2, 0, 1, qwk_gu_f121_c2) QW_GU(121, 2, 121, 2, qwk_gu_f121_c2_s121_c2) QW_GU(121, 2, 8, 16, qwk_gu_f121_c2_s8_c16)
 QW_GU(QW_F_ABLATE, 2, 0, 1, qwk_gu_f122_c2) // measurement: the launch above without its arithmetic
 QW_GU(121, 1, 0, 1, qwk_gu_f121_c1) QW_GU(121, 1, 121, 1, qwk_gu_f121_c1_s121_c1) QW_GU(121, 1, 8, 1, qwk_gu_f121_c1_s8_c1)
+#endif
+// routed rows of the other GGUF types (Q4_K, Q5_K, Q6_K, IQ4_NL, IQ4_XS: kernels/moe_gg.metal:336-395), the type an argument
+#if QW_IN_PART(1)
+QW_GU(QW_F_RT, 1, 0, 1, qwk_gu_rt) QW_GU(QW_F_RT, 1, 21, 1, qwk_gu_rt_s21_c1) QW_GU(QW_F_RT, 1, 8, 1, qwk_gu_rt_s8_c1)
 #endif
 
 // ================================================================ front part of a layer (kernels/moe_gg.metal:534-590)
@@ -1149,11 +1180,13 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
 #define QW_PRE(WF, F, CH, NAME)                                                                          \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {                           \
         __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[(QW_WG / 64) * 64]; } L; \
+        QW_DSTAMP(3);                                                                                   \
         if (blockIdx.x < a.nrouter) {                                                                   \
             if (WF == 1) pre_router_mfma(a.r, L.xf, L.part);                                            \
             else pre_router<WF>(a, L.xf);                                                               \
+            QW_DSTAMP(4);                                                                               \
         }                                                                                               \
-        else if (F != 0) pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part);                              \
+        else if (F != 0) { pre_shared<F ? F : 8, CH>(a, L.lut, L.xf, L.part); QW_DSTAMP(5); }            \
     }
 #if QW_IN_PART(2)
 QW_PRE(1, 0, 1, qwk_pre_w1) QW_PRE(30, 0, 1, qwk_pre_w30)
@@ -1584,6 +1617,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
     const uint32_t base = a.nbr / nq, rem = a.nbr % nq, t0 = q * base + (q < rem ? q : rem);
     uint32_t nt = base + (q < rem ? 1 : 0);
     if (nt > 4) nt = 4; // (the host admits 16 tokens in four quarters, 8 in two)
+    QW_DSTAMP(6);
     // one memory round trip: the record (U, experts, masks, this quarter's slot bytes and gating weights) and the table,
     // through registers (a workgroup has nothing else to do meanwhile, and plain loads move more bytes per clock
     // than the direct ones)
@@ -1617,6 +1651,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         }
     }
     __syncthreads();
+    QW_DSTAMP(7);
     // the unique experts this quarter's tokens picked, in record order: every wave makes the whole list (all write the
     // same values to the same places), so that none waits for another before it asks for its first weights
     uint32_t nv = 0;
@@ -1656,6 +1691,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         for (uint32_t it = 0; it < PER; it++)
             if (at[it] != ~0u) L.hrows[at[it]] = t[it];
         __syncthreads();
+        QW_DSTAMP(8);
     };
     // the routed experts first (every wave has tiles there, so every wave's first weights are on their way before the
     // rows are asked for); the shared expert's tiles go to the waves that the routed deal gave one tile fewer
@@ -1665,6 +1701,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, 1, nv * tpw, ready);
     }
     ready(); // (for symmetry only: both runs call it, with or without tiles)
+    QW_DSTAMP(9);
     __syncthreads();
     for (uint32_t j = tid; j < nt * rw; j += blockDim.x) { // rank order, then the shared expert (qwk_cmb's arithmetic)
         const uint32_t t = j >> (4 + __builtin_ctz(tpw)), i = j & (rw - 1), r = g * rw + i;
@@ -1677,6 +1714,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         o = __builtin_fmaf(w[K], sh, o);
         a.out[(size_t)(t0 + t) * a.D + r] = qw_f2h(o);
     }
+    QW_DSTAMP(14);
 }
 #define QW_DNQ(F, CH, FSD, CHSD, NAME)                                                              \
     extern "C" __global__ __launch_bounds__(QW_WG_DN) void NAME(qwk_dn_args a) {                    \
@@ -1867,18 +1905,10 @@ QW_GUD(0, 1, qwk_gud_f121_c2) QW_GUD(121, 2, qwk_gud_f121_c2_s121_c2) QW_GUD(8, 
 #endif
 
 // Any I (multiple of the block size): one tile at a time, operand A straight from global memory.
-template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+template <int F> __device__ __forceinline__ void dn_any_tiles(const qwk_dn_args &a, const u2 *lut, const qw_sel_cache *sc, uint32_t w0, uint32_t nw) {
     typedef qw_chunk<F, 1> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
-    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
-    if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook (IQ3_S never meets it here)
-    qw_sel_load(*sc, a.sel, K, gnb);
-    __syncthreads();
-    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
-    if (FSD != 0) {
-        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, 1>(a, lut, w0, nw);
-    }
-    const uint32_t cpr = a.I / C::BLK_K;
+    const uint32_t tpe = a.D / 16, ntasks = sc->U * tpe, cpr = a.I / C::BLK_K;
     for (uint32_t task = w0; task < ntasks; task += nw) {
         const uint32_t u = task / tpe, r = 16 * (task % tpe) + n, m = sc->mask[u];
         qw_afrag_glb<true> af = {nullptr, nullptr};
@@ -1897,6 +1927,54 @@ template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_
         }
     }
 }
+template <int F, int FSD> __device__ __forceinline__ void dn_any_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+    if (F == 21 || FSD == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    if (F == 20 || FSD == 20) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook (IQ3_S never meets it here)
+    qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+    __syncthreads();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x /* wave-major: see gu_body */;
+    if (FSD != 0) {
+        if (a.Wsd) shared_down_tiles<FSD == 0 ? 8 : FSD, 1>(a, lut, w0, nw);
+    }
+    dn_any_tiles<F>(a, lut, sc, w0, nw);
+}
+// The same with both ggml types as arguments (qwk_dn_args.fd, fsd): every pair of types the reference's kernel takes
+// (kernels/moe_gg.metal:336-395) that has no build of its own above. IQ3_S reads the big table, the 4-bit codebooks the
+// byte table behind it.
+__device__ __forceinline__ void dn_rt_body(const qwk_dn_args &a, u2 *lut, qw_sel_cache *sc) {
+    const u2 *tab = lut + QW_LUT_ENTRIES;
+    if (a.fd == 21 || a.fsd == 21) qw_lut_copy(lut, (const u2 *)a.glut);
+    qw_kq_tab_build((uint32_t *)tab);
+    qw_sel_load(*sc, a.sel, a.topk, a.gnb);
+    __syncthreads();
+    const uint32_t nw = gridDim.x * (blockDim.x >> 6), w0 = qw_wave() * gridDim.x + blockIdx.x;
+    if (a.Wsd) switch (a.fsd) {
+        case 8: shared_down_tiles<8, 1>(a, lut, w0, nw); break;
+        case 21: shared_down_tiles<21, 1>(a, lut, w0, nw); break;
+        case 20: shared_down_tiles<20, 1>(a, tab, w0, nw); break;
+        case 12: shared_down_tiles<12, 1>(a, tab, w0, nw); break;
+        case 13: shared_down_tiles<13, 1>(a, tab, w0, nw); break;
+        case 14: shared_down_tiles<14, 1>(a, tab, w0, nw); break;
+        case 23: shared_down_tiles<23, 1>(a, tab, w0, nw); break;
+        default: break; // (the host launches this kernel for these seven only)
+        }
+    switch (a.fd) {
+    case 8: dn_any_tiles<8>(a, lut, sc, w0, nw); break;
+    case 21: dn_any_tiles<21>(a, lut, sc, w0, nw); break;
+    case 20: dn_any_tiles<20>(a, tab, sc, w0, nw); break;
+    case 12: dn_any_tiles<12>(a, tab, sc, w0, nw); break;
+    case 13: dn_any_tiles<13>(a, tab, sc, w0, nw); break;
+    case 14: dn_any_tiles<14>(a, tab, sc, w0, nw); break;
+    case 23: dn_any_tiles<23>(a, tab, sc, w0, nw); break;
+    default: break;
+    }
+}
+#if QW_IN_PART(2)
+extern "C" __global__ __launch_bounds__(QW_WG) void qwk_dn_rt(qwk_dn_args a) {
+    __shared__ struct { u2 lut[QW_LUT_ENTRIES + QW_KQ_TAB / 2]; qw_sel_cache sc; } L;
+    dn_rt_body(a, L.lut, &L.sc);
+}
+#endif
 #define QW_DN_ANY(F, FSD, NAME)                                                       \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_dn_args a) {         \
         __shared__ struct { u2 lut[(F == 21 || FSD == 21) ? QW_LUT_ENTRIES : (F == 20 || FSD == 20) ? QW_KQ_TAB / 2 : 1]; qw_sel_cache sc; } L; \

@@ -94,7 +94,7 @@ template <> struct qw_kq<12> {
         c = qw_h2f((uint16_t)(r[0] >> 16)) * (float)mn;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 32 * S + 8 * kg + i; }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 32 * S + 8 * kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 32 * S + 8 * kg); }
 };
 
 // ---------------------------------------------------------------- Q5_K: 176 bytes, d, dmin, scales[12] @4, qh[32] @16, qs[128] @48
@@ -126,7 +126,7 @@ template <> struct qw_kq<13> {
         c = qw_h2f((uint16_t)(r[0] >> 16)) * (float)mn;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 32 * S + 8 * kg + i; }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 32 * S + 8 * kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 32 * S + 8 * kg); }
 };
 
 // ---------------------------------------------------------------- Q6_K: 210 bytes, ql[128] @0, qh[64] @128, int8 scales[16] @192, d @208
@@ -157,7 +157,7 @@ template <> struct qw_kq<14> {
         c = 0.0f;
     }
     template <int G> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 16 * G + 4 * kg + i; }
-    template <int G> static __device__ __forceinline__ h4 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return af.at4(kb + 16 * G + 4 * kg); }
+    template <int G, class AFK> static __device__ __forceinline__ h4 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return af.at4(kb + 16 * G + 4 * kg); }
 };
 
 // ---------------------------------------------------------------- the 4-bit codebook formats
@@ -172,7 +172,7 @@ __device__ __forceinline__ h8 qw_iq4_bytes(const uint32_t *tab, uint32_t q) {
     raw[3] = __builtin_amdgcn_perm(t3, t2, 0x07060302u);
     return __builtin_bit_cast(h8, raw);
 }
-__device__ __forceinline__ h8 qw_iq4_xfrag(const qw_afrag_kq &af, uint32_t k32, uint32_t kg) { // x[4 kg .. + 4], x[16 + 4 kg .. + 4] of a 32-block
+template <class AFK> __device__ __forceinline__ h8 qw_iq4_xfrag(const AFK &af, uint32_t k32, uint32_t kg) { // x[4 kg .. + 4], x[16 + 4 kg .. + 4] of a 32-block
     const h4 a = af.at4(k32 + 4 * kg), b = af.at4(k32 + 16 + 4 * kg);
     return h8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
 }
@@ -198,7 +198,7 @@ template <> struct qw_kq<23> {
         c = 0.0f;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 32 * S + qw_iq4_pos(kg, i); }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return qw_iq4_xfrag(af, kb + 32 * S, kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return qw_iq4_xfrag(af, kb + 32 * S, kg); }
 };
 
 // IQ4_NL: 18 bytes, d @0, qs[16] @2 (2-byte aligned); one step.
@@ -217,7 +217,7 @@ template <> struct qw_kq<20> {
         c = 0.0f;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return qw_iq4_pos(kg, i); }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return qw_iq4_xfrag(af, kb, kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return qw_iq4_xfrag(af, kb, kg); }
 };
 
 // ---------------------------------------------------------------- plain rows: 32 values a step, 8 consecutive values a lane group
@@ -236,7 +236,7 @@ template <> struct qw_kq<1> { // binary16
         c = 0.0f;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 8 * kg + i; }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 8 * kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 8 * kg); }
 };
 
 // bfloat16 weights go to the bfloat16 matrix instruction unchanged; the binary16 activations are split there into two
@@ -256,7 +256,7 @@ template <> struct qw_kq<30> {
         c = 0.0f;
     }
     template <int S> static __device__ __forceinline__ uint32_t pos(uint32_t kg, uint32_t i) { return 8 * kg + i; }
-    template <int S> static __device__ __forceinline__ h8 xfrag(const qw_afrag_kq &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 8 * kg); }
+    template <int S, class AFK> static __device__ __forceinline__ h8 xfrag(const AFK &af, uint32_t kb, uint32_t kg) { return af.at8(kb + 8 * kg); }
 };
 __device__ __forceinline__ float qw_w2f(_Float16 v) { return (float)v; }
 __device__ __forceinline__ float qw_w2f(__bf16 v) { return (float)v; }
@@ -352,6 +352,7 @@ template <int NB> struct qw_chunk<20, NB> {
             acc += qw_h2f(d[b]) * sub;
         }
     }
+    template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
     // NG groups of 16 activation rows (binary16, one plane, global memory) against the same decoded weights
     template <int NG> __device__ __forceinline__ void mac_groups(const u2 *lut, const uint16_t *const (&rows)[NG], uint32_t k0, uint32_t kg, f4 (&acc)[NG]) const {
@@ -484,3 +485,69 @@ template <int NB> struct qw_chunk_kq<QW_F_PACKED_Q6, NB> {
         for (int i = 0; i < NB; i++) qw_kq_block<14>(b[i], tab, af, k0 + BLK_K * i, kg, acc);
     }
 };
+
+// ---------------------------------------------------------------- the same decoders in the MoE kernels' chunk interface
+// qw_chunk<F, NB> for Q4_K, Q5_K, Q6_K and IQ4_XS rows (kernels/moe_gg.metal:336-395 of the reference takes them for
+// the routed experts too): GGUF-order rows loaded in quad order, operand A from any of the fragment providers (one plane
+// or hi + lo). "lut" is the 256-entry byte table of qw_kq_tab_build (read by IQ4_XS only). The minimum term of Q4_K and
+// Q5_K needs the sum of the step's 32 activations per token: one more matrix instruction against a fragment of ones
+// delivers it in the accumulator's own layout, whatever the provider. Built for coverage of the formats, not tuned.
+template <class AF, bool LO> struct qw_kq_plane { // one plane of a provider, in the at8 / at4 interface of xfrag
+    const AF &af;
+    __device__ __forceinline__ h8 at8(uint32_t k) const {
+        if constexpr (LO) return af.lo(k);
+        else return af.hi(k);
+    }
+    __device__ __forceinline__ h4 at4(uint32_t k) const {
+        if constexpr (LO) return af.lo4(k);
+        else return af.hi4(k);
+    }
+};
+template <int F, int S, class AF> __device__ __forceinline__ void qw_kq_step_af(const qw_kq<F> &b, const uint32_t *tab, const AF &af, uint32_t kb, uint32_t kg, f4 &acc) {
+    typename qw_kq<F>::W w;
+    float a, c;
+    b.template dec<S>(tab, kg, w, a, c);
+    const qw_kq_plane<AF, false> ph = {af};
+    const qw_kq_plane<AF, true> pl = {af};
+    const auto xh = qw_kq<F>::template xfrag<S>(ph, kb, kg);
+    f4 sub = {0, 0, 0, 0};
+    if constexpr (qw_kq<F>::KSTEP == 16) {
+        sub = qw_mfma16(xh, w, sub);
+        if (AF::has_lo) sub = qw_mfma16(qw_kq<F>::template xfrag<S>(pl, kb, kg), w, sub);
+    } else {
+        sub = qw_mfma(xh, w, sub);
+        if (AF::has_lo) sub = qw_mfma(qw_kq<F>::template xfrag<S>(pl, kb, kg), w, sub);
+        if constexpr (qw_kq<F>::HAS_MIN) {
+            const _Float16 o = (_Float16)1.0f;
+            const h8 ones = {o, o, o, o, o, o, o, o};
+            f4 xs = {0, 0, 0, 0};
+            xs = qw_mfma(xh, ones, xs);
+            if (AF::has_lo) xs = qw_mfma(qw_kq<F>::template xfrag<S>(pl, kb, kg), ones, xs);
+            acc -= c * xs;
+        }
+    }
+    acc += a * sub;
+}
+template <int F, class AF, int S = 0> __device__ __forceinline__ void qw_kq_block_af(const qw_kq<F> &b, const uint32_t *tab, const AF &af, uint32_t kb, uint32_t kg, f4 &acc) {
+    if constexpr (S < (int)qw_kq<F>::STEPS) {
+        qw_kq_step_af<F, S>(b, tab, af, kb, kg, acc);
+        qw_kq_block_af<F, AF, S + 1>(b, tab, af, kb, kg, acc);
+    }
+}
+template <int F, int NB> struct qw_chunk_kqa : qw_chunk_kq<F, NB> {
+    template <class AF> __device__ __forceinline__ void mac(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+#pragma unroll
+        for (int i = 0; i < NB; i++) qw_kq_block_af<F>(this->b[i], (const uint32_t *)lut, af, k0 + qw_kq<F>::BLK_K * i, kg, acc);
+    }
+    template <class AF> __device__ __forceinline__ void mac_lean(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    template <class AF> __device__ __forceinline__ void mac_half(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const { mac(lut, af, k0, kg, acc); }
+    // operand A from the two H planes in global memory, read by the lanes whose token is in use
+    template <class AF> __device__ __forceinline__ void mac_gather(const u2 *lut, const AF &af, uint32_t k0, uint32_t kg, f4 &acc) const {
+        const qw_afrag_glb<true> g = {af.on ? af.rowhi : nullptr, af.on ? af.rowlo : nullptr};
+        mac(lut, g, k0, kg, acc);
+    }
+};
+template <int NB> struct qw_chunk<12, NB> : qw_chunk_kqa<12, NB> {};
+template <int NB> struct qw_chunk<13, NB> : qw_chunk_kqa<13, NB> {};
+template <int NB> struct qw_chunk<14, NB> : qw_chunk_kqa<14, NB> {};
+template <int NB> struct qw_chunk<23, NB> : qw_chunk_kqa<23, NB> {};

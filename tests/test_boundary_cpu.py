@@ -93,7 +93,9 @@ def test_define_blocks_of_the_reference_register_its_kernel_names():
     ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 17\n", "NB"),
     ("#define qmv_gg x\n#define GF 21\n#define KD 2048\n#define RB 880\n#define NB 8\n#define YT bfloat\n", "YT"),
     (ENGINE_MOE % 32 + "#define GG_PART 0\n", "NB"),
-    (ENGINE_MOE % 8 + "#define GG_PART 2\n#define FGU 23\n#define FSD 21\n", "23"),                           # IQ4_XS
+    (ENGINE_MOE % 8 + "#define GG_PART 2\n#define FGU 10\n#define FSD 21\n", "types 10"),                     # Q2_K routed rows
+    (ENGINE_MOE % 8 + "#define GG_PART 2\n#define FGU 23\n#define FSD 11\n", "23/11"),                        # Q3_K shared down
+    ("#define E 64\n#define TOPK 10\n#define D 2560\n#define I 640\n#define NB 8\n#define GG_PART 3\n#define FD 12\n", "I 640"),  # Q4_K rows want I a multiple of 256
     (ENGINE_MOE % 8 + "#define GG_PART 1\n#define FSG 21\n#define FSU 8\n#define RBF 1\n", "equal"),
     (ENGINE_MOE % 8 + "#define GG_PART 6\n", "GG_PART"),
     ("#define E 512\n#define TOPK 10\n#define D 2000\n#define I 512\n#define NB 8\n#define GG_PART 3\n#define FD 21\n", "D 2000"),
@@ -102,6 +104,16 @@ def test_define_blocks_of_the_reference_register_its_kernel_names():
 def test_unsupported_blocks_fail_with_a_message(block, needle):
     ok, err, names = compile_check(block)
     assert not ok and needle in err and names == []
+
+
+@pytest.mark.parametrize("fgu,fsd,fd", [(23, 21, 23), (12, 13, 14), (20, 14, 12), (21, 12, 13), (8, 23, 20)])
+def test_routed_rows_of_the_other_types_are_taken(fgu, fsd, fd):
+    """kernels/moe_gg.metal:336-395 of the reference: Q4_K, Q5_K, Q6_K, IQ4_NL and IQ4_XS beside IQ3_S and Q8_0, for the
+    routed rows and for the shared down rows."""
+    ok, err, names = compile_check(ENGINE_MOE % 8 + "#define GG_PART 2\n#define FGU %d\n#define FSD %d\n" % (fgu, fsd))
+    assert ok and names == ["moe_gu_gg"], err
+    ok, err, names = compile_check(ENGINE_MOE % 8 + "#define GG_PART 3\n#define FD %d\n" % fd)
+    assert ok and sorted(names) == ["moe_cmb_gg", "moe_dn_gg"], err
 
 
 def test_later_definitions_win_and_whitespace_is_tolerated():

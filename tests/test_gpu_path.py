@@ -326,6 +326,15 @@ def test_moe_layer_parity(gpu, oracle, nb, fmt):
     (256, 640, 16, 1, 4, 8, 20, 8, 20, True),        # the narrowest layer, one pick per token, tile-major IQ4_NL rows
     (512, 1280, 16, 16, 3, 21, 20, 21, 20, True),    # IQ4_NL rows wider than the staged 640: the any-shape kernel; every expert picked
     (2560, 640, 512, 10, 16, 21, 20, 8, 8, True),    # 512 experts at the reference model's shape, Q8_0 shared expert
+    # the other types the reference's kernels take for routed rows (kernels/moe_gg.metal:336-395): the kernels whose type is an argument
+    (2048, 512, 64, 10, 16, 23, 23, 21, 21, True),   # IQ4_XS routed rows beside an IQ3_S shared expert
+    (2560, 768, 64, 10, 9, 12, 12, 12, 12, True),    # Q4_K everywhere (the minimum term; shared gate/up through the multi-format matvec)
+    (1024, 512, 32, 4, 5, 14, 14, 8, 14, False),     # Q6_K routed rows and shared down, Q8_0 shared gate/up
+    (1536, 256, 48, 6, 13, 13, 13, 8, 8, True),      # Q5_K routed rows
+    (768, 256, 16, 2, 3, 20, 20, 21, 21, False),     # IQ4_NL gate/up; D off the front launch's shapes: the shared IQ3_S gate/up rides in the routed launch
+    (1280, 512, 32, 8, 2, 12, 23, 8, 8, False),      # Q4_K gate/up, IQ4_XS down, the Q8_0 shared gate/up in the routed launch
+    (2048, 512, 64, 10, 8, 21, 14, 21, 13, True),    # IQ3_S gate/up (tile-major) with Q6_K down rows and a Q5_K shared down
+    (2048, 512, 64, 10, 1, 23, 12, 23, 23, True),    # one token
 ])
 def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
     """Shapes and format mixes off the benchmark's: every kernel variant the host can pick is reached by one of them."""
@@ -343,6 +352,33 @@ def test_moe_layer_shapes(gpu, oracle, D, I, E, K, nb, fgu, fd, fsh, fshd, dev):
     ref = oracle.moe_layer_f64(m, lg, x)
     assert np.isfinite(out.astype(np.float64)).all()
     assert maxrel(out, ref) <= TOL, maxrel(out, ref)
+    dl.free()
+    path.close()
+
+
+@pytest.mark.parametrize("fgu,fd,fsh,fshd,D,want", [
+    (23, 23, 21, 21, 2048, ("qwk_gu_rt", "qwk_dn_rt")),       # the shared gate/up in the front launch
+    (12, 14, 8, 13, 1280, ("qwk_gu_rt_s8_c1", "qwk_dn_rt")),  # ... in the routed launch (D off the front launch's shapes)
+    (21, 21, 21, 12, 2048, ("qwk_gu_f121_c2", "qwk_dn_rt")),  # only the shared down rows are of another type
+    (20, 20, 21, 21, 768, ("qwk_gu_rt_s21_c1", "qwk_dn_rt")), # IQ4_NL routed down beside IQ3_S shared down: no build of their own
+])
+def test_types_without_a_build_of_their_own_take_the_argument_kernels(gpu, oracle, fgu, fd, fsh, fshd, D, want):
+    """kernels/moe_gg.metal:336-395 of the reference: every pair of the seven quantised types is a layer it can run. The
+    pairs off the fast builds go through qwk_gu_rt* / qwk_dn_rt (the type an argument); against the float64 layer."""
+    I, E, K, nb = 512, 32, 6, 11
+    rng = np.random.default_rng(fgu * 100 + fd + fshd)
+    m = synth.moe_layer(rng, D, I, E, fgu=fgu, fd=fd, fsh=fsh, fshd=fshd)
+    m["topk"] = K
+    x = synth.activations(rng, nb, D)
+    dl = DeviceLayer(gpu, m, device_only=True)
+    path = q.Path(gpu, D, I, E, K, 16)
+    gpu.profile(True)
+    out, lg, _, _ = run_moe(gpu, path, dl, x, nb)
+    names = [n for n, _ in gpu.profile_entries()]
+    gpu.profile(False)
+    assert all(w in names for w in want), names
+    assert np.isfinite(out.astype(np.float64)).all()
+    assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
     dl.free()
     path.close()
 

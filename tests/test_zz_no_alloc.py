@@ -22,7 +22,8 @@ def devptr(gpu, buf):
 @pytest.mark.parametrize("shape", [(2048, 512, 64, 10, 21, 21, 21, 21, 21, 1), (2560, 640, 32, 10, 21, 20, 8, 8, 8, 1), (1024, 256, 128, 8, 8, 8, 8, 8, 8, 1),
                                    (2560, 640, 32, 10, 21, 20, 12, 23, 20, 1),    # shared gate/up in the K-quant / IQ4 family: the front launch that carries them
                                    (2048, 512, 64, 10, 21, 21, 21, 21, 21, 30),   # bfloat16 router
-                                   (2560, 640, 32, 6, 21, 20, 12, 23, 20, 30)])   # both: the shared gate/up as a launch of its own beside a bfloat16 router
+                                   (2560, 640, 32, 6, 21, 20, 12, 23, 20, 30),    # both: the shared gate/up as a launch of its own beside a bfloat16 router
+                                   (2048, 512, 32, 8, 23, 14, 8, 8, 12, 1)])      # routed rows of the other types (the kernels whose type is an argument)
 def test_no_alloc_layer_equals_the_allocating_entry_point(gpu, oracle, shape):
     D, I, E, K, fgu, fd, fsg, fsu, fsd, rt = shape
     rng = np.random.default_rng(D + E + fsg + rt)
