@@ -323,7 +323,8 @@ struct qw_afrag_gather {
 // ---------------------------------------------------------------- chunks: the unit of prefetch
 // A chunk is NB consecutive blocks of one weight row, held in registers by the lane that decodes them. Kernels keep
 // DEPTH chunks per wave (two or three): while one is decoded and multiplied, the loads of the next one or two are in
-// flight. With 10 waves per compute unit and 7 to 14 KB per wave in flight this covers the HBM latency.
+// flight. With 12 waves per compute unit and 3.5 to 7 KB per wave in flight this covers the HBM latency; more in flight
+// than that slows the device-wide streams down (see qw_chunk<QW_F_PACKED, NB>).
 template <int F, int NB> struct qw_chunk;
 
 template <int NB> struct qw_chunk<21, NB> {
@@ -553,7 +554,10 @@ template <int NB> struct qw_chunk<21, NB> {
 // and no transpose. p is the (wave-uniform) address of the chunk's first slab, the second argument the lane.
 template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = QW_SLAB_BYTES;
-    static constexpr int DEPTH = 3;
+    // One chunk ahead, not two: with every wave of the device streaming, more loads in flight made the launches slower
+    // (24 layers at 16 tokens, ms: 1.80 with two chunks ahead in the routed gate/up and down launches, 1.70 with one, 1.85
+    // and 1.95 with three and four in the gate/up launch; the grouped product of the packing path 4 % faster with one).
+    static constexpr int DEPTH = 2;
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t lane) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -579,7 +583,7 @@ template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
 // QW_F_ABLATE: the same loads and lane moves, no decoding and no matrix instructions (a measurement; see qw_kargs.h).
 template <int NB> struct qw_chunk<QW_F_ABLATE, NB> : qw_chunk<QW_F_PACKED, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = QW_SLAB_BYTES;
-    static constexpr int DEPTH = 3;
+    static constexpr int DEPTH = 2;
     template <class AF> __device__ __forceinline__ void mac_lean(const u2 *, const AF &, uint32_t, uint32_t, f4 &acc) const {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -783,6 +787,51 @@ __device__ __forceinline__ void qw_task_stream(uint32_t ntasks, uint32_t w0, uin
 #pragma unroll
     for (int i = 0; i + 1 < DEPTH; i++)
         if (left > (uint32_t)i) consume(buf[i]);
+}
+
+// The same streaming with the tasks taken from a queue instead of a fixed stride: `first` is the wave's first task,
+// next() returns its next one whenever it has asked for all chunks of the current one (any value >= ntasks: none left,
+// and none ever again). A workgroup's waves share a counter in LDS behind next(): the hardware serves the older waves of
+// a compute unit first, so with a fixed deal the first waves finish their tiles long before the last ones and the unit
+// runs its last third with a few waves' loads in flight; from a queue every wave works until the workgroup's tiles are gone.
+// Each chunk buffer carries the task and chunk it was loaded for.
+template <class C, int DEPTH = C::DEPTH, class N, class R, class U, class S>
+__device__ __forceinline__ void qw_task_queue(uint32_t ntasks, uint32_t first, N next, uint32_t cpr, uint32_t cstride, uint32_t kl, R rowp, U use, S ready, const uint8_t *spare = nullptr) {
+    if (first >= ntasks) {
+        ready();
+        return;
+    }
+    C buf[DEPTH];
+    uint32_t btask[DEPTH], bchunk[DEPTH];
+    uint32_t lt = first, lc = 0;
+    const uint8_t *lrow = rowp(lt);
+    // (every step issues one chunk's loads whatever happens, as in qw_task_stream: past the last task they read valid, cached memory)
+    const uint8_t *const past = spare && cpr * cstride <= 65536u ? spare : lrow;
+    auto load = [&](int i) {
+        btask[i] = lt, bchunk[i] = lc;
+        buf[i].load(lrow + (size_t)lc * cstride, kl);
+        if (++lc == cpr) {
+            lc = 0;
+            if (lt < ntasks) lt = next();
+            lrow = lt < ntasks ? rowp(lt) : past;
+        }
+    };
+#pragma unroll
+    for (int i = 0; i + 1 < DEPTH; i++) load(i);
+    ready();
+    for (bool done = false; !done;) {
+#pragma unroll
+        for (int i = 0; i < DEPTH; i++) {
+            if (!done) { // (a guard, not a break: the loop unrolls and every buffer keeps its registers)
+                load((i + DEPTH - 1) % DEPTH);
+                if (btask[i] >= ntasks) done = true;
+                else {
+                    buf[i].transpose();
+                    use(btask[i], bchunk[i], buf[i]);
+                }
+            }
+        }
+    }
 }
 
 

@@ -602,6 +602,7 @@ extern "C" __global__ __launch_bounds__(256) void qwk_router_w30(qwk_router_args
 struct qw_sel_cache { // the part of the selection record a weight kernel needs, in LDS
     uint32_t U, ue[256], mask[256];
     uint8_t slot[256 * 16];
+    uint32_t qnext; // the workgroup's tile queue (gu_tasks): how many of its tiles have been handed out
 };
 struct qw_sel_scratch {
     uint32_t ids[256], lead[8], first[1024];
@@ -938,8 +939,11 @@ struct qw_h_global {
         qw_store_u16(H + o + hplane, lo);
     }
 };
-template <int F, int CH, class S, class HS>
-__device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, const qw_sel_cache *sc, uint32_t w0, uint32_t nw, S ready, HS &hs) {
+// QUEUE: the workgroup's tiles (blockIdx.x, blockIdx.x + gridDim.x, ...) go to its waves from the counter sc->qnext, which
+// the caller has set to the number of waves before a barrier (wave w starts with the w-th of them); else wave w0 of nw takes
+// tiles w0, w0 + nw, ...
+template <int F, int CH, bool QUEUE, class S, class HS>
+__device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, const u4 *xf, qw_sel_cache *sc, uint32_t w0, uint32_t nw, S ready, HS &hs) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, gnb = a.gnb;
     const uint32_t U = a.shared ? 1 : sc->U, tpe = a.I / 8, ntasks = U * tpe;
@@ -952,7 +956,7 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
         else return (nl < 8 ? a.Wg : a.Wu) + ((size_t)e * a.I + 8 * (task % tpe) + (nl & 7)) * a.rowbytes;
     };
     f4 acc = {0, 0, 0, 0};
-    qw_task_stream<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, F == QW_F_PACKED || F == QW_F_ABLATE ? lane : lane & 3, rowp, [&](uint32_t task, uint32_t ci, const C &c) {
+    auto use = [&](uint32_t task, uint32_t ci, const C &c) {
         c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
         if (ci + 1 != cpr) return;
         const uint32_t u = task / tpe, j0 = 8 * (task % tpe);
@@ -971,7 +975,18 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
             }
         }
         acc = f4{0, 0, 0, 0};
-    }, ready, qw_has_lut(F) ? (const uint8_t *)a.glut : nullptr);
+    };
+    const uint32_t kl = F == QW_F_PACKED || F == QW_F_ABLATE ? lane : lane & 3;
+    const uint8_t *spare = qw_has_lut(F) ? (const uint8_t *)a.glut : nullptr;
+    if constexpr (QUEUE) {
+        auto next = [&]() -> uint32_t {
+            uint32_t j = 0;
+            if (lane == 0) j = atomicAdd(&sc->qnext, 1u);
+            // (a workgroup's tiles lie gridDim.x tiles apart: neighbouring tiles on one compute unit measured slower, 38.4 -> 40.3 us)
+            return blockIdx.x + gridDim.x * (uint32_t)__builtin_amdgcn_readfirstlane((int)j);
+        };
+        qw_task_queue<C>(ntasks, blockIdx.x + gridDim.x * qw_wave(), next, cpr, CH * C::BLK_B, kl, rowp, use, ready, spare);
+    } else qw_task_stream<C>(ntasks, w0, nw, cpr, CH * C::BLK_B, kl, rowp, use, ready, spare);
 }
 
 // FGU: routed gate/up format; FSG: shared gate/up format done by the same launch (0 = none).
@@ -985,6 +1000,7 @@ __device__ __forceinline__ void gu_tasks(const qwk_gu_args &a, const u2 *lut, co
 template <int FGU, int CHGU, int FSG, int CHSG, class HS, class SEL>
 __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, qw_sel_cache *sc, qw_sel_scratch *ss, HS &hs, bool all_w, SEL selected) {
     bool staged = false, tabled = false;
+    if (threadIdx.x == 0) sc->qnext = blockDim.x >> 6; // (nothing below writes it; a barrier follows on every path)
     if (threadIdx.x == 0) QW_WSTAMP(12);
     QW_DSTAMP(0);
     if constexpr (FGU == QW_F_RT) qw_kq_tab_build((uint32_t *)(lut + (qw_has_lut(FSG) ? QW_LUT_ENTRIES : 0))); // (published by the barriers below)
@@ -1043,21 +1059,21 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
             sa.Wu = a.Wsu;
             sa.rowbytes = a.sg_rowbytes;
             sa.shared = 1;
-            gu_tasks<FSG == 0 ? 8 : FSG, CHSG>(sa, lut, xf, nullptr, w0, nw, ready, hs);
+            gu_tasks<FSG == 0 ? 8 : FSG, CHSG, false>(sa, lut, xf, nullptr, w0, nw, ready, hs);
         }
     }
-    // the waves that did a shared tile come last in the routed deal, so that the work stays level
+    // the routed tiles: from the workgroup's queue (a wave that did a shared tile simply takes its next one later)
     if constexpr (FGU == QW_F_RT) { // the other GGUF types, one block a chunk; their byte table lies behind the IQ3_S table
         const u2 *tab = lut + (qw_has_lut(FSG) ? QW_LUT_ENTRIES : 0);
         switch (a.fgu) {
-        case 12: gu_tasks<12, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
-        case 13: gu_tasks<13, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
-        case 14: gu_tasks<14, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
-        case 20: gu_tasks<20, 8>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
-        case 23: gu_tasks<23, 1>(a, tab, xf, sc, nw - 1 - w0, nw, ready, hs); break;
+        case 12: gu_tasks<12, 1, true>(a, tab, xf, sc, 0, 0, ready, hs); break;
+        case 13: gu_tasks<13, 1, true>(a, tab, xf, sc, 0, 0, ready, hs); break;
+        case 14: gu_tasks<14, 1, true>(a, tab, xf, sc, 0, 0, ready, hs); break;
+        case 20: gu_tasks<20, 8, true>(a, tab, xf, sc, 0, 0, ready, hs); break;
+        case 23: gu_tasks<23, 1, true>(a, tab, xf, sc, 0, 0, ready, hs); break;
         default: break; // (the host launches this kernel for these five only)
         }
-    } else gu_tasks<FGU, CHGU>(a, lut, xf, sc, nw - 1 - w0, nw, ready, hs);
+    } else gu_tasks<FGU, CHGU, true>(a, lut, xf, sc, 0, 0, ready, hs);
     QW_WSTAMP(qw_wave());
     QW_DSTAMP(2);
 }
