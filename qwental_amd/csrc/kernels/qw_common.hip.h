@@ -16,6 +16,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "qw_kargs.h"
 #define QW_CODES_QUAL __constant__ const
 #include "iq3s_codes.h"
@@ -309,6 +310,7 @@ struct qw_afrag_gather {
     h8 (&hi)[4];
     h8 (&lo)[4];
     static constexpr bool has_lo = true;
+    static constexpr bool stacked = false; // (true: both planes of a token in one operand A, the provider of the down launch by token shares)
     __device__ __forceinline__ void fetch4(uint32_t koff, uint32_t kstep) const {
         if (on) {
 #pragma unroll
@@ -487,8 +489,19 @@ template <int NB> struct qw_chunk<21, NB> {
                     for (int i = 0; i < 4; i++) raw[i] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, (uint32_t)raw[i]) * ff);
                     const h8 wv = __builtin_bit_cast(h8, raw);
                     sub0 = qw_mfma(af.hi[jj], wv, sub0);
-                    sub1 = qw_mfma(af.lo[jj], wv, sub1);
+                    if constexpr (!AF::stacked) sub1 = qw_mfma(af.lo[jj], wv, sub1);
                 }
+            }
+            if constexpr (AF::stacked) {
+                // operand A rows 0 .. 3 held the hi plane, rows 4 .. 7 the lo plane of the same tokens: the lo sums lie
+                // in the lanes 16 further (k-group 1). Each output row depends on its own operand A row only, so both
+                // sums have the bits the two instructions above would give; only lanes 0 .. 15 hold a result.
+                // (The elements are copied to scalars first: __builtin_bit_cast applied to a vector element directly read
+                // element 0 whatever the index.)
+                const int from = (int)(((threadIdx.x & 63) + 16) & 63) * 4;
+                const float a0 = sub0[0], a1 = sub0[1], a2 = sub0[2], a3 = sub0[3];
+                sub1 = f4{__builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, a0))), __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, a1))),
+                          __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, a2))), __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, a3)))};
             }
             acc += s[b].d * (sub0 + sub1);
         }

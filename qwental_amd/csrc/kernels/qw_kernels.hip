@@ -1544,7 +1544,7 @@ struct qw_dnq_lds {
     float wl[4 * 11];               // gating weights of the quarter's tokens
     uint32_t ue[QW_DNQ_MAXU], slot4[QW_DNQ_MAXU]; // expert of unique index u; the slot bytes of the quarter's four tokens
     uint16_t mask[QW_DNQ_MAXU], vlist[48];        // token mask of u; the unique indices this quarter needs
-    uint32_t U, nv;
+    uint32_t U, nv, q[2];
 };
 // Operand A from the staged rows, in the manner of qw_afrag_gather: lane m < 4 is local token m, its row chosen per
 // expert; four fragments per plane at a time inside one predicated region, into registers the caller keeps (and has
@@ -1555,6 +1555,10 @@ template <uint32_t ROWS> struct qw_afrag_rows {
     h8 (&hi)[4];
     h8 (&lo)[4];
     static constexpr bool has_lo = true;
+    static constexpr bool stacked = false;
+    __device__ __forceinline__ void place(const u4 *hi0, const u4 *lo0, uint32_t m, uint32_t r, bool picked) {
+        on = picked && m < 4, hi_ = hi0 + r, lo_ = lo0 + r; // (read only where on: one of the staged rows then)
+    }
     __device__ __forceinline__ void fetch4(uint32_t koff, uint32_t kstep) const {
         if (on) {
 #pragma unroll
@@ -1565,16 +1569,37 @@ template <uint32_t ROWS> struct qw_afrag_rows {
         }
     }
 };
+// The same rows with both planes in one operand A: lane m < 4 supplies the hi plane of local token m, lane 4 + m its lo
+// plane, so that one matrix instruction does the work of two (a share has at most four tokens: eight of the sixteen
+// operand rows are in use instead of four). For the chunk types whose mac_gather knows the stacked form.
+template <uint32_t ROWS> struct qw_afrag_rows2 {
+    const u4 *hi_, *lo_; // hi_: this lane's row in its plane; lo_ unused
+    bool on;
+    h8 (&hi)[4];
+    h8 (&lo)[4];
+    static constexpr bool has_lo = true;
+    static constexpr bool stacked = true;
+    __device__ __forceinline__ void place(const u4 *hi0, const u4 *lo0, uint32_t m, uint32_t r, bool picked) {
+        on = picked && m < 8, hi_ = (m & 4 ? lo0 : hi0) + r;
+    }
+    __device__ __forceinline__ void fetch4(uint32_t koff, uint32_t kstep) const {
+        if (on) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) hi[i] = __builtin_bit_cast(h8, hi_[((koff + i * kstep) >> 3) * ROWS]);
+        }
+    }
+};
 // What dnq_run reads and writes in LDS (the two kernels that hold it lay their LDS out differently).
 struct qw_dnq_view {
     const u4 *hrows;       // [plane][8 k-values][row], 16 bytes each, ROWS rows: row = local token * (topk + 1) + slot
     float *part;           // [local token][slot][row of the group]
     const uint32_t *ue, *slot4;
     const uint16_t *mask, *vlist;
+    uint32_t *q;           // two counters: the routed tiles handed out (starts at the number of waves: wave w begins with tile w), the shared ones (starts at 0)
 };
 // The tiles of `nv` experts (shared: the one shared expert) for this workgroup's tpw tiles, dealt to its waves.
 template <int F, int CH, bool SHARED, uint32_t ROWS, class S>
-__device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, const qw_dnq_view &L, uint32_t g, uint32_t t0, uint32_t nt, uint32_t nv, uint32_t dealt, S ready) {
+__device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, const qw_dnq_view &L, uint32_t g, uint32_t t0, uint32_t nt, uint32_t nv, S ready) {
     typedef qw_chunk<F, CH> C;
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, K = a.topk, tpe = a.D / 16, tpw = a.tpw, cpr = a.I / (C::BLK_K * CH), rw = 16 * tpw;
     const uint32_t ts = (uint32_t)__builtin_ctz(tpw), tm = tpw - 1; // tpw is a power of two
@@ -1582,10 +1607,25 @@ __device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, con
     f4 acc = {0, 0, 0, 0};
     const u4 *const lo0 = L.hrows + a.I / 8 * ROWS;
     h8 xhi[4] = {}, xlo[4] = {};
+    // (tile-major IQ3_S: both planes in one matrix instruction; the Q8_0 form adds the planes inside the accumulator, which one instruction cannot reproduce bit for bit)
+#ifdef QW_DNQ_NOSTACK
     qw_afrag_rows<ROWS> af = {L.hrows, lo0, false, xhi, xlo};
+#else
+    typename std::conditional<F == QW_F_PACKED, qw_afrag_rows2<ROWS>, qw_afrag_rows<ROWS>>::type af = {L.hrows, lo0, false, xhi, xlo};
+#endif
     auto expert = [&](uint32_t task) { return SHARED ? 0u : (uint32_t)L.vlist[task >> ts]; };
-    const uint32_t nw = blockDim.x >> 6, w0 = (qw_wave() + nw - dealt % nw) % nw; // the deal goes on where the last one (dealt tiles) stopped
-    qw_task_stream<C>(nv * tpw, w0, nw, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
+    // the workgroup's tiles go to its waves from a queue (qw_task_queue): a wave that is done takes the next one, and the
+    // shared expert's tiles go to the waves that leave the routed ones first
+    auto next = [&]() -> uint32_t {
+        uint32_t j = 0;
+        if (lane == 0) j = atomicAdd(&L.q[SHARED ? 1 : 0], 1u);
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)j);
+    };
+#ifdef QW_DNQ_NOQUEUE
+    qw_task_stream<C>(nv * tpw, qw_wave(), blockDim.x >> 6, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
+#else
+    qw_task_queue<C>(nv * tpw, SHARED ? next() : qw_wave(), next, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
+#endif
         [&](uint32_t task) {
             const uint32_t tile = g * tpw + (task & tm);
             const uint8_t *W = SHARED ? a.Wsd : a.Wd + (size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)L.ue[expert(task)]) * (qw_tiled(F) ? tpe : a.D) * a.rowbytes;
@@ -1598,8 +1638,7 @@ __device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, con
             if (ci == 0) { // this lane's operand A row for the task's expert
                 const uint32_t tl = m & 3, mk = SHARED ? qw_all_tokens(a.snbr) >> t0 : (uint32_t)L.mask[u] >> t0;
                 const uint32_t r = tl * (K + 1) + (SHARED ? K : (L.slot4[u] >> (8 * tl)) & 255);
-                af.on = m < nt && ((mk >> m) & 1);
-                af.hi_ = L.hrows + r, af.lo_ = lo0 + r; // (read only where on: one of the 44 rows then)
+                af.place(L.hrows, lo0, m, r, tl < nt && ((mk >> tl) & 1));
                 // a lane that is off keeps the fragments of an earlier expert: they feed output rows that are never
                 // stored (a matrix-core output row depends on its own operand A row only)
             }
@@ -1657,7 +1696,7 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
             L.ue[i] = ue[i], L.mask[i] = (uint16_t)mk[i], L.slot4[i] = s4;
         }
         for (uint32_t i = tid; i < nt * (K + 1); i += blockDim.x) L.wl[i] = wg[i];
-        if (tid == 0) L.U = *(const uint32_t *)a.sel;
+        if (tid == 0) L.U = *(const uint32_t *)a.sel, L.q[0] = blockDim.x >> 6, L.q[1] = 0;
         if (qw_has_lut(F) || qw_has_lut(FSD)) {
 #pragma unroll
             for (uint32_t it = 0; it < PER; it++) {
@@ -1711,10 +1750,10 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
     };
     // the routed experts first (every wave has tiles there, so every wave's first weights are on their way before the
     // rows are asked for); the shared expert's tiles go to the waves that the routed deal gave one tile fewer
-    const qw_dnq_view V = {L.hrows, L.part, L.ue, L.slot4, L.mask, L.vlist};
-    dnq_run<F, CH, false, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, nv, 0, ready);
+    const qw_dnq_view V = {L.hrows, L.part, L.ue, L.slot4, L.mask, L.vlist, L.q};
+    dnq_run<F, CH, false, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, nv, ready);
     if (FSD != 0) {
-        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, 1, nv * tpw, ready);
+        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, 1, ready);
     }
     ready(); // (for symmetry only: both runs call it, with or without tiles)
     QW_DSTAMP(9);
@@ -1788,7 +1827,7 @@ struct qw_gud_lds {
     float wl[QW_GUD_SHARE * 11];
     uint32_t ue[QW_DNQ_MAXU], slot4[QW_DNQ_MAXU];
     uint16_t mask[QW_DNQ_MAXU], vlist[32];
-    uint32_t hcount, bail;
+    uint32_t hcount, bail, dq[2];
 };
 static_assert(sizeof(qw_gud_lds) <= 160 * 1024, "LDS of the fused launch");
 static_assert(QW_GUD_SHARE * 11 * 32 <= 2 * 11 * 64, "part holds three tokens by two tiles or two tokens by four");
@@ -1822,7 +1861,7 @@ template <int FSD, int CHSD> __device__ __forceinline__ void gud_body(const qwk_
             for (uint32_t j = 0; j < nt; j++) s4 |= (uint32_t)L.sc.slot[i * gnb + t0 + j] << (8 * j);
             L.ue[i] = L.sc.ue[i], L.mask[i] = (uint16_t)L.sc.mask[i], L.slot4[i] = s4;
         }
-        if (tid == 0) L.hcount = 0, L.bail = 0;
+        if (tid == 0) L.hcount = 0, L.bail = 0, L.dq[0] = blockDim.x >> 6, L.dq[1] = 0;
         uint32_t U = L.sc.U;
         if (U > GU) U = GU;
         const uint32_t want = (1u << nt) - 1;
@@ -1888,11 +1927,11 @@ template <int FSD, int CHSD> __device__ __forceinline__ void gud_body(const qwk_
         meet();
         return;
     }
-    const qw_dnq_view V = {L.big.hrows, L.u.part, L.ue, L.slot4, L.mask, L.vlist};
+    const qw_dnq_view V = {L.big.hrows, L.u.part, L.ue, L.slot4, L.mask, L.vlist, L.dq};
     // the routed experts first; the shared expert's tiles go to the waves that the routed deal gave one tile fewer
-    dnq_run<F, CH, false, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, nv, 0, meet);
+    dnq_run<F, CH, false, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, nv, meet);
     if (FSD != 0) {
-        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, 1, nv * tpw, meet);
+        if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_GUD_ROWS>(d, L.lut, V, g, t0, nt, 1, meet);
     }
     meet();
     QW_STAMP(8);
