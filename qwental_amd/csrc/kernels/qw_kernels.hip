@@ -1673,23 +1673,28 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
     uint32_t nt = base + (q < rem ? 1 : 0);
     if (nt > 4) nt = 4; // (the host admits 16 tokens in four quarters, 8 in two)
     QW_DSTAMP(6);
-    // one memory round trip: the record (U, experts, masks, this quarter's slot bytes and gating weights) and the table,
-    // through registers (a workgroup has nothing else to do meanwhile, and plain loads move more bytes per clock
-    // than the direct ones)
+    // one memory round trip: the record (U, experts, masks, this quarter's slot bytes and gating weights), every H row of the
+    // quarter's tokens (which rows they are does not depend on the record) and the table. The rows go through registers into
+    // LDS in fragment order; a wave's load takes 8 rows x 128 bytes (whole cache lines), lanes 0 .. 31 the first 64 bytes
+    // of a row, 32 .. 63 the rest.
     {
+        const uint32_t upr = a.I / 8, cbs = upr / 8, used = nt * (K + 1), nrb = (used + 7) / 8, nunits = 2 * nrb * cbs, wv = qw_wave();
+        constexpr uint32_t NW = QW_WG_DN / 64, RPER = (2 * 6 * 8 + NW - 1) / NW; // 2 planes x 6 row blocks x 8 column blocks at most
+        u4 rowv[RPER];
+        uint32_t at[RPER];
+#pragma unroll
+        for (uint32_t it = 0; it < RPER; it++) {
+            const uint32_t unit = wv + it * NW, cb = unit % cbs, rest = unit / cbs, rb = rest % nrb, pl = rest / nrb;
+            const uint32_t r = 8 * rb + ((lane >> 2) & 7), c = 8 * cb + 4 * (lane >> 5) + (lane & 3);
+            const bool on = unit < nunits && r < used;
+            at[it] = on ? (pl * upr + c) * QW_DNQ_ROWS + r : ~0u;
+            // (a unit that is off reads the first bytes of H: a load under a condition made the compiler keep the whole array in scratch memory)
+            rowv[it] = *(const u4 *)(on ? a.H + pl * (size_t)a.hplane + ((size_t)t0 * (K + 1) + r) * a.I + 8 * c : a.H);
+        }
         const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mk = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
         const uint8_t *sl = a.sel + QW_SEL_OFF_SLOT(gnb, K);
         const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K)) + t0 * (K + 1);
-        constexpr uint32_t N = QW_LUT_BYTES / 16, PER = (N + QW_WG_DN - 1) / QW_WG_DN;
-        const uint32_t rot = blockIdx.x * 320u; // every workgroup starts at another place of the table
-        u4 tab[PER];
-        if (qw_has_lut(F) || qw_has_lut(FSD)) {
-#pragma unroll
-            for (uint32_t it = 0; it < PER; it++) {
-                const uint32_t i = tid + it * QW_WG_DN;
-                if (i < N) tab[it] = ((const u4 *)a.glut)[(i + rot) & (N - 1)];
-            }
-        }
+        if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // (straight into LDS: the registers hold the rows)
         for (uint32_t i = tid; i < GU; i += blockDim.x) {
             uint32_t s4 = 0;
             for (uint32_t j = 0; j < nt; j++) s4 |= (uint32_t)sl[i * gnb + t0 + j] << (8 * j);
@@ -1697,13 +1702,10 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         }
         for (uint32_t i = tid; i < nt * (K + 1); i += blockDim.x) L.wl[i] = wg[i];
         if (tid == 0) L.U = *(const uint32_t *)a.sel, L.q[0] = blockDim.x >> 6, L.q[1] = 0;
-        if (qw_has_lut(F) || qw_has_lut(FSD)) {
 #pragma unroll
-            for (uint32_t it = 0; it < PER; it++) {
-                const uint32_t i = tid + it * QW_WG_DN;
-                if (i < N) ((u4 *)lut)[(i + rot) & (N - 1)] = tab[it];
-            }
-        }
+        for (uint32_t it = 0; it < RPER; it++)
+            if (at[it] != ~0u) L.hrows[at[it]] = rowv[it];
+        qw_lds_arrive();
     }
     __syncthreads();
     QW_DSTAMP(7);
@@ -1725,37 +1727,13 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         if (nv > 48) nv = 48; // (four tokens of ten experts: 40 at most)
     }
     const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0;
-    bool staged = false;
-    // once per wave, behind its first weight loads: every H row of the quarter's tokens into LDS in fragment order.
-    // A wave's load takes 8 rows x 128 bytes (whole cache lines), lanes 0 .. 31 the first 64 bytes of a row, 32 .. 63 the rest
-    auto ready = [&] {
-        if (staged) return;
-        staged = true;
-        const uint32_t upr = a.I / 8, cbs = upr / 8, used = nt * (K + 1), nrb = (used + 7) / 8, nunits = 2 * nrb * cbs, wv = qw_wave();
-        constexpr uint32_t NW = QW_WG_DN / 64, PER = (2 * 6 * 8 + NW - 1) / NW; // 2 planes x 6 row blocks x 8 column blocks at most
-        u4 t[PER];
-        uint32_t at[PER];
-#pragma unroll
-        for (uint32_t it = 0; it < PER; it++) {
-            const uint32_t unit = wv + it * NW, cb = unit % cbs, rest = unit / cbs, rb = rest % nrb, pl = rest / nrb;
-            const uint32_t r = 8 * rb + ((lane >> 2) & 7), c = 8 * cb + 4 * (lane >> 5) + (lane & 3);
-            at[it] = unit < nunits && r < used ? (pl * upr + c) * QW_DNQ_ROWS + r : ~0u;
-            if (at[it] != ~0u) t[it] = *(const u4 *)(a.H + pl * (size_t)a.hplane + ((size_t)t0 * (K + 1) + r) * a.I + 8 * c);
-        }
-#pragma unroll
-        for (uint32_t it = 0; it < PER; it++)
-            if (at[it] != ~0u) L.hrows[at[it]] = t[it];
-        __syncthreads();
-        QW_DSTAMP(8);
-    };
-    // the routed experts first (every wave has tiles there, so every wave's first weights are on their way before the
-    // rows are asked for); the shared expert's tiles go to the waves that the routed deal gave one tile fewer
+    auto ready = [] {}; // (everything the tiles need is in LDS already)
+    // the routed experts first; the shared expert's tiles go to the waves that leave the routed ones first
     const qw_dnq_view V = {L.hrows, L.part, L.ue, L.slot4, L.mask, L.vlist, L.q};
     dnq_run<F, CH, false, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, nv, ready);
     if (FSD != 0) {
         if (nsh) dnq_run<FSD == 0 ? F : FSD, CHSD, true, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, 1, ready);
     }
-    ready(); // (for symmetry only: both runs call it, with or without tiles)
     QW_DSTAMP(9);
     __syncthreads();
     for (uint32_t j = tid; j < nt * rw; j += blockDim.x) { // rank order, then the shared expert (qwk_cmb's arithmetic)
