@@ -1,10 +1,11 @@
 // HIP kernels of the quantized decode path for gfx950. One code object; gpu_hip.c loads it and launches these
 // entry points by name. Each kernel takes one argument record from qw_kargs.h by value.
 //
-// Shape of the weight-streaming kernels (dense matvec, gate/up, down): persistent workgroups of 512 threads, one
+// Shape of the weight-streaming kernels (dense matvec, gate/up, down): persistent workgroups of 512 or 768 threads, one
 // per compute unit (the 64 KB pre-signed table plus the staged activations fill most of the 160 KB LDS). Each wave
-// walks its own list of 16-row tiles through a two-chunk register pipeline: the loads of the next chunk are issued
-// before the current one is decoded, so every wave keeps about one tile of weight bytes in flight.
+// walks 16-row tiles through a register pipeline of chunks: the loads of the next chunk (for some formats the next two)
+// are issued before the current one is decoded. In the routed gate/up launch and the down launch by token shares the
+// tiles of a workgroup go to its waves from a queue in LDS, elsewhere every wave has its own fixed list.
 #include "qw_common.hip.h"
 #include "qw_kquants.hip.h"
 
@@ -1608,11 +1609,7 @@ __device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, con
     const u4 *const lo0 = L.hrows + a.I / 8 * ROWS;
     h8 xhi[4] = {}, xlo[4] = {};
     // (tile-major IQ3_S: both planes in one matrix instruction; the Q8_0 form adds the planes inside the accumulator, which one instruction cannot reproduce bit for bit)
-#ifdef QW_DNQ_NOSTACK
-    qw_afrag_rows<ROWS> af = {L.hrows, lo0, false, xhi, xlo};
-#else
     typename std::conditional<F == QW_F_PACKED, qw_afrag_rows2<ROWS>, qw_afrag_rows<ROWS>>::type af = {L.hrows, lo0, false, xhi, xlo};
-#endif
     auto expert = [&](uint32_t task) { return SHARED ? 0u : (uint32_t)L.vlist[task >> ts]; };
     // the workgroup's tiles go to its waves from a queue (qw_task_queue): a wave that is done takes the next one, and the
     // shared expert's tiles go to the waves that leave the routed ones first
@@ -1621,11 +1618,7 @@ __device__ __forceinline__ void dnq_run(const qwk_dn_args &a, const u2 *lut, con
         if (lane == 0) j = atomicAdd(&L.q[SHARED ? 1 : 0], 1u);
         return (uint32_t)__builtin_amdgcn_readfirstlane((int)j);
     };
-#ifdef QW_DNQ_NOQUEUE
-    qw_task_stream<C>(nv * tpw, qw_wave(), blockDim.x >> 6, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
-#else
     qw_task_queue<C>(nv * tpw, SHARED ? next() : qw_wave(), next, cpr, CH * C::BLK_B, qw_tiled(F) ? lane : lane & 3,
-#endif
         [&](uint32_t task) {
             const uint32_t tile = g * tpw + (task & tm);
             const uint8_t *W = SHARED ? a.Wsd : a.Wd + (size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)L.ue[expert(task)]) * (qw_tiled(F) ? tpe : a.D) * a.rowbytes;
