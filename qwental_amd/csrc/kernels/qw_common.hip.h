@@ -322,6 +322,15 @@ struct qw_afrag_gather {
     }
 };
 
+// A provider that holds its fragments in registers (member x[], declared `indexed`) is read by position, the others by
+// K offset: idx is a constant wherever the loops around the call are unrolled, so x[idx] is a register, not an address.
+template <class T, class = void> struct qw_is_indexed : std::false_type {};
+template <class T> struct qw_is_indexed<T, std::void_t<decltype(T::indexed)>> : std::true_type {};
+template <class AF> __device__ __forceinline__ h8 qw_af_hi(const AF &af, int idx, uint32_t koff) {
+    if constexpr (qw_is_indexed<AF>::value) return af.x[idx];
+    else return af.hi(koff);
+}
+
 // ---------------------------------------------------------------- chunks: the unit of prefetch
 // A chunk is NB consecutive blocks of one weight row, held in registers by the lane that decodes them. Kernels keep
 // DEPTH chunks per wave (two or three): while one is decoded and multiplied, the loads of the next one or two are in
@@ -406,7 +415,7 @@ template <int NB> struct qw_chunk<21, NB> {
             h8 xh[8], xl[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                xh[j] = af.hi(kb + 8 * j);
+                xh[j] = qw_af_hi(af, 8 * b + j, kb + 8 * j);
                 if (AF::has_lo) xl[j] = af.lo(kb + 8 * j);
             }
             block_mfma(b, w, xh, xl, AF::has_lo, acc);
@@ -682,7 +691,7 @@ template <int NB> struct qw_chunk<8, NB> {
             const h8 w = qw_q8_cvt(q[b]);
             const uint32_t kb = k0 + 32 * b + 8 * kg;
             f4 sub = {0, 0, 0, 0};
-            sub = qw_mfma(af.hi(kb), w, sub);
+            sub = qw_mfma(qw_af_hi(af, b, kb), w, sub);
             if (AF::has_lo) sub = qw_mfma(af.lo(kb), w, sub);
             acc += qw_h2f(d[b]) * sub;
         }

@@ -1124,25 +1124,48 @@ template <int WF> __device__ __forceinline__ void pre_router(const qwk_pre_args 
 // and wave 0 adds them in wave order. A token's logits do not depend on the other token columns.
 // Eight waves take part whatever the workgroup's size: the split of K and the order of the final sum, hence the bits
 // of the logits, are the same in every kernel that holds this router.
+// Up to this many tokens the front launch reads operand A straight from memory instead of staging all of x in LDS: a
+// wave then reads only the K range it multiplies (8 KB of 64 at sixteen tokens) and no barrier stands before the first
+// product — but every lane of an operand reads its own token's row, 64 requests an instruction, which the address unit
+// serialises: with 8 or 16 tokens the staged form is 1 to 2 us faster, with one or two the direct one (24 layers at one
+// token: 0.638 -> 0.618 ms).
+#define QW_PRE_DIRECT_NB 2u
 __device__ __forceinline__ void pre_router_mfma(const qwk_router_args &a, u4 *xf, f4 *part) {
     const uint32_t lane = qw_lane(), n = lane & 15, kg = lane >> 4, wave = qw_wave(), nwv = QW_WG / 64;
     const uint32_t row = 16 * blockIdx.x + n;
     const uint16_t *wrow = row < a.E ? (const uint16_t *)a.Wr + (size_t)row * a.D : (const uint16_t *)a.Wsg; // rows past E repeat the gate vector; not stored
     f4 acc = {0, 0, 0, 0};
-    // the first pass's weights are in flight while x is staged
     u4 w[8];
     uint32_t k0 = wave < nwv ? 256 * wave : a.D; // (waves past the eighth: nothing)
-    if (k0 < a.D)
+    if (a.nb <= QW_PRE_DIRECT_NB) {
+        // lane (n, kg) supplies eight activations of token n per step; token columns past the batch read token 0's row,
+        // their results are never stored
+        const uint16_t *xrow = a.x + (size_t)(n < a.nb ? n : 0) * a.D;
+        u4 xa[8];
+        if (k0 < a.D)
 #pragma unroll
-        for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 32 * j + 8 * kg);
-    qw_stage_x(xf, a.x, a.D, a.D, a.nb);
-    __syncthreads();
-    for (; k0 < a.D; k0 += 256 * nwv) {
+            for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 32 * j + 8 * kg), xa[j] = *(const u4 *)(xrow + k0 + 32 * j + 8 * kg);
+        for (; k0 < a.D; k0 += 256 * nwv) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) acc = qw_mfma(__builtin_bit_cast(h8, xf[((k0 + 32 * j + 8 * kg) >> 3) * 16 + n]), __builtin_bit_cast(h8, w[j]), acc);
-        if (k0 + 256 * nwv < a.D)
+            for (int j = 0; j < 8; j++) acc = qw_mfma(__builtin_bit_cast(h8, xa[j]), __builtin_bit_cast(h8, w[j]), acc);
+            if (k0 + 256 * nwv < a.D)
 #pragma unroll
-            for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 256 * nwv + 32 * j + 8 * kg);
+                for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 256 * nwv + 32 * j + 8 * kg), xa[j] = *(const u4 *)(xrow + k0 + 256 * nwv + 32 * j + 8 * kg);
+        }
+    } else {
+        // the first pass's weights are in flight while x is staged
+        if (k0 < a.D)
+#pragma unroll
+            for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 32 * j + 8 * kg);
+        qw_stage_x(xf, a.x, a.D, a.D, a.nb);
+        __syncthreads();
+        for (; k0 < a.D; k0 += 256 * nwv) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc = qw_mfma(__builtin_bit_cast(h8, xf[((k0 + 32 * j + 8 * kg) >> 3) * 16 + n]), __builtin_bit_cast(h8, w[j]), acc);
+            if (k0 + 256 * nwv < a.D)
+#pragma unroll
+                for (int j = 0; j < 8; j++) w[j] = *(const u4 *)(wrow + k0 + 256 * nwv + 32 * j + 8 * kg);
+        }
     }
     part[wave * 64 + lane] = acc;
     __syncthreads();
@@ -1153,6 +1176,20 @@ __device__ __forceinline__ void pre_router_mfma(const qwk_router_args &a, u4 *xf
         for (uint32_t j = 0; j < 4; j++)
             if (4 * kg + j < a.nb) a.logits[(size_t)(4 * kg + j) * (a.E + 1) + row] = acc[j];
 }
+// Operand A of one chunk held in registers: the fragments a lane needs for its chunk, asked for together with the chunk's
+// weights (read by position: qw_af_hi). BLK_K = 256: a lane's slice of a block is 64 values, eight steps of 8; BLK_K = 32:
+// one step a block.
+template <int BLK_K, int NB> struct qw_afrag_regs {
+    static constexpr int NX = BLK_K == 256 ? 8 * NB : NB;
+    static constexpr bool indexed = true, has_lo = false;
+    h8 x[NX];
+    __device__ __forceinline__ void load(const uint16_t *row, uint32_t k0, uint32_t kg) { // row: this lane's token
+#pragma unroll
+        for (int i = 0; i < NX; i++) x[i] = *(const h8 *)(row + k0 + (BLK_K == 256 ? 64 * kg + 256 * (i >> 3) + 8 * (i & 7) : 8 * kg + 32 * i));
+    }
+    __device__ __forceinline__ h8 hi(uint32_t) const { return h8{}; } // (not used: the provider is indexed)
+    __device__ __forceinline__ h8 lo(uint32_t) const { return h8{}; }
+};
 template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pre_args &pa, u2 *lut, u4 *xf, f4 *part) {
     typedef qw_chunk<F, CH> C;
     const qwk_gu_args &a = pa.g;
@@ -1165,17 +1202,34 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
         if constexpr (F == QW_F_PACKED) c.load(a.Wg + (size_t)tile * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane);
         else c.load(((lane >> 2) < 8 ? a.Wg : a.Wu) + ((size_t)8 * tile + ((lane >> 2) & 7)) * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane & 3);
     }
-    // the table and the activations behind the weights, all awaited once: one memory round trip before the barrier
-    if (qw_has_lut(F)) qw_lut_copy_issue(lut, (const u2 *)a.glut);
-    qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
-    qw_lds_arrive();
-    __syncthreads();
     f4 acc = {0, 0, 0, 0};
-    if (on) {
-        c.transpose();
-        const qw_afrag_lds af = {xf, n};
-        c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
-        part[wave * 64 + lane] = acc;
+    if (a.nbr <= QW_PRE_DIRECT_NB) {
+        // one or two tokens: the chunk's activations straight into registers, the table behind the weights; all awaited
+        // once. Token columns past the batch read token 0's row; their results are never stored.
+        qw_afrag_regs<C::BLK_K, CH> af;
+        if (on) af.load(a.x + (size_t)(n < a.nbr ? n : 0) * a.D, ci * CH * C::BLK_K, kg);
+        if (qw_has_lut(F)) {
+            qw_lut_copy_issue(lut, (const u2 *)a.glut);
+            qw_lds_arrive();
+            __syncthreads();
+        }
+        if (on) {
+            c.transpose();
+            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+            part[wave * 64 + lane] = acc;
+        }
+    } else {
+        // the table and the activations behind the weights, all awaited once: one memory round trip before the barrier
+        if (qw_has_lut(F)) qw_lut_copy_issue(lut, (const u2 *)a.glut);
+        qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
+        qw_lds_arrive();
+        __syncthreads();
+        if (on) {
+            c.transpose();
+            const qw_afrag_lds af = {xf, n};
+            c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
+            part[wave * 64 + lane] = acc;
+        }
     }
     __syncthreads();
     if (!on || ci != 0) return;
