@@ -336,7 +336,10 @@ def qmv_table(gpu, reps=5, nmat=64):
                         b.buf(0, W, i * N * rb)
                         b.dispatch((N + 7) // 8, 1, 1, 256, 1, 1)
                     best = min(best, b.end())
-                out["%s_B%d%s" % ("iq3_s" if ft == 21 else "q8_0", nb, "_valu" if valu else "")] = {"us_per_matvec": best / nmat * 1e6, "GBps": algo / (best / nmat) / 1e9}
+                # (frac_of_peak: the launch's algorithmic bytes over its time against the 8 TB/s of the data sheet; at this size a
+                # launch is mostly its own fixed cost, an empty launch of the same grid takes 2.5 us)
+                out["%s_B%d%s" % ("iq3_s" if ft == 21 else "q8_0", nb, "_valu" if valu else "")] = {"us_per_matvec": best / nmat * 1e6, "GBps": algo / (best / nmat) / 1e9,
+                                                                                                  "algorithmic_bytes": algo, "frac_of_peak": algo / (best / nmat) / 1e9 / HBM_PEAK_GBS}
         W.free()
     path.close()
     x.free()
