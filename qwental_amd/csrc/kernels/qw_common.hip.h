@@ -841,17 +841,29 @@ __device__ __forceinline__ void qw_task_queue(uint32_t ntasks, uint32_t first, N
 #pragma unroll
     for (int i = 0; i + 1 < DEPTH; i++) load(i);
     ready();
-    for (bool done = false; !done;) {
-#pragma unroll
-        for (int i = 0; i < DEPTH; i++) {
-            if (!done) { // (a guard, not a break: the loop unrolls and every buffer keeps its registers)
-                load((i + DEPTH - 1) % DEPTH);
-                if (btask[i] >= ntasks) done = true;
-                else {
-                    buf[i].transpose();
-                    use(btask[i], bchunk[i], buf[i]);
-                }
-            }
+    // One phase per chunk buffer, written out instead of an unrolled loop with a flag: the wave leaves from inside a
+    // phase, so the only way back to the top is the one on which every load but the last phase's has been waited for,
+    // and the youngest chunk stays in flight across the turn (with the flag, the leaving path met the top of the loop
+    // and the compiler emptied the queue there on every turn).
+    static_assert(DEPTH >= 1 && DEPTH <= 4, "chunk buffers");
+    auto phase = [&](auto I) -> bool {
+        constexpr int i = decltype(I)::value;
+        load((i + DEPTH - 1) % DEPTH);
+        if (btask[i] >= ntasks) return false;
+        buf[i].transpose();
+        use(btask[i], bchunk[i], buf[i]);
+        return true;
+    };
+    for (;;) {
+        if (!phase(std::integral_constant<int, 0>{})) break;
+        if constexpr (DEPTH > 1) {
+            if (!phase(std::integral_constant<int, 1>{})) break;
+        }
+        if constexpr (DEPTH > 2) {
+            if (!phase(std::integral_constant<int, 2>{})) break;
+        }
+        if constexpr (DEPTH > 3) {
+            if (!phase(std::integral_constant<int, 3>{})) break;
         }
     }
 }
@@ -877,6 +889,36 @@ __device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut) {
     for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i < N; i += blockDim.x) {
         const uint32_t j = (i + rot) & (N - 1); // a multiple of 64, the same in every lane
         qw_load_to_lds(src + j + lane, dst + j);
+    }
+}
+// The same copy with a fixed number of loads in every wave (NW waves a workgroup), for a caller that counts the loads
+// it has outstanding: a wave whose share is short copies an earlier piece once more (same bytes to the same place).
+template <uint32_t NW> constexpr uint32_t qw_lut_copy_loads() { return (QW_LUT_BYTES / 16 + 64 * NW - 1) / (64 * NW); }
+template <uint32_t NW> __device__ __forceinline__ void qw_lut_copy_issue_n(u2 *lut, const u2 *glut) {
+    const u4 *src = (const u4 *)glut;
+    u4 *dst = (u4 *)lut;
+    constexpr uint32_t N = QW_LUT_BYTES / 16;
+    const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63, w64 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64;
+#pragma unroll
+    for (uint32_t it = 0; it < qw_lut_copy_loads<NW>(); it++) {
+        uint32_t i = w64 + it * 64 * NW;
+        if (i >= N) i -= 64 * NW;
+        const uint32_t j = (i + rot) & (N - 1);
+        qw_load_to_lds(src + j + lane, dst + j);
+    }
+}
+// Likewise the activations of qw_stage_x_issue for up to MAXN / 32 values a row: a fixed number of loads in every wave,
+// and the rows past nb repeat row nb - 1 instead of holding zeros (they feed matrix-core output rows that nobody reads).
+template <uint32_t NW, uint32_t MAXN> constexpr uint32_t qw_stage_x_loads() { return (MAXN + 64 * NW - 1) / (64 * NW); }
+template <uint32_t NW, uint32_t MAXN> __device__ __forceinline__ void qw_stage_x_issue_n(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
+    const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 320u) % n, lane = threadIdx.x & 63, w64 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64;
+    const uint32_t last = nb ? nb - 1 : 0;
+#pragma unroll
+    for (uint32_t it = 0; it < qw_stage_x_loads<NW, MAXN>(); it++) {
+        uint32_t i0 = w64 + it * 64 * NW;
+        while (i0 >= n) i0 -= n;
+        const uint32_t base = i0 + rot < n ? i0 + rot : i0 + rot - n, i = base + lane, c = i >> 4, m = i & 15;
+        qw_load_to_lds((const u4 *)(x + (size_t)(m < nb ? m : last) * xstride + 8 * c), xf + base);
     }
 }
 __device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {

@@ -31,6 +31,18 @@ __device__ uint32_t *qw_stamp_ptr;
 #define QW_DSTAMP(k) do {} while (0)
 #define QW_WSTAMP(k) do {} while (0)
 #endif
+#if defined(QW_STAMPS) && QW_STAMPS == 3 // steps of the selection in the routed gate/up launch: 16 stamps a wave, kept in LDS until the launch ends
+__shared__ uint32_t qw_sst[12 * 16];
+#undef QW_DSTAMP
+#define QW_DSTAMP(k) do {} while (0)
+#define QW_SSTAMP(k) do { if ((threadIdx.x & 63) == 0) qw_sst[(threadIdx.x >> 6) * 16 + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#define QW_SDEP(v) asm volatile("" :: "v"(v))
+#define QW_SST_FLUSH() do { QW_SSTAMP(15); __syncthreads(); if (qw_stamp_ptr && blockIdx.x < 32 && threadIdx.x < 192) qw_stamp_ptr[512 + 192 * blockIdx.x + threadIdx.x] = qw_sst[threadIdx.x]; } while (0)
+#else
+#define QW_SSTAMP(k) do {} while (0)
+#define QW_SDEP(v) do {} while (0)
+#define QW_SST_FLUSH() do {} while (0)
+#endif
 #ifdef QW_STAMPS
 #define QW_WG_END_STAMP(k) do { __syncthreads(); QW_DSTAMP(k); } while (0)
 #else
@@ -664,7 +676,8 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
     }
 }
 
-// The same result without the chain of K dependent wave-wide maxima. Every lane finds the maximum of its PER keys;
+// The same result without the chain of K dependent wave-wide maxima. Lane l holds experts l, l + 64, ... here (which lane
+// holds a key does not matter to this form, and a wave's load is then 256 contiguous bytes). Every lane finds the maximum of its PER keys;
 // a value T0 that at least K of the 64 lane maxima reach bounds the answer from below: at least K keys are >= T0, so
 // no key below T0 can be picked. The keys >= T0 (K of them, or a few more) are gathered one to a lane, each is ranked among
 // them by (key descending, expert ascending) - the order of the repeated maximum with ties to the lowest index - and
@@ -674,18 +687,32 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
 // ws: 144 dwords of LDS scratch per token for this wave. need_w: also the gating weights (softmax over the picked
 // logits in rank order, sigmoid of the shared-expert logit).
 // issued(): called once the loads of the logits are issued (the place for the caller's own prefetches: loads return in
-// the order of issue, and the logits are needed first).
-template <int PER, int T, class H>
+// the order of issue, and the logits are needed first); it issues at least NDMA vector memory loads in every wave, and
+// the keys are used as soon as no more than NDMA loads of the wave are outstanding.
+template <int PER, int T, uint32_t NDMA, class H>
 __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, uint32_t E, uint32_t K, const uint32_t (&tok)[T], const bool (&on)[T], float *w, uint32_t *ids, uint32_t *ws,
                                                         uint32_t lane, bool need_w, H issued) {
     uint32_t k[T][PER], M[T], T0[T], c[T], pos[T][PER];
+    // The loads of the logits are written out, and so is the wait for them: issued() asks for NDMA more loads (straight
+    // into LDS, wanted much later), the loads of a wave return in the order of issue, and the compiler waits for
+    // everything outstanding when loads into registers and loads into LDS are in flight together. Nothing may read k
+    // between here and the wait (the registers are not valid yet).
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        const float *p = logits + (size_t)tok[t] * (E + 1) + lane; // (a wave reads 256 contiguous bytes a load)
+#pragma unroll
+        for (int j = 0; j < PER; j++) asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(k[t][j]) : "v"(p), "n"(j * 256) : "memory");
+    }
+    QW_DSTAMP(12);
+    QW_SSTAMP(3);
+    issued();
+    QW_DSTAMP(13);
+    QW_SSTAMP(4);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
 #pragma unroll
     for (int t = 0; t < T; t++)
 #pragma unroll
-        for (int j = 0; j < PER; j++) k[t][j] = __builtin_bit_cast(uint32_t, logits[(size_t)tok[t] * (E + 1) + lane * PER + j]);
-    QW_DSTAMP(12);
-    issued();
-    QW_DSTAMP(13);
+        for (int j = 0; j < PER; j++) asm volatile("" : "+v"(k[t][j])); // (every use of k follows the wait)
 #pragma unroll
     for (int t = 0; t < T; t++) {
         M[t] = 0;
@@ -693,14 +720,19 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
         for (int j = 0; j < PER; j++) k[t][j] = qw_fkey(__builtin_bit_cast(float, k[t][j])), M[t] = max(M[t], k[t][j]);
         T0[t] = 0;
     }
+    QW_SDEP(M[T - 1]);
+    QW_SSTAMP(5);
     // T0: the largest value with bits [lo, 32) such that at least K lane maxima reach it, found bit by bit with a
     // ballot each (scalar work but for the comparison). The upper 16 bits are nearly always enough to leave at most
     // 64 keys; otherwise the lower 16 follow, which makes T0 the K-th largest lane maximum itself.
-    auto refine = [&](int t, int hi, int lo) {
-        for (int b = hi; b >= lo; b--) {
-            const uint32_t cd = T0[t] | (1u << b);
-            if ((uint32_t)__popcll(__ballot(M[t] >= cd)) >= K) T0[t] = cd;
-        }
+    // (the tokens of `which` side by side: a step is a chain of vector compare -> scalar count -> scalar select)
+    auto refine = [&](uint32_t which, int hi, int lo) {
+        for (int b = hi; b >= lo; b--)
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                const uint32_t cd = T0[t] | (1u << b);
+                if (((which >> t) & 1) && (uint32_t)__popcll(__ballot(M[t] >= cd)) >= K) T0[t] = cd;
+            }
     };
     // gather the keys >= T0: position = candidates of earlier j, plus those of lower lanes at this j
     auto gather = [&](int t) {
@@ -712,24 +744,28 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
             c[t] += (uint32_t)__popcll(bal);
         }
     };
-    uint32_t fail = 0;
+    uint32_t fail = 0, more = 0;
+    refine((1u << T) - 1, 31, 16);
 #pragma unroll
     for (int t = 0; t < T; t++) {
-        refine(t, 31, 16);
         gather(t);
-        if (c[t] > 64) {
-            refine(t, 15, 0);
-            gather(t);
-        }
+        if (c[t] > 64) more |= 1u << t;
+    }
+    if (more) refine(more, 15, 0);
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        if ((more >> t) & 1) gather(t);
         if (c[t] > 64 || !on[t]) fail |= 1u << t;
     }
+    QW_SDEP(pos[T - 1][PER - 1]);
+    QW_SSTAMP(6);
 #pragma unroll
     for (int t = 0; t < T; t++) {
         if ((fail >> t) & 1) continue;
         u2 *cand = (u2 *)(ws + 144 * t); // (key, expert) of candidate p
 #pragma unroll
         for (int j = 0; j < PER; j++)
-            if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], lane * PER + j};
+            if (k[t][j] >= T0[t]) cand[pos[t][j]] = u2{k[t][j], j * 64 + lane};
     }
     uint32_t mk[T], me[T], rank[T];
 #pragma unroll
@@ -739,24 +775,36 @@ __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, ui
         mk[t] = lane < c[t] ? mine.x : 0, me[t] = lane < c[t] ? ~mine.y : 0;
         rank[t] = 0;
     }
+    QW_SDEP(mk[T - 1]);
+    QW_SSTAMP(7);
+    // (all tokens against candidate lane l in one step; lanes past a token's own count hold the least value and add nothing)
+    uint32_t cm = 0;
 #pragma unroll
-    for (int t = 0; t < T; t++) {
-        if ((fail >> t) & 1) continue;
-        const unsigned long long mine = (unsigned long long)mk[t] << 32 | me[t];
-        for (uint32_t q0 = 0; q0 < c[t]; q0 += 16) // candidates sixteen at a time, read from their lanes
+    for (int t = 0; t < T; t++)
+        if (!((fail >> t) & 1)) cm = max(cm, c[t]);
+    for (uint32_t q0 = 0; q0 < cm; q0 += 16) // candidates sixteen at a time, read from their lanes
 #pragma unroll
-            for (uint32_t q = 0; q < 16; q++) {
-                if (q >= 8 && q0 + q >= c[t]) break; // uniform: ten to twelve candidates are the common case
-                const uint32_t l = q0 ? (q0 + q) & 63 : q;
+        for (uint32_t q = 0; q < 16; q++) {
+            if (q >= 8 && q0 + q >= cm) break; // uniform: ten to twelve candidates are the common case
+            const uint32_t l = q0 ? (q0 + q) & 63 : q;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                const unsigned long long mine = (unsigned long long)mk[t] << 32 | me[t];
                 const unsigned long long o = (unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)mk[t], (int)l) << 32 | (uint32_t)__builtin_amdgcn_readlane((int)me[t], (int)l);
                 rank[t] += o > mine;
             }
+        }
+#pragma unroll
+    for (int t = 0; t < T; t++) {
+        if ((fail >> t) & 1) continue;
         uint32_t *pkr = ws + 144 * t + 128; // key of rank r
         if (lane < c[t] && rank[t] < K) {
             ids[tok[t] * K + rank[t]] = ~me[t];
             pkr[rank[t]] = mk[t];
         }
     }
+    QW_SDEP(rank[T - 1]);
+    QW_SSTAMP(8);
     if (!need_w) return fail; // the gating weights are only wanted by the workgroup that writes the record
 #pragma unroll
     for (int t = 0; t < T; t++) {
@@ -804,54 +852,73 @@ __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 ||
 // The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
 // floats per wave (288 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
 // store: this workgroup writes the record; need_w: it wants the gating weights in s.w (store implies it).
-template <class H>
+// issued(): runs once in every wave, behind the wave's loads of its first tokens' logits when it has tokens; NDMA as in
+// select_tokens_ranked.
+template <uint32_t NDMA = 0, class H>
 __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued, bool need_w = false) {
     need_w = need_w || store;
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
-    // nothing the token loop writes is cleared here (rows of w past the batch only), so no barrier separates the two
-    for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
-    for (uint32_t i = tid; i < GU; i += nth) c.ue[i] = 0, c.mask[i] = 0;
-    for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
-    if (tid < 8) s.lead[tid] = 0;
-    for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
-    QW_DSTAMP(11);
-    if (fast) { // two tokens per wave at a time when there are more tokens than waves; lgs gives a wave 288 dwords
+    QW_SDEP(E + K + gnb + a.nbr);
+    QW_SSTAMP(1);
+    // nothing the token loop writes is cleared here (rows of w past the batch only), so no barrier separates the two,
+    // and with the fast form the clearing waits until the logits have been asked for
+    auto issued_clear = [&] {
+        issued();
+        for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
+        for (uint32_t i = tid; i < GU; i += nth) c.ue[i] = 0, c.mask[i] = 0;
+        for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
+        if (tid < 8) s.lead[tid] = 0;
+        for (uint32_t i = a.nbr * (K + 1) + tid; i < gnb * (K + 1); i += nth) s.w[i] = 0;
+        QW_DSTAMP(11);
+        QW_SSTAMP(2);
+    };
+    if (fast) { // a first pass of straight-line code: a wave takes one token, or two when there are more tokens than waves (lgs gives a wave 288 dwords)
         uint32_t *ws = (uint32_t *)lgs + 288 * wave;
         const uint32_t trot = a.nbr ? blockIdx.x % a.nbr : 0; // the workgroups of a launch read the tokens' logits in different orders
         auto rot = [&](uint32_t tt) { return tt + trot < a.nbr ? tt + trot : tt + trot - a.nbr; };
         const bool pairs = E <= 512; // sixteen keys a lane: one token at a time (registers)
-        for (uint32_t tt = wave; tt < a.nbr; tt += (pairs ? 2 : 1) * nwv) {
+        auto slow = [&](uint32_t tok) { // the repeated maximum
+            switch (E) {
+            case 64: select_tokens<1, 1>(a.logits, E, K, tok, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 128: select_tokens<2, 1>(a.logits, E, K, tok, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 256: select_tokens<4, 1>(a.logits, E, K, tok, nwv, a.nbr, s.w, s.ids, lane); break;
+            case 512: select_tokens<8, 1>(a.logits, E, K, tok, nwv, a.nbr, s.w, s.ids, lane); break;
+            default: select_tokens<16, 1>(a.logits, E, K, tok, nwv, a.nbr, s.w, s.ids, lane); break;
+            }
+        };
+        if (wave < a.nbr) {
+            const uint32_t tt = wave;
             const bool two = pairs && tt + nwv < a.nbr;
             const uint32_t tk[2] = {rot(tt), two ? rot(tt + nwv) : rot(tt)};
             const bool on2[2] = {true, two}, on1[1] = {true};
             const uint32_t t1[1] = {tk[0]};
             uint32_t fail;
             switch (E) {
-            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
-            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
-            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
-            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
-            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued); break;
+            case 64: fail = two ? select_tokens_ranked<1, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<1, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
+            case 128: fail = two ? select_tokens_ranked<2, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<2, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
+            case 256: fail = two ? select_tokens_ranked<4, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<4, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
+            case 512: fail = two ? select_tokens_ranked<8, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<8, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
+            default: fail = select_tokens_ranked<16, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
             }
-            for (uint32_t i = 0; i < 2; i++) { // more than 64 keys tie at the bound: the repeated maximum instead
-                if (!((fail >> i) & 1) || (i == 1 && !two)) continue;
-                switch (E) {
-                case 64: select_tokens<1, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
-                case 128: select_tokens<2, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
-                case 256: select_tokens<4, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
-                case 512: select_tokens<8, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
-                default: select_tokens<16, 1>(a.logits, E, K, tk[i], nwv, a.nbr, s.w, s.ids, lane); break;
-                }
-            }
+            for (uint32_t i = 0; i < 2; i++) // more than 64 keys tie at the bound
+                if (((fail >> i) & 1) && (i == 0 || two)) slow(tk[i]);
+        } else issued_clear();
+        // tokens that the first pass does not reach (more than the waves when a lane holds sixteen keys, more than twice the waves otherwise)
+        for (uint32_t tt = wave + (pairs ? 2 : 1) * nwv; tt < a.nbr; tt += nwv) {
+            const uint32_t t1[1] = {rot(tt)};
+            const bool on1[1] = {true};
+            if (pairs || select_tokens_ranked<16, 1, 0>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, [] {})) slow(t1[0]);
         }
     } else {
+        issued_clear();
         for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
-    issued(); // the waves without a token
     QW_DSTAMP(15);
+    QW_SSTAMP(9);
     __syncthreads();
+    QW_SSTAMP(10);
     if (a.nbr == 1) { // one token: its picks are the unique experts, in rank order (what the steps below would leave)
         if (tid < K) c.ue[tid] = s.ids[tid], c.mask[tid] = 1, c.slot[tid * gnb] = (uint8_t)tid;
         if (tid == 0) c.U = K;
@@ -859,6 +926,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     } else {
     if (tid < UM) atomicMin(&s.first[s.ids[tid]], tid); // first flat index of every picked expert
     __syncthreads();
+    QW_SSTAMP(11);
     // lead = this pair is its expert's first; every wave leaves the ballot of its leads (UM <= 256: four waves)
     uint32_t f = 0;
     bool lead = false;
@@ -871,6 +939,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         if (lane == 0) s.lead[2 * wave] = (uint32_t)bal, s.lead[2 * wave + 1] = (uint32_t)(bal >> 32);
     }
     __syncthreads();
+    QW_SSTAMP(12);
     // unique index of a pair = number of leads before its expert's first pair
     if (tid < UM) {
         uint32_t u = 0;
@@ -889,6 +958,7 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
     }
     __syncthreads();
     }
+    QW_SSTAMP(13);
     if (!store) return;
     // the record, in one pass of dword stores: U | ue[GU] | mask[GU] | slot[GU][gnb] | w[gnb][K + 1]
     uint32_t *out = (uint32_t *)a.sel;
@@ -1004,6 +1074,7 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
     if (threadIdx.x == 0) sc->qnext = blockDim.x >> 6; // (nothing below writes it; a barrier follows on every path)
     if (threadIdx.x == 0) QW_WSTAMP(12);
     QW_DSTAMP(0);
+    QW_SSTAMP(0);
     if constexpr (FGU == QW_F_RT) qw_kq_tab_build((uint32_t *)(lut + (qw_has_lut(FSG) ? QW_LUT_ENTRIES : 0))); // (published by the barriers below)
     if (a.logits) { // the selection, made here by every workgroup
         const qwk_select_args sa = {a.logits, const_cast<uint8_t *>(a.sel), a.nbr, a.E, a.topk, a.gnb};
@@ -1012,15 +1083,20 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
             // their place (they follow in ready()).
             constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
             const bool early = a.D * 2 + (QW_WG_GU / 64) * 288 / 4 <= QW_XF_MAXK * 2;
-            bool fetched = false;
-            select_all(sa, *ss, *sc, (float *)(early ? xf + a.D * 2 : xf), blockIdx.x == 0, [&] {
-                if (fetched) return;
-                fetched = true;
-                if (lutp) qw_lut_copy_issue(lut, (const u2 *)a.glut);
-                if (early) qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
+            // (the table and the activations are asked for behind the logits, a fixed number of loads a wave, so that the
+            // selection goes on as soon as the logits are there; when the activations have to wait for the scratch's place,
+            // the table is copied twice to keep that number: one selection per kernel instead of two)
+            constexpr uint32_t NWV = QW_WG_GU / 64, XN = QW_XF_MAXK * 2 - NWV * 288 / 4, NT = qw_lut_copy_loads<NWV>(), NX = qw_stage_x_loads<NWV, XN>();
+            static_assert(NT == NX, "two copies of equal length");
+            // (a kernel without the table counts nothing: its selection waits for whatever it has asked for)
+            select_all<lutp ? NT + NX : 0>(sa, *ss, *sc, (float *)(early ? xf + a.D * 2 : xf), blockIdx.x == 0, [&] {
+                if (lutp) qw_lut_copy_issue_n<NWV>(lut, (const u2 *)a.glut);
+                if (early) qw_stage_x_issue_n<NWV, XN>(xf, a.x, a.D, a.D, a.nbr);
+                else if (lutp) qw_lut_copy_issue_n<NWV>(lut, (const u2 *)a.glut);
             }, all_w);
             qw_lds_arrive();
             __syncthreads();
+            QW_SSTAMP(14);
             staged = early;
             tabled = true;
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
@@ -1084,6 +1160,7 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
         qw_h_global hs = {a.H, a.hplane};                                                                      \
         gu_body<FGU, CHGU, FSG, CHSG>(a, L.lut, L.xf, &L.sc, &L.ss, hs, false, [] {});                           \
         QW_WG_END_STAMP(10);                                                                                    \
+        QW_SST_FLUSH();                                                                                         \
     }
 // K = D a multiple of 512: 2 IQ3_S blocks or 16 Q8_0 blocks a chunk; any other K: 1.
 #if QW_IN_PART(1)
@@ -1720,15 +1797,30 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
     uint32_t nt = base + (q < rem ? 1 : 0);
     if (nt > 4) nt = 4; // (the host admits 16 tokens in four quarters, 8 in two)
     QW_DSTAMP(6);
-    // one memory round trip: the record (U, experts, masks, this quarter's slot bytes and gating weights), every H row of the
-    // quarter's tokens (which rows they are does not depend on the record) and the table. The rows go through registers into
-    // LDS in fragment order; a wave's load takes 8 rows x 128 bytes (whole cache lines), lanes 0 .. 31 the first 64 bytes
-    // of a row, 32 .. 63 the rest.
+    // Everything is asked for at once, in the order in which it is wanted: the record (U, experts, masks, this quarter's slot
+    // bytes and gating weights), every H row of the quarter's tokens (which rows they are does not depend on the record)
+    // and the table - all through registers, so that the waits are exact (with loads straight into LDS in flight the
+    // compiler waits for everything outstanding). The record goes to LDS as soon as it is there, the waves list the
+    // experts and ask for their first tiles; rows and table follow into LDS while those tiles are on their way (ready()).
+    // A wave's row load takes 8 rows x 128 bytes (whole cache lines), lanes 0 .. 31 the first 64 bytes of a row, 32 .. 63 the rest.
+    constexpr uint32_t NW = QW_WG_DN / 64, RPER = (2 * 6 * 8 + NW - 1) / NW; // 2 planes x 6 row blocks x 8 column blocks at most
+    constexpr bool TAB = qw_has_lut(F) || qw_has_lut(FSD);
+    constexpr uint32_t TPER = TAB ? (QW_LUT_BYTES / 16 + QW_WG_DN - 1) / QW_WG_DN : 0;
+    u4 rowv[RPER], tabv[TPER ? TPER : 1];
+    uint32_t at[RPER], tat[TPER ? TPER : 1];
     {
+        const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mk = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
+        const uint8_t *sl = a.sel + QW_SEL_OFF_SLOT(gnb, K);
+        const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K)) + t0 * (K + 1);
+        // (GU <= 160 and nt * (K + 1) <= 44: one element a thread; a thread without one reads element 0)
+        const bool rec = tid < GU, hasw = tid < nt * (K + 1);
+        const uint32_t ri = rec ? tid : 0;
+        const uint32_t r_ue = ue[ri], r_mk = mk[ri], r_U = *(const uint32_t *)a.sel;
+        uint32_t r_sl[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; j++) r_sl[j] = sl[ri * gnb + t0 + (j < nt ? j : 0)];
+        const float r_w = wg[hasw ? tid : 0];
         const uint32_t upr = a.I / 8, cbs = upr / 8, used = nt * (K + 1), nrb = (used + 7) / 8, nunits = 2 * nrb * cbs, wv = qw_wave();
-        constexpr uint32_t NW = QW_WG_DN / 64, RPER = (2 * 6 * 8 + NW - 1) / NW; // 2 planes x 6 row blocks x 8 column blocks at most
-        u4 rowv[RPER];
-        uint32_t at[RPER];
 #pragma unroll
         for (uint32_t it = 0; it < RPER; it++) {
             const uint32_t unit = wv + it * NW, cb = unit % cbs, rest = unit / cbs, rb = rest % nrb, pl = rest / nrb;
@@ -1738,21 +1830,24 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
             // (a unit that is off reads the first bytes of H: a load under a condition made the compiler keep the whole array in scratch memory)
             rowv[it] = *(const u4 *)(on ? a.H + pl * (size_t)a.hplane + ((size_t)t0 * (K + 1) + r) * a.I + 8 * c : a.H);
         }
-        const uint32_t *ue = (const uint32_t *)(a.sel + QW_SEL_OFF_UE(gnb, K)), *mk = (const uint32_t *)(a.sel + QW_SEL_OFF_MASK(gnb, K));
-        const uint8_t *sl = a.sel + QW_SEL_OFF_SLOT(gnb, K);
-        const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K)) + t0 * (K + 1);
-        if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // (straight into LDS: the registers hold the rows)
-        for (uint32_t i = tid; i < GU; i += blockDim.x) {
-            uint32_t s4 = 0;
-            for (uint32_t j = 0; j < nt; j++) s4 |= (uint32_t)sl[i * gnb + t0 + j] << (8 * j);
-            L.ue[i] = ue[i], L.mask[i] = (uint16_t)mk[i], L.slot4[i] = s4;
-        }
-        for (uint32_t i = tid; i < nt * (K + 1); i += blockDim.x) L.wl[i] = wg[i];
-        if (tid == 0) L.U = *(const uint32_t *)a.sel, L.q[0] = blockDim.x >> 6, L.q[1] = 0;
+        if constexpr (TAB) { // every workgroup starts at another place of the table (as qw_lut_copy_issue); the last piece of some threads repeats an earlier one
 #pragma unroll
-        for (uint32_t it = 0; it < RPER; it++)
-            if (at[it] != ~0u) L.hrows[at[it]] = rowv[it];
-        qw_lds_arrive();
+            for (uint32_t it = 0; it < TPER; it++) {
+                uint32_t i = tid + it * QW_WG_DN;
+                if (i >= QW_LUT_BYTES / 16) i -= QW_WG_DN;
+                tat[it] = (i + blockIdx.x * 320u) & (QW_LUT_BYTES / 16 - 1);
+                tabv[it] = ((const u4 *)a.glut)[tat[it]];
+            }
+        }
+        if (rec) {
+            uint32_t s4 = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; j++)
+                if (j < nt) s4 |= r_sl[j] << (8 * j);
+            L.ue[tid] = r_ue, L.mask[tid] = (uint16_t)r_mk, L.slot4[tid] = s4;
+        }
+        if (hasw) L.wl[tid] = r_w;
+        if (tid == 0) L.U = r_U, L.q[0] = blockDim.x >> 6, L.q[1] = 0;
     }
     __syncthreads();
     QW_DSTAMP(7);
@@ -1774,7 +1869,20 @@ __device__ __forceinline__ void dnq_body(const qwk_dn_args &a, u2 *lut, qw_dnq_l
         if (nv > 48) nv = 48; // (four tokens of ten experts: 40 at most)
     }
     const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0;
-    auto ready = [] {}; // (everything the tiles need is in LDS already)
+    bool staged = false;
+    auto ready = [&] { // called by every wave once it has asked for its first tile
+        if (staged) return;
+        staged = true;
+#pragma unroll
+        for (uint32_t it = 0; it < RPER; it++)
+            if (at[it] != ~0u) L.hrows[at[it]] = rowv[it];
+        if constexpr (TAB) {
+#pragma unroll
+            for (uint32_t it = 0; it < TPER; it++) ((u4 *)lut)[tat[it]] = tabv[it];
+        }
+        __syncthreads();
+        QW_DSTAMP(8);
+    };
     // the routed experts first; the shared expert's tiles go to the waves that leave the routed ones first
     const qw_dnq_view V = {L.hrows, L.part, L.ue, L.slot4, L.mask, L.vlist, L.q};
     dnq_run<F, CH, false, QW_DNQ_ROWS>(a, lut, V, g, t0, nt, nv, ready);
