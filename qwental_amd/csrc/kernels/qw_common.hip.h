@@ -574,12 +574,17 @@ template <int NB> struct qw_chunk<21, NB> {
 
 // Packed IQ3_S (see qwk_pack_args): the slab already lies in matrix-core lane order; three coalesced loads per block
 // and no transpose. p is the (wave-uniform) address of the chunk's first slab, the second argument the lane.
+#ifndef QW_PACKED_DEPTH
+#define QW_PACKED_DEPTH 2
+#endif
 template <int NB> struct qw_chunk<QW_F_PACKED, NB> : qw_chunk<21, NB> {
     static constexpr uint32_t BLK_K = 256, BLK_B = QW_SLAB_BYTES;
     // One chunk ahead, not two: with every wave of the device streaming, more loads in flight made the launches slower
     // (24 layers at 16 tokens, ms: 1.80 with two chunks ahead in the routed gate/up and down launches, 1.70 with one, 1.85
-    // and 1.95 with three and four in the gate/up launch; the grouped product of the packing path 4 % faster with one).
-    static constexpr int DEPTH = 2;
+    // and 1.95 with three and four in the gate/up launch; the grouped product of the packing path 4 % faster with one;
+    // measured again after the queue loop stopped emptying the queue at every turn: two ahead 1.74 against 1.67).
+    // QW_PACKED_DEPTH: for working builds that measure this.
+    static constexpr int DEPTH = QW_PACKED_DEPTH;
     __device__ __forceinline__ void load(const uint8_t *p, uint32_t lane) {
 #pragma unroll
         for (int b = 0; b < NB; b++) {
