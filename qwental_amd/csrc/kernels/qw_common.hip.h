@@ -269,9 +269,11 @@ struct qw_afrag_lds2 {
 // caller runs qw_lds_arrive() and a barrier before the fragments are read.
 __device__ __forceinline__ void qw_load_to_lds(const u4 *src_lane, u4 *dst_wave);
 __device__ __forceinline__ void qw_lds_arrive();
-__device__ __forceinline__ void qw_stage_x_issue(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
+// part, nparts: the calling wave is number `part` of the `nparts` waves that do the copy (default: all of the workgroup).
+__device__ __forceinline__ void qw_stage_x_issue(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb, uint32_t part = ~0u, uint32_t nparts = 0) {
     const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 320u) % n, lane = threadIdx.x & 63; // n and rot are multiples of 64
-    for (uint32_t i0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i0 < n; i0 += blockDim.x) {
+    if (part == ~0u) part = threadIdx.x >> 6, nparts = blockDim.x >> 6;
+    for (uint32_t i0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)part) * 64; i0 < n; i0 += 64 * nparts) {
         const uint32_t base = i0 + rot < n ? i0 + rot : i0 + rot - n, i = base + lane, c = i >> 4, m = i & 15;
         if (m < nb) qw_load_to_lds((const u4 *)(x + (size_t)m * xstride + 8 * c), xf + base);
         else xf[i] = u4{0, 0, 0, 0};
@@ -886,44 +888,16 @@ __device__ __forceinline__ void qw_lds_arrive() { __builtin_amdgcn_s_waitcnt(0);
 // Issue the copy of the 64 KB table into LDS (direct loads, a wave takes 64 entries at a time). Every workgroup of a
 // launch starts at a different place of the table (a rotation by its index), so that at any moment the workgroups
 // ask different memory channels. The caller runs qw_lds_arrive() and a barrier before the table is read.
-__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut) {
+// part, nparts: as in qw_stage_x_issue.
+__device__ __forceinline__ void qw_lut_copy_issue(u2 *lut, const u2 *glut, uint32_t part = ~0u, uint32_t nparts = 0) {
     const u4 *src = (const u4 *)glut;
     u4 *dst = (u4 *)lut;
     constexpr uint32_t N = QW_LUT_BYTES / 16;
     const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63;
-    for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64; i < N; i += blockDim.x) {
+    if (part == ~0u) part = threadIdx.x >> 6, nparts = blockDim.x >> 6;
+    for (uint32_t i = (uint32_t)__builtin_amdgcn_readfirstlane((int)part) * 64; i < N; i += 64 * nparts) {
         const uint32_t j = (i + rot) & (N - 1); // a multiple of 64, the same in every lane
         qw_load_to_lds(src + j + lane, dst + j);
-    }
-}
-// The same copy with a fixed number of loads in every wave (NW waves a workgroup), for a caller that counts the loads
-// it has outstanding: a wave whose share is short copies an earlier piece once more (same bytes to the same place).
-template <uint32_t NW> constexpr uint32_t qw_lut_copy_loads() { return (QW_LUT_BYTES / 16 + 64 * NW - 1) / (64 * NW); }
-template <uint32_t NW> __device__ __forceinline__ void qw_lut_copy_issue_n(u2 *lut, const u2 *glut) {
-    const u4 *src = (const u4 *)glut;
-    u4 *dst = (u4 *)lut;
-    constexpr uint32_t N = QW_LUT_BYTES / 16;
-    const uint32_t rot = blockIdx.x * 320u, lane = threadIdx.x & 63, w64 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64;
-#pragma unroll
-    for (uint32_t it = 0; it < qw_lut_copy_loads<NW>(); it++) {
-        uint32_t i = w64 + it * 64 * NW;
-        if (i >= N) i -= 64 * NW;
-        const uint32_t j = (i + rot) & (N - 1);
-        qw_load_to_lds(src + j + lane, dst + j);
-    }
-}
-// Likewise the activations of qw_stage_x_issue for up to MAXN / 32 values a row: a fixed number of loads in every wave,
-// and the rows past nb repeat row nb - 1 instead of holding zeros (they feed matrix-core output rows that nobody reads).
-template <uint32_t NW, uint32_t MAXN> constexpr uint32_t qw_stage_x_loads() { return (MAXN + 64 * NW - 1) / (64 * NW); }
-template <uint32_t NW, uint32_t MAXN> __device__ __forceinline__ void qw_stage_x_issue_n(u4 *xf, const uint16_t *x, uint32_t xstride, uint32_t K, uint32_t nb) {
-    const uint32_t n = (K >> 3) * 16, rot = (blockIdx.x * 320u) % n, lane = threadIdx.x & 63, w64 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)) * 64;
-    const uint32_t last = nb ? nb - 1 : 0;
-#pragma unroll
-    for (uint32_t it = 0; it < qw_stage_x_loads<NW, MAXN>(); it++) {
-        uint32_t i0 = w64 + it * 64 * NW;
-        while (i0 >= n) i0 -= n;
-        const uint32_t base = i0 + rot < n ? i0 + rot : i0 + rot - n, i = base + lane, c = i >> 4, m = i & 15;
-        qw_load_to_lds((const u4 *)(x + (size_t)(m < nb ? m : last) * xstride + 8 * c), xf + base);
     }
 }
 __device__ __forceinline__ void qw_lut_copy(u2 *lut, const u2 *glut) {

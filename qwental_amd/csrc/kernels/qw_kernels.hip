@@ -686,33 +686,21 @@ __device__ __forceinline__ void select_tokens(const float *logits, uint32_t E, u
 // it: more than 64 keys reach T0 (many equal logits) and the caller falls back to select_tokens.
 // ws: 144 dwords of LDS scratch per token for this wave. need_w: also the gating weights (softmax over the picked
 // logits in rank order, sigmoid of the shared-expert logit).
-// issued(): called once the loads of the logits are issued (the place for the caller's own prefetches: loads return in
-// the order of issue, and the logits are needed first); it issues at least NDMA vector memory loads in every wave, and
-// the keys are used as soon as no more than NDMA loads of the wave are outstanding.
-template <int PER, int T, uint32_t NDMA, class H>
+// issued(): called once the loads of the logits are issued (work that needs no memory: with loads straight into LDS
+// outstanding beside them the compiler would wait for everything at the first use of a key).
+template <int PER, int T, class H>
 __device__ __forceinline__ uint32_t select_tokens_ranked(const float *logits, uint32_t E, uint32_t K, const uint32_t (&tok)[T], const bool (&on)[T], float *w, uint32_t *ids, uint32_t *ws,
                                                         uint32_t lane, bool need_w, H issued) {
     uint32_t k[T][PER], M[T], T0[T], c[T], pos[T][PER];
-    // The loads of the logits are written out, and so is the wait for them: issued() asks for NDMA more loads (straight
-    // into LDS, wanted much later), the loads of a wave return in the order of issue, and the compiler waits for
-    // everything outstanding when loads into registers and loads into LDS are in flight together. Nothing may read k
-    // between here and the wait (the registers are not valid yet).
 #pragma unroll
-    for (int t = 0; t < T; t++) {
-        const float *p = logits + (size_t)tok[t] * (E + 1) + lane; // (a wave reads 256 contiguous bytes a load)
+    for (int t = 0; t < T; t++)
 #pragma unroll
-        for (int j = 0; j < PER; j++) asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(k[t][j]) : "v"(p), "n"(j * 256) : "memory");
-    }
+        for (int j = 0; j < PER; j++) k[t][j] = __builtin_bit_cast(uint32_t, logits[(size_t)tok[t] * (E + 1) + j * 64 + lane]); // (a wave reads 256 contiguous bytes)
     QW_DSTAMP(12);
     QW_SSTAMP(3);
     issued();
     QW_DSTAMP(13);
     QW_SSTAMP(4);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-#pragma unroll
-    for (int t = 0; t < T; t++)
-#pragma unroll
-        for (int j = 0; j < PER; j++) asm volatile("" : "+v"(k[t][j])); // (every use of k follows the wait)
 #pragma unroll
     for (int t = 0; t < T; t++) {
         M[t] = 0;
@@ -852,20 +840,22 @@ __device__ __forceinline__ bool qw_select_fast_e(uint32_t E) { return E == 64 ||
 // The whole selection by one workgroup (a multiple of 64 threads, at least nbr * topk of them). lgs: LDS scratch, 1024
 // floats per wave (288 are used when E is 64 * {1, 2, 4, 8, 16}). c is complete for every thread on return.
 // store: this workgroup writes the record; need_w: it wants the gating weights in s.w (store implies it).
-// issued(): runs once in every wave, behind the wave's loads of its first tokens' logits when it has tokens; NDMA as in
-// select_tokens_ranked.
-template <uint32_t NDMA = 0, class H>
-__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H issued, bool need_w = false) {
+// NSTAGE: the workgroup's last NSTAGE waves take no tokens; each of them runs stage(part, NSTAGE) instead, the caller's
+// copies into LDS (table, activations). A wave that asks for 128 KB of such copies sits in the issue of those loads for
+// 2 to 3 us - the copies go at the rate of the unit's path into LDS - so a wave that did both made its keys that much
+// later; the waves with tokens ask for nothing but their logits.
+template <uint32_t NSTAGE = 0, class H>
+__device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scratch &s, qw_sel_cache &c, float *lgs, bool store, H stage, bool need_w = false) {
     need_w = need_w || store;
     const uint32_t tid = threadIdx.x, nth = blockDim.x, wave = qw_wave(), lane = qw_lane(), nwv = nth >> 6;
     const uint32_t E = a.E, K = a.topk, gnb = a.gnb, GU = gnb * K, UM = a.nbr * K;
     const bool fast = qw_select_fast_e(E);
+    const uint32_t tw = nwv - NSTAGE; // the waves that take tokens
     QW_SDEP(E + K + gnb + a.nbr);
     QW_SSTAMP(1);
     // nothing the token loop writes is cleared here (rows of w past the batch only), so no barrier separates the two,
-    // and with the fast form the clearing waits until the logits have been asked for
-    auto issued_clear = [&] {
-        issued();
+    // and a wave clears its part once it has asked for what it reads
+    auto clear = [&] {
         for (uint32_t i = tid; i < E; i += nth) s.first[i] = 0xffffffffu;
         for (uint32_t i = tid; i < GU; i += nth) c.ue[i] = 0, c.mask[i] = 0;
         for (uint32_t i = tid; i < GU * gnb / 4; i += nth) ((uint32_t *)c.slot)[i] = 0;
@@ -874,7 +864,11 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         QW_DSTAMP(11);
         QW_SSTAMP(2);
     };
-    if (fast) { // a first pass of straight-line code: a wave takes one token, or two when there are more tokens than waves (lgs gives a wave 288 dwords)
+    if (NSTAGE != 0 && wave >= tw) { // (uniform)
+        stage(wave - tw, NSTAGE);
+        QW_SSTAMP(4);
+        clear();
+    } else if (fast) { // a wave takes one token, or two when there are more tokens than such waves (lgs gives a wave 288 dwords)
         uint32_t *ws = (uint32_t *)lgs + 288 * wave;
         const uint32_t trot = a.nbr ? blockIdx.x % a.nbr : 0; // the workgroups of a launch read the tokens' logits in different orders
         auto rot = [&](uint32_t tt) { return tt + trot < a.nbr ? tt + trot : tt + trot - a.nbr; };
@@ -890,30 +884,30 @@ __device__ __forceinline__ void select_all(const qwk_select_args &a, qw_sel_scra
         };
         if (wave < a.nbr) {
             const uint32_t tt = wave;
-            const bool two = pairs && tt + nwv < a.nbr;
-            const uint32_t tk[2] = {rot(tt), two ? rot(tt + nwv) : rot(tt)};
+            const bool two = pairs && tt + tw < a.nbr;
+            const uint32_t tk[2] = {rot(tt), two ? rot(tt + tw) : rot(tt)};
             const bool on2[2] = {true, two}, on1[1] = {true};
             const uint32_t t1[1] = {tk[0]};
             uint32_t fail;
             switch (E) {
-            case 64: fail = two ? select_tokens_ranked<1, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<1, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
-            case 128: fail = two ? select_tokens_ranked<2, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<2, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
-            case 256: fail = two ? select_tokens_ranked<4, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<4, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
-            case 512: fail = two ? select_tokens_ranked<8, 2, NDMA>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, issued_clear) : select_tokens_ranked<8, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
-            default: fail = select_tokens_ranked<16, 1, NDMA>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, issued_clear); break;
+            case 64: fail = two ? select_tokens_ranked<1, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, clear) : select_tokens_ranked<1, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, clear); break;
+            case 128: fail = two ? select_tokens_ranked<2, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, clear) : select_tokens_ranked<2, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, clear); break;
+            case 256: fail = two ? select_tokens_ranked<4, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, clear) : select_tokens_ranked<4, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, clear); break;
+            case 512: fail = two ? select_tokens_ranked<8, 2>(a.logits, E, K, tk, on2, s.w, s.ids, ws, lane, need_w, clear) : select_tokens_ranked<8, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, clear); break;
+            default: fail = select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, clear); break;
             }
             for (uint32_t i = 0; i < 2; i++) // more than 64 keys tie at the bound
                 if (((fail >> i) & 1) && (i == 0 || two)) slow(tk[i]);
-        } else issued_clear();
-        // tokens that the first pass does not reach (more than the waves when a lane holds sixteen keys, more than twice the waves otherwise)
-        for (uint32_t tt = wave + (pairs ? 2 : 1) * nwv; tt < a.nbr; tt += nwv) {
+        } else clear();
+        // tokens that the first pass does not reach (more than such waves when a lane holds sixteen keys, more than twice as many otherwise)
+        for (uint32_t tt = wave + (pairs ? 2 : 1) * tw; tt < a.nbr; tt += tw) {
             const uint32_t t1[1] = {rot(tt)};
             const bool on1[1] = {true};
-            if (pairs || select_tokens_ranked<16, 1, 0>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, [] {})) slow(t1[0]);
+            if (pairs || select_tokens_ranked<16, 1>(a.logits, E, K, t1, on1, s.w, s.ids, ws, lane, need_w, [] {})) slow(t1[0]);
         }
     } else {
-        issued_clear();
-        for (uint32_t t = wave; t < a.nbr; t += nwv) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
+        clear();
+        for (uint32_t t = wave; t < a.nbr; t += tw) select_token_any(a.logits + (size_t)t * (E + 1), lgs + (size_t)wave * 1024, E, K, t, s.w, s.ids, lane);
     }
     QW_DSTAMP(15);
     QW_SSTAMP(9);
@@ -980,7 +974,7 @@ extern "C" __global__ __launch_bounds__(1024) void qwk_select(qwk_select_args a)
     __shared__ qw_sel_scratch s;
     __shared__ qw_sel_cache c;
     __shared__ float lgs[16 * 1024];
-    select_all(a, s, c, lgs, true, [] {});
+    select_all(a, s, c, lgs, true, [](uint32_t, uint32_t) {});
 }
 #endif
 
@@ -1083,16 +1077,10 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
             // their place (they follow in ready()).
             constexpr bool lutp = qw_has_lut(FGU) || qw_has_lut(FSG);
             const bool early = a.D * 2 + (QW_WG_GU / 64) * 288 / 4 <= QW_XF_MAXK * 2;
-            // (the table and the activations are asked for behind the logits, a fixed number of loads a wave, so that the
-            // selection goes on as soon as the logits are there; when the activations have to wait for the scratch's place,
-            // the table is copied twice to keep that number: one selection per kernel instead of two)
-            constexpr uint32_t NWV = QW_WG_GU / 64, XN = QW_XF_MAXK * 2 - NWV * 288 / 4, NT = qw_lut_copy_loads<NWV>(), NX = qw_stage_x_loads<NWV, XN>();
-            static_assert(NT == NX, "two copies of equal length");
-            // (a kernel without the table counts nothing: its selection waits for whatever it has asked for)
-            select_all<lutp ? NT + NX : 0>(sa, *ss, *sc, (float *)(early ? xf + a.D * 2 : xf), blockIdx.x == 0, [&] {
-                if (lutp) qw_lut_copy_issue_n<NWV>(lut, (const u2 *)a.glut);
-                if (early) qw_stage_x_issue_n<NWV, XN>(xf, a.x, a.D, a.D, a.nbr);
-                else if (lutp) qw_lut_copy_issue_n<NWV>(lut, (const u2 *)a.glut);
+            // (four of the twelve waves ask for the table and the activations, the others make the selection meanwhile)
+            select_all<4>(sa, *ss, *sc, (float *)(early ? xf + a.D * 2 : xf), blockIdx.x == 0, [&](uint32_t part, uint32_t nparts) {
+                if (lutp) qw_lut_copy_issue(lut, (const u2 *)a.glut, part, nparts);
+                if (early) qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr, part, nparts);
             }, all_w);
             qw_lds_arrive();
             __syncthreads();
@@ -1101,7 +1089,7 @@ __device__ __forceinline__ void gu_body(const qwk_gu_args &a, u2 *lut, u4 *xf, q
             tabled = true;
         } else { // other expert counts need 1024 floats of scratch per wave: everything lies where x is staged afterwards
             qw_sel_scratch &so = *(qw_sel_scratch *)xf;
-            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [] {}, all_w);
+            select_all(sa, so, *sc, (float *)(xf + (sizeof(qw_sel_scratch) + 15) / 16), blockIdx.x == 0, [](uint32_t, uint32_t) {}, all_w);
             if (all_w) { // (the caller reads the weights from ss)
                 for (uint32_t i = threadIdx.x; i < a.gnb * (a.topk + 1); i += blockDim.x) ss->w[i] = so.w[i];
                 __syncthreads();
@@ -2696,7 +2684,10 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
     const uint32_t tid = threadIdx.x, l32 = tid & 31, i = blockIdx.x * 8 + (tid >> 5), t0 = blockIdx.y * QW_HC_TG;
     const uint32_t nt = a.nb - t0 < QW_HC_TG ? a.nb - t0 : QW_HC_TG;
     const size_t HCD = (size_t)QW_HC * a.D;
-    // the weights first: their round trip overlaps what follows
+    // Everything a thread will read is asked for here and without conditions (a lane without a token or a thread without
+    // an element reads what element 0 would: valid memory, the value unused), so that the launch is one memory round
+    // trip. Loads under conditions were a round trip each: the weights and h, out, the inject sums, the sums of squares,
+    // the mix_down sums - five in a row.
     uint32_t u[QW_HC][5];
 #pragma unroll
     for (uint32_t q = 0; q < QW_HC; q++) {
@@ -2704,18 +2695,41 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
 #pragma unroll
         for (int k = 0; k < 5; k++) u[q][k] = wr[k];
     }
-    // lane l < 4 QW_HC_TG of a group owns token l / 4 of the workgroup's and the stream qw_sum4 leaves with it: its h, out
-    // and norm weight are asked for now as well
+    // lane l < 4 QW_HC_TG of a group owns token l / 4 of the workgroup's and the stream qw_sum4 leaves with it
     const uint32_t ts = l32 / QW_HC, sq = 2 * (l32 & 1) + ((l32 >> 1) & 1);
     const bool mine = ts < nt;
+    const uint32_t tsc = mine ? ts : 0;
     const float wn = a.w[(size_t)sq * a.D + i];
-    float hv = 0, ov = 0;
-    if (mine) {
-        hv = a.h[(t0 + ts) * HCD + (size_t)sq * a.D + i];
-        if (a.apply) ov = qw_h2f(a.out[(size_t)(t0 + ts) * a.D + i]);
+    const float hv = a.h[(t0 + tsc) * HCD + (size_t)sq * a.D + i];
+    // (out is not read unless it is applied: it may never have been written, nor the inject sums)
+    const uint16_t ovr = *(a.apply ? a.out + (size_t)(t0 + tsc) * a.D + i : (const uint16_t *)a.h);
+    const bool hasj = tid < nt * QW_HC; // this thread makes the values of (token jt / HC, stream jt % HC)
+    const uint32_t jt = hasj ? tid : 0;
+    const float *injp = a.apply ? a.inj + (t0 + jt / QW_HC) * QW_HC * QW_HC : a.pd;
+    float iq[QW_HC];
+#pragma unroll
+    for (uint32_t q = 0; q < QW_HC; q++) iq[q] = injp[q * QW_HC + jt % QW_HC];
+    // the middle step's inputs (hc_mid's arithmetic below, element tid + 256 e): sums of squares, mix_down sums, inject sums
+    constexpr uint32_t EPT = (QW_HC_TG * QW_HC_LR + 255) / 256;
+    const float *pd = a.pd + (size_t)t0 * QW_HC * QW_HC_PDS;
+    float sq_raw = 0, ij_raw = 0, p[EPT][QW_HC];
+    if (!GIVEN) {
+        sq_raw = pd[jt * QW_HC_PDS + QW_HC_LR + QW_HC];
+        const uint32_t ji = tid < nt * QW_HC * QW_HC ? tid : 0; // (t, s, q)
+        ij_raw = pd[(ji / QW_HC) * QW_HC_PDS + QW_HC_LR + ji % QW_HC];
+#pragma unroll
+        for (uint32_t e = 0; e < EPT; e++) {
+            const uint32_t j = tid + e * 256, jc = j < nt * QW_HC_LR ? j : 0, t = jc / QW_HC_LR, r = jc % QW_HC_LR;
+#pragma unroll
+            for (uint32_t q = 0; q < QW_HC; q++) p[e][q] = pd[(t * QW_HC + q) * QW_HC_PDS + r];
+        }
     }
-    // (before the middle step: its loads then share that step's round trip)
-    if (tid < nt * QW_HC) js[tid / QW_HC][tid % QW_HC] = a.apply ? hc_coef(a.inj + (t0 + tid / QW_HC) * QW_HC * QW_HC, tid % QW_HC) : 0.0f;
+    if (hasj) {
+        float t = 0;
+#pragma unroll
+        for (uint32_t q = 0; q < QW_HC; q++) t += iq[q];
+        js[tid / QW_HC][tid % QW_HC] = a.apply ? 2.0f / (1.0f + expf(-t / QW_HC)) : 0.0f; // hc_coef
+    }
     if (GIVEN) {
         for (uint32_t j0 = tid; j0 < nt * QW_HC_LR; j0 += 8 * blockDim.x) { // eight loads in flight a thread
             float v[8];
@@ -2726,10 +2740,24 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
                 if (j0 + e * blockDim.x < nt * QW_HC_LR) (&sx[0][0])[j0 + e * blockDim.x] = v[e];
         }
         if (tid < nt * QW_HC) rs[tid / QW_HC][tid % QW_HC] = a.rs[t0 * QW_HC + tid];
-    } else {
-        hc_mid(a, t0, nt, &rs[0][0], &sx[0][0], blockIdx.x == 0 && a.want_inj ? a.injo : nullptr);
+    } else { // hc_mid for the workgroup's tokens, on the values read above
+        if (hasj) (&rs[0][0])[tid] = rsqrtf(sq_raw / (float)a.D + 1e-6f);
+        __syncthreads();
+#pragma unroll
+        for (uint32_t e = 0; e < EPT; e++) {
+            const uint32_t j = tid + e * 256, t = j / QW_HC_LR;
+            if (j < nt * QW_HC_LR) {
+                float d = 0;
+#pragma unroll
+                for (uint32_t q = 0; q < QW_HC; q++) d = fmaf(rs[t][q], p[e][q], d);
+                d /= QW_HC;
+                (&sx[0][0])[j] = d / (1.0f + __expf(-d));
+            }
+        }
+        if (blockIdx.x == 0 && a.want_inj && tid < nt * QW_HC * QW_HC) a.injo[t0 * QW_HC * QW_HC + tid] = (&rs[0][0])[tid / QW_HC] * ij_raw;
     }
     __syncthreads();
+    const float ov = qw_h2f(ovr);
     float v[QW_HC][10];
 #pragma unroll
     for (uint32_t q = 0; q < QW_HC; q++)
