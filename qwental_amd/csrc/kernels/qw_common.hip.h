@@ -177,6 +177,7 @@ __device__ __forceinline__ h8 qw_q8_cvt(u2 q) {
 // implies that all but the N youngest loads have returned. A store reads its data registers when it is issued, and it
 // has completed when the kernel ends, which is when its readers start. INVARIANT for every user: what is stored this way
 // is never read back from memory inside the same kernel (the compiler would not wait for the store before such a read).
+// (the default cache policy: the same stores marked nontemporal or of device scope made the step 1.2 % and 0.4 % slower)
 __device__ __forceinline__ void qw_store_u16(uint16_t *p, uint16_t v) { asm volatile("global_store_short %0, %1, off" : : "v"(p), "v"((uint32_t)v) : "memory"); }
 __device__ __forceinline__ void qw_store_f32(float *p, float v) { asm volatile("global_store_dword %0, %1, off" : : "v"(p), "v"(v) : "memory"); }
 
