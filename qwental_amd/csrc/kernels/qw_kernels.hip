@@ -1582,20 +1582,38 @@ __device__ __forceinline__ f4 dnc_tile(const qwk_dn_args &a, const u2 *lut, cons
 template <int F, int CH, int FSD, int CHSD>
 __device__ __forceinline__ void dnc_body(const qwk_dn_args &a, u2 *lut, float *part /* [QW_DNC_MAXNB][topk + 1][16] */, float *wl /* [QW_DNC_MAXNB][topk + 1] */, qw_sel_cache *sc) {
     const uint32_t K = a.topk, gnb = a.gnb, tpe = a.D / 16, tile = blockIdx.x, lane = qw_lane(), n = lane & 15, kg = lane >> 4, nwv = blockDim.x >> 6;
+    // The table through registers, asked for first and stored behind the record (published by the barrier of ready()): a
+    // copy straight into LDS kept every wave in the issue of its loads for more than a microsecond, between the record and
+    // the first weights (which need the record).
+    constexpr bool TAB = qw_has_lut(F) || qw_has_lut(FSD);
+    constexpr uint32_t TPER = TAB ? (QW_LUT_BYTES / 16 + QW_WG_DN - 1) / QW_WG_DN : 0;
+    u4 tabv[TPER ? TPER : 1];
+    uint32_t tat[TPER ? TPER : 1];
+    if constexpr (TAB) { // (every workgroup starts at another place of the table; the last piece of some threads repeats an earlier one)
+#pragma unroll
+        for (uint32_t it = 0; it < TPER; it++) {
+            uint32_t i = threadIdx.x + it * QW_WG_DN;
+            if (i >= QW_LUT_BYTES / 16) i -= QW_WG_DN;
+            tat[it] = (i + blockIdx.x * 320u) & (QW_LUT_BYTES / 16 - 1);
+            tabv[it] = ((const u4 *)a.glut)[tat[it]];
+        }
+    }
     qw_sel_load(*sc, a.sel, K, gnb);
     const float *wg = (const float *)(a.sel + QW_SEL_OFF_W(gnb, K));
     for (uint32_t i = threadIdx.x; i < a.nbr * (K + 1); i += blockDim.x) wl[i] = wg[i];
-    if (qw_has_lut(F) || qw_has_lut(FSD)) qw_lut_copy_issue(lut, (const u2 *)a.glut); // awaited in ready()
     if (F == QW_F_PACKED_NL || FSD == QW_F_PACKED_NL) qw_kq_tab_build((uint32_t *)lut); // the byte table of the 4-bit codebook instead
+    if constexpr (TAB) {
+#pragma unroll
+        for (uint32_t it = 0; it < TPER; it++) ((u4 *)lut)[tat[it]] = tabv[it];
+    }
     __syncthreads();
     uint32_t U = (uint32_t)__builtin_amdgcn_readfirstlane((int)sc->U);
     if (U > gnb * K) U = gnb * K;
     const uint32_t nsh = (FSD != 0 && a.Wsd) ? 1 : 0, V = nsh + U;
     bool staged = false;
-    auto ready = [&] { // once per wave, behind its first weight loads: the table has landed, for every wave
+    auto ready = [&] { // once per wave, behind its first weight loads
         if (staged) return;
         staged = true;
-        qw_lds_arrive();
         __syncthreads();
     };
     for (uint32_t v = qw_wave(); v < V; v += nwv) {
