@@ -43,6 +43,13 @@ __shared__ uint32_t qw_sst[12 * 16];
 #define QW_SDEP(v) do {} while (0)
 #define QW_SST_FLUSH() do {} while (0)
 #endif
+#if defined(QW_STAMPS) && QW_STAMPS == 4 // steps of the front launch only
+#undef QW_DSTAMP
+#define QW_DSTAMP(k) do {} while (0)
+#define QW_PSTAMP(k) do { if (threadIdx.x == 0 && qw_stamp_ptr) qw_stamp_ptr[512 + 16 * blockIdx.x + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define QW_PSTAMP(k) do {} while (0)
+#endif
 #ifdef QW_STAMPS
 #define QW_WG_END_STAMP(k) do { __syncthreads(); QW_DSTAMP(k); } while (0)
 #else
@@ -1262,6 +1269,7 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
     const uint32_t cpr = a.D / (C::BLK_K * CH), tpw = nwv / cpr; // tiles per workgroup (the host checks cpr <= waves)
     const uint32_t tile = (blockIdx.x - pa.nrouter) * tpw + wave / cpr, ci = wave % cpr;
     const bool on = wave < tpw * cpr && tile < a.I / 8;
+    QW_PSTAMP(1);
     C c;
     if (on) {
         if constexpr (F == QW_F_PACKED) c.load(a.Wg + (size_t)tile * a.rowbytes + (size_t)ci * CH * C::BLK_B, lane);
@@ -1285,18 +1293,24 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
         }
     } else {
         // the table and the activations behind the weights, all awaited once: one memory round trip before the barrier
+        QW_PSTAMP(2);
         if (qw_has_lut(F)) qw_lut_copy_issue(lut, (const u2 *)a.glut);
         qw_stage_x_issue(xf, a.x, a.D, a.D, a.nbr);
+        QW_PSTAMP(3);
         qw_lds_arrive();
+        QW_PSTAMP(4);
         __syncthreads();
+        QW_PSTAMP(5);
         if (on) {
             c.transpose();
             const qw_afrag_lds af = {xf, n};
             c.mac_lean(lut, af, ci * CH * C::BLK_K, kg, acc);
             part[wave * 64 + lane] = acc;
         }
+        QW_PSTAMP(6);
     }
     __syncthreads();
+    QW_PSTAMP(7);
     if (!on || ci != 0) return;
     acc = part[wave * 64 + lane];
     for (uint32_t i = 1; i < cpr; i++) acc += part[(wave + i) * 64 + lane]; // chunk order
@@ -1312,11 +1326,13 @@ template <int F, int CH> __device__ __forceinline__ void pre_shared(const qwk_pr
             a.H[o + a.hplane] = __builtin_bit_cast(uint16_t, lo);
         }
     }
+    QW_PSTAMP(8);
 }
 #define QW_PRE(WF, F, CH, NAME)                                                                          \
     extern "C" __global__ __launch_bounds__(QW_WG) void NAME(qwk_pre_args a) {                           \
         __shared__ struct { u2 lut[qw_has_lut(F) ? QW_LUT_ENTRIES : 1]; u4 xf[QW_XF_MAXK * 2]; f4 part[(QW_WG / 64) * 64]; } L; \
         QW_DSTAMP(3);                                                                                   \
+        QW_PSTAMP(0);                                                                                   \
         if (blockIdx.x < a.nrouter) {                                                                   \
             if (WF == 1) pre_router_mfma(a.r, L.xf, L.part);                                            \
             else pre_router<WF>(a, L.xf);                                                               \
