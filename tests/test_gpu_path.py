@@ -277,6 +277,62 @@ def test_selection_close_values_and_every_expert_count(gpu, oracle, E):
     assert list(ids[3]) == [E // 2, E // 2 + 1, E // 2 + 2] + list(range(7))
 
 
+@pytest.mark.parametrize("E,nb", [(64, 16), (512, 16), (1024, 16), (512, 11), (1024, 9), (256, 2)])
+def test_selection_inside_the_gate_up_launch_on_crafted_logits(gpu, oracle, E, nb):
+    """The gate/up launch makes the selection itself: eight of its twelve waves take the tokens (two a wave above eight
+    tokens; with 1024 experts one a wave and a second pass), the other four copy the table and the activations. One-hot
+    activations make the router's logits equal to chosen binary16 values, so the cases of the stand-alone selection's
+    tests reach that code too: more than 64 equal keys at the bound (the repeated-maximum fallback), every value eight
+    times, one-ulp ramps up and down, close negative values, zeros of both signs. The record must be the oracle's."""
+    D, I, K = 512, 256, 10
+    rng = np.random.default_rng(900 + E + nb)
+    m = synth.moe_layer(rng, D, I, E)  # every expert's rows: any of them may be picked
+    m["topk"] = K
+    cols = rng.normal(0, 1, (nb, E)).astype(np.float16)
+    n = min(E, 200)
+
+    def put(t, v):
+        if t < nb:
+            cols[t] = np.asarray(v, np.float32).astype(np.float16)
+
+    r = np.full(E, 0.5, np.float32)
+    r[E // 2:E // 2 + 3] = 0.75
+    put(0, r)                                                                        # all equal but three
+    put(1, np.repeat(rng.normal(0, 1, E // 8).astype(np.float16).astype(np.float32), 8))  # every value eight times
+    up = rng.normal(0, 0.1, E).astype(np.float32)
+    up[:n] = 1.0 + np.arange(n) * 2.0 ** -10                                         # ascending by one binary16 ulp
+    put(2, up)
+    dn = rng.normal(0, 0.1, E).astype(np.float32)
+    dn[:n] = 1.0 + np.arange(n)[::-1] * 2.0 ** -10                                   # descending
+    put(3, dn)
+    put(4, -2.0 - rng.permutation(E).astype(np.float32) * 2.0 ** -9 * (1024 // E))   # all negative, all close, all distinct
+    z = np.zeros(E, np.float32)
+    z[1::2] = -0.0
+    z[[E // 3, E // 3 + 1]] = 2.0 ** -14
+    put(5, z)                                                                        # zeros of both signs and two small values
+    assert np.array_equal(cols.astype(np.float32).astype(np.float16), cols)
+    m["Wr"][:, :nb] = cols.T
+    x = np.zeros((nb, D), np.float16)
+    x[np.arange(nb), np.arange(nb)] = 1.0                                           # logit[t][e] = Wr[e][t]
+    path = q.Path(gpu, D, I, E, K, 16)
+    dl = DeviceLayer(gpu, m)
+    gpu.profile(True)
+    out, lg, selraw, _ = run_moe(gpu, path, dl, x, nb)
+    names = [nm for nm, _ in gpu.profile_entries()]
+    gpu.profile(False)
+    assert "qwk_select" not in names and any(nm.startswith("qwk_gu_") for nm in names), names
+    assert np.array_equal(lg[:, :E], cols.astype(np.float32))
+    gnb = 8 if nb <= 8 else 16
+    _check_sel(oracle.Sel(selraw, gnb, K), oracle.select(lg, K, gnb), nb, K)
+    ids = oracle.topk_ids(lg, K)
+    assert list(ids[0]) == [E // 2, E // 2 + 1, E // 2 + 2] + list(range(7))
+    if nb > 3:
+        assert list(ids[2]) == list(range(n - 1, n - 11, -1)) and list(ids[3]) == list(range(10))
+    assert maxrel(out, oracle.moe_layer_f64(m, lg, x)) <= TOL
+    path.close()
+    dl.free()
+
+
 # ---------------------------------------------------------------- one MoE layer
 @pytest.mark.parametrize("nb,fmt", [(1, 21), (3, 21), (8, 21), (16, 21), (8, 8), (16, 8)])
 def test_moe_layer_parity(gpu, oracle, nb, fmt):
