@@ -50,6 +50,13 @@ __shared__ uint32_t qw_sst[12 * 16];
 #else
 #define QW_PSTAMP(k) do {} while (0)
 #endif
+#if defined(QW_STAMPS) && QW_STAMPS == 5 // steps of the hyper-connection's launches (workgroups 0 .. 255 of each)
+#undef QW_DSTAMP
+#define QW_DSTAMP(k) do {} while (0)
+#define QW_HSTAMP(k) do { const uint32_t wg_ = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z); if (threadIdx.x == 0 && qw_stamp_ptr && wg_ < 256) qw_stamp_ptr[512 + 16 * wg_ + (k)] = (uint32_t)__builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define QW_HSTAMP(k) do {} while (0)
+#endif
 #ifdef QW_STAMPS
 #define QW_WG_END_STAMP(k) do { __syncthreads(); QW_DSTAMP(k); } while (0)
 #else
@@ -2591,6 +2598,7 @@ template <int W> __device__ __forceinline__ float qw_sum4(float d0, float d1, fl
 template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_args &a, float (*part)[QW_HC_TG][17]) {
     const uint32_t rb = blockIdx.x, s = blockIdx.y, t0 = blockIdx.z * QW_HC_TG, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, nwv = blockDim.x >> 6;
     const uint32_t nt = a.nb - t0 < QW_HC_TG ? a.nb - t0 : QW_HC_TG;
+    QW_HSTAMP(0);
     const bool is_inj = rb == QW_HC_LR / R;
     const uint32_t nrow = is_inj ? QW_HC : R; // rows of this block (uniform)
     const size_t HCD = (size_t)QW_HC * a.D, c0 = (size_t)s * a.D + 8 * tid;
@@ -2608,6 +2616,7 @@ template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_
             if (a.apply) ou[tt] = *(const u4 *)(a.out + (size_t)(t0 + tt) * a.D + 8 * tid); // not read otherwise: it may never have been written
         }
     }
+    QW_HSTAMP(1);
 #pragma unroll
     for (uint32_t tt = 0; tt < QW_HC_TG; tt++) {
         if (tt >= nt) break;
@@ -2624,6 +2633,7 @@ template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_
 #pragma unroll
         for (int k = 0; k < 8; k++) ss = fmaf(v[k], v[k], ss), x[k] = v[k] * (k < 4 ? w0[k] : w1[k - 4]);
         ss = qw_wave_sum(ss);
+        if (tt == 0) QW_HSTAMP(2);
         if (lane == 0) part[wave][tt][16] = ss;
 #pragma unroll
         for (uint32_t r0 = 0; r0 < R; r0 += 4) {
@@ -2642,7 +2652,9 @@ template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_
             if (lane < 4) part[wave][tt][r0 + 2 * (lane & 1) + (lane >> 1)] = f;
         }
     }
+    QW_HSTAMP(3);
     __syncthreads();
+    QW_HSTAMP(4);
     for (uint32_t j = tid; j < nt * 17; j += blockDim.x) {
         const uint32_t tt = j / 17, r = j % 17;
         if (r < 16 && r >= nrow) continue;
@@ -2652,6 +2664,7 @@ template <uint32_t R> __device__ __forceinline__ void hc_down_body(const qwk_hc_
         if (r < 16) pd[(is_inj ? QW_HC_LR : rb * R) + r] = sum;
         else if (rb == 0) pd[QW_HC_LR + QW_HC] = sum;
     }
+    QW_HSTAMP(5);
 }
 #if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(512) void qwk_hc_down_r4(qwk_hc_args a) {
@@ -2718,6 +2731,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
     const uint32_t tid = threadIdx.x, l32 = tid & 31, i = blockIdx.x * 8 + (tid >> 5), t0 = blockIdx.y * QW_HC_TG;
     const uint32_t nt = a.nb - t0 < QW_HC_TG ? a.nb - t0 : QW_HC_TG;
     const size_t HCD = (size_t)QW_HC * a.D;
+    QW_HSTAMP(8);
     // Everything a thread will read is asked for here and without conditions (a lane without a token or a thread without
     // an element reads what element 0 would: valid memory, the value unused), so that the launch is one memory round
     // trip. Loads under conditions were a round trip each: the weights and h, out, the inject sums, the sums of squares,
@@ -2758,6 +2772,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
             for (uint32_t q = 0; q < QW_HC; q++) p[e][q] = pd[(t * QW_HC + q) * QW_HC_PDS + r];
         }
     }
+    QW_HSTAMP(9);
     if (hasj) {
         float t = 0;
 #pragma unroll
@@ -2777,6 +2792,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
     } else { // hc_mid for the workgroup's tokens, on the values read above
         if (hasj) (&rs[0][0])[tid] = rsqrtf(sq_raw / (float)a.D + 1e-6f);
         __syncthreads();
+        QW_HSTAMP(10);
 #pragma unroll
         for (uint32_t e = 0; e < EPT; e++) {
             const uint32_t j = tid + e * 256, t = j / QW_HC_LR;
@@ -2791,6 +2807,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
         if (blockIdx.x == 0 && a.want_inj && tid < nt * QW_HC * QW_HC) a.injo[t0 * QW_HC * QW_HC + tid] = (&rs[0][0])[tid / QW_HC] * ij_raw;
     }
     __syncthreads();
+    QW_HSTAMP(11);
     const float ov = qw_h2f(ovr);
     float v[QW_HC][10];
 #pragma unroll
@@ -2814,6 +2831,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
         const float f = qw_sum4<32>(d[0], d[1], d[2], d[3], l32); // this lane's stream, summed over the group
         uv = ts == t ? f : uv;
     }
+    QW_HSTAMP(12);
     // the gates and the mix over the streams: the four streams of a token are neighbouring lanes
     float m = 0;
     if (mine) {
@@ -2827,6 +2845,7 @@ template <bool GIVEN> __device__ __forceinline__ void hc_up_body(const qwk_hc_ar
     m += __shfl_xor(m, 1);
     m += __shfl_xor(m, 2);
     if (mine && sq == 0) a.x[(size_t)(t0 + ts) * a.D + i] = qw_f2h(m / QW_HC);
+    QW_HSTAMP(13);
 }
 #if QW_IN_PART(5)
 extern "C" __global__ __launch_bounds__(256) void qwk_hc_up(qwk_hc_args a) { hc_up_body<false>(a); }
